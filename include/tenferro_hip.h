@@ -176,8 +176,8 @@ int32_t tfh_subscripts_n_inputs(const tfh_subscripts* s);
 int32_t tfh_subscripts_input_rank(const tfh_subscripts* s, int32_t i);
 /* Copies the labels of input i (or of the output when i == -1) into out[cap]; returns the rank. */
 int32_t tfh_subscripts_labels(const tfh_subscripts* s, int32_t i, uint32_t* out, int32_t cap);
-/* Pairs implied by parentheses (empty when the notation had none).  Returns the pair count. */
-int32_t tfh_subscripts_pairs(const tfh_subscripts* s, int32_t* out_pairs, int32_t cap_pairs);
+/* The parenthesisation as written, operands by index: "ij,(jk,kl)->il" gives "0,(1,2)". */
+int32_t tfh_subscripts_nesting(const tfh_subscripts* s, char* buf, size_t cap);
 
 /* ContractionTree::optimize(subscripts, shapes) (:303-318): minimum total operation count;
  * exhaustive over subsets up to 12 operands, greedy beyond.  If the subscripts carry

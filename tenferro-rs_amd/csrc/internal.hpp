@@ -1,0 +1,129 @@
+// internal.hpp -- types shared by the host side of the backend (not part of the C ABI).
+#pragma once
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../include/tenferro_hip.h"
+
+namespace tfh {
+
+// ---- error reporting -----------------------------------------------------------------------------
+// Each failing call records one of tenferro_device::Error's variants (tenferro-device/src/lib.rs:108-159)
+// in a thread-local slot and returns its status code.
+int32_t set_error(int32_t status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int32_t set_shape_mismatch(const int64_t* expected, int n_expected, const int64_t* got, int n_got);
+int32_t set_rank_mismatch(int64_t expected, int64_t got);
+void clear_error();
+
+inline bool is_complex(int dt) { return dt == TFH_C64 || dt == TFH_C128; }
+inline bool is_double(int dt) { return dt == TFH_F64 || dt == TFH_C128; }
+inline size_t dtype_size(int dt) {
+    switch (dt) {
+        case TFH_F32: return 4;
+        case TFH_F64: return 8;
+        case TFH_C64: return 8;
+        case TFH_C128: return 16;
+        default: return 0;
+    }
+}
+// Host scalar of any dtype widened to (re, im) doubles.
+struct Scalar {
+    double re = 0, im = 0;
+    bool is_zero() const { return re == 0 && im == 0; }
+    bool is_one() const { return re == 1 && im == 0; }
+};
+inline Scalar load_scalar(int dt, const void* p) {
+    Scalar s;
+    if (is_double(dt)) {
+        s.re = ((const double*)p)[0];
+        if (is_complex(dt)) s.im = ((const double*)p)[1];
+    } else {
+        s.re = ((const float*)p)[0];
+        if (is_complex(dt)) s.im = ((const float*)p)[1];
+    }
+    return s;
+}
+
+// One loop axis with an element stride per tensor slot (0 = the tensor does not carry it).
+struct Axis {
+    int64_t n;
+    int64_t s[3];
+    uint32_t label;
+};
+
+// ---- plan ----------------------------------------------------------------------------------------
+struct GroupedState;  // device tables of a grouped plan (gemm.cpp)
+}  // namespace tfh
+
+struct tfh_plan {
+    int32_t dtype = 0;
+    int32_t op = 0;
+    int32_t reduce_op = 0;
+    std::vector<uint32_t> modes_a, modes_b, modes_c;
+    std::vector<std::pair<uint32_t, uint32_t>> pairs;
+    int32_t n_inputs = 0;
+    // expected shapes, inputs first then output; for a grouped plan n_groups*(n_inputs+1) entries
+    std::vector<std::vector<int64_t>> shapes;
+    int32_t n_groups = 0;  // 0 = not grouped
+    tfh::GroupedState* grouped = nullptr;
+    ~tfh_plan();
+};
+
+namespace tfh {
+
+// Validation + normalisation of a descriptor: BatchedGemm is rewritten as a Contract over synthetic
+// labels; returns TFH_OK or records an error.
+int32_t make_plan(int32_t dtype, const tfh_desc* desc, const int64_t* const* shapes, const int32_t* ranks,
+                  int32_t n_tensors, tfh_plan& plan);
+int32_t check_view_against(const std::vector<int64_t>& shape, const tfh_view& v, const char* what);
+
+// Mode classification of a binary contraction (tenferro-prims/src/lib.rs:136-138).
+struct ContractAxes {
+    std::vector<Axis> batch, M, N, K;  // s[0]=A, s[1]=B, s[2]=C
+};
+int32_t classify_contract(const std::vector<uint32_t>& ma, const int64_t* dims_a, const int64_t* str_a,
+                          const std::vector<uint32_t>& mb, const int64_t* dims_b, const int64_t* str_b,
+                          const std::vector<uint32_t>& mc, const int64_t* dims_c, const int64_t* str_c,
+                          ContractAxes& out);
+// Drops extent-1 axes and merges neighbours that are contiguous in every slot in [0, nslots).
+// Order is preserved (axis i+1 is "inside" axis i when they merge).
+void fuse_axes(std::vector<Axis>& ax, int nslots);
+
+// ---- kernel launchers (each enqueues on `stream`, returns a tfh_status) ----------------------------
+// B = alpha*op(A) + beta*B over axes (s[0] = in stride, s[1] = out stride); op = conj if `conj`.
+int32_t launch_copy(int dtype, const void* in, void* out, std::vector<Axis> axes, Scalar alpha, Scalar beta,
+                    bool conj, void* stream);
+// out = value over axes (s[0] = out stride)
+int32_t launch_fill(int dtype, void* out, std::vector<Axis> axes, Scalar value, void* stream);
+// C = alpha*A.*B + beta*C over axes (s[0]=A, s[1]=B, s[2]=C)
+int32_t launch_emul(int dtype, const void* a, const void* b, void* c, std::vector<Axis> axes, Scalar alpha,
+                    Scalar beta, void* stream);
+// C[kept] = alpha*reduce(A[kept, red]) + beta*C ; kept: s[0]=A, s[1]=C ; red: s[0]=A
+int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, std::vector<Axis> red, int reduce_op,
+                      Scalar alpha, Scalar beta, void* stream);
+// C = alpha*A*B + beta*C over classified axes
+int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes axes, Scalar alpha,
+                        Scalar beta, void* stream);
+int32_t grouped_plan_init(tfh_plan& plan);
+int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* inputs, Scalar beta, tfh_view* outputs,
+                       void* stream);
+void grouped_state_destroy(GroupedState* g);
+
+// ---- per-stream scratch memory ----------------------------------------------------------------------
+// Workspace: one growing buffer per stream; kernels on a stream are ordered, so successive calls
+// reuse it.  Valid until the next workspace() call on the same stream.
+int32_t workspace(void* stream, size_t bytes, void** out);
+// Intermediates of an einsum tree: stream-ordered cached allocations (free returns the block to the
+// stream's cache; reuse on the same stream needs no synchronisation).
+int32_t pool_alloc(void* stream, size_t bytes, void** out);
+void pool_free(void* stream, void* ptr);
+int32_t hip_check(int err, const char* what);
+
+// Byte pointer of a view's element 0.
+inline char* view_ptr(const tfh_view& v, int dtype) { return (char*)v.base + v.offset * (int64_t)dtype_size(dtype); }
+
+}  // namespace tfh

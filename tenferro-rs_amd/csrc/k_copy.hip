@@ -1,0 +1,478 @@
+// k_copy.hip -- strided N-d data movement for gfx950: Permute (tenferro-prims/src/lib.rs:194-202),
+// conj (tenferro-tensor/src/lib.rs:622-658), fill (zeros/ones, :336-347) and ElementwiseMul
+// (tenferro-prims/src/lib.rs:241-244).
+//
+// One kernel family.  The host picks a tile: up to four axes with power-of-two tile extents, chosen so
+// that the tile holds a >=512-byte contiguous run on the input side AND on the output side.  A block
+// reads the tile in input-memory order (coalesced), parks it in LDS, and writes it in output-memory
+// order (coalesced); in-tile coordinates are shifts and masks, the per-block origin is decomposed once.
+// HBM-bound: algorithmic bytes = 2 * elements * sizeof(T).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+
+#include "internal.hpp"
+
+namespace tfh {
+namespace {
+
+constexpr int MAXT = 4;    // tile axes
+constexpr int MAXG = 16;   // grid axes
+constexpr int THREADS = 256;
+
+struct CopyArgs {
+    const void* in;
+    const void* in2;       // second input (elementwise mul)
+    void* out;
+    int32_t nt, ng;
+    int32_t tile_elems;    // product of tile extents (power of two)
+    int32_t pad_;
+    // tile axes in read order (ascending input stride) and in write order (ascending output stride)
+    int32_t r_shift[MAXT], r_mask[MAXT], r_id[MAXT];
+    int64_t r_si[MAXT];
+    int32_t w_shift[MAXT], w_mask[MAXT], w_id[MAXT], w_rpos[MAXT];
+    int64_t w_so[MAXT], w_si[MAXT], w_si2[MAXT];
+    int64_t t_n[MAXT];     // full extent of tile axis id
+    // grid axes (every axis with more than one tile)
+    int64_t g_count[MAXG], g_si[MAXG], g_si2[MAXG], g_so[MAXG];
+    int32_t g_tid[MAXG];   // tile axis id advanced by this grid axis, or -1
+    int32_t g_text[MAXG];  // tile extent of that axis (1 if untiled)
+    double alpha_re, alpha_im, beta_re, beta_im;
+    int32_t conj, use_beta;
+};
+
+__device__ __forceinline__ int swz(int r) { return r + (r >> 5); }
+
+struct BlockOrigin {
+    int64_t in, in2, out;
+    int64_t lim[MAXT];  // remaining extent of each tile axis at this block
+};
+
+__device__ __forceinline__ BlockOrigin block_origin(const CopyArgs& a) {
+    BlockOrigin o;
+    o.in = o.in2 = o.out = 0;
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) o.lim[t] = t < a.nt ? a.t_n[t] : 1;
+    uint64_t bid = (uint64_t)blockIdx.x + (uint64_t)blockIdx.y * gridDim.x;
+    for (int g = 0; g < a.ng; ++g) {
+        uint64_t q = bid / (uint64_t)a.g_count[g];
+        int64_t c = (int64_t)(bid - q * (uint64_t)a.g_count[g]);
+        bid = q;
+        o.in += c * a.g_si[g];
+        o.in2 += c * a.g_si2[g];
+        o.out += c * a.g_so[g];
+        int t = a.g_tid[g];
+        if (t >= 0) {
+#pragma unroll
+            for (int k = 0; k < MAXT; ++k)
+                if (k == t) o.lim[k] -= c * a.g_text[g];
+        }
+    }
+    return o;
+}
+
+// ---- element operations -----------------------------------------------------------------------------
+template <class V>
+struct RawOp {  // bit-exact move
+    static constexpr bool kNeedsOld = false;
+    __device__ V operator()(V x, V, const CopyArgs&) const { return x; }
+};
+template <class R>
+struct RealOp {  // out = alpha*x + beta*old
+    __device__ R operator()(R x, R old, const CopyArgs& a) const {
+        R r = (R)a.alpha_re * x;
+        if (a.use_beta) r += (R)a.beta_re * old;
+        return r;
+    }
+};
+template <class V, class R>
+struct CplxOp {  // V = float2/double2
+    __device__ V operator()(V x, V old, const CopyArgs& a) const {
+        R xr = x.x, xi = a.conj ? -x.y : x.y;
+        R ar = (R)a.alpha_re, ai = (R)a.alpha_im;
+        V r;
+        r.x = ar * xr - ai * xi;
+        r.y = ar * xi + ai * xr;
+        if (a.use_beta) {
+            R br = (R)a.beta_re, bi = (R)a.beta_im;
+            r.x += br * old.x - bi * old.y;
+            r.y += br * old.y + bi * old.x;
+        }
+        return r;
+    }
+};
+template <class V>
+struct ConjOp {  // bit-exact conj: flip the sign of the imaginary part
+    __device__ V operator()(V x, V, const CopyArgs&) const {
+        x.y = -x.y;
+        return x;
+    }
+};
+
+template <class V, class Op, int EPT, bool READ_OLD>
+__global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    V* lds = reinterpret_cast<V*>(smem_raw);
+    const BlockOrigin o = block_origin(a);
+    const V* in = reinterpret_cast<const V*>(a.in) + o.in;
+    V* out = reinterpret_cast<V*>(a.out) + o.out;
+    const int tid = threadIdx.x;
+    V regs[EPT];
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+        int r = u * THREADS + tid;
+        bool ok = r < a.tile_elems;
+        int64_t off = 0;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t) {
+            if (t < a.nt) {
+                int c = (r >> a.r_shift[t]) & a.r_mask[t];
+                off += (int64_t)c * a.r_si[t];
+                int id = a.r_id[t];
+                int64_t lim = id == 0 ? o.lim[0] : id == 1 ? o.lim[1] : id == 2 ? o.lim[2] : o.lim[3];
+                ok &= c < lim;
+            }
+        }
+        if (ok) regs[u] = in[off];
+    }
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+        int r = u * THREADS + tid;
+        if (r < a.tile_elems) lds[swz(r)] = regs[u];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+        int w = u * THREADS + tid;
+        bool ok = w < a.tile_elems;
+        int64_t off = 0;
+        int r = 0;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t) {
+            if (t < a.nt) {
+                int c = (w >> a.w_shift[t]) & a.w_mask[t];
+                off += (int64_t)c * a.w_so[t];
+                r += c * a.w_rpos[t];
+                int id = a.w_id[t];
+                int64_t lim = id == 0 ? o.lim[0] : id == 1 ? o.lim[1] : id == 2 ? o.lim[2] : o.lim[3];
+                ok &= c < lim;
+            }
+        }
+        if (ok) {
+            V x = lds[swz(r)];
+            V old = x;
+            if (READ_OLD) old = out[off];
+            out[off] = op(x, old, a);
+        }
+    }
+}
+
+// Direct (no LDS) kernels in write order: fill and elementwise multiply.
+template <class V>
+__global__ void __launch_bounds__(THREADS) fill_kernel(CopyArgs a, V value, int ept) {
+    const BlockOrigin o = block_origin(a);
+    V* out = reinterpret_cast<V*>(a.out) + o.out;
+    for (int u = 0; u < ept; ++u) {
+        int w = u * THREADS + threadIdx.x;
+        bool ok = w < a.tile_elems;
+        int64_t off = 0;
+        for (int t = 0; t < a.nt; ++t) {
+            int c = (w >> a.w_shift[t]) & a.w_mask[t];
+            off += (int64_t)c * a.w_so[t];
+            ok &= c < o.lim[a.w_id[t]];
+        }
+        if (ok) out[off] = value;
+    }
+}
+
+template <class R, bool CX>
+__global__ void __launch_bounds__(THREADS) emul_kernel(CopyArgs a, int ept) {
+    constexpr int NC = CX ? 2 : 1;
+    const BlockOrigin o = block_origin(a);
+    const R* A = reinterpret_cast<const R*>(a.in) + o.in * NC;
+    const R* B = reinterpret_cast<const R*>(a.in2) + o.in2 * NC;
+    R* C = reinterpret_cast<R*>(a.out) + o.out * NC;
+    for (int u = 0; u < ept; ++u) {
+        int w = u * THREADS + threadIdx.x;
+        bool ok = w < a.tile_elems;
+        int64_t oa = 0, ob = 0, oc = 0;
+        for (int t = 0; t < a.nt; ++t) {
+            int c = (w >> a.w_shift[t]) & a.w_mask[t];
+            oa += (int64_t)c * a.w_si[t];
+            ob += (int64_t)c * a.w_si2[t];
+            oc += (int64_t)c * a.w_so[t];
+            ok &= c < o.lim[a.w_id[t]];
+        }
+        if (!ok) continue;
+        R ar = (R)a.alpha_re, ai = (R)a.alpha_im;
+        if (CX) {
+            R xr = A[oa * 2], xi = A[oa * 2 + 1], yr = B[ob * 2], yi = B[ob * 2 + 1];
+            R pr = xr * yr - xi * yi, pi = xr * yi + xi * yr;
+            R rr = ar * pr - ai * pi, ri = ar * pi + ai * pr;
+            if (a.use_beta) {
+                R br = (R)a.beta_re, bi = (R)a.beta_im, cr = C[oc * 2], ci = C[oc * 2 + 1];
+                rr += br * cr - bi * ci;
+                ri += br * ci + bi * cr;
+            }
+            C[oc * 2] = rr;
+            C[oc * 2 + 1] = ri;
+        } else {
+            R r = ar * (A[oa] * B[ob]);
+            if (a.use_beta) r += (R)a.beta_re * C[oc];
+            C[oc] = r;
+        }
+    }
+}
+
+// ---- host side: tile selection --------------------------------------------------------------------------
+int ceil_log2(int64_t n) {
+    int l = 0;
+    while (((int64_t)1 << l) < n) ++l;
+    return l;
+}
+
+struct TilePlan {
+    CopyArgs args;
+    dim3 grid;
+    int ept;
+};
+
+// axes: s[0] = input stride, s[1] = output stride, s[2] = second input stride (emul only).
+// order_slot: which slot defines the read order (0) -- the write order is always slot 1.
+int32_t plan_tiles(std::vector<Axis> axes, int elem_bytes, int max_tile_elems, bool two_sided, TilePlan& tp) {
+    CopyArgs& a = tp.args;
+    std::memset(&a, 0, sizeof a);
+    for (auto& x : axes)
+        if (x.n == 0) {
+            tp.grid = dim3(0, 0, 0);
+            return TFH_OK;
+        }
+    // canonical order: output stride descending, then merge what is contiguous on every side
+    std::stable_sort(axes.begin(), axes.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[1]) > std::llabs(y.s[1]); });
+    fuse_axes(axes, 3);
+    if (axes.empty()) axes.push_back(Axis{1, {0, 0, 0}, 0});
+    const int na = (int)axes.size();
+    if (na > MAXG) return set_error(TFH_ERR_INVALID_ARGUMENT, "more than %d non-mergeable axes", MAXG);
+    for (auto& x : axes)
+        if (x.n > 1 && x.s[1] == 0) return set_error(TFH_ERR_STRIDED, "output view has stride 0 on an axis of extent %lld (elements would alias)", (long long)x.n);
+    auto key_in = [&](int i) { return axes[i].s[0] == 0 ? INT64_MAX : std::llabs(axes[i].s[0]); };
+    std::vector<int> out_order(na), in_order(na);
+    for (int i = 0; i < na; ++i) out_order[i] = in_order[i] = i;
+    std::stable_sort(out_order.begin(), out_order.end(), [&](int x, int y) { return std::llabs(axes[x].s[1]) < std::llabs(axes[y].s[1]); });
+    std::stable_sort(in_order.begin(), in_order.end(), [&](int x, int y) { return key_in(x) < key_in(y); });
+
+    std::vector<int> tl(na, 0);  // log2 tile extent per axis
+    auto full = [&](int i) { return ceil_log2(axes[i].n); };
+    auto tile_axes = [&]() { int c = 0; for (int i = 0; i < na; ++i) c += tl[i] > 0; return c; };
+    auto prod_log2 = [&]() { int p = 0; for (int i = 0; i < na; ++i) p += tl[i]; return p; };
+    const int budget = ceil_log2(max_tile_elems);
+    const int run_target = ceil_log2(std::max(1, 512 / elem_bytes));
+    auto take_run = [&](const std::vector<int>& order) {
+        int run = 0;
+        for (int i : order) {
+            if (run >= run_target) break;
+            if (tl[i] == 0 && tile_axes() >= MAXT) break;
+            int want = std::min(full(i), run_target - run);
+            want = std::max(want, tl[i]);
+            want = std::min(want, tl[i] + budget - prod_log2());
+            tl[i] = want;
+            run += want;
+            if (want < full(i)) break;
+        }
+    };
+    take_run(out_order);
+    if (two_sided) take_run(in_order);
+    // spend the rest of the budget: alternately lengthen the output-side and the input-side run
+    for (int side = 0; prod_log2() < budget; side ^= 1) {
+        bool grew = false;
+        for (int pass = 0; pass < 2 && !grew; ++pass) {
+            const std::vector<int>& order = ((side ^ pass) == 0 || !two_sided) ? out_order : in_order;
+            for (int i : order) {
+                if (tl[i] < full(i) && (tl[i] > 0 || tile_axes() < MAXT)) {
+                    ++tl[i];
+                    grew = true;
+                    break;
+                }
+                if (tl[i] < full(i)) break;  // cannot extend this run past a partial axis
+            }
+        }
+        if (!grew) break;
+    }
+    // tile axis ids
+    std::vector<int> ids;
+    for (int i = 0; i < na; ++i)
+        if (tl[i] > 0) ids.push_back(i);
+    a.nt = (int)ids.size();
+    a.tile_elems = 1 << prod_log2();
+    auto id_of = [&](int axis) { return (int)(std::find(ids.begin(), ids.end(), axis) - ids.begin()); };
+    for (int t = 0; t < a.nt; ++t) a.t_n[t] = axes[ids[t]].n;
+    // read order / write order
+    std::vector<int> rd, wr;
+    for (int i : in_order) if (tl[i] > 0) rd.push_back(i);
+    for (int i : out_order) if (tl[i] > 0) wr.push_back(i);
+    std::vector<int> rshift(na, 0);
+    int sh = 0;
+    for (int t = 0; t < a.nt; ++t) {
+        int i = rd[t];
+        a.r_shift[t] = sh;
+        a.r_mask[t] = (1 << tl[i]) - 1;
+        a.r_id[t] = id_of(i);
+        a.r_si[t] = axes[i].s[0];
+        rshift[i] = sh;
+        sh += tl[i];
+    }
+    sh = 0;
+    for (int t = 0; t < a.nt; ++t) {
+        int i = wr[t];
+        a.w_shift[t] = sh;
+        a.w_mask[t] = (1 << tl[i]) - 1;
+        a.w_id[t] = id_of(i);
+        a.w_rpos[t] = 1 << rshift[i];
+        a.w_so[t] = axes[i].s[1];
+        a.w_si[t] = axes[i].s[0];
+        a.w_si2[t] = axes[i].s[2];
+        sh += tl[i];
+    }
+    // grid axes
+    a.ng = 0;
+    uint64_t blocks = 1;
+    for (int i = 0; i < na; ++i) {
+        int64_t text = (int64_t)1 << tl[i];
+        int64_t cnt = (axes[i].n + text - 1) / text;
+        if (cnt <= 1) continue;
+        int g = a.ng++;
+        a.g_count[g] = cnt;
+        a.g_si[g] = axes[i].s[0] * text;
+        a.g_si2[g] = axes[i].s[2] * text;
+        a.g_so[g] = axes[i].s[1] * text;
+        a.g_tid[g] = tl[i] > 0 ? id_of(i) : -1;
+        a.g_text[g] = (int32_t)text;
+        blocks *= (uint64_t)cnt;
+    }
+    if (blocks > (uint64_t)0x7fffffff * 65535ull) return set_error(TFH_ERR_INVALID_ARGUMENT, "tensor too large for one launch");
+    uint32_t gx = (uint32_t)std::min<uint64_t>(blocks, 0x7fffffffull);
+    uint32_t gy = (uint32_t)((blocks + gx - 1) / gx);
+    if ((uint64_t)gx * gy != blocks) {  // keep the grid exact: x*y must equal the block count
+        gx = 1u << 30;
+        while (blocks % gx) gx >>= 1;
+        gy = (uint32_t)(blocks / gx);
+        if (gy > 65535u) return set_error(TFH_ERR_INVALID_ARGUMENT, "tensor too large for one launch");
+    }
+    tp.grid = dim3(gx, gy, 1);
+    tp.ept = (a.tile_elems + THREADS - 1) / THREADS;
+    return TFH_OK;
+}
+
+void set_scalars(CopyArgs& a, Scalar alpha, Scalar beta, bool conj) {
+    a.alpha_re = alpha.re;
+    a.alpha_im = alpha.im;
+    a.beta_re = beta.re;
+    a.beta_im = beta.im;
+    a.conj = conj;
+    a.use_beta = !beta.is_zero();
+}
+
+template <class V, class Op>
+int32_t run_copy(const TilePlan& tp, Op op, bool read_old, hipStream_t st) {
+    size_t lds = (size_t)(tp.args.tile_elems + tp.args.tile_elems / 32 + 1) * sizeof(V);
+    const int ept = tp.ept;
+#define TFH_LAUNCH(E)                                                                                     \
+    do {                                                                                                  \
+        if (read_old) hipLaunchKernelGGL((copy_kernel<V, Op, E, true>), tp.grid, dim3(THREADS), lds, st, tp.args, op);   \
+        else hipLaunchKernelGGL((copy_kernel<V, Op, E, false>), tp.grid, dim3(THREADS), lds, st, tp.args, op);           \
+    } while (0)
+    if (ept <= 1) TFH_LAUNCH(1);
+    else if (ept <= 4) TFH_LAUNCH(4);
+    else if (ept <= 8) TFH_LAUNCH(8);
+    else TFH_LAUNCH(16);
+#undef TFH_LAUNCH
+    return hip_check(hipGetLastError(), "copy kernel launch");
+}
+
+bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+}  // namespace
+
+int32_t launch_copy(int dtype, const void* in, void* out, std::vector<Axis> axes, Scalar alpha, Scalar beta, bool conj,
+                    void* stream) {
+    const int eb = (int)dtype_size(dtype);
+    if (!aligned(in, eb) || !aligned(out, eb)) return set_error(TFH_ERR_STRIDED, "view base is not aligned to the element size (%d bytes)", eb);
+    for (auto& x : axes) x.s[2] = 0;
+    TilePlan tp;
+    const int max_tile = eb >= 16 ? 2048 : 4096;
+    if (int32_t e = plan_tiles(axes, eb, max_tile, true, tp)) return e;
+    if (tp.grid.x == 0) return TFH_OK;
+    tp.args.in = in;
+    tp.args.out = out;
+    set_scalars(tp.args, alpha, beta, conj);
+    hipStream_t st = (hipStream_t)stream;
+    const bool cx = is_complex(dtype);
+    const bool raw = alpha.is_one() && beta.is_zero() && !(conj && cx);
+    if (raw) {
+        switch (eb) {
+            case 4: return run_copy<uint32_t>(tp, RawOp<uint32_t>(), false, st);
+            case 8: return run_copy<uint64_t>(tp, RawOp<uint64_t>(), false, st);
+            default: return run_copy<double2>(tp, RawOp<double2>(), false, st);
+        }
+    }
+    const bool rb = !beta.is_zero();
+    if (alpha.is_one() && beta.is_zero() && conj) {
+        if (dtype == TFH_C64) return run_copy<float2>(tp, ConjOp<float2>(), false, st);
+        return run_copy<double2>(tp, ConjOp<double2>(), false, st);
+    }
+    switch (dtype) {
+        case TFH_F32: return run_copy<float>(tp, RealOp<float>(), rb, st);
+        case TFH_F64: return run_copy<double>(tp, RealOp<double>(), rb, st);
+        case TFH_C64: return run_copy<float2>(tp, CplxOp<float2, float>(), rb, st);
+        default: return run_copy<double2>(tp, CplxOp<double2, double>(), rb, st);
+    }
+}
+
+int32_t launch_fill(int dtype, void* out, std::vector<Axis> axes, Scalar value, void* stream) {
+    const int eb = (int)dtype_size(dtype);
+    if (!aligned(out, eb)) return set_error(TFH_ERR_STRIDED, "view base is not aligned to the element size (%d bytes)", eb);
+    for (auto& x : axes) {  // slot 1 is the output everywhere in the tile planner
+        x.s[1] = x.s[0];
+        x.s[0] = x.s[2] = 0;
+    }
+    TilePlan tp;
+    if (int32_t e = plan_tiles(axes, eb, 4096, false, tp)) return e;
+    if (tp.grid.x == 0) return TFH_OK;
+    tp.args.out = out;
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case TFH_F32: hipLaunchKernelGGL(fill_kernel<float>, tp.grid, dim3(THREADS), 0, st, tp.args, (float)value.re, tp.ept); break;
+        case TFH_F64: hipLaunchKernelGGL(fill_kernel<double>, tp.grid, dim3(THREADS), 0, st, tp.args, value.re, tp.ept); break;
+        case TFH_C64: hipLaunchKernelGGL(fill_kernel<float2>, tp.grid, dim3(THREADS), 0, st, tp.args, make_float2((float)value.re, (float)value.im), tp.ept); break;
+        default: hipLaunchKernelGGL(fill_kernel<double2>, tp.grid, dim3(THREADS), 0, st, tp.args, make_double2(value.re, value.im), tp.ept); break;
+    }
+    return hip_check(hipGetLastError(), "fill kernel launch");
+}
+
+int32_t launch_emul(int dtype, const void* a, const void* b, void* c, std::vector<Axis> axes, Scalar alpha, Scalar beta,
+                    void* stream) {
+    // incoming slots: s[0]=A, s[1]=B, s[2]=C -> planner slots: 0 = A, 1 = output, 2 = B
+    for (auto& x : axes) std::swap(x.s[1], x.s[2]);
+    const int eb = (int)dtype_size(dtype);
+    const int rb = is_double(dtype) ? 8 : 4;
+    if (!aligned(a, rb) || !aligned(b, rb) || !aligned(c, rb)) return set_error(TFH_ERR_STRIDED, "view base is not aligned");
+    TilePlan tp;
+    if (int32_t e = plan_tiles(axes, eb, 2048, false, tp)) return e;
+    if (tp.grid.x == 0) return TFH_OK;
+    tp.args.in = a;
+    tp.args.in2 = b;
+    tp.args.out = c;
+    set_scalars(tp.args, alpha, beta, false);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case TFH_F32: hipLaunchKernelGGL((emul_kernel<float, false>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
+        case TFH_F64: hipLaunchKernelGGL((emul_kernel<double, false>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
+        case TFH_C64: hipLaunchKernelGGL((emul_kernel<float, true>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
+        default: hipLaunchKernelGGL((emul_kernel<double, true>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
+    }
+    return hip_check(hipGetLastError(), "elementwise kernel launch");
+}
+
+}  // namespace tfh

@@ -1,0 +1,764 @@
+// k_gemm.hip -- binary tensor contraction on the gfx950 matrix cores: PrimDescriptor::Contract and
+// BatchedGemm (tenferro-prims/src/lib.rs:227-239, 156-168) and the grouped (variable-size) form.
+//
+// C[b, m, n] = alpha * sum_k A[b, m, k] * B[b, k, n] + beta * C, where b, m, n, k are *fused mode
+// groups*: each operand element is addressed as base + off_batch(b) + off_row(m) + off_k(k), and every
+// off_* is either a single stride or a table built on the device from the group's extents and strides.
+// The permutation a contraction implies is therefore applied while the tiles are loaded ("permute on
+// load"); nothing is materialised.
+//
+// Block = 256 threads = 4 waves (2x2), tile BM x BN x BK, double-buffered in LDS with the k index
+// contiguous for both operands.  The inner product runs on v_mfma_f64_16x16x4_f64 /
+// v_mfma_f32_16x16x4_f32: lane l feeds A[l%16][l/16] and B[l/16][l%16]; a lane reads FOUR consecutive
+// k values at once (one or two ds_read_b128) and uses them in four successive MFMAs, which permutes k
+// identically for A and B and is harmless under the sum.
+// complex128/complex64 run on the real MFMA: the A tile keeps (re, im) interleaved along k, the B tile
+// is expanded on its way into LDS to the real 2x2 block [[br, bi], [-bi, br]], so that the real product
+// A'(M x 2K) * B'(2K x 2N) is the interleaved complex C(M x N).  conj is a sign flip in the same place.
+// MFMA-bound: algorithmic flops = 2*M*N*K (x4 for complex).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <array>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+
+#include "internal.hpp"
+
+namespace tfh {
+namespace {
+
+constexpr int THREADS = 256;
+
+typedef double d4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+struct OffFn {
+    const int64_t* tab;  // offsets per fused index, or null
+    int64_t stride;      // used when tab == null
+};
+__device__ __forceinline__ int64_t off_of(const OffFn& f, int64_t i) { return f.tab ? f.tab[i] : i * f.stride; }
+
+struct GroupProblem {   // one problem of a grouped launch (plain strided matrices)
+    const void* A;
+    const void* B;
+    void* C;
+    int64_t M, N, K;
+    int64_t sam, sak, sbk, sbn, scm, scn;
+};
+
+struct GemmArgs {
+    const void* A;
+    const void* B;
+    void* C;
+    int64_t M, N, K, nbatch;
+    OffFn am, ak, bk, bn, cm, cn, ab, bb, cb;
+    int32_t a_kfast, b_kfast, conj_a, conj_b;
+    int32_t nsplit, use_beta;
+    int64_t k_per_split;
+    void* partial;
+    int32_t tiles_m, tiles_n;
+    double alpha_re, alpha_im, beta_re, beta_im;
+    const GroupProblem* problems;  // grouped launch when non-null
+    const int4* tile_map;          // per block: (problem, tile_m, tile_n, 0)
+};
+
+template <class R> struct Mfma;
+template <> struct Mfma<double> {
+    typedef d4 acc_t;
+    __device__ static __forceinline__ d4 run(double a, double b, d4 c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+    // accumulator register r of lane l holds row (l/16) + 4r, column l%16
+    __device__ static __forceinline__ int row(int lane, int r) { return (lane >> 4) + 4 * r; }
+};
+template <> struct Mfma<float> {
+    typedef f4 acc_t;
+    __device__ static __forceinline__ f4 run(float a, float b, f4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+    // accumulator register r of lane l holds row 4*(l/16) + r, column l%16
+    __device__ static __forceinline__ int row(int lane, int r) { return 4 * (lane >> 4) + r; }
+};
+
+template <class R, bool CX> struct ElemT;
+template <> struct ElemT<float, false> { typedef float type; };
+template <> struct ElemT<double, false> { typedef double type; };
+template <> struct ElemT<float, true> { typedef float2 type; };
+template <> struct ElemT<double, true> { typedef double2 type; };
+
+// One operand tile loader: ROWS x BKE elements per stage, NU per thread.
+template <class R, bool CX, int ROWS, int BKE>
+struct Loader {
+    typedef typename ElemT<R, CX>::type E;
+    static constexpr int NU = ROWS * BKE / THREADS;
+    static_assert(ROWS * BKE % THREADS == 0, "tile must divide over the block");
+    const E* base;
+    int64_t rowoff[NU];   // kfast: one per u.  rfast: [0] only
+    int rows_left;        // valid rows in this tile
+    bool kfast;
+    OffFn fk;
+
+    __device__ __forceinline__ void init(const void* p, int64_t boff, const OffFn& frow, const OffFn& fk_, int64_t row0,
+                                         int64_t nrows, bool kfast_) {
+        base = reinterpret_cast<const E*>(p) + boff;
+        kfast = kfast_;
+        fk = fk_;
+        int64_t left = nrows - row0;
+        rows_left = left > ROWS ? ROWS : (int)left;
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+            int row = kfast ? (u * THREADS + t) / BKE : (u * THREADS + t) % ROWS;
+            int64_t r = row0 + (row < rows_left ? row : 0);
+            rowoff[u] = (kfast || u == 0) ? off_of(frow, r) : rowoff[0];
+        }
+    }
+    // k0: first element index of the stage; kend: end of this block's k range
+    __device__ __forceinline__ void load(E (&v)[NU], int64_t k0, int64_t kend) const {
+        const int t = threadIdx.x;
+        if (kfast) {
+            const int kk = t % BKE;
+            const bool kok = k0 + kk < kend;
+            const int64_t ko = kok ? off_of(fk, k0 + kk) : 0;
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                int row = (u * THREADS + t) / BKE;
+                E z = E();
+                v[u] = (kok && row < rows_left) ? base[rowoff[u] + ko] : z;
+            }
+        } else {
+            const int row = t % ROWS;
+            const bool rok = row < rows_left;
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                int kk = (u * THREADS + t) / ROWS;
+                bool kok = k0 + kk < kend;
+                E z = E();
+                v[u] = (kok && rok) ? base[rowoff[0] + off_of(fk, kok ? k0 + kk : 0)] : z;
+            }
+        }
+    }
+    __device__ __forceinline__ void coords(int u, int& row, int& kk) const {
+        const int id = u * THREADS + threadIdx.x;
+        if (kfast) {
+            row = id / BKE;
+            kk = id % BKE;
+        } else {
+            row = id % ROWS;
+            kk = id / ROWS;
+        }
+    }
+};
+
+template <class R, bool CX, int BM, int BN>
+struct Cfg {
+    static constexpr int BKR = sizeof(R) == 8 ? 16 : 32;  // real k per stage
+    static constexpr int BKE = CX ? BKR / 2 : BKR;        // elements of k per stage
+    static constexpr int PAD = 16 / sizeof(R);
+    static constexpr int PITCH = BKR + PAD;
+    static constexpr int BNE = CX ? BN / 2 : BN;          // element columns per tile
+    static constexpr int WM = BM / 2, WN = BN / 2;        // wave tile
+    static constexpr int TM = WM / 16, TN = WN / 16;
+    static constexpr size_t LDS_BYTES = (size_t)2 * (BM + BN) * PITCH * sizeof(R);
+};
+
+template <class R, bool CX, int BM, int BN>
+__global__ void __launch_bounds__(THREADS) gemm_kernel(GemmArgs g) {
+    typedef Cfg<R, CX, BM, BN> C_;
+    typedef typename ElemT<R, CX>::type E;
+    typedef typename Mfma<R>::acc_t acc_t;
+    constexpr int BKR = C_::BKR, BKE = C_::BKE, PITCH = C_::PITCH, BNE = C_::BNE, TM = C_::TM, TN = C_::TN;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    R* As = reinterpret_cast<R*>(smem_raw);                 // [2][BM][PITCH]
+    R* Bs = As + 2 * BM * PITCH;                            // [2][BN][PITCH]
+
+    // ---- which tile ---------------------------------------------------------------------------------
+    int64_t M = g.M, N = g.N, K = g.K;
+    const void* Ap = g.A;
+    const void* Bp = g.B;
+    void* Cp = g.C;
+    OffFn am = g.am, ak = g.ak, bk = g.bk, bn = g.bn, cm = g.cm, cn = g.cn;
+    int tile_m, tile_n;
+    int64_t batch = 0;
+    int split = 0;
+    if (g.problems) {
+        const int4 tm = g.tile_map[blockIdx.x];
+        const GroupProblem& p = g.problems[tm.x];
+        M = p.M; N = p.N; K = p.K;
+        Ap = p.A; Bp = p.B; Cp = p.C;
+        am.stride = p.sam; ak.stride = p.sak; bk.stride = p.sbk; bn.stride = p.sbn; cm.stride = p.scm; cn.stride = p.scn;
+        tile_m = tm.y;
+        tile_n = tm.z;
+    } else {
+        tile_n = blockIdx.x % g.tiles_n;
+        tile_m = blockIdx.x / g.tiles_n;
+        split = blockIdx.z % g.nsplit;
+        batch = blockIdx.z / g.nsplit;
+    }
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BNE;
+    const int64_t kbeg = (int64_t)split * g.k_per_split;
+    const int64_t kend = (g.nsplit > 1 && kbeg + g.k_per_split < K) ? kbeg + g.k_per_split : K;
+
+    Loader<R, CX, BM, BKE> la;
+    Loader<R, CX, BNE, BKE> lb;
+    la.init(Ap, g.problems ? 0 : off_of(g.ab, batch), am, ak, m0, M, g.a_kfast);
+    lb.init(Bp, g.problems ? 0 : off_of(g.bb, batch), bn, bk, n0, N, g.b_kfast);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm0 = (wave >> 1) * C_::WM, wn0 = (wave & 1) * C_::WN;
+    const int lrow = lane & 15, lgrp = lane >> 4;
+
+    acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
+
+    E va[Loader<R, CX, BM, BKE>::NU], vb[Loader<R, CX, BNE, BKE>::NU];
+
+    auto store_tiles = [&](int buf) {
+        R* as = As + buf * BM * PITCH;
+        R* bs = Bs + buf * BN * PITCH;
+#pragma unroll
+        for (int u = 0; u < Loader<R, CX, BM, BKE>::NU; ++u) {
+            int row, kk;
+            la.coords(u, row, kk);
+            if constexpr (CX) {
+                E x = va[u];
+                if (g.conj_a) x.y = -x.y;
+                *reinterpret_cast<E*>(as + row * PITCH + 2 * kk) = x;
+            } else {
+                as[row * PITCH + kk] = va[u];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < Loader<R, CX, BNE, BKE>::NU; ++u) {
+            int row, kk;
+            lb.coords(u, row, kk);
+            if constexpr (CX) {
+                E x = vb[u];
+                if (g.conj_b) x.y = -x.y;
+                E r0, r1;           // B'[2k][2n] = br, B'[2k+1][2n] = -bi ; B'[2k][2n+1] = bi, B'[2k+1][2n+1] = br
+                r0.x = x.x; r0.y = -x.y;
+                r1.x = x.y; r1.y = x.x;
+                *reinterpret_cast<E*>(bs + (2 * row) * PITCH + 2 * kk) = r0;
+                *reinterpret_cast<E*>(bs + (2 * row + 1) * PITCH + 2 * kk) = r1;
+            } else {
+                bs[row * PITCH + kk] = vb[u];
+            }
+        }
+    };
+
+    const int64_t nstage = kend > kbeg ? (kend - kbeg + BKE - 1) / BKE : 0;
+    if (nstage > 0) {
+        la.load(va, kbeg, kend);
+        lb.load(vb, kbeg, kend);
+        store_tiles(0);
+    }
+    __syncthreads();
+    for (int64_t s = 0; s < nstage; ++s) {
+        const int buf = (int)(s & 1);
+        const bool more = s + 1 < nstage;
+        if (more) {
+            la.load(va, kbeg + (s + 1) * BKE, kend);
+            lb.load(vb, kbeg + (s + 1) * BKE, kend);
+        }
+        const R* as = As + buf * BM * PITCH + (wm0 + lrow) * PITCH + 4 * lgrp;
+        const R* bs = Bs + buf * BN * PITCH + (wn0 + lrow) * PITCH + 4 * lgrp;
+#pragma unroll
+        for (int c = 0; c < BKR / 16; ++c) {
+            R a[TM][4], b[TN][4];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const R* p = as + i * 16 * PITCH + c * 16;
+                if constexpr (sizeof(R) == 8) {
+                    double2 lo = *reinterpret_cast<const double2*>(p), hi = *reinterpret_cast<const double2*>(p + 2);
+                    a[i][0] = lo.x; a[i][1] = lo.y; a[i][2] = hi.x; a[i][3] = hi.y;
+                } else {
+                    float4 q = *reinterpret_cast<const float4*>(p);
+                    a[i][0] = q.x; a[i][1] = q.y; a[i][2] = q.z; a[i][3] = q.w;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const R* p = bs + j * 16 * PITCH + c * 16;
+                if constexpr (sizeof(R) == 8) {
+                    double2 lo = *reinterpret_cast<const double2*>(p), hi = *reinterpret_cast<const double2*>(p + 2);
+                    b[j][0] = lo.x; b[j][1] = lo.y; b[j][2] = hi.x; b[j][3] = hi.y;
+                } else {
+                    float4 q = *reinterpret_cast<const float4*>(p);
+                    b[j][0] = q.x; b[j][1] = q.y; b[j][2] = q.z; b[j][3] = q.w;
+                }
+            }
+#pragma unroll
+            for (int k4 = 0; k4 < 4; ++k4)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<R>::run(a[i][k4], b[j][k4], acc[i][j]);
+        }
+        if (more) store_tiles(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue ---------------------------------------------------------------------------------------
+    // real column index inside the tile: wn0 + 16 j + lrow ; for complex, column 2n+p is part p of element n
+    const int64_t NR = CX ? 2 * N : N;           // real columns of C
+    const int64_t n0r = CX ? 2 * n0 : n0;
+    if (g.nsplit > 1) {
+        R* P = reinterpret_cast<R*>(g.partial) + ((int64_t)split * g.nbatch + batch) * M * NR;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                int64_t row = m0 + wm0 + 16 * i + Mfma<R>::row(lane, r);
+                if (row >= M) continue;
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    int64_t col = n0r + wn0 + 16 * j + lrow;
+                    if (col < NR) P[row * NR + col] = acc[i][j][r];
+                }
+            }
+        return;
+    }
+    R* Cb = reinterpret_cast<R*>(Cp) + (g.problems ? 0 : off_of(g.cb, batch)) * (CX ? 2 : 1);
+    const R ar = (R)g.alpha_re, ai = (R)g.alpha_im, br = (R)g.beta_re, bi = (R)g.beta_im;
+    int64_t coff[TN];
+    bool cok[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        int64_t col = n0r + wn0 + 16 * j + lrow;
+        cok[j] = col < NR;
+        int64_t n = CX ? col >> 1 : col;
+        coff[j] = cok[j] ? off_of(cn, n) * (CX ? 2 : 1) + (CX ? (col & 1) : 0) : 0;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            int64_t row = m0 + wm0 + 16 * i + Mfma<R>::row(lane, r);
+            const bool rok = row < M;
+            const int64_t roff = rok ? off_of(cm, row) * (CX ? 2 : 1) : 0;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                R v = acc[i][j][r];
+                const bool ok = rok && cok[j];
+                R* dst = Cb + roff + coff[j];
+                if constexpr (CX) {
+                    // even lanes hold re, odd lanes hold im of the same element: exchange with the neighbour
+                    R other = __shfl_xor(v, 1);
+                    R old = (g.use_beta && ok) ? *dst : R(0);
+                    R old_other = __shfl_xor(old, 1);
+                    const bool im = lane & 1;
+                    R re_v = im ? other : v, im_v = im ? v : other;
+                    R re_o = im ? old_other : old, im_o = im ? old : old_other;
+                    R out = im ? (ar * im_v + ai * re_v) : (ar * re_v - ai * im_v);
+                    if (g.use_beta) out += im ? (br * im_o + bi * re_o) : (br * re_o - bi * im_o);
+                    if (ok) *dst = out;
+                } else {
+                    if (ok) {
+                        R out = ar * v;
+                        if (g.use_beta) out += br * *dst;
+                        *dst = out;
+                    }
+                }
+            }
+        }
+}
+
+// Sums split-K partials in split order and applies alpha/beta.  One thread per element.
+template <class R, bool CX>
+__global__ void __launch_bounds__(THREADS) splitk_finalize_kernel(GemmArgs g) {
+    const int64_t total = g.nbatch * g.M * g.N;
+    const int64_t idx = (int64_t)blockIdx.x * THREADS + threadIdx.x;
+    if (idx >= total) return;
+    const int64_t n = idx % g.N, t = idx / g.N, m = t % g.M, b = t / g.M;
+    constexpr int NC = CX ? 2 : 1;
+    const R* P = reinterpret_cast<const R*>(g.partial);
+    const int64_t plane = g.nbatch * g.M * g.N * NC;
+    R sr = 0, si = 0;
+    for (int s = 0; s < g.nsplit; ++s) {
+        const R* p = P + s * plane + ((b * g.M + m) * g.N + n) * NC;
+        sr += p[0];
+        if (CX) si += p[1];
+    }
+    R* dst = reinterpret_cast<R*>(g.C) + (off_of(g.cb, b) + off_of(g.cm, m) + off_of(g.cn, n)) * NC;
+    const R ar = (R)g.alpha_re, ai = (R)g.alpha_im, br = (R)g.beta_re, bi = (R)g.beta_im;
+    if (CX) {
+        R rr = ar * sr - ai * si, ri = ar * si + ai * sr;
+        if (g.use_beta) {
+            R cr = dst[0], ci = dst[1];
+            rr += br * cr - bi * ci;
+            ri += br * ci + bi * cr;
+        }
+        dst[0] = rr;
+        dst[1] = ri;
+    } else {
+        R r = ar * sr;
+        if (g.use_beta) r += br * dst[0];
+        dst[0] = r;
+    }
+}
+
+// Offsets of every fused index of an axis group (last axis fastest): tab[i] = sum_d idx_d * stride_d.
+struct TableJob {
+    int64_t* dst;
+    int64_t n;
+    int32_t naxes;
+    int64_t dims[TFH_MAX_RANK], strides[TFH_MAX_RANK];
+};
+__global__ void __launch_bounds__(THREADS) build_table_kernel(TableJob j) {
+    int64_t i = (int64_t)blockIdx.x * THREADS + threadIdx.x;
+    if (i >= j.n) return;
+    int64_t lin = i, off = 0;
+    for (int d = j.naxes - 1; d >= 0; --d) {
+        int64_t q = lin / j.dims[d];
+        off += (lin - q * j.dims[d]) * j.strides[d];
+        lin = q;
+    }
+    j.dst[i] = off;
+}
+
+int64_t prod(const std::vector<Axis>& ax) {
+    int64_t p = 1;
+    for (auto& a : ax) p *= a.n;
+    return p;
+}
+int64_t min_stride(const std::vector<Axis>& ax, int slot) {
+    int64_t m = INT64_MAX;
+    for (auto& a : ax)
+        if (a.n > 1 && a.s[slot] != 0) m = std::min<int64_t>(m, std::llabs(a.s[slot]));
+    return m;
+}
+void order_by(std::vector<Axis>& ax, int slot) {
+    // slowest first, fastest (smallest stride) last; zero strides first
+    std::stable_sort(ax.begin(), ax.end(), [slot](const Axis& x, const Axis& y) {
+        int64_t a = std::llabs(x.s[slot]), b = std::llabs(y.s[slot]);
+        if (a == 0) a = INT64_MAX;
+        if (b == 0) b = INT64_MAX;
+        return a > b;
+    });
+}
+
+template <class R, bool CX, int BM, int BN>
+void launch_tile(const GemmArgs& g, dim3 grid, hipStream_t st) {
+    size_t lds = Cfg<R, CX, BM, BN>::LDS_BYTES;
+    static bool once = [] {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<R, CX, BM, BN>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg<R, CX, BM, BN>::LDS_BYTES);
+        return true;
+    }();
+    (void)once;
+    hipLaunchKernelGGL((gemm_kernel<R, CX, BM, BN>), grid, dim3(THREADS), lds, st, g);
+}
+
+template <class R, bool CX>
+void launch_any_tile(const GemmArgs& g, dim3 grid, int bm, hipStream_t st) {
+    if (bm == 128) launch_tile<R, CX, 128, 128>(g, grid, st);
+    else launch_tile<R, CX, 64, 64>(g, grid, st);
+}
+
+void launch_dtype(int dtype, const GemmArgs& g, dim3 grid, int bm, hipStream_t st) {
+    switch (dtype) {
+        case TFH_F32: launch_any_tile<float, false>(g, grid, bm, st); break;
+        case TFH_F64: launch_any_tile<double, false>(g, grid, bm, st); break;
+        case TFH_C64: launch_any_tile<float, true>(g, grid, bm, st); break;
+        default: launch_any_tile<double, true>(g, grid, bm, st); break;
+    }
+}
+
+int bke_of(int dtype) {
+    int bkr = is_double(dtype) ? 16 : 32;
+    return is_complex(dtype) ? bkr / 2 : bkr;
+}
+
+}  // namespace
+
+int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes ax, Scalar alpha, Scalar beta,
+                        void* stream) {
+    const int rb = is_double(dtype) ? 8 : 4;
+    const size_t eb = dtype_size(dtype);
+    if (((uintptr_t)a % eb) || ((uintptr_t)b % eb) || ((uintptr_t)c % rb))
+        return set_error(TFH_ERR_STRIDED, "view base is not aligned to the element size");
+    hipStream_t st = (hipStream_t)stream;
+    int64_t nb = prod(ax.batch), M = prod(ax.M), N = prod(ax.N), K = prod(ax.K);
+    if (nb == 0 || M == 0 || N == 0) return TFH_OK;
+    for (auto* grp : {&ax.batch, &ax.M, &ax.N})
+        for (auto& x : *grp)
+            if (x.n > 1 && x.s[2] == 0) return set_error(TFH_ERR_STRIDED, "output view has stride 0 on an axis of extent %lld", (long long)x.n);
+    if (K == 0) {
+        // empty sum: C = beta*C
+        std::vector<Axis> out;
+        for (auto* grp : {&ax.batch, &ax.M, &ax.N})
+            for (auto& x : *grp) out.push_back(Axis{x.n, {x.s[2], x.s[2], 0}, x.label});
+        if (beta.is_zero()) return launch_fill(dtype, c, out, Scalar{0, 0}, stream);
+        return launch_copy(dtype, c, c, out, beta, Scalar{0, 0}, false, stream);
+    }
+    // lanes of the epilogue run along n: put C's fastest axis in the N group (swap operands if needed)
+    if (min_stride(ax.M, 2) < min_stride(ax.N, 2)) {
+        std::swap(a, b);
+        std::swap(ax.M, ax.N);
+        std::swap(M, N);
+        for (auto* grp : {&ax.batch, &ax.M, &ax.N, &ax.K})
+            for (auto& x : *grp) std::swap(x.s[0], x.s[1]);
+    }
+    // loaders run their lanes along k when the operand is contiguous in k, along the row index otherwise
+    const bool a_kfast = min_stride(ax.K, 0) <= min_stride(ax.M, 0);
+    const bool b_kfast = min_stride(ax.K, 1) <= min_stride(ax.N, 1);
+    order_by(ax.M, a_kfast ? 2 : 0);
+    order_by(ax.N, 2);
+    order_by(ax.K, a_kfast ? 0 : (b_kfast ? 1 : 0));
+    order_by(ax.batch, 2);
+    fuse_axes(ax.M, 3);
+    fuse_axes(ax.N, 3);
+    fuse_axes(ax.K, 3);
+    fuse_axes(ax.batch, 3);
+
+    GemmArgs g;
+    std::memset(&g, 0, sizeof g);
+    g.A = a; g.B = b; g.C = c;
+    g.M = M; g.N = N; g.K = K; g.nbatch = nb;
+    g.a_kfast = a_kfast; g.b_kfast = b_kfast;
+    g.alpha_re = alpha.re; g.alpha_im = alpha.im; g.beta_re = beta.re; g.beta_im = beta.im;
+    g.use_beta = !beta.is_zero();
+
+    // tile shape, split-K
+    const bool cx = is_complex(dtype);
+    const int64_t NR = cx ? 2 * N : N;
+    int bm = (M >= 96 && NR >= 96) ? 128 : 64;
+    auto tiles_for = [&](int t) { return ((M + t - 1) / t) * ((NR + t - 1) / t) * nb; };
+    const int bke = bke_of(dtype);
+    const int64_t kstages = (K + bke - 1) / bke;
+    // too few 128x128 tiles to fill 256 CUs and too little k to split: fall back to 64x64 tiles
+    if (bm == 128 && tiles_for(128) < 192 && kstages < 32 && tiles_for(64) >= 2 * tiles_for(128)) bm = 64;
+    const int64_t tiles = tiles_for(bm);
+    int nsplit = 1;
+    if (tiles < 256 && kstages >= 16) {
+        nsplit = (int)std::min<int64_t>((512 + tiles - 1) / tiles, kstages / 8);
+        nsplit = std::max(1, std::min(nsplit, 64));
+    }
+    int64_t kps = ((kstages + nsplit - 1) / nsplit) * bke;
+    nsplit = (int)((K + kps - 1) / kps);
+    g.nsplit = nsplit;
+    g.k_per_split = kps;
+    g.tiles_m = (int)((M + bm - 1) / bm);
+    g.tiles_n = (int)((NR + bm - 1) / bm);
+    if ((int64_t)g.tiles_m * g.tiles_n > 0x7fffffffll || nb * nsplit > 65535)
+        return set_error(TFH_ERR_INVALID_ARGUMENT, "contraction too large for one launch (tiles %lld, batch*split %lld)",
+                         (long long)g.tiles_m * g.tiles_n, (long long)(nb * nsplit));
+
+    // workspace: offset tables for every multi-axis group, then the split-K partials
+    struct Want { std::vector<Axis>* grp; int slot; OffFn* fn; int64_t n; };
+    Want wants[9] = {{&ax.M, 0, &g.am, M}, {&ax.K, 0, &g.ak, K}, {&ax.K, 1, &g.bk, K}, {&ax.N, 1, &g.bn, N}, {&ax.M, 2, &g.cm, M},
+                     {&ax.N, 2, &g.cn, N}, {&ax.batch, 0, &g.ab, nb}, {&ax.batch, 1, &g.bb, nb}, {&ax.batch, 2, &g.cb, nb}};
+    size_t table_bytes = 0;
+    for (auto& w : wants)
+        if (w.grp->size() > 1) table_bytes += ((size_t)w.n * sizeof(int64_t) + 255) & ~(size_t)255;
+    size_t partial_bytes = nsplit > 1 ? (size_t)nsplit * nb * M * NR * rb : 0;
+    char* ws = nullptr;
+    if (table_bytes + partial_bytes) {
+        void* p = nullptr;
+        if (int32_t e = workspace(stream, table_bytes + partial_bytes, &p)) return e;
+        ws = (char*)p;
+    }
+    size_t cursor = 0;
+    for (auto& w : wants) {
+        if (w.grp->size() <= 1) {
+            w.fn->tab = nullptr;
+            w.fn->stride = w.grp->empty() ? 0 : (*w.grp)[0].s[w.slot];
+            continue;
+        }
+        TableJob j;
+        std::memset(&j, 0, sizeof j);
+        j.dst = (int64_t*)(ws + cursor);
+        j.n = w.n;
+        j.naxes = (int)w.grp->size();
+        for (int d = 0; d < j.naxes; ++d) {
+            j.dims[d] = (*w.grp)[d].n;
+            j.strides[d] = (*w.grp)[d].s[w.slot];
+        }
+        hipLaunchKernelGGL(build_table_kernel, dim3((uint32_t)((w.n + THREADS - 1) / THREADS)), dim3(THREADS), 0, st, j);
+        w.fn->tab = j.dst;
+        w.fn->stride = 0;
+        cursor += ((size_t)w.n * sizeof(int64_t) + 255) & ~(size_t)255;
+    }
+    if (nsplit > 1) g.partial = ws + cursor;
+    dim3 grid((uint32_t)(g.tiles_m * g.tiles_n), 1, (uint32_t)(nb * nsplit));
+    launch_dtype(dtype, g, grid, bm, st);
+    if (int32_t e = hip_check(hipGetLastError(), "contraction kernel launch")) return e;
+    if (nsplit > 1) {
+        int64_t total = nb * M * N;
+        dim3 g2((uint32_t)((total + THREADS - 1) / THREADS));
+        switch (dtype) {
+            case TFH_F32: hipLaunchKernelGGL((splitk_finalize_kernel<float, false>), g2, dim3(THREADS), 0, st, g); break;
+            case TFH_F64: hipLaunchKernelGGL((splitk_finalize_kernel<double, false>), g2, dim3(THREADS), 0, st, g); break;
+            case TFH_C64: hipLaunchKernelGGL((splitk_finalize_kernel<float, true>), g2, dim3(THREADS), 0, st, g); break;
+            default: hipLaunchKernelGGL((splitk_finalize_kernel<double, true>), g2, dim3(THREADS), 0, st, g); break;
+        }
+        if (int32_t e = hip_check(hipGetLastError(), "split-K finalize launch")) return e;
+    }
+    return TFH_OK;
+}
+
+// ---- grouped launch ------------------------------------------------------------------------------------------
+struct GroupedState {
+    std::vector<int4> tile_map_host;
+    int bm = 128;
+    std::mutex mu;
+    int4* tile_map_dev = nullptr;       // uploaded on first execute
+    GroupProblem* problems_dev = nullptr;
+    int device = -1;
+};
+
+void grouped_state_destroy(GroupedState* s) {
+    if (!s) return;
+    if (s->tile_map_dev) (void)hipFree(s->tile_map_dev);
+    if (s->problems_dev) (void)hipFree(s->problems_dev);
+    delete s;
+}
+
+int32_t grouped_plan_init(tfh_plan& plan) {
+    // Tile list over all problems, heaviest tiles (largest K) first so the tail of the launch is short.
+    auto* gs = new (std::nothrow) GroupedState();
+    if (!gs) return set_error(TFH_ERR_DEVICE, "out of host memory");
+    const bool cx = is_complex(plan.dtype);
+    struct T { int p, tm, tn; int64_t k; };
+    std::vector<T> tiles;
+    int64_t small = 0;
+    std::vector<std::array<int64_t, 3>> mnk((size_t)plan.n_groups);
+    for (int gi = 0; gi < plan.n_groups; ++gi) {
+        // extents of the fused groups from the labels: batch modes are not allowed in a grouped plan
+        const auto& sa = plan.shapes[(size_t)gi * 3 + 0];
+        const auto& sb = plan.shapes[(size_t)gi * 3 + 1];
+        int64_t M = 1, N = 1, K = 1;
+        for (size_t d = 0; d < plan.modes_a.size(); ++d) {
+            uint32_t l = plan.modes_a[d];
+            bool in_b = std::find(plan.modes_b.begin(), plan.modes_b.end(), l) != plan.modes_b.end();
+            bool in_c = std::find(plan.modes_c.begin(), plan.modes_c.end(), l) != plan.modes_c.end();
+            if (in_b && in_c) {
+                delete gs;
+                return set_error(TFH_ERR_INVALID_ARGUMENT, "grouped contraction does not take batch modes (mode %u)", l);
+            }
+            if (in_c) M *= sa[d];
+            else K *= sa[d];
+        }
+        for (size_t d = 0; d < plan.modes_b.size(); ++d) {
+            uint32_t l = plan.modes_b[d];
+            bool in_a = std::find(plan.modes_a.begin(), plan.modes_a.end(), l) != plan.modes_a.end();
+            bool in_c = std::find(plan.modes_c.begin(), plan.modes_c.end(), l) != plan.modes_c.end();
+            if (in_c) N *= sb[d];
+            else if (!in_a) K *= sb[d];
+        }
+        mnk[(size_t)gi] = {M, N, K};
+        if (M < 96 || (cx ? 2 * N : N) < 96) ++small;
+    }
+    gs->bm = small * 2 > plan.n_groups ? 64 : 128;
+    for (int gi = 0; gi < plan.n_groups; ++gi) {
+        int64_t M = mnk[(size_t)gi][0], N = mnk[(size_t)gi][1], K = mnk[(size_t)gi][2];
+        int64_t NR = cx ? 2 * N : N;
+        for (int64_t tm = 0; tm * gs->bm < M; ++tm)
+            for (int64_t tn = 0; tn * gs->bm < NR; ++tn) tiles.push_back({gi, (int)tm, (int)tn, K});
+    }
+    std::stable_sort(tiles.begin(), tiles.end(), [](const T& x, const T& y) { return x.k > y.k; });
+    for (auto& t : tiles) gs->tile_map_host.push_back(make_int4(t.p, t.tm, t.tn, 0));
+    plan.grouped = gs;
+    return TFH_OK;
+}
+
+namespace {
+// Writes a batch of problem records into device memory from kernel arguments (no host staging buffer,
+// so the call is asynchronous and capturable).
+constexpr int PROBS_PER_SET = 32;
+struct ProblemSet {
+    GroupProblem p[PROBS_PER_SET];
+    int32_t first, count;
+};
+__global__ void set_problems_kernel(GroupProblem* dst, ProblemSet s) {
+    int i = threadIdx.x;
+    if (i < s.count) dst[s.first + i] = s.p[i];
+}
+}  // namespace
+
+int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* inputs, Scalar beta, tfh_view* outputs,
+                       void* stream) {
+    GroupedState* gs = plan.grouped;
+    hipStream_t st = (hipStream_t)stream;
+    const int dtype = plan.dtype;
+    const size_t eb = dtype_size(dtype);
+    std::vector<GroupProblem> probs((size_t)plan.n_groups);
+    for (int gi = 0; gi < plan.n_groups; ++gi) {
+        const tfh_view& va = inputs[(size_t)gi * 2 + 0];
+        const tfh_view& vb = inputs[(size_t)gi * 2 + 1];
+        const tfh_view& vc = outputs[gi];
+        if (int32_t e = check_view_against(plan.shapes[(size_t)gi * 3 + 0], va, "grouped input A")) return e;
+        if (int32_t e = check_view_against(plan.shapes[(size_t)gi * 3 + 1], vb, "grouped input B")) return e;
+        if (int32_t e = check_view_against(plan.shapes[(size_t)gi * 3 + 2], vc, "grouped output")) return e;
+        ContractAxes ax;
+        if (int32_t e = classify_contract(plan.modes_a, va.dims, va.strides, plan.modes_b, vb.dims, vb.strides, plan.modes_c,
+                                          vc.dims, vc.strides, ax))
+            return e;
+        order_by(ax.M, 2);
+        order_by(ax.N, 2);
+        order_by(ax.K, 0);
+        fuse_axes(ax.M, 3);
+        fuse_axes(ax.N, 3);
+        fuse_axes(ax.K, 3);
+        if (ax.M.size() > 1 || ax.N.size() > 1 || ax.K.size() > 1 || !ax.batch.empty())
+            return set_error(TFH_ERR_INVALID_ARGUMENT, "grouped contraction: operands of group %d are not plain strided matrices", gi);
+        GroupProblem& p = probs[(size_t)gi];
+        p.A = view_ptr(va, dtype);
+        p.B = view_ptr(vb, dtype);
+        p.C = view_ptr(vc, dtype);
+        if (((uintptr_t)p.A % eb) || ((uintptr_t)p.B % eb) || ((uintptr_t)p.C % eb))
+            return set_error(TFH_ERR_STRIDED, "view base is not aligned to the element size");
+        p.M = prod(ax.M); p.N = prod(ax.N); p.K = prod(ax.K);
+        p.sam = ax.M.empty() ? 0 : ax.M[0].s[0];
+        p.scm = ax.M.empty() ? 0 : ax.M[0].s[2];
+        p.sbn = ax.N.empty() ? 0 : ax.N[0].s[1];
+        p.scn = ax.N.empty() ? 0 : ax.N[0].s[2];
+        p.sak = ax.K.empty() ? 0 : ax.K[0].s[0];
+        p.sbk = ax.K.empty() ? 0 : ax.K[0].s[1];
+        if ((p.M > 1 && p.scm == 0) || (p.N > 1 && p.scn == 0)) return set_error(TFH_ERR_STRIDED, "output view has stride 0");
+    }
+    {
+        std::lock_guard<std::mutex> lk(gs->mu);
+        int dev = 0;
+        if (int32_t e = hip_check(hipGetDevice(&dev), "hipGetDevice")) return e;
+        if (!gs->tile_map_dev || gs->device != dev) {
+            if (gs->tile_map_dev) (void)hipFree(gs->tile_map_dev);
+            if (gs->problems_dev) (void)hipFree(gs->problems_dev);
+            gs->tile_map_dev = nullptr;
+            gs->problems_dev = nullptr;
+            size_t nb = gs->tile_map_host.size() * sizeof(int4);
+            if (int32_t e = hip_check(hipMalloc((void**)&gs->tile_map_dev, std::max<size_t>(nb, 16)), "hipMalloc(tile map)")) return e;
+            if (int32_t e = hip_check(hipMalloc((void**)&gs->problems_dev, sizeof(GroupProblem) * (size_t)plan.n_groups), "hipMalloc(problem table)")) return e;
+            if (nb)
+                if (int32_t e = hip_check(hipMemcpy(gs->tile_map_dev, gs->tile_map_host.data(), nb, hipMemcpyHostToDevice), "upload tile map")) return e;
+            gs->device = dev;
+        }
+    }
+    if (gs->tile_map_host.empty()) return TFH_OK;
+    for (int first = 0; first < plan.n_groups; first += PROBS_PER_SET) {
+        ProblemSet s;
+        s.first = first;
+        s.count = std::min(PROBS_PER_SET, plan.n_groups - first);
+        std::memcpy(s.p, probs.data() + first, sizeof(GroupProblem) * (size_t)s.count);
+        hipLaunchKernelGGL(set_problems_kernel, dim3(1), dim3(64), 0, st, gs->problems_dev, s);
+    }
+    GemmArgs g;
+    std::memset(&g, 0, sizeof g);
+    g.nbatch = 1;
+    g.nsplit = 1;
+    g.a_kfast = 1;   // per-problem choice is not available in one launch: assume row-major operands,
+    g.b_kfast = 0;   // i.e. A contiguous in k, B contiguous in n (the block-sparse "ij,jk->ik" case)
+    // pick the mapping from the first problem's strides
+    g.a_kfast = std::llabs(probs[0].sak) <= std::llabs(probs[0].sam) || probs[0].M == 1;
+    g.b_kfast = std::llabs(probs[0].sbk) <= std::llabs(probs[0].sbn) || probs[0].N == 1;
+    g.alpha_re = alpha.re; g.alpha_im = alpha.im; g.beta_re = beta.re; g.beta_im = beta.im;
+    g.use_beta = !beta.is_zero();
+    g.problems = gs->problems_dev;
+    g.tile_map = gs->tile_map_dev;
+    dim3 grid((uint32_t)gs->tile_map_host.size(), 1, 1);
+    launch_dtype(dtype, g, grid, gs->bm, st);
+    return hip_check(hipGetLastError(), "grouped contraction launch");
+}
+
+}  // namespace tfh

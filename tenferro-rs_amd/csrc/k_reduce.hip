@@ -1,0 +1,433 @@
+// k_reduce.hip -- multi-axis strided reduction for gfx950: PrimDescriptor::Reduce
+// (tenferro-prims/src/lib.rs:170-180), C[kept] = alpha*reduce_op(A[kept, reduced]) + beta*C.
+//
+// The 256 threads of a block tile the axes that are fastest in A's memory (kept or reduced alike), so
+// every wave reads contiguous runs.  A thread walks the remaining reduced extent serially (odometer,
+// no division in the loop), lanes that share an output combine through an LDS tree over the thread-id
+// bits that belong to reduced axes, and the lanes whose reduced bits are zero write the output.
+// When few outputs meet a long reduction the reduced range is split over blockIdx.y into partial
+// results that a second small kernel folds in a fixed order (deterministic, no atomics).
+// HBM-bound: algorithmic bytes = (input elements + output elements) * sizeof(T).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+
+#include "internal.hpp"
+
+namespace tfh {
+namespace {
+
+constexpr int MAXT = 4;
+constexpr int MAXG = 16;
+constexpr int MAXR = 4;  // serial (outer) reduced axes
+constexpr int THREADS = 256;
+
+struct ReduceArgs {
+    const void* in;
+    void* out;
+    double* partial;       // [nchunks][kept_slots] accumulators (complex: 2 doubles each)
+    int32_t nt, ng, nr;
+    int32_t tile_elems;
+    int32_t red_bits;      // thread-id bits owned by reduced tile axes
+    int32_t op;
+    int32_t nchunks;
+    int32_t use_beta;
+    // thread tile, in A-memory order
+    int32_t t_shift[MAXT], t_mask[MAXT], t_red[MAXT];
+    int64_t t_sa[MAXT], t_sc[MAXT], t_n[MAXT];
+    // kept outer axes -> blockIdx.x
+    int64_t g_count[MAXG], g_sa[MAXG], g_sc[MAXG];
+    int32_t g_tid[MAXG], g_text[MAXG];
+    // serial reduced axes (innermost first)
+    int64_t r_count[MAXR], r_sa[MAXR], r_n[MAXR];
+    int32_t r_tid[MAXR], r_text[MAXR];
+    int64_t r_total;       // product of r_count
+    int64_t kept_slots;    // gridDim.x * kept lanes per block
+    double alpha_re, alpha_im, beta_re, beta_im;
+};
+
+template <bool CX>
+struct Acc {
+    double re, im;
+};
+
+__device__ __forceinline__ double combine(double a, double b, int op) {
+    return op == TFH_REDUCE_SUM ? a + b : (op == TFH_REDUCE_MAX ? fmax(a, b) : fmin(a, b));
+}
+__device__ __forceinline__ double identity(int op) {
+    return op == TFH_REDUCE_SUM ? 0.0 : (op == TFH_REDUCE_MAX ? -INFINITY : INFINITY);
+}
+
+struct ThreadPos {
+    int64_t in, out;      // element offsets of this thread (block origin + in-tile position)
+    int64_t lim[MAXT];    // remaining extent of each tile axis at this block
+    int32_t tc[MAXT];     // in-tile coordinate per tile axis
+    bool ok;              // inside the tensor on every kept tile axis
+    bool red_ok;          // inside the tensor on every reduced tile axis
+    int32_t kept_lane;    // index of this thread among the block's kept lanes
+    bool writer;          // reduced bits all zero
+};
+
+__device__ __forceinline__ ThreadPos thread_pos(const ReduceArgs& a) {
+    ThreadPos p;
+    p.in = p.out = 0;
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) p.lim[t] = t < a.nt ? a.t_n[t] : 1;
+    uint64_t bid = blockIdx.x;
+    for (int g = 0; g < a.ng; ++g) {
+        uint64_t q = bid / (uint64_t)a.g_count[g];
+        int64_t c = (int64_t)(bid - q * (uint64_t)a.g_count[g]);
+        bid = q;
+        p.in += c * a.g_sa[g];
+        p.out += c * a.g_sc[g];
+        int t = a.g_tid[g];
+#pragma unroll
+        for (int k = 0; k < MAXT; ++k)
+            if (k == t) p.lim[k] -= c * a.g_text[g];
+    }
+    const int tid = threadIdx.x;
+    p.ok = tid < a.tile_elems;
+    p.writer = true;
+    p.red_ok = true;
+    p.kept_lane = 0;
+    int kshift = 0;
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) {
+        p.tc[t] = 0;
+        if (t < a.nt) {
+            int c = (tid >> a.t_shift[t]) & a.t_mask[t];
+            p.tc[t] = c;
+            p.in += (int64_t)c * a.t_sa[t];
+            if (a.t_red[t]) {
+                p.writer &= c == 0;
+                p.red_ok &= c < a.t_n[t];
+            } else {
+                p.out += (int64_t)c * a.t_sc[t];
+                p.ok &= c < p.lim[t];
+                p.kept_lane |= c << kshift;
+                kshift += __popc(a.t_mask[t]);
+            }
+        }
+    }
+    return p;
+}
+
+template <class R, bool CX>
+__global__ void __launch_bounds__(THREADS) reduce_kernel(ReduceArgs a) {
+    constexpr int NC = CX ? 2 : 1;
+    __shared__ double lds[THREADS * NC];
+    const ThreadPos p = thread_pos(a);
+    const R* A = reinterpret_cast<const R*>(a.in) + p.in * NC;
+    const int op = a.op;
+    double acc_re = identity(op), acc_im = 0.0;
+    // this block's slice of the serial reduced range
+    const int64_t per = (a.r_total + a.nchunks - 1) / a.nchunks;
+    const int64_t it0 = (int64_t)blockIdx.y * per;
+    const int64_t it1 = it0 + per < a.r_total ? it0 + per : a.r_total;
+    // odometer start
+    int64_t c[MAXR];
+    int64_t off = 0;
+    {
+        int64_t lin = it0;
+#pragma unroll
+        for (int r = 0; r < MAXR; ++r) {
+            c[r] = 0;
+            if (r < a.nr) {
+                int64_t q = lin / a.r_count[r];
+                c[r] = lin - q * a.r_count[r];
+                lin = q;
+                off += c[r] * a.r_sa[r];
+            }
+        }
+    }
+    // in-tile coordinate of this thread along the tile axis each serial axis extends (0 if none)
+    int64_t tcr[MAXR];
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) {
+        tcr[r] = 0;
+        if (r < a.nr) {
+            int t = a.r_tid[r];
+#pragma unroll
+            for (int k = 0; k < MAXT; ++k)
+                if (k == t) tcr[r] = p.tc[k];
+        }
+    }
+    const bool load_ok = p.ok && p.red_ok;
+    constexpr int U = 8;  // independent loads in flight per thread
+    for (int64_t it = it0; it < it1; it += U) {
+        int64_t offs[U];
+        bool oks[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            bool ok = load_ok && it + u < it1;
+#pragma unroll
+            for (int r = 0; r < MAXR; ++r)
+                if (r < a.nr) ok &= c[r] * a.r_text[r] + tcr[r] < a.r_n[r];
+            oks[u] = ok;
+            offs[u] = off;
+            // advance the odometer
+            off += a.r_sa[0];
+            if (++c[0] == a.r_count[0]) {
+                off -= a.r_sa[0] * a.r_count[0];
+                c[0] = 0;
+#pragma unroll
+                for (int r = 1; r < MAXR; ++r) {
+                    if (r < a.nr) {
+                        off += a.r_sa[r];
+                        if (++c[r] < a.r_count[r]) break;
+                        off -= a.r_sa[r] * a.r_count[r];
+                        c[r] = 0;
+                    }
+                }
+            }
+        }
+        R vre[U], vim[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            vre[u] = vim[u] = R(0);
+            if (oks[u]) {
+                vre[u] = A[offs[u] * NC];
+                if (CX) vim[u] = A[offs[u] * NC + 1];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (oks[u]) {
+                if (CX) {
+                    acc_re += (double)vre[u];
+                    acc_im += (double)vim[u];
+                } else {
+                    acc_re = combine(acc_re, (double)vre[u], op);
+                }
+            }
+        }
+    }
+    // combine lanes that share an output: tree over the reduced thread-id bits
+    const int tid = threadIdx.x;
+    if (a.red_bits) {
+        lds[tid * NC] = acc_re;
+        if (CX) lds[tid * NC + 1] = acc_im;
+        __syncthreads();
+        for (int b = 7; b >= 0; --b) {
+            const int bit = 1 << b;
+            if (a.red_bits & bit) {
+                if (!(tid & bit)) {
+                    lds[tid * NC] = combine(lds[tid * NC], lds[(tid | bit) * NC], op);
+                    if (CX) lds[tid * NC + 1] += lds[(tid | bit) * NC + 1];
+                }
+                __syncthreads();
+            }
+        }
+        acc_re = lds[tid * NC];
+        if (CX) acc_im = lds[tid * NC + 1];
+    }
+    if (!(p.writer && p.ok)) return;
+    if (a.nchunks > 1) {
+        int64_t slot = ((int64_t)blockIdx.y * a.kept_slots + (int64_t)blockIdx.x * THREADS + p.kept_lane) * NC;
+        a.partial[slot] = acc_re;
+        if (CX) a.partial[slot + 1] = acc_im;
+        return;
+    }
+    R* C = reinterpret_cast<R*>(a.out) + p.out * NC;
+    if (CX) {
+        double rr = a.alpha_re * acc_re - a.alpha_im * acc_im, ri = a.alpha_re * acc_im + a.alpha_im * acc_re;
+        if (a.use_beta) {
+            double cr = C[0], ci = C[1];
+            rr += a.beta_re * cr - a.beta_im * ci;
+            ri += a.beta_re * ci + a.beta_im * cr;
+        }
+        C[0] = (R)rr;
+        C[1] = (R)ri;
+    } else {
+        double r = a.alpha_re * acc_re;
+        if (a.use_beta) r += a.beta_re * (double)C[0];
+        C[0] = (R)r;
+    }
+}
+
+// Second pass of a split reduction: fold the partials of every chunk, in chunk order.
+template <class R, bool CX>
+__global__ void __launch_bounds__(THREADS) reduce_finalize_kernel(ReduceArgs a) {
+    constexpr int NC = CX ? 2 : 1;
+    const ThreadPos p = thread_pos(a);
+    if (!(p.writer && p.ok)) return;
+    const int op = a.op;
+    double acc_re = identity(op), acc_im = 0.0;
+    for (int ch = 0; ch < a.nchunks; ++ch) {
+        int64_t slot = ((int64_t)ch * a.kept_slots + (int64_t)blockIdx.x * THREADS + p.kept_lane) * NC;
+        acc_re = combine(acc_re, a.partial[slot], op);
+        if (CX) acc_im += a.partial[slot + 1];
+    }
+    R* C = reinterpret_cast<R*>(a.out) + p.out * NC;
+    if (CX) {
+        double rr = a.alpha_re * acc_re - a.alpha_im * acc_im, ri = a.alpha_re * acc_im + a.alpha_im * acc_re;
+        if (a.use_beta) {
+            double cr = C[0], ci = C[1];
+            rr += a.beta_re * cr - a.beta_im * ci;
+            ri += a.beta_re * ci + a.beta_im * cr;
+        }
+        C[0] = (R)rr;
+        C[1] = (R)ri;
+    } else {
+        double r = a.alpha_re * acc_re;
+        if (a.use_beta) r += a.beta_re * (double)C[0];
+        C[0] = (R)r;
+    }
+}
+
+int ceil_log2(int64_t n) {
+    int l = 0;
+    while (((int64_t)1 << l) < n) ++l;
+    return l;
+}
+
+}  // namespace
+
+int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, std::vector<Axis> red, int reduce_op,
+                      Scalar alpha, Scalar beta, void* stream) {
+    const int rb = is_double(dtype) ? 8 : 4;
+    if (((uintptr_t)a % rb) || ((uintptr_t)c % rb)) return set_error(TFH_ERR_STRIDED, "view base is not aligned");
+    for (auto& x : kept)
+        if (x.n == 0) return TFH_OK;  // no outputs
+    int64_t nred = 1;
+    for (auto& x : red) nred *= x.n;
+    if (nred == 0) {
+        // empty reduction: every output is alpha*identity + beta*C; sum -> 0
+        if (reduce_op != TFH_REDUCE_SUM) return set_error(TFH_ERR_INVALID_ARGUMENT, "max/min over an empty extent");
+        red.clear();
+        // scale C by beta through the copy kernel (in = out, alpha = 0 is not safe for NaN; use fill when beta == 0)
+        std::vector<Axis> ax;
+        for (auto& x : kept) ax.push_back(Axis{x.n, {x.s[1], x.s[1], 0}, x.label});
+        if (beta.is_zero()) return launch_fill(dtype, c, ax, Scalar{0, 0}, stream);
+        return launch_copy(dtype, c, c, ax, beta, Scalar{0, 0}, false, stream);
+    }
+    // merge axes (kept and reduced separately; slot 0 = A, slot 1 = C)
+    std::stable_sort(kept.begin(), kept.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[1]) > std::llabs(y.s[1]); });
+    for (auto& x : kept) x.s[2] = 0;
+    fuse_axes(kept, 2);
+    for (auto& x : red) x.s[1] = x.s[2] = 0;
+    std::stable_sort(red.begin(), red.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[0]) > std::llabs(y.s[0]); });
+    fuse_axes(red, 1);
+    for (auto& x : kept)
+        if (x.s[1] == 0) return set_error(TFH_ERR_STRIDED, "output view has stride 0 on an axis of extent %lld", (long long)x.n);
+    struct Ax {
+        Axis a;
+        bool red;
+        int tl;  // log2 tile extent
+    };
+    std::vector<Ax> all;
+    for (auto& x : kept) all.push_back({x, false, 0});
+    for (auto& x : red) all.push_back({x, true, 0});
+    if ((int)all.size() > MAXG) return set_error(TFH_ERR_INVALID_ARGUMENT, "more than %d non-mergeable axes", MAXG);
+    auto key = [](const Ax& x) { return x.a.s[0] == 0 ? INT64_MAX : std::llabs(x.a.s[0]); };
+    std::stable_sort(all.begin(), all.end(), [&](const Ax& x, const Ax& y) { return key(x) < key(y); });
+    ReduceArgs ra;
+    std::memset(&ra, 0, sizeof ra);
+    int bits = 8, nt = 0;
+    for (auto& x : all) {
+        if (bits == 0 || nt == MAXT) break;
+        int t = std::min(ceil_log2(x.a.n), bits);
+        if (t == 0) continue;
+        x.tl = t;
+        bits -= t;
+        ++nt;
+    }
+    int shift = 0;
+    ra.nt = 0;
+    std::vector<int> tid_of(all.size(), -1);
+    for (size_t i = 0; i < all.size(); ++i) {
+        if (all[i].tl == 0) continue;
+        int t = ra.nt++;
+        tid_of[i] = t;
+        ra.t_shift[t] = shift;
+        ra.t_mask[t] = (1 << all[i].tl) - 1;
+        ra.t_red[t] = all[i].red;
+        ra.t_sa[t] = all[i].a.s[0];
+        ra.t_sc[t] = all[i].a.s[1];
+        ra.t_n[t] = all[i].a.n;
+        if (all[i].red) ra.red_bits |= ra.t_mask[t] << shift;
+        shift += all[i].tl;
+    }
+    ra.tile_elems = 1 << shift;
+    // kept outer axes -> grid.x ; reduced outer axes -> serial loop
+    uint64_t blocks = 1;
+    ra.r_total = 1;
+    for (int r = 0; r < MAXR; ++r) {
+        ra.r_count[r] = 1;
+        ra.r_n[r] = 1;
+        ra.r_text[r] = 1;
+        ra.r_tid[r] = -1;
+    }
+    for (size_t i = 0; i < all.size(); ++i) {
+        int64_t text = (int64_t)1 << all[i].tl;
+        int64_t cnt = (all[i].a.n + text - 1) / text;
+        if (cnt <= 1) continue;
+        if (all[i].red) {
+            if (ra.nr == MAXR) return set_error(TFH_ERR_INVALID_ARGUMENT, "more than %d non-mergeable reduced axes outside the thread tile", MAXR);
+            int r = ra.nr++;
+            ra.r_count[r] = cnt;
+            ra.r_sa[r] = all[i].a.s[0] * text;
+            ra.r_n[r] = all[i].a.n;
+            ra.r_tid[r] = tid_of[i];
+            ra.r_text[r] = (int32_t)text;
+            ra.r_total *= cnt;
+        } else {
+            int g = ra.ng++;
+            ra.g_count[g] = cnt;
+            ra.g_sa[g] = all[i].a.s[0] * text;
+            ra.g_sc[g] = all[i].a.s[1] * text;
+            ra.g_tid[g] = tid_of[i];
+            ra.g_text[g] = (int32_t)text;
+            blocks *= (uint64_t)cnt;
+        }
+    }
+    if (ra.nr == 0) ra.nr = 1;  // a single pass through the loop
+    if (blocks > 0x7fffffffull) return set_error(TFH_ERR_INVALID_ARGUMENT, "tensor too large for one launch");
+    // split a long serial range when there are too few blocks to fill 256 CUs
+    int nchunks = 1;
+    if (blocks < 1024 && ra.r_total >= 64) {
+        nchunks = (int)std::min<int64_t>((2048 + (int64_t)blocks - 1) / (int64_t)blocks, ra.r_total / 16);
+        nchunks = std::max(1, std::min(nchunks, 65535));
+    }
+    ra.nchunks = nchunks;
+    ra.kept_slots = (int64_t)blocks * THREADS;
+    ra.in = a;
+    ra.out = c;
+    ra.op = reduce_op;
+    ra.alpha_re = alpha.re;
+    ra.alpha_im = alpha.im;
+    ra.beta_re = beta.re;
+    ra.beta_im = beta.im;
+    ra.use_beta = !beta.is_zero();
+    const bool cx = is_complex(dtype);
+    if (nchunks > 1) {
+        void* ws = nullptr;
+        size_t bytes = (size_t)nchunks * (size_t)ra.kept_slots * (cx ? 2 : 1) * sizeof(double);
+        if (int32_t e = workspace(stream, bytes, &ws)) return e;
+        ra.partial = (double*)ws;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid((uint32_t)blocks, (uint32_t)nchunks, 1), block(THREADS);
+    switch (dtype) {
+        case TFH_F32: hipLaunchKernelGGL((reduce_kernel<float, false>), grid, block, 0, st, ra); break;
+        case TFH_F64: hipLaunchKernelGGL((reduce_kernel<double, false>), grid, block, 0, st, ra); break;
+        case TFH_C64: hipLaunchKernelGGL((reduce_kernel<float, true>), grid, block, 0, st, ra); break;
+        default: hipLaunchKernelGGL((reduce_kernel<double, true>), grid, block, 0, st, ra); break;
+    }
+    if (int32_t e = hip_check(hipGetLastError(), "reduce kernel launch")) return e;
+    if (nchunks > 1) {
+        dim3 g2((uint32_t)blocks, 1, 1);
+        switch (dtype) {
+            case TFH_F32: hipLaunchKernelGGL((reduce_finalize_kernel<float, false>), g2, block, 0, st, ra); break;
+            case TFH_F64: hipLaunchKernelGGL((reduce_finalize_kernel<double, false>), g2, block, 0, st, ra); break;
+            case TFH_C64: hipLaunchKernelGGL((reduce_finalize_kernel<float, true>), g2, block, 0, st, ra); break;
+            default: hipLaunchKernelGGL((reduce_finalize_kernel<double, true>), g2, block, 0, st, ra); break;
+        }
+        if (int32_t e = hip_check(hipGetLastError(), "reduce finalize launch")) return e;
+    }
+    return TFH_OK;
+}
+
+}  // namespace tfh

@@ -1,0 +1,201 @@
+// runtime.cpp -- device, memory, stream and event entry points of the C ABI plus the per-stream
+// scratch memory the kernels use.  Mirrors the device model of tenferro-device/src/lib.rs:30-105 and
+// the GPU-async vocabulary of tenferro-tensor/src/lib.rs:301-309, 660-713.
+#include <hip/hip_runtime.h>
+
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include "internal.hpp"
+
+namespace tfh {
+
+int32_t hip_check(int err, const char* what) {
+    if (err == hipSuccess) return TFH_OK;
+    return set_error(TFH_ERR_DEVICE, "%s: %s", what, hipGetErrorString((hipError_t)err));
+}
+
+namespace {
+struct StreamScratch {
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+    std::multimap<size_t, void*> free_blocks;   // cached intermediates by size
+    std::map<void*, size_t> live;
+};
+std::mutex g_mu;
+std::map<std::pair<int, void*>, StreamScratch> g_scratch;   // (device, stream)
+
+StreamScratch* scratch_for(void* stream, int32_t* err) {
+    int dev = 0;
+    *err = hip_check(hipGetDevice(&dev), "hipGetDevice");
+    if (*err) return nullptr;
+    return &g_scratch[{dev, stream}];
+}
+}  // namespace
+
+int32_t workspace(void* stream, size_t bytes, void** out) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    int32_t err;
+    StreamScratch* s = scratch_for(stream, &err);
+    if (!s) return err;
+    if (bytes > s->ws_bytes) {
+        if (s->ws) {
+            // kernels already enqueued may still read the old buffer
+            if (int32_t e = hip_check(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize")) return e;
+            (void)hipFree(s->ws);
+            s->ws = nullptr;
+            s->ws_bytes = 0;
+        }
+        size_t want = std::max<size_t>(bytes + bytes / 4, (size_t)1 << 20);
+        if (int32_t e = hip_check(hipMalloc(&s->ws, want), "hipMalloc(workspace)")) return e;
+        s->ws_bytes = want;
+    }
+    *out = s->ws;
+    return TFH_OK;
+}
+
+int32_t pool_alloc(void* stream, size_t bytes, void** out) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    int32_t err;
+    StreamScratch* s = scratch_for(stream, &err);
+    if (!s) return err;
+    bytes = std::max<size_t>((bytes + 255) & ~(size_t)255, 256);
+    auto it = s->free_blocks.lower_bound(bytes);
+    if (it != s->free_blocks.end() && it->first <= bytes + bytes / 4) {
+        *out = it->second;
+        s->live[*out] = it->first;
+        s->free_blocks.erase(it);
+        return TFH_OK;
+    }
+    void* p = nullptr;
+    if (int32_t e = hip_check(hipMalloc(&p, bytes), "hipMalloc(intermediate)")) return e;
+    s->live[p] = bytes;
+    *out = p;
+    return TFH_OK;
+}
+
+void pool_free(void* stream, void* ptr) {
+    if (!ptr) return;
+    std::lock_guard<std::mutex> lk(g_mu);
+    int32_t err;
+    StreamScratch* s = scratch_for(stream, &err);
+    if (!s) return;
+    auto it = s->live.find(ptr);
+    if (it == s->live.end()) return;
+    // stream-ordered reuse: the next user of this block is enqueued on the same stream
+    s->free_blocks.emplace(it->second, ptr);
+    s->live.erase(it);
+}
+
+}  // namespace tfh
+
+using tfh::hip_check;
+using tfh::set_error;
+
+extern "C" {
+
+int32_t tfh_release_workspaces(void) {
+    std::lock_guard<std::mutex> lk(tfh::g_mu);
+    if (int32_t e = hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize")) return e;
+    for (auto& kv : tfh::g_scratch) {
+        if (kv.second.ws) (void)hipFree(kv.second.ws);
+        kv.second.ws = nullptr;
+        kv.second.ws_bytes = 0;
+        for (auto& b : kv.second.free_blocks) (void)hipFree(b.second);
+        kv.second.free_blocks.clear();
+    }
+    return TFH_OK;
+}
+
+int32_t tfh_device_count(int32_t* n) {
+    if (!n) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
+    int c = 0;
+    hipError_t e = hipGetDeviceCount(&c);
+    if (e == hipErrorNoDevice) {
+        *n = 0;
+        (void)hipGetLastError();
+        return TFH_OK;
+    }
+    if (int32_t s = hip_check(e, "hipGetDeviceCount")) return s;
+    *n = c;
+    return TFH_OK;
+}
+
+int32_t tfh_set_device(int32_t device_id) { return hip_check(hipSetDevice(device_id), "hipSetDevice"); }
+
+int32_t tfh_preferred_compute_devices(int32_t space_kind, int64_t space_id, int32_t op_kind, tfh_compute_device* out,
+                                      int32_t cap, int32_t* n) {
+    // preferred_compute_devices(space, op_kind) (tenferro-device/src/lib.rs:92-105).  This library
+    // computes on HIP devices only: GpuMemory{id} -> [Hip{id}] when that device exists.
+    if (!n) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
+    *n = 0;
+    if (op_kind < TFH_KIND_CONTRACT || op_kind > TFH_KIND_ELEMENTWISE_MUL) return set_error(TFH_ERR_INVALID_ARGUMENT, "unknown OpKind %d", op_kind);
+    static const char* kinds[] = {"Contract", "BatchedGemm", "Reduce", "Trace", "Permute", "ElementwiseMul"};
+    if (space_kind == TFH_SPACE_GPU_MEMORY) {
+        int32_t count = 0;
+        if (int32_t e = tfh_device_count(&count)) return e;
+        if (space_id >= 0 && space_id < count) {
+            if (out && cap > 0) {
+                out[0].kind = TFH_DEVICE_HIP;
+                out[0].device_id = (int32_t)space_id;
+            }
+            *n = 1;
+            return TFH_OK;
+        }
+        return set_error(TFH_ERR_NO_COMPATIBLE_DEVICE, "no compatible compute device for %s on GpuMemory { space_id: %lld }",
+                         kinds[op_kind], (long long)space_id);
+    }
+    if (space_kind == TFH_SPACE_MAIN_MEMORY)
+        return set_error(TFH_ERR_NO_COMPATIBLE_DEVICE, "no compatible compute device for %s on MainMemory", kinds[op_kind]);
+    return set_error(TFH_ERR_INVALID_ARGUMENT, "unknown memory space kind %d", space_kind);
+}
+
+int32_t tfh_malloc(size_t bytes, void** out) {
+    if (!out) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
+    *out = nullptr;
+    return hip_check(hipMalloc(out, bytes ? bytes : 1), "hipMalloc");
+}
+int32_t tfh_free(void* ptr) { return hip_check(hipFree(ptr), "hipFree"); }
+int32_t tfh_memcpy_h2d(void* dst, const void* src, size_t bytes, tfh_stream stream) {
+    return hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream), "hipMemcpyAsync(h2d)");
+}
+int32_t tfh_memcpy_d2h(void* dst, const void* src, size_t bytes, tfh_stream stream) {
+    return hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream), "hipMemcpyAsync(d2h)");
+}
+int32_t tfh_memcpy_d2d(void* dst, const void* src, size_t bytes, tfh_stream stream) {
+    return hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream), "hipMemcpyAsync(d2d)");
+}
+
+int32_t tfh_stream_create(tfh_stream* out) {
+    if (!out) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
+    hipStream_t s = nullptr;
+    if (int32_t e = hip_check(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreate")) return e;
+    *out = s;
+    return TFH_OK;
+}
+int32_t tfh_stream_destroy(tfh_stream s) { return hip_check(hipStreamDestroy((hipStream_t)s), "hipStreamDestroy"); }
+int32_t tfh_stream_synchronize(tfh_stream s) { return hip_check(hipStreamSynchronize((hipStream_t)s), "hipStreamSynchronize"); }
+
+int32_t tfh_event_create(tfh_event* out) {
+    if (!out) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
+    hipEvent_t e = nullptr;
+    if (int32_t s = hip_check(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreate")) return s;
+    *out = e;
+    return TFH_OK;
+}
+int32_t tfh_event_destroy(tfh_event e) { return hip_check(hipEventDestroy((hipEvent_t)e), "hipEventDestroy"); }
+int32_t tfh_event_record(tfh_event e, tfh_stream s) { return hip_check(hipEventRecord((hipEvent_t)e, (hipStream_t)s), "hipEventRecord"); }
+int32_t tfh_event_synchronize(tfh_event e) { return hip_check(hipEventSynchronize((hipEvent_t)e), "hipEventSynchronize"); }
+int32_t tfh_event_query(tfh_event e, int32_t* ready) {
+    if (!ready) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
+    hipError_t r = hipEventQuery((hipEvent_t)e);
+    if (r == hipSuccess) { *ready = 1; return TFH_OK; }
+    if (r == hipErrorNotReady) { *ready = 0; (void)hipGetLastError(); return TFH_OK; }
+    return hip_check(r, "hipEventQuery");
+}
+int32_t tfh_stream_wait_event(tfh_stream s, tfh_event e) {
+    return hip_check(hipStreamWaitEvent((hipStream_t)s, (hipEvent_t)e, 0), "hipStreamWaitEvent");
+}
+
+}  // extern "C"

@@ -1,0 +1,496 @@
+"""GPU parity: the HIP backend, called through the C ABI, against the CPU oracle on the same seeded
+inputs.  Bit-exact for data movement; relative Frobenius error <= 1e-12 for f64/complex128 and
+<= 1e-5 for f32/complex64 (the tolerances the backend is specified to)."""
+import itertools
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.float32: 1e-5, np.float64: 1e-12, np.complex64: 1e-5, np.complex128: 1e-12}
+ALL = [np.float32, np.float64, np.complex64, np.complex128]
+
+
+@pytest.fixture(scope="module")
+def tf():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import tenferro_rs_amd as tf
+    tf.lib()
+    return tf
+
+
+def rand(rng, shape, dtype):
+    x = rng.standard_normal(shape)
+    if np.issubdtype(dtype, np.complexfloating):
+        x = x + 1j * rng.standard_normal(shape)
+    return x.astype(dtype)
+
+
+def relerr(x, ref):
+    d = np.linalg.norm((np.asarray(x, np.complex128) - ref).ravel())
+    n = np.linalg.norm(np.asarray(ref).ravel())
+    return d / n if n > 0 else d
+
+
+def dev(tf, arr):
+    """Device Tensor with the same dims, element strides and offset as the numpy view `arr`."""
+    import torch
+    root = arr
+    while root.base is not None:
+        root = root.base
+    flat = np.ascontiguousarray(root).reshape(-1) if root.flags.c_contiguous else None
+    if flat is None or (arr.size and not np.shares_memory(flat, arr)):
+        arr = np.ascontiguousarray(arr)
+        flat = arr.reshape(-1)
+    isz = arr.dtype.itemsize
+    off = (arr.ctypes.data - flat.ctypes.data) // isz if arr.size else 0
+    buf = torch.from_numpy(flat.copy()).cuda()
+    return tf.Tensor(buf, list(arr.shape), [s // isz for s in arr.strides], off, tf.GpuMemory(0), tf.dtype_code(arr.dtype))
+
+
+def lab(s):
+    return [ord(c) for c in s]
+
+
+# ------------------------------------------------------------------------------------------------ permute
+@pytest.mark.parametrize("dtype", ALL)
+def test_permute_all_rank4_perms_bit_exact(tf, oracle, dtype):
+    rng = np.random.default_rng(21)
+    a = rand(rng, (5, 12, 7, 9), dtype)
+    da = dev(tf, a)
+    for perm in itertools.permutations(range(4)):
+        shape = [a.shape[p] for p in perm]
+        out = tf.Tensor.empty(shape, tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Permute([0, 1, 2, 3], list(perm)), [a.shape, shape])
+        tf.HipBackend.execute(plan, 1.0, [da], 0.0, out)
+        ref = np.empty(shape, dtype)
+        oracle.permute(a, [0, 1, 2, 3], ref, list(perm))
+        assert out.to_numpy().tobytes() == ref.tobytes(), perm
+
+
+@pytest.mark.parametrize("shape,perm", [((33, 65), (1, 0)), ((1, 7, 1, 5), (3, 2, 1, 0)), ((130, 3, 70), (2, 0, 1)),
+                                        ((4, 4, 4, 4, 4, 4, 4), (6, 2, 4, 0, 5, 1, 3)), ((2000,), (0,)), ((3, 1000), (1, 0)),
+                                        ((0, 5), (1, 0)), ((), ())])
+def test_permute_shapes_bit_exact(tf, oracle, shape, perm):
+    rng = np.random.default_rng(22)
+    a = rng.standard_normal(shape)
+    oshape = [shape[p] for p in perm]
+    out = tf.Tensor.empty(oshape, tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+    modes = list(range(len(shape)))
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute(modes, list(perm)), [shape, oshape])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, a)], 0.0, out)
+    ref = np.empty(oshape)
+    if a.size:
+        oracle.permute(a, modes, ref, list(perm))
+    assert out.to_numpy().tobytes() == ref.tobytes()
+
+
+def test_permute_special_values_bitwise(tf):
+    a = np.array([[0.0, -0.0, np.inf, 1.0], [-np.inf, np.nan, 5e-324, -1.0]])
+    out = tf.Tensor.empty([4, 2], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute([0, 1], [1, 0]), [[2, 4], [4, 2]])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, a)], 0.0, out)
+    assert out.to_numpy().tobytes() == np.ascontiguousarray(a.T).tobytes()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex128])
+def test_permute_strided_negative_alpha_beta_and_column_major(tf, oracle, dtype):
+    rng = np.random.default_rng(23)
+    big = rand(rng, (16, 18, 20), dtype)
+    a = big[::2, ::-1, 1:19:3]
+    b0 = np.asfortranarray(rand(rng, (a.shape[2], a.shape[0], a.shape[1]), dtype))   # column-major output
+    alpha, beta = (0.5 - 2j, 1.5 + 1j) if np.iscomplexobj(a) else (0.5, -1.5)
+    ref = b0.copy(order="F")
+    oracle.permute(a, [0, 1, 2], ref, [2, 0, 1], alpha=alpha, beta=beta)
+    db = dev(tf, b0.T).permute([2, 1, 0])
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Permute([0, 1, 2], [2, 0, 1]), [a.shape, b0.shape])
+    tf.HipBackend.execute(plan, alpha, [dev(tf, a)], beta, db)
+    assert relerr(db.to_numpy(), ref) < TOL[dtype]
+
+
+def test_permute_config2_full_size_bit_exact(tf, oracle):
+    # the 16^6 f64 tensor permuted to (5,2,0,4,1,3): bit-exact against the oracle, and the inverse permutation
+    # restores the input (involution)
+    from tenferro_rs_amd import inputs
+    a = inputs.uniform(1002, 0, (16,) * 6)
+    perm = [5, 2, 0, 4, 1, 3]
+    da = dev(tf, a)
+    out = tf.Tensor.empty([16] * 6, tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute(list(range(6)), perm), [[16] * 6, [16] * 6])
+    tf.HipBackend.execute(plan, 1.0, [da], 0.0, out)
+    ref = np.empty((16,) * 6)
+    oracle.permute(a, list(range(6)), ref, perm)
+    got = out.to_numpy()
+    assert got.tobytes() == ref.tobytes()
+    back = tf.Tensor.empty([16] * 6, tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+    inv = [int(i) for i in np.argsort(perm)]
+    plan2 = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute(list(range(6)), inv), [[16] * 6, [16] * 6])
+    tf.HipBackend.execute(plan2, 1.0, [out], 0.0, back)
+    assert back.to_numpy().tobytes() == a.tobytes()
+
+
+# ------------------------------------------------------------------------------------------------ reduce
+@pytest.mark.parametrize("dtype", ALL)
+def test_reduce_sum_keep_sets(tf, oracle, dtype):
+    rng = np.random.default_rng(24)
+    a = rand(rng, (6, 17, 5, 33), dtype)
+    da = dev(tf, a)
+    for keep in [(0,), (1, 3), (3, 0), (2, 1, 0), (), (0, 1, 2, 3), (3,), (2,)]:
+        shape = [a.shape[k] for k in keep]
+        ref = np.empty(shape, dtype)
+        oracle.reduce(a, range(4), ref, list(keep))
+        out = tf.Tensor.empty(shape, tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Reduce([0, 1, 2, 3], list(keep), tf.ReduceOp.Sum), [a.shape, shape])
+        tf.HipBackend.execute(plan, 1.0, [da], 0.0, out)
+        assert relerr(out.to_numpy(), ref) < TOL[dtype], keep
+
+
+def test_reduce_closed_forms_exact_and_long_reductions(tf):
+    # integers: exact in f64 whatever the summation order
+    shape = (6, 50, 4, 30)
+    a = np.arange(np.prod(shape), dtype=np.float64).reshape(shape)
+    out = tf.Tensor.empty([6, 4], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Reduce([0, 1, 2, 3], [0, 2], tf.ReduceOp.Sum), [shape, [6, 4]])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, a)], 0.0, out)
+    assert np.array_equal(out.to_numpy(), a.sum(axis=(1, 3)))
+    # full reduction of 2^22 ones -> split over blocks, two passes
+    ones = np.ones(1 << 22)
+    s = tf.Tensor.empty([], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Reduce([0], [], tf.ReduceOp.Sum), [[1 << 22], []])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, ones)], 0.0, s)
+    assert s.to_numpy() == float(1 << 22)
+    # few outputs, long strided reduction
+    b = np.arange(3 * 70000, dtype=np.float64).reshape(70000, 3)
+    o = tf.Tensor.empty([3], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Reduce([0, 1], [1], tf.ReduceOp.Sum), [[70000, 3], [3]])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, b)], 0.0, o)
+    assert np.array_equal(o.to_numpy(), b.sum(axis=0))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_reduce_max_min_alpha_beta_strided(tf, oracle, dtype):
+    rng = np.random.default_rng(25)
+    big = rand(rng, (14, 40, 18), dtype)
+    a = big[::2, ::-1, ::3]
+    da = dev(tf, a)
+    for op, name in [(tf.ReduceOp.Max, oracle.MAX), (tf.ReduceOp.Min, oracle.MIN)]:
+        ref = np.empty((a.shape[2], a.shape[0]), dtype)
+        oracle.reduce(a, [0, 1, 2], ref, [2, 0], op=name)
+        out = tf.Tensor.empty(list(ref.shape), tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Reduce([0, 1, 2], [2, 0], op), [a.shape, ref.shape])
+        tf.HipBackend.execute(plan, 1.0, [da], 0.0, out)
+        assert np.array_equal(out.to_numpy(), ref)
+    c0 = rand(rng, (a.shape[2], a.shape[0]), dtype)
+    ref = c0.copy()
+    oracle.reduce(a, [0, 1, 2], ref, [2, 0], alpha=2.0, beta=-0.5)
+    dc = dev(tf, c0)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Reduce([0, 1, 2], [2, 0], tf.ReduceOp.Sum), [a.shape, c0.shape])
+    tf.HipBackend.execute(plan, 2.0, [da], -0.5, dc)
+    assert relerr(dc.to_numpy(), ref) < TOL[dtype]
+
+
+def test_reduce_config2_full_size(tf, oracle):
+    # sum over axes 1 and 4 of the permuted 16^6 tensor: <= 1e-12 against the oracle; all-ones gives 256 exactly
+    from tenferro_rs_amd import inputs
+    p = inputs.uniform(1002, 0, (16,) * 6).transpose(5, 2, 0, 4, 1, 3).copy()
+    modes_a, modes_c = [5, 2, 0, 4, 1, 3], [5, 0, 4, 3]
+    ref = np.empty((16,) * 4)
+    oracle.reduce(p, modes_a, ref, modes_c)
+    out = tf.Tensor.empty([16] * 4, tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Reduce(modes_a, modes_c, tf.ReduceOp.Sum), [[16] * 6, [16] * 4])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, p)], 0.0, out)
+    assert relerr(out.to_numpy(), ref) < 1e-12
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, np.ones((16,) * 6))], 0.0, out)
+    assert np.all(out.to_numpy() == 256.0)
+
+
+# ------------------------------------------------------------------------------------------------ contract
+CASES = [
+    ("mk", "kn", "mn", dict(m=37, k=53, n=29)),
+    ("km", "nk", "nm", dict(m=20, k=300, n=17)),
+    ("mk", "kn", "mn", dict(m=300, k=77, n=260)),                  # 128x128 tiles with ragged edges
+    ("km", "kn", "mn", dict(m=200, k=45, n=136)),                  # both operands contiguous along the row index
+    ("mk", "nk", "nm", dict(m=130, k=100, n=150)),                 # output contiguous along m: operands swap
+    ("bmk", "bkn", "bmn", dict(b=3, m=70, k=31, n=40)),
+    ("ajbk", "kcj", "abc", dict(a=6, j=8, b=7, k=12, c=20)),       # config-1 pattern: multi-mode M and K
+    ("awc", "asx", "wcsx", dict(a=33, w=3, c=10, s=2, x=9)),       # config-3 step 1
+    ("mk", "k", "m", dict(m=150, k=300)),
+    ("i", "i", "", dict(i=5000)),                                  # split-K down to a scalar
+    ("i", "j", "ij", dict(i=19, j=23)),
+    ("bij", "jk", "bik", dict(b=4, i=30, j=14, k=25)),
+    ("abij", "abjk", "abik", dict(a=2, b=3, i=14, j=15, k=16)),
+    ("xmk", "kn", "mn", dict(x=4, m=16, k=7, n=15)),
+    ("mk", "kn", "mn", dict(m=64, k=4096, n=64)),                  # split-K
+]
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("case", CASES, ids=[c[0] + "," + c[1] + "->" + c[2] + str(i) for i, c in enumerate(CASES)])
+def test_contract_against_oracle(tf, oracle, dtype, case):
+    ma, mb, mc, ext = case
+    rng = np.random.default_rng(26)
+    a = rand(rng, [ext[l] for l in ma], dtype)
+    b = rand(rng, [ext[l] for l in mb], dtype)
+    cshape = [ext[l] for l in mc]
+    ref = np.empty(cshape, dtype)
+    oracle.contract(a, lab(ma), b, lab(mb), ref, lab(mc))
+    out = dev(tf, np.full(cshape, np.nan, dtype))      # beta == 0 must not read the NaNs
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [a.shape, b.shape, cshape])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
+    assert relerr(out.to_numpy(), ref) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_contract_integer_inputs_exact(tf, dtype):
+    # small integers: products and sums are exact, so MFMA accumulation order cannot matter
+    rng = np.random.default_rng(27)
+
+    def ints(shape):
+        x = rng.integers(-3, 4, shape).astype(np.float64)
+        if np.issubdtype(dtype, np.complexfloating):
+            x = x + 1j * rng.integers(-3, 4, shape)
+        return x.astype(dtype)
+
+    a, b = ints((150, 90, 3)), ints((90, 3, 140))
+    out = tf.Tensor.empty([3, 150, 140], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract([0, 1, 2], [1, 2, 3], [2, 0, 3]), [a.shape, b.shape, [3, 150, 140]])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
+    assert np.array_equal(out.to_numpy(), np.einsum("mkb,kbn->bmn", a, b).astype(dtype))
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.complex128, np.float32])
+def test_contract_alpha_beta_strided_views(tf, oracle, dtype):
+    rng = np.random.default_rng(28)
+    alpha, beta = (0.7 - 1.1j, -0.3 + 0.2j) if np.issubdtype(dtype, np.complexfloating) else (0.7, -0.3)
+    big = rand(rng, (140, 90), dtype)
+    av = big[::2, ::-2]                       # 70 x 45, negative stride
+    b = rand(rng, (45, 50), dtype)
+    c0 = rand(rng, (70, 100), dtype)
+    cv = c0[:, ::2]                           # strided output
+    ref = c0.copy()
+    oracle.contract(av, [0, 1], b, [1, 2], ref[:, ::2], [0, 2], alpha=alpha, beta=beta)
+    dc = dev(tf, cv)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract([0, 1], [1, 2], [0, 2]), [av.shape, b.shape, cv.shape])
+    tf.HipBackend.execute(plan, alpha, [dev(tf, av), dev(tf, b)], beta, dc)
+    assert relerr(dc.to_numpy(), ref[:, ::2]) < TOL[dtype]
+    # broadcast (stride-0) operand
+    row = rand(rng, (1, 45), dtype)
+    bc = np.broadcast_to(row, (70, 45))
+    ref2 = np.empty((70, 50), dtype)
+    oracle.contract(bc, [0, 1], b, [1, 2], ref2, [0, 2])
+    out = tf.Tensor.empty([70, 50], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    tbc = dev(tf, row).broadcast([70, 45])
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract([0, 1], [1, 2], [0, 2]), [[70, 45], b.shape, [70, 50]])
+    tf.HipBackend.execute(plan, 1.0, [tbc, dev(tf, b)], 0.0, out)
+    assert relerr(out.to_numpy(), ref2) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_batched_gemm(tf, oracle, dtype):
+    rng = np.random.default_rng(29)
+    a, b = rand(rng, (2, 3, 50, 70), dtype), rand(rng, (2, 3, 70, 40), dtype)
+    ref = np.empty((2, 3, 50, 40), dtype)
+    oracle.batched_gemm(a, b, ref, n_batch=2)
+    out = tf.Tensor.empty([2, 3, 50, 40], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.BatchedGemm([2, 3], 50, 40, 70), [a.shape, b.shape, ref.shape])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
+    assert relerr(out.to_numpy(), ref) < TOL[dtype]
+
+
+def test_config0_matmul_512_f64(tf, oracle):
+    from tenferro_rs_amd import inputs
+    a, b = inputs.uniform(1000, 0, (512, 512)), inputs.uniform(1000, 1, (512, 512))
+    ref = np.empty((512, 512))
+    oracle.contract(a, lab("ij"), b, lab("jk"), ref, lab("ik"))
+    c = tf.einsum("ij,jk->ik", [dev(tf, a), dev(tf, b)])
+    assert c.dims() == [512, 512]
+    assert relerr(c.to_numpy(), ref) < 1e-12
+
+
+def test_config1_full_size_f32(tf, oracle):
+    # "ajbk,kcj->abc", a=64 j=128 b=64 k=96 c=256, standard normal f32: <= 1e-5 against the oracle
+    # (the oracle accumulates f32 products in f64)
+    from tenferro_rs_amd import inputs
+    A = inputs.normal(1001, 0, (64, 128, 64, 96), np.float32)
+    B = inputs.normal(1001, 1, (96, 256, 128), np.float32)
+    ref = np.empty((64, 64, 256), np.float32)
+    oracle.contract(A, lab("ajbk"), B, lab("kcj"), ref, lab("abc"))
+    c = tf.einsum("ajbk,kcj->abc", [dev(tf, A), dev(tf, B)])
+    assert relerr(c.to_numpy(), ref) < 1e-5
+
+
+# ------------------------------------------------------------------------------------------------ grouped
+def _grouped_case(tf, oracle, dims, dtype, seed):
+    from tenferro_rs_amd import inputs
+    As = [inputs.uniform(seed, 3 * g, (i, j), dtype) for g, (i, j, k) in enumerate(dims)]
+    Bs = [inputs.uniform(seed, 3 * g + 1, (j, k), dtype) for g, (i, j, k) in enumerate(dims)]
+    outs = [tf.Tensor.empty([i, k], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype) for (i, j, k) in dims]
+    desc = tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik"))
+    plan = tf.HipBackend.plan_grouped(dtype, desc, [[[i, j], [j, k], [i, k]] for (i, j, k) in dims])
+    tf.HipBackend.execute_grouped(plan, 1.0, [(dev(tf, a), dev(tf, b)) for a, b in zip(As, Bs)], 0.0, outs)
+    worst = 0.0
+    for a, b, o in zip(As, Bs, outs):
+        ref = np.empty((a.shape[0], b.shape[1]), dtype)
+        oracle.contract(a, lab("ij"), b, lab("jk"), ref, lab("ik"))
+        worst = max(worst, relerr(o.to_numpy(), ref))
+    return worst
+
+
+def test_grouped_small_ragged(tf, oracle):
+    dims = [(5, 7, 3), (64, 64, 64), (130, 33, 70), (1, 1, 1), (200, 128, 17)]
+    assert _grouped_case(tf, oracle, dims, np.float64, 77) < 1e-12
+
+
+def test_config4_grouped_full_size(tf, oracle):
+    # 128 blocks, i,j,k iid from {64,...,1024}: every block <= 1e-12 against the oracle, one launch
+    from tenferro_rs_amd import inputs
+    dims = inputs.draw_block_dims(1004, 128)
+    assert _grouped_case(tf, oracle, dims, np.float64, 1004) < 1e-12
+
+
+# ------------------------------------------------------------------------------------------------ elementwise, conj, fill, trace family
+@pytest.mark.parametrize("dtype", ALL)
+def test_elementwise_mul_conj_fill(tf, oracle, dtype):
+    rng = np.random.default_rng(30)
+    a, b = rand(rng, (9, 40, 21), dtype), rand(rng, (21, 40, 9), dtype).transpose(2, 1, 0)
+    c0 = rand(rng, (9, 40, 21), dtype)
+    ref = c0.copy()
+    oracle.elementwise_mul(a, b, ref, alpha=2.0, beta=1.0)
+    dc = dev(tf, c0)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.ElementwiseMul(), [a.shape, b.shape, c0.shape])
+    tf.HipBackend.execute(plan, 2.0, [dev(tf, a), dev(tf, b)], 1.0, dc)
+    assert relerr(dc.to_numpy(), ref) < TOL[dtype]
+    da = dev(tf, a)
+    assert np.array_equal(da.conj().to_numpy(), np.conj(a))
+    assert np.array_equal(da.into_conj().to_numpy(), np.conj(a))
+    ones = tf.Tensor.ones([7, 33], tf.GpuMemory(0), tf.MemoryOrder.ColumnMajor, dtype)
+    assert np.array_equal(ones.to_numpy(), np.ones((7, 33), dtype))
+    assert ones.strides() == [1, 7]
+
+
+def test_conj_reference_doc_example(tf):
+    # tenferro-tensor/src/lib.rs:612-620
+    a = dev(tf, np.array([1 + 2j, 3 - 4j]))
+    assert np.array_equal(a.conj().to_numpy(), np.array([1 - 2j, 3 + 4j]))
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.complex128])
+def test_trace_anti_trace_anti_diag(tf, oracle, dtype):
+    rng = np.random.default_rng(31)
+    a = rand(rng, (14, 5, 14, 3), dtype)
+    ref = np.empty((3, 5), dtype)
+    oracle.trace(a, [0, 1, 2, 3], ref, [3, 1], pairs=[(0, 2)])
+    out = tf.Tensor.empty([3, 5], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Trace([0, 1, 2, 3], [3, 1], [(0, 2)]), [a.shape, [3, 5]])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, a)], 0.0, out)
+    assert relerr(out.to_numpy(), ref) < 1e-12
+    g = rand(rng, (3, 5), dtype)
+    back0 = rand(rng, (14, 5, 14, 3), dtype)
+    for op_, ofn, am, av in [(tf.PrimDescriptor.AntiTrace, oracle.anti_trace, [3, 1], g),
+                             (tf.PrimDescriptor.AntiDiag, oracle.anti_diag, [3, 1, 0], rand(rng, (3, 5, 14), dtype))]:
+        for alpha, beta in [(1.0, 0.0), (2.0, 1.0), (0.5, -1.5)]:
+            ref = back0.copy()
+            ofn(av, am, ref, [0, 1, 2, 3], pairs=[(0, 2)], alpha=alpha, beta=beta)
+            dc = dev(tf, back0)
+            plan = tf.HipBackend.plan(dtype, op_(am, [0, 1, 2, 3], [(0, 2)]), [av.shape, back0.shape])
+            tf.HipBackend.execute(plan, alpha, [dev(tf, av)], beta, dc)
+            assert relerr(dc.to_numpy(), ref) < 1e-12
+
+
+# ------------------------------------------------------------------------------------------------ einsum
+PATTERNS = ["ij,jk->ik", "ii->", "i,j->ij", "i,i->", "ij,j->i", "ii->i", "ijk->", "bij,bjk->bik", "abij,abjk->abik",
+            "bij,jk->bik", "ij,jk,kl->il", "ij->ji", "ij,ij->ij", "iij,jk->ik", "i->ii", "i->iii", "ij,(jk,kl)->il",
+            "ijx,jk->ik"]
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.complex128, np.float32])
+@pytest.mark.parametrize("pattern", PATTERNS)
+def test_einsum_pattern_catalogue(tf, oracle, dtype, pattern):
+    # tenferro-einsum/src/lib.rs:37-93, against the brute-force einsum of the oracle
+    rng = np.random.default_rng(32)
+    ext = dict(i=13, j=14, k=15, l=6, a=2, b=3, x=4)
+    ins, out = pattern.replace("(", "").replace(")", "").split("->")
+    terms = ins.split(",")
+    ops = [rand(rng, [ext[l] for l in t], dtype) for t in terms]
+    oshape = [ext[l] for l in out]
+    ref = np.empty(oshape, dtype)
+    oracle.einsum_naive(ops, [lab(t) for t in terms], ref, lab(out))
+    res = tf.einsum(pattern, [dev(tf, o) for o in ops])
+    assert res.dims() == oshape
+    assert relerr(res.to_numpy(), ref) < TOL[dtype]
+
+
+def test_einsum_reference_doc_examples(tf):
+    # tenferro-einsum/src/lib.rs:52-63, 76-93
+    v = dev(tf, np.array([1.0, 2.0, 3.0]))
+    d = tf.einsum("i->ii", [v])
+    assert d.dims() == [3, 3] and np.array_equal(d.to_numpy(), np.diag([1.0, 2.0, 3.0]))
+    assert tf.einsum("i->iii", [v]).dims() == [3, 3, 3]
+    z = lambda *s: tf.Tensor.zeros(list(s), tf.GpuMemory(0), tf.MemoryOrder.ColumnMajor)
+    assert tf.einsum("bij,bjk->bik", [z(10, 3, 4), z(10, 4, 5)]).dims() == [10, 3, 5]
+    assert tf.einsum("abij,abjk->abik", [z(2, 3, 4, 5), z(2, 3, 5, 6)]).dims() == [2, 3, 4, 6]
+    assert tf.einsum("bij,jk->bik", [z(10, 3, 4), z(4, 5)]).dims() == [10, 3, 5]
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.complex128])
+def test_einsum_every_tree_of_a_small_network_agrees(tf, oracle, dtype):
+    rng = np.random.default_rng(33)
+    ext = dict(a=9, c=8, x=7, y=6, w=3, v=4, s=2, t=2)
+    terms, out = ["awc", "asx", "wstv", "cty"], "xvy"
+    ops = [rand(rng, [ext[l] for l in t], dtype) for t in terms]
+    ref = np.empty([ext[l] for l in out], dtype)
+    oracle.einsum_naive(ops, [lab(t) for t in terms], ref, lab(out))
+    subs = tf.Subscripts.new([lab(t) for t in terms], lab(out))
+    dops = [dev(tf, o) for o in ops]
+    orders = [[(0, 1), (4, 2), (5, 3)], [(0, 2), (1, 4), (5, 3)], [(1, 2), (0, 3), (4, 5)], [(2, 3), (0, 1), (4, 5)], [(0, 3), (4, 2), (5, 1)]]
+    for pairs in orders:
+        tree = tf.ContractionTree.from_pairs(subs, [o.shape for o in ops], pairs)
+        res = tf.einsum_with_plan(tree, dops)
+        assert relerr(res.to_numpy(), ref) < 1e-12, pairs
+    # alpha/beta into a pre-allocated output, twice (accumulate)
+    tree = tf.ContractionTree.optimize(subs, [o.shape for o in ops])
+    c0 = rand(rng, ref.shape, dtype)
+    dc = dev(tf, c0)
+    tf.einsum_with_plan_into(tree, dops, 2.0, -1.0, dc)
+    assert relerr(dc.to_numpy(), 2 * ref - c0) < 1e-12
+    tf.einsum_with_plan_into(tree, dops, 1.0, 1.0, dc)
+    assert relerr(dc.to_numpy(), 3 * ref - c0) < 1e-12
+
+
+def test_einsum_async_chaining(tf):
+    # tenferro-einsum/src/lib.rs:158-177: the second call chains on the first result's event
+    rng = np.random.default_rng(34)
+    a, b = rng.standard_normal((300, 400)), rng.standard_normal((400, 400))
+    da, db = dev(tf, a), dev(tf, b)
+    c = tf.einsum("ij,jk->ik", [da, db])
+    assert c.event is not None
+    d = tf.einsum("ij,jk->ik", [c, db])
+    d.wait()
+    assert d.is_ready() and d.event is None
+    assert relerr(d.to_numpy(), a @ b @ b) < 1e-12
+
+
+def test_execute_errors(tf):
+    a = tf.Tensor.zeros([3, 4], tf.GpuMemory(0), tf.MemoryOrder.RowMajor)
+    b = tf.Tensor.zeros([4, 5], tf.GpuMemory(0), tf.MemoryOrder.RowMajor)
+    c = tf.Tensor.zeros([3, 5], tf.GpuMemory(0), tf.MemoryOrder.RowMajor)
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Contract([0, 1], [1, 2], [0, 2]), [[3, 4], [4, 5], [3, 5]])
+    with pytest.raises(tf.ShapeMismatch) as e:
+        tf.HipBackend.execute(plan, 1.0, [b, b], 0.0, c)
+    assert e.value.expected == [3, 4] and e.value.got == [4, 5]
+    with pytest.raises(tf.RankMismatch):
+        tf.HipBackend.execute(plan, 1.0, [a, b], 0.0, tf.Tensor.zeros([15], tf.GpuMemory(0), tf.MemoryOrder.RowMajor))
+    with pytest.raises(tf.InvalidArgument):
+        tf.HipBackend.execute(plan, 1.0, [a], 0.0, c)
+    with pytest.raises(tf.Strided):
+        tf.HipBackend.execute(plan, 1.0, [a, b], 0.0, tf.Tensor.zeros([3, 1], tf.GpuMemory(0), tf.MemoryOrder.RowMajor).broadcast([3, 5]))
+    host = tf.Tensor.from_slice(np.zeros(12), [3, 4], tf.MemoryOrder.ColumnMajor)
+    with pytest.raises(tf.CrossMemorySpaceOperation):
+        tf.einsum("ij,jk->ik", [host, b])
+    with pytest.raises(tf.NoCompatibleComputeDevice):
+        tf.einsum("ij,jk->ik", [host, tf.Tensor.from_slice(np.zeros(20), [4, 5], tf.MemoryOrder.ColumnMajor)])
+    assert [str(d) for d in tf.preferred_compute_devices(tf.GpuMemory(0), tf.OpKind.Contract)] == ["hip:0"]
+    with pytest.raises(tf.NoCompatibleComputeDevice):
+        tf.preferred_compute_devices(tf.GpuMemory(99), tf.OpKind.Contract)
