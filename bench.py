@@ -1,0 +1,314 @@
+#!/usr/bin/env python3
+"""Benchmark of the tensor-contraction hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs c1,c2,c3,c4] [--no-cpu]
+
+Prints ONE JSON line.  The headline (`value`) is configuration 1 of BASELINE.json -- the f32 einsum
+"ajbk,kcj->abc" (a=64, j=128, b=64, k=96, c=256) -- as whole-step TFLOP/s with inputs resident in
+HBM; `all_configs` carries the same measurements for configurations 2 (permute + reduce of a 16^6
+f64 tensor), 3 (complex128 MPS-MPO environment update, four operands) and 4 (128-block grouped f64
+GEMM).  A "step" is one pass of the workload: one contraction, one permute+reduce, one einsum tree,
+one grouped launch.
+
+`roofline.achieved` is algorithmic flops (or bytes) of the dominant kernel divided by that kernel's
+average duration, measured with HIP events recorded on the launch stream inside the timed region.
+`cpu_baseline` is the CPU oracle (a port: the reference has no CPU backend to time) on the host
+cores of this machine, on the same inputs; its result is also the parity check of the run.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"hbm": 8000.0, "f32": 157.3, "f64": 78.6}   # GB/s, TFLOP/s (MI355X published peaks)
+METRIC = "contraction TFLOP/s & % MFMA peak (f64/f32); permute/reduce GB/s & % HBM peak"
+
+
+def lab(s):
+    return [ord(c) for c in s]
+
+
+def relerr(x, ref):
+    d = np.linalg.norm((x - ref).ravel())
+    n = np.linalg.norm(ref.ravel())
+    return float(d / n) if n > 0 else float(d)
+
+
+class Harness:
+    def __init__(self, steps, warmup, cpu):
+        import torch
+        import tenferro_rs_amd as tf
+        from tenferro_rs_amd import inputs
+        self.torch, self.tf, self.inputs = torch, tf, inputs
+        self.steps, self.warmup, self.cpu = steps, warmup, cpu
+        tf.lib()
+        if cpu:
+            from oracle import tfo
+            tfo.lib()
+            self.tfo = tfo
+            self.cores = tfo.num_threads()
+
+    def gpu(self, arr):
+        return self.tf.Tensor.from_torch(self.torch.from_numpy(np.ascontiguousarray(arr)).cuda())
+
+    def empty(self, shape, dtype):
+        return self.tf.Tensor.empty(list(shape), self.tf.GpuMemory(0), self.tf.MemoryOrder.RowMajor, dtype)
+
+    def timed(self, step, kinds):
+        """step(i) enqueues one pass.  Returns (ms per step, {kind: (ms per launch, launches per step)})."""
+        torch, tf = self.torch, self.tf
+        for i in range(self.warmup):
+            step(i)
+        torch.cuda.synchronize()
+        tf.profile_enable(True)
+        t0 = time.perf_counter()
+        for i in range(self.steps):
+            step(self.warmup + i)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        out = {}
+        for k in kinds:
+            ms, n = tf.profile_collect(k)
+            out[k] = (ms / max(n, 1), n / self.steps)
+        tf.profile_enable(False)
+        return (t1 - t0) * 1e3 / self.steps, out
+
+    def cpu_time(self, fn, reps):
+        best = None
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        return best
+
+    def bound_execute(self, plan, inputs, output, alpha=1.0, beta=0.0):
+        """Pre-marshalled tfh_execute call: the hot loop does no Python-side packing."""
+        tf = self.tf
+        L = tf.lib()
+        views = (tf.tfh_view * len(inputs))(*[tf.view_of(t) for t in inputs])
+        vo = tf.view_of(output)
+        al, be = tf._scalar_c(plan.dtype, alpha), tf._scalar_c(plan.dtype, beta)
+        st = tf.current_stream()
+        n = len(inputs)
+
+        def call():
+            rc = L.tfh_execute(plan._h, al, views, n, be, C.byref(vo), st)
+            if rc:
+                tf._check(rc)
+        call.keep = (views, vo, al, be, inputs, output, plan)
+        return call
+
+
+# ------------------------------------------------------------------------------------------------- config 1
+def run_c1(h):
+    tf, inputs = h.tf, h.inputs
+    a, j, b, k, c = 64, 128, 64, 96, 256
+    A = inputs.normal(1001, 0, (a, j, b, k), np.float32)
+    B = inputs.normal(1001, 1, (k, c, j), np.float32)
+    flops = 2.0 * a * b * c * j * k
+    algo_bytes = 4.0 * (A.size + B.size + a * b * c)
+    nset = 3   # rotate operand sets so the 201 MB operand is not served from the 256 MB last-level cache
+    As = [h.gpu(A) for _ in range(nset)]
+    Bd = h.gpu(B)
+    outs = [h.empty((a, b, c), np.float32) for _ in range(nset)]
+    plan = tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Contract(lab("ajbk"), lab("kcj"), lab("abc")),
+                              [A.shape, B.shape, (a, b, c)])
+    calls = [h.bound_execute(plan, [As[i], Bd], outs[i]) for i in range(nset)]
+    ms, prof = h.timed(lambda i: calls[i % nset](), [tf.PROF_CONTRACT])
+    kms, per_step = prof[tf.PROF_CONTRACT]
+    res = {
+        "workload": "einsum ajbk,kcj->abc f32 a=64 j=128 b=64 k=96 c=256 (GEMM view M=4096 N=256 K=12288)",
+        "dtype": "f32", "ms_per_step": ms, "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
+        "roofline": {"bound": "mfma", "achieved": flops / (kms * 1e-3) / 1e12, "peak": PEAK["f32"], "unit": "TFLOP/s",
+                     "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f32"], "traffic": None,
+                     "kernel": "gemm_kernel<float,false,128,128>", "kernel_ms": kms, "launches_per_step": per_step},
+    }
+    if h.cpu:
+        ref = np.empty((a, b, c), np.float32)
+        t = h.cpu_time(lambda: h.tfo.contract(A, lab("ajbk"), B, lab("kcj"), ref, lab("abc")), 2)
+        res["cpu_baseline"] = {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": h.cores, "kind": "port",
+                               "sample": "the full contraction (25.8 GFLOP), best of 2", "seconds": t}
+        res["parity"] = {"rel_frobenius": relerr(outs[0].to_numpy().astype(np.float64), ref.astype(np.float64)), "tolerance": 1e-5}
+    return res
+
+
+# ------------------------------------------------------------------------------------------------- config 2
+def run_c2(h):
+    tf, inputs = h.tf, h.inputs
+    shape = (16,) * 6
+    perm = [5, 2, 0, 4, 1, 3]
+    X = inputs.uniform(1002, 0, shape)
+    nset = 3   # 3 x (134 MB in + 134 MB out) > 256 MB last-level cache: every pass misses
+    Xs = [h.gpu(X) for _ in range(nset)]
+    Ps = [h.empty(shape, np.float64) for _ in range(nset)]
+    Rs = [h.empty((16,) * 4, np.float64) for _ in range(nset)]
+    pplan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute(list(range(6)), perm), [shape, shape])
+    modes_a, modes_c = perm, [5, 0, 4, 3]          # sum over output axes 1 and 4 of the permuted tensor
+    rplan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Reduce(modes_a, modes_c, tf.ReduceOp.Sum), [shape, (16,) * 4])
+    pcalls = [h.bound_execute(pplan, [Xs[i]], Ps[i]) for i in range(nset)]
+    rcalls = [h.bound_execute(rplan, [Ps[i]], Rs[i]) for i in range(nset)]
+    pbytes = 2.0 * X.nbytes
+    rbytes = float(X.nbytes + 16 ** 4 * 8)
+
+    def step(i):
+        pcalls[i % nset]()
+        rcalls[i % nset]()
+    ms, prof = h.timed(step, [tf.PROF_COPY, tf.PROF_REDUCE])
+    pms, rms = prof[tf.PROF_COPY][0], prof[tf.PROF_REDUCE][0]
+    res = {
+        "workload": "f64 16^6 tensor: permute to (5,2,0,4,1,3), then sum over output axes 1 and 4",
+        "dtype": "f64", "ms_per_step": ms, "value": (pbytes + rbytes) / (ms * 1e-3) / 1e9, "unit": "GB/s",
+        "permute": {"roofline": {"bound": "hbm", "achieved": pbytes / (pms * 1e-3) / 1e9, "peak": PEAK["hbm"], "unit": "GB/s",
+                                 "frac": pbytes / (pms * 1e-3) / 1e9 / PEAK["hbm"], "traffic": None,
+                                 "kernel": "copy_kernel<u64>", "kernel_ms": pms}, "algorithmic_bytes": pbytes},
+        "reduce": {"roofline": {"bound": "hbm", "achieved": rbytes / (rms * 1e-3) / 1e9, "peak": PEAK["hbm"], "unit": "GB/s",
+                                "frac": rbytes / (rms * 1e-3) / 1e9 / PEAK["hbm"], "traffic": None,
+                                "kernel": "reduce_kernel<double>", "kernel_ms": rms}, "algorithmic_bytes": rbytes},
+    }
+    if h.cpu:
+        P = np.empty(shape)
+        R = np.empty((16,) * 4)
+        tp = h.cpu_time(lambda: h.tfo.permute(X, list(range(6)), P, perm), 3)
+        tr = h.cpu_time(lambda: h.tfo.reduce(P, modes_a, R, modes_c), 3)
+        res["cpu_baseline"] = {"permute": {"value": pbytes / tp / 1e9, "unit": "GB/s", "seconds": tp},
+                               "reduce": {"value": rbytes / tr / 1e9, "unit": "GB/s", "seconds": tr},
+                               "cores": h.cores, "kind": "port", "sample": "the full 16^6 tensor, best of 3"}
+        res["parity"] = {"permute_bit_exact": bool(Ps[0].to_numpy().tobytes() == P.tobytes()),
+                         "reduce_rel_frobenius": relerr(Rs[0].to_numpy(), R), "tolerance": 1e-12}
+    return res
+
+
+# ------------------------------------------------------------------------------------------------- config 3
+def run_c3(h):
+    tf, inputs = h.tf, h.inputs
+    chi, D, d = 1024, 16, 2
+    sig = 1.0 / np.sqrt(chi)
+    Lh = inputs.complex_normal(1003, 0, (chi, D, chi), sig)
+    Ah = inputs.complex_normal(1003, 1, (chi, d, chi), sig)
+    Wh = inputs.complex_normal(1003, 2, (D, d, d, D), sig)
+    Ach = np.conj(Ah)                                  # 4th operand: conj(A), materialised outside the timed region
+    terms, out = ["awc", "asx", "wstv", "cty"], "xvy"
+    host = [Lh, Ah, Wh, Ach]
+    subs = tf.Subscripts.parse(",".join(terms) + "->" + out)
+    tree = tf.ContractionTree.optimize(subs, [x.shape for x in host])
+    flops = 8.0 * tree.mac_count
+    ops = [h.gpu(x) for x in host]
+    res_t = h.empty((chi, D, chi), np.complex128)
+    ms, prof = h.timed(lambda i: tf.einsum_with_plan_into(tree, ops, 1.0, 0.0, res_t), [tf.PROF_CONTRACT])
+    kms, per_step = prof[tf.PROF_CONTRACT]
+    total_kms = kms * per_step
+    res = {
+        "workload": "einsum awc,asx,wstv,cty->xvy complex128 chi=1024 D=16 d=2 (tree from the optimiser)",
+        "dtype": "c128 on f64 MFMA", "ms_per_step": ms, "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "flops_per_step": flops, "tree_steps": tree.steps, "min_flop_tree": bool(abs(flops - 558.3e9) < 0.1e9),
+        "peak_intermediate_bytes": tree.peak_intermediate * 16,
+        "roofline": {"bound": "mfma", "achieved": flops / (total_kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
+                     "frac": flops / (total_kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": None,
+                     "kernel": "gemm_kernel<double,true,...> x3 (the three pairwise contractions of the tree)",
+                     "kernel_ms": total_kms, "launches_per_step": per_step},
+    }
+    if h.cpu:
+        ref = np.empty((chi, D, chi), np.complex128)
+        t = h.cpu_time(lambda: h.tfo.einsum_pairs(host, [lab(t_) for t_ in terms], ref, lab(out), tree.steps), 1)
+        res["cpu_baseline"] = {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": h.cores, "kind": "port",
+                               "sample": "the full tree (558.3 GFLOP), one pass", "seconds": t}
+        res["parity"] = {"rel_frobenius": relerr(res_t.to_numpy(), ref), "tolerance": 1e-12}
+    return res
+
+
+# ------------------------------------------------------------------------------------------------- config 4
+def run_c4(h):
+    tf, inputs = h.tf, h.inputs
+    dims = inputs.draw_block_dims(1004, 128)
+    As = [inputs.uniform(1004, 3 * g, (i, j)) for g, (i, j, k) in enumerate(dims)]
+    Bs = [inputs.uniform(1004, 3 * g + 1, (j, k)) for g, (i, j, k) in enumerate(dims)]
+    flops = float(sum(2 * i * j * k for i, j, k in dims))
+    algo_bytes = float(sum(8 * (i * j + j * k + i * k) for i, j, k in dims))
+    dA, dB = [h.gpu(x) for x in As], [h.gpu(x) for x in Bs]
+    outs = [h.empty((i, k), np.float64) for i, j, k in dims]
+    plan = tf.HipBackend.plan_grouped(np.float64, tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik")),
+                                      [[[i, j], [j, k], [i, k]] for i, j, k in dims])
+    pairs = list(zip(dA, dB))
+    ms, prof = h.timed(lambda i: tf.HipBackend.execute_grouped(plan, 1.0, pairs, 0.0, outs), [tf.PROF_CONTRACT])
+    kms, per_step = prof[tf.PROF_CONTRACT]
+    res = {
+        "workload": "128 independent ij,jk->ik f64 blocks, i,j,k iid from {64,...,1024}, one grouped launch",
+        "dtype": "f64", "ms_per_step": ms, "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
+        "roofline": {"bound": "mfma", "achieved": flops / (kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
+                     "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": None,
+                     "kernel": "gemm_kernel<double,false,128,128> (grouped)", "kernel_ms": kms, "launches_per_step": per_step},
+    }
+    if h.cpu:
+        refs = [np.empty((i, k)) for i, j, k in dims]
+
+        def cpu():
+            for a, b, r in zip(As, Bs, refs):
+                h.tfo.contract(a, lab("ij"), b, lab("jk"), r, lab("ik"))
+        t = h.cpu_time(cpu, 1)
+        res["cpu_baseline"] = {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": h.cores, "kind": "port",
+                               "sample": "all 128 blocks, one pass", "seconds": t}
+        res["parity"] = {"max_rel_frobenius": max(relerr(o.to_numpy(), r) for o, r in zip(outs, refs)), "tolerance": 1e-12}
+    return res
+
+
+RUNNERS = {"c1": run_c1, "c2": run_c2, "c3": run_c3, "c4": run_c4}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--configs", default="c1,c2,c3,c4")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus %d is not supported\n" % args.gpus)
+        sys.exit(2)
+    h = Harness(args.steps, args.warmup, not args.no_cpu)
+    wanted = [c.strip() for c in args.configs.split(",") if c.strip()]
+    if "c1" not in wanted:
+        wanted.insert(0, "c1")
+    results = {}
+    for name in wanted:
+        results[name] = RUNNERS[name](h)
+        h.torch.cuda.synchronize()
+        h.torch.cuda.empty_cache()
+        h.tf.lib().tfh_release_workspaces()
+    c1 = results["c1"]
+    line = {
+        "metric": METRIC, "value": c1["value"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": c1["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config 1: " + c1["workload"], "inputs": "seeded N(0,1), resident in HBM, 3 rotating operand sets"},
+        "roofline": c1["roofline"],
+        "cpu_baseline": c1.get("cpu_baseline"),
+        "parity": c1.get("parity"),
+        "all_configs": results,
+    }
+    print(json.dumps(line))
+    bad = []
+    for name, r in results.items():
+        p = r.get("parity") or {}
+        for k, v in p.items():
+            if k.endswith("frobenius") and v > p["tolerance"]:
+                bad.append((name, k, v))
+            if k.endswith("bit_exact") and not v:
+                bad.append((name, k, v))
+    if bad:
+        sys.stderr.write("PARITY FAILURE: %r\n" % bad)
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()

@@ -255,6 +255,13 @@ int32_t tfh_event_synchronize(tfh_event e);             /* Tensor::wait */
 int32_t tfh_event_query(tfh_event e, int32_t* ready);   /* Tensor::is_ready */
 int32_t tfh_stream_wait_event(tfh_stream s, tfh_event e);  /* chaining without a host wait (tenferro-einsum/src/lib.rs:146-177) */
 
+/* Measurement aid (no counterpart in the reference): while enabled, the dominant kernel of every
+ * contraction (kind 0), copy/permute (kind 1) and reduction (kind 2) launch is bracketed by HIP events
+ * on its own stream.  tfh_profile_collect waits for them and returns the summed duration and the
+ * launch count of one kind since the last enable, then forgets those records. */
+int32_t tfh_profile_enable(int32_t on);
+int32_t tfh_profile_collect(int32_t kind, double* total_ms, int32_t* launches);
+
 /* Releases the cached workspace and intermediate buffers of every stream (after a synchronize). */
 int32_t tfh_release_workspaces(void);
 

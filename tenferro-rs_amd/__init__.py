@@ -103,6 +103,8 @@ def lib():
         L.tfh_compute_device_format.argtypes = [C.c_int32, C.c_int64, C.c_char_p, C.c_size_t]
         L.tfh_preferred_compute_devices.argtypes = [C.c_int32, C.c_int64, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p]
         L.tfh_has_extension.argtypes = [C.c_int32, C.c_int32]
+        L.tfh_profile_enable.argtypes = [C.c_int32]
+        L.tfh_profile_collect.argtypes = [C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_int32)]
         L.tfh_subscripts_labels.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]
         L.tfh_subscripts_nesting.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t]
         L.tfh_plan_describe.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t]
@@ -867,3 +869,19 @@ def einsum_with_subscripts_owned(subscripts, operands, stream=None):
 def einsum_owned(subscripts, operands, stream=None):
     """:460-465"""
     return einsum_with_subscripts_owned(Subscripts.parse(subscripts), operands, stream)
+
+
+# ---------------------------------------------------------------------------------------------- measurement aid
+PROF_CONTRACT, PROF_COPY, PROF_REDUCE = 0, 1, 2
+
+
+def profile_enable(on=True):
+    """Bracket the dominant kernel of every launch with HIP events on its stream (tfh_profile_enable)."""
+    _check(lib().tfh_profile_enable(1 if on else 0))
+
+
+def profile_collect(kind):
+    """(total milliseconds, launches) of one kernel kind since profile_enable."""
+    ms, n = C.c_double(), C.c_int32()
+    _check(lib().tfh_profile_collect(kind, C.byref(ms), C.byref(n)))
+    return ms.value, n.value

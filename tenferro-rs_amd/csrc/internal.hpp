@@ -122,6 +122,10 @@ int32_t workspace(void* stream, size_t bytes, void** out);
 int32_t pool_alloc(void* stream, size_t bytes, void** out);
 void pool_free(void* stream, void* ptr);
 int32_t hip_check(int err, const char* what);
+// Event bracket around a dominant kernel while profiling is enabled (runtime.cpp); -1 when disabled.
+enum { PROF_CONTRACT = 0, PROF_COPY = 1, PROF_REDUCE = 2 };
+int prof_begin(int kind, void* stream);
+void prof_end(int token, void* stream);
 
 // Byte pointer of a view's element 0.
 inline char* view_ptr(const tfh_view& v, int dtype) { return (char*)v.base + v.offset * (int64_t)dtype_size(dtype); }

@@ -378,6 +378,7 @@ template <class V, class Op>
 int32_t run_copy(const TilePlan& tp, Op op, bool read_old, hipStream_t st) {
     size_t lds = (size_t)(tp.args.tile_elems + tp.args.tile_elems / 32 + 1) * sizeof(V);
     const int ept = tp.ept;
+    const int prof = prof_begin(PROF_COPY, st);
 #define TFH_LAUNCH(E)                                                                                     \
     do {                                                                                                  \
         if (read_old) hipLaunchKernelGGL((copy_kernel<V, Op, E, true>), tp.grid, dim3(THREADS), lds, st, tp.args, op);   \
@@ -388,6 +389,7 @@ int32_t run_copy(const TilePlan& tp, Op op, bool read_old, hipStream_t st) {
     else if (ept <= 8) TFH_LAUNCH(8);
     else TFH_LAUNCH(16);
 #undef TFH_LAUNCH
+    prof_end(prof, st);
     return hip_check(hipGetLastError(), "copy kernel launch");
 }
 

@@ -582,7 +582,9 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     }
     if (nsplit > 1) g.partial = ws + cursor;
     dim3 grid((uint32_t)(g.tiles_m * g.tiles_n), 1, (uint32_t)(nb * nsplit));
+    const int prof = prof_begin(PROF_CONTRACT, stream);
     launch_dtype(dtype, g, grid, bm, st);
+    prof_end(prof, stream);
     if (int32_t e = hip_check(hipGetLastError(), "contraction kernel launch")) return e;
     if (nsplit > 1) {
         int64_t total = nb * M * N;
@@ -757,7 +759,9 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
     g.problems = gs->problems_dev;
     g.tile_map = gs->tile_map_dev;
     dim3 grid((uint32_t)gs->tile_map_host.size(), 1, 1);
+    const int prof = prof_begin(PROF_CONTRACT, stream);
     launch_dtype(dtype, g, grid, gs->bm, st);
+    prof_end(prof, stream);
     return hip_check(hipGetLastError(), "grouped contraction launch");
 }
 

@@ -48,11 +48,6 @@ struct ReduceArgs {
     double alpha_re, alpha_im, beta_re, beta_im;
 };
 
-template <bool CX>
-struct Acc {
-    double re, im;
-};
-
 __device__ __forceinline__ double combine(double a, double b, int op) {
     return op == TFH_REDUCE_SUM ? a + b : (op == TFH_REDUCE_MAX ? fmax(a, b) : fmin(a, b));
 }
@@ -410,12 +405,14 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
     }
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((uint32_t)blocks, (uint32_t)nchunks, 1), block(THREADS);
+    const int prof = prof_begin(PROF_REDUCE, stream);
     switch (dtype) {
         case TFH_F32: hipLaunchKernelGGL((reduce_kernel<float, false>), grid, block, 0, st, ra); break;
         case TFH_F64: hipLaunchKernelGGL((reduce_kernel<double, false>), grid, block, 0, st, ra); break;
         case TFH_C64: hipLaunchKernelGGL((reduce_kernel<float, true>), grid, block, 0, st, ra); break;
         default: hipLaunchKernelGGL((reduce_kernel<double, true>), grid, block, 0, st, ra); break;
     }
+    prof_end(prof, stream);
     if (int32_t e = hip_check(hipGetLastError(), "reduce kernel launch")) return e;
     if (nchunks > 1) {
         dim3 g2((uint32_t)blocks, 1, 1);

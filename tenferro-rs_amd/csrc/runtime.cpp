@@ -88,12 +88,85 @@ void pool_free(void* stream, void* ptr) {
     s->live.erase(it);
 }
 
+namespace {
+struct ProfRec {
+    int kind;
+    hipEvent_t a, b;
+};
+std::mutex g_prof_mu;
+bool g_prof_on = false;
+std::vector<ProfRec> g_prof;
+std::vector<hipEvent_t> g_prof_pool;
+hipEvent_t prof_event() {
+    if (!g_prof_pool.empty()) {
+        hipEvent_t e = g_prof_pool.back();
+        g_prof_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    (void)hipEventCreate(&e);
+    return e;
+}
+}  // namespace
+
+int prof_begin(int kind, void* stream) {
+    if (!g_prof_on) return -1;
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    ProfRec r{kind, prof_event(), prof_event()};
+    if (!r.a || !r.b) return -1;
+    (void)hipEventRecord(r.a, (hipStream_t)stream);
+    g_prof.push_back(r);
+    return (int)g_prof.size() - 1;
+}
+void prof_end(int token, void* stream) {
+    if (token < 0) return;
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    if (token < (int)g_prof.size()) (void)hipEventRecord(g_prof[(size_t)token].b, (hipStream_t)stream);
+}
+
 }  // namespace tfh
 
 using tfh::hip_check;
 using tfh::set_error;
 
 extern "C" {
+
+int32_t tfh_profile_enable(int32_t on) {
+    std::lock_guard<std::mutex> lk(tfh::g_prof_mu);
+    for (auto& r : tfh::g_prof) {
+        (void)hipEventSynchronize(r.b);
+        tfh::g_prof_pool.push_back(r.a);
+        tfh::g_prof_pool.push_back(r.b);
+    }
+    tfh::g_prof.clear();
+    tfh::g_prof_on = on != 0;
+    return TFH_OK;
+}
+
+int32_t tfh_profile_collect(int32_t kind, double* total_ms, int32_t* launches) {
+    if (!total_ms || !launches) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
+    std::lock_guard<std::mutex> lk(tfh::g_prof_mu);
+    double total = 0;
+    int n = 0;
+    std::vector<tfh::ProfRec> keep;
+    for (auto& r : tfh::g_prof) {
+        if (r.kind != kind) {
+            keep.push_back(r);
+            continue;
+        }
+        if (int32_t e = hip_check(hipEventSynchronize(r.b), "hipEventSynchronize")) return e;
+        float ms = 0;
+        if (int32_t e = hip_check(hipEventElapsedTime(&ms, r.a, r.b), "hipEventElapsedTime")) return e;
+        total += ms;
+        ++n;
+        tfh::g_prof_pool.push_back(r.a);
+        tfh::g_prof_pool.push_back(r.b);
+    }
+    tfh::g_prof.swap(keep);
+    *total_ms = total;
+    *launches = n;
+    return TFH_OK;
+}
 
 int32_t tfh_release_workspaces(void) {
     std::lock_guard<std::mutex> lk(tfh::g_mu);
