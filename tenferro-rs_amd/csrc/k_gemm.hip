@@ -84,69 +84,6 @@ template <> struct ElemT<double, false> { typedef double type; };
 template <> struct ElemT<float, true> { typedef float2 type; };
 template <> struct ElemT<double, true> { typedef double2 type; };
 
-// One operand tile loader: ROWS x BKE elements per stage, NU per thread.
-template <class R, bool CX, int ROWS, int BKE>
-struct Loader {
-    typedef typename ElemT<R, CX>::type E;
-    static constexpr int NU = ROWS * BKE / THREADS;
-    static_assert(ROWS * BKE % THREADS == 0, "tile must divide over the block");
-    const E* base;
-    int64_t rowoff[NU];   // kfast: one per u.  rfast: [0] only
-    int rows_left;        // valid rows in this tile
-    bool kfast;
-    OffFn fk;
-
-    __device__ __forceinline__ void init(const void* p, int64_t boff, const OffFn& frow, const OffFn& fk_, int64_t row0,
-                                         int64_t nrows, bool kfast_) {
-        base = reinterpret_cast<const E*>(p) + boff;
-        kfast = kfast_;
-        fk = fk_;
-        int64_t left = nrows - row0;
-        rows_left = left > ROWS ? ROWS : (int)left;
-        const int t = threadIdx.x;
-#pragma unroll
-        for (int u = 0; u < NU; ++u) {
-            int row = kfast ? (u * THREADS + t) / BKE : (u * THREADS + t) % ROWS;
-            int64_t r = row0 + (row < rows_left ? row : 0);
-            rowoff[u] = (kfast || u == 0) ? off_of(frow, r) : rowoff[0];
-        }
-    }
-    // k0: first element index of the stage; kend: end of this block's k range
-    __device__ __forceinline__ void load(E (&v)[NU], int64_t k0, int64_t kend) const {
-        const int t = threadIdx.x;
-        if (kfast) {
-            const int kk = t % BKE;
-            const bool kok = k0 + kk < kend;
-            const int64_t ko = kok ? off_of(fk, k0 + kk) : 0;
-#pragma unroll
-            for (int u = 0; u < NU; ++u) {
-                int row = (u * THREADS + t) / BKE;
-                E z = E();
-                v[u] = (kok && row < rows_left) ? base[rowoff[u] + ko] : z;
-            }
-        } else {
-            const int row = t % ROWS;
-            const bool rok = row < rows_left;
-#pragma unroll
-            for (int u = 0; u < NU; ++u) {
-                int kk = (u * THREADS + t) / ROWS;
-                bool kok = k0 + kk < kend;
-                E z = E();
-                v[u] = (kok && rok) ? base[rowoff[0] + off_of(fk, kok ? k0 + kk : 0)] : z;
-            }
-        }
-    }
-    __device__ __forceinline__ void coords(int u, int& row, int& kk) const {
-        const int id = u * THREADS + threadIdx.x;
-        if (kfast) {
-            row = id / BKE;
-            kk = id % BKE;
-        } else {
-            row = id % ROWS;
-            kk = id / ROWS;
-        }
-    }
-};
 
 template <class R, bool CX, int BM, int BN>
 struct Cfg {
@@ -157,18 +94,64 @@ struct Cfg {
     static constexpr int BNE = CX ? BN / 2 : BN;          // element columns per tile
     static constexpr int WM = BM / 2, WN = BN / 2;        // wave tile
     static constexpr int TM = WM / 16, TN = WN / 16;
-    static constexpr size_t LDS_BYTES = (size_t)2 * (BM + BN) * PITCH * sizeof(R);
+    static constexpr int NUA = BM * BKE / THREADS, NUB = BNE * BKE / THREADS;   // elements per thread per stage
+    static constexpr size_t TILE_BYTES = (size_t)2 * (BM + BN) * PITCH * sizeof(R);
+    static constexpr size_t LDS_BYTES = TILE_BYTES + (size_t)(BM + BNE) * sizeof(int64_t);
+    static_assert(BM * BKE % THREADS == 0 && BNE * BKE % THREADS == 0, "tile must divide over the block");
+    static_assert(THREADS % BKE == 0 && THREADS % BM == 0 && THREADS % BNE == 0, "thread mapping");
 };
 
+// Loads this thread's share of one operand tile (ROWS x BKE elements) into registers.  Every address is
+// valid (row and k indices are clamped); `kmask` bit u tells whether element u lies inside the k range,
+// rows outside the matrix are zeroed when the tile is written to LDS.
+template <class E, int ROWS, int BKE, int NU>
+__device__ __forceinline__ void load_tile(E (&v)[NU], uint32_t& kmask, const E* __restrict__ base, const int64_t* rowoff_lds,
+                                          int64_t rowoff_fixed, bool kfast, const OffFn& fk, int64_t k0, int64_t kend) {
+    const int t = threadIdx.x;
+    if (kfast) {
+        const int kk = t % BKE;
+        const bool kok = k0 + kk < kend;
+        const int64_t ko = off_of(fk, kok ? k0 + kk : k0);
+        kmask = kok ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int u = 0; u < NU; ++u) v[u] = base[rowoff_lds[t / BKE + u * (THREADS / BKE)] + ko];
+    } else {
+        kmask = 0;
+        int64_t ko[NU];
+        if (fk.tab) {
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                const int64_t kidx = k0 + t / ROWS + u * (THREADS / ROWS);
+                const bool kok = kidx < kend;
+                kmask |= (kok ? 1u : 0u) << u;
+                ko[u] = fk.tab[kok ? kidx : k0];
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                const int64_t kidx = k0 + t / ROWS + u * (THREADS / ROWS);
+                const bool kok = kidx < kend;
+                kmask |= (kok ? 1u : 0u) << u;
+                ko[u] = (kok ? kidx : k0) * fk.stride;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NU; ++u) v[u] = base[rowoff_fixed + ko[u]];
+    }
+}
+
 template <class R, bool CX, int BM, int BN>
-__global__ void __launch_bounds__(THREADS) gemm_kernel(GemmArgs g) {
+__global__ void __launch_bounds__(THREADS, 2) gemm_kernel(GemmArgs g) {
     typedef Cfg<R, CX, BM, BN> C_;
     typedef typename ElemT<R, CX>::type E;
     typedef typename Mfma<R>::acc_t acc_t;
     constexpr int BKR = C_::BKR, BKE = C_::BKE, PITCH = C_::PITCH, BNE = C_::BNE, TM = C_::TM, TN = C_::TN;
+    constexpr int NUA = C_::NUA, NUB = C_::NUB;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     R* As = reinterpret_cast<R*>(smem_raw);                 // [2][BM][PITCH]
     R* Bs = As + 2 * BM * PITCH;                            // [2][BN][PITCH]
+    int64_t* rowA = reinterpret_cast<int64_t*>(smem_raw + C_::TILE_BYTES);   // [BM]  row offsets of this tile
+    int64_t* rowB = rowA + BM;                                               // [BNE]
 
     // ---- which tile ---------------------------------------------------------------------------------
     int64_t M = g.M, N = g.N, K = g.K;
@@ -196,13 +179,18 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(GemmArgs g) {
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BNE;
     const int64_t kbeg = (int64_t)split * g.k_per_split;
     const int64_t kend = (g.nsplit > 1 && kbeg + g.k_per_split < K) ? kbeg + g.k_per_split : K;
-
-    Loader<R, CX, BM, BKE> la;
-    Loader<R, CX, BNE, BKE> lb;
-    la.init(Ap, g.problems ? 0 : off_of(g.ab, batch), am, ak, m0, M, g.a_kfast);
-    lb.init(Bp, g.problems ? 0 : off_of(g.bb, batch), bn, bk, n0, N, g.b_kfast);
+    const int rowsA = (int)(M - m0 < BM ? M - m0 : BM), rowsB = (int)(N - n0 < BNE ? N - n0 : BNE);
+    const bool a_kfast = g.a_kfast, b_kfast = g.b_kfast;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // row offsets of the tile (clamped to the last valid row so that every load address is valid)
+    for (int r = tid; r < BM; r += THREADS) rowA[r] = off_of(am, m0 + (r < rowsA ? r : rowsA - 1));
+    for (int r = tid; r < BNE; r += THREADS) rowB[r] = off_of(bn, n0 + (r < rowsB ? r : rowsB - 1));
+    __syncthreads();
+    const E* baseA = reinterpret_cast<const E*>(Ap) + (g.problems ? 0 : off_of(g.ab, batch));
+    const E* baseB = reinterpret_cast<const E*>(Bp) + (g.problems ? 0 : off_of(g.bb, batch));
+    const int64_t fixedA = rowA[tid % BM], fixedB = rowB[tid % BNE];
+
     const int wm0 = (wave >> 1) * C_::WM, wn0 = (wave & 1) * C_::WN;
     const int lrow = lane & 15, lgrp = lane >> 4;
 
@@ -212,88 +200,81 @@ __global__ void __launch_bounds__(THREADS) gemm_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
 
-    E va[Loader<R, CX, BM, BKE>::NU], vb[Loader<R, CX, BNE, BKE>::NU];
+    E va[NUA], vb[NUB];
+    uint32_t maskA = 0, maskB = 0;
 
     auto store_tiles = [&](int buf) {
         R* as = As + buf * BM * PITCH;
         R* bs = Bs + buf * BN * PITCH;
 #pragma unroll
-        for (int u = 0; u < Loader<R, CX, BM, BKE>::NU; ++u) {
-            int row, kk;
-            la.coords(u, row, kk);
+        for (int u = 0; u < NUA; ++u) {
+            const int row = a_kfast ? tid / BKE + u * (THREADS / BKE) : tid % BM;
+            const int kk = a_kfast ? tid % BKE : tid / BM + u * (THREADS / BM);
+            const bool ok = row < rowsA && ((maskA >> u) & 1u);
+            E x = va[u];
             if constexpr (CX) {
-                E x = va[u];
-                if (g.conj_a) x.y = -x.y;
+                x.x = ok ? x.x : R(0);
+                x.y = ok ? (g.conj_a ? -x.y : x.y) : R(0);
                 *reinterpret_cast<E*>(as + row * PITCH + 2 * kk) = x;
             } else {
-                as[row * PITCH + kk] = va[u];
+                as[row * PITCH + kk] = ok ? x : R(0);
             }
         }
 #pragma unroll
-        for (int u = 0; u < Loader<R, CX, BNE, BKE>::NU; ++u) {
-            int row, kk;
-            lb.coords(u, row, kk);
+        for (int u = 0; u < NUB; ++u) {
+            const int row = b_kfast ? tid / BKE + u * (THREADS / BKE) : tid % BNE;
+            const int kk = b_kfast ? tid % BKE : tid / BNE + u * (THREADS / BNE);
+            const bool ok = row < rowsB && ((maskB >> u) & 1u);
+            E x = vb[u];
             if constexpr (CX) {
-                E x = vb[u];
-                if (g.conj_b) x.y = -x.y;
+                const R xr = ok ? x.x : R(0);
+                const R xi = ok ? (g.conj_b ? -x.y : x.y) : R(0);
                 E r0, r1;           // B'[2k][2n] = br, B'[2k+1][2n] = -bi ; B'[2k][2n+1] = bi, B'[2k+1][2n+1] = br
-                r0.x = x.x; r0.y = -x.y;
-                r1.x = x.y; r1.y = x.x;
+                r0.x = xr; r0.y = -xi;
+                r1.x = xi; r1.y = xr;
                 *reinterpret_cast<E*>(bs + (2 * row) * PITCH + 2 * kk) = r0;
                 *reinterpret_cast<E*>(bs + (2 * row + 1) * PITCH + 2 * kk) = r1;
             } else {
-                bs[row * PITCH + kk] = vb[u];
+                bs[row * PITCH + kk] = ok ? x : R(0);
             }
         }
     };
 
     const int64_t nstage = kend > kbeg ? (kend - kbeg + BKE - 1) / BKE : 0;
     if (nstage > 0) {
-        la.load(va, kbeg, kend);
-        lb.load(vb, kbeg, kend);
+        load_tile<E, BM, BKE, NUA>(va, maskA, baseA, rowA, fixedA, a_kfast, ak, kbeg, kend);
+        load_tile<E, BNE, BKE, NUB>(vb, maskB, baseB, rowB, fixedB, b_kfast, bk, kbeg, kend);
         store_tiles(0);
     }
     __syncthreads();
+    constexpr int NS = BKR / 4;   // MFMA k-steps per stage
     for (int64_t s = 0; s < nstage; ++s) {
         const int buf = (int)(s & 1);
         const bool more = s + 1 < nstage;
         if (more) {
-            la.load(va, kbeg + (s + 1) * BKE, kend);
-            lb.load(vb, kbeg + (s + 1) * BKE, kend);
+            load_tile<E, BM, BKE, NUA>(va, maskA, baseA, rowA, fixedA, a_kfast, ak, kbeg + (s + 1) * BKE, kend);
+            load_tile<E, BNE, BKE, NUB>(vb, maskB, baseB, rowB, fixedB, b_kfast, bk, kbeg + (s + 1) * BKE, kend);
         }
-        const R* as = As + buf * BM * PITCH + (wm0 + lrow) * PITCH + 4 * lgrp;
-        const R* bs = Bs + buf * BN * PITCH + (wn0 + lrow) * PITCH + 4 * lgrp;
+        // lane l feeds A[row l%16][k = 4*step + l/16] and B[k = 4*step + l/16][col l%16]
+        const R* as = As + buf * BM * PITCH + (wm0 + lrow) * PITCH + lgrp;
+        const R* bs = Bs + buf * BN * PITCH + (wn0 + lrow) * PITCH + lgrp;
+        R a[2][TM], b[2][TN];
 #pragma unroll
-        for (int c = 0; c < BKR / 16; ++c) {
-            R a[TM][4], b[TN][4];
+        for (int i = 0; i < TM; ++i) a[0][i] = as[i * 16 * PITCH];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const R* p = as + i * 16 * PITCH + c * 16;
-                if constexpr (sizeof(R) == 8) {
-                    double2 lo = *reinterpret_cast<const double2*>(p), hi = *reinterpret_cast<const double2*>(p + 2);
-                    a[i][0] = lo.x; a[i][1] = lo.y; a[i][2] = hi.x; a[i][3] = hi.y;
-                } else {
-                    float4 q = *reinterpret_cast<const float4*>(p);
-                    a[i][0] = q.x; a[i][1] = q.y; a[i][2] = q.z; a[i][3] = q.w;
-                }
+        for (int j = 0; j < TN; ++j) b[0][j] = bs[j * 16 * PITCH];
+#pragma unroll
+        for (int st = 0; st < NS; ++st) {
+            if (st + 1 < NS) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) a[(st + 1) & 1][i] = as[i * 16 * PITCH + 4 * (st + 1)];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) b[(st + 1) & 1][j] = bs[j * 16 * PITCH + 4 * (st + 1)];
             }
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const R* p = bs + j * 16 * PITCH + c * 16;
-                if constexpr (sizeof(R) == 8) {
-                    double2 lo = *reinterpret_cast<const double2*>(p), hi = *reinterpret_cast<const double2*>(p + 2);
-                    b[j][0] = lo.x; b[j][1] = lo.y; b[j][2] = hi.x; b[j][3] = hi.y;
-                } else {
-                    float4 q = *reinterpret_cast<const float4*>(p);
-                    b[j][0] = q.x; b[j][1] = q.y; b[j][2] = q.z; b[j][3] = q.w;
-                }
-            }
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int k4 = 0; k4 < 4; ++k4)
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<R>::run(a[i][k4], b[j][k4], acc[i][j]);
+                for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<R>::run(a[st & 1][i], b[st & 1][j], acc[i][j]);
         }
         if (more) store_tiles(buf ^ 1);
         __syncthreads();
