@@ -14,7 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libtenferro_hip.so")
-SOURCES = ["errors.cpp", "plan.cpp", "prims.cpp", "einsum.cpp", "runtime.cpp", "k_copy.hip", "k_reduce.hip", "k_gemm.hip"]
+SOURCES = ["errors.cpp", "plan.cpp", "prims.cpp", "einsum.cpp", "runtime.cpp", "k_copy.hip", "k_reduce.hip", "k_gemm.hip",
+           "k_gemm128_f32.hip", "k_gemm128_f64.hip", "k_gemm128_c64.hip", "k_gemm128_c128.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed-fp32 instruction selection is switched off for all device code
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Wall", "-Wno-unused-function",
@@ -43,7 +44,7 @@ def _compile(src, force):
 def build(force=False, verbose=False):
     os.makedirs(OBJ, exist_ok=True)
     srcs = [os.path.join(CSRC, s) for s in SOURCES]
-    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
+    with ThreadPoolExecutor(max_workers=min(12, len(srcs))) as ex:
         results = list(ex.map(lambda s: _compile(s, force), srcs))
     objs = [o for o, _ in results]
     if verbose:

@@ -1,0 +1,81 @@
+// gemm_common.hpp -- argument block and MFMA wrappers shared by the contraction kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace tfh {
+namespace gemm {
+
+constexpr int THREADS = 256;
+
+typedef double d4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+struct OffFn {
+    const int64_t* tab;  // offsets per fused index, or null
+    int64_t stride;      // used when tab == null
+};
+__device__ __forceinline__ int64_t off_of(const OffFn& f, int64_t i) { return f.tab ? f.tab[i] : i * f.stride; }
+
+// Byte offsets modulo 2^32 for the 128x128 kernel: the host rebases each operand to its lowest reachable
+// address and guarantees that the reachable span is below 4 GiB, so sums of wrapped components are exact.
+struct Off32 {
+    const uint32_t* tab;  // byte offsets per fused index, or null
+    uint32_t stride;      // byte stride (wrapped) when tab == null
+};
+__device__ __forceinline__ uint32_t off32_of(const Off32& f, int64_t i) { return f.tab ? f.tab[i] : (uint32_t)i * f.stride; }
+
+struct GroupProblem {   // one problem of a grouped launch (plain strided matrices)
+    const void* A;
+    const void* B;
+    void* C;
+    int64_t M, N, K;
+    int64_t sam, sak, sbk, sbn, scm, scn;
+};
+
+struct GemmArgs {
+    const void* A;
+    const void* B;
+    void* C;
+    int64_t M, N, K, nbatch;
+    OffFn am, ak, bk, bn, cm, cn, ab, bb, cb;
+    int32_t a_kfast, b_kfast, conj_a, conj_b;
+    int32_t nsplit, use_beta;
+    int64_t k_per_split;
+    void* partial;
+    int32_t tiles_m, tiles_n;
+    double alpha_re, alpha_im, beta_re, beta_im;
+    // 128x128 kernel only: operand bases moved to the lowest reachable address + wrapped byte offsets
+    const char* A32;
+    const char* B32;
+    Off32 am32, ak32, bk32, bn32;
+    uint32_t bias_a32, bias_b32;   // byte distance from the rebased base back to element 0
+    const GroupProblem* problems;  // grouped launch when non-null
+    const int4* tile_map;          // per block: (problem, tile_m, tile_n, 0)
+};
+
+template <class R> struct Mfma;
+template <> struct Mfma<double> {
+    typedef d4 acc_t;
+    __device__ static __forceinline__ d4 run(double a, double b, d4 c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+    // accumulator register r of lane l holds row (l/16) + 4r, column l%16
+    __device__ static __forceinline__ int row(int lane, int r) { return (lane >> 4) + 4 * r; }
+};
+template <> struct Mfma<float> {
+    typedef f4 acc_t;
+    __device__ static __forceinline__ f4 run(float a, float b, f4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+    // accumulator register r of lane l holds row 4*(l/16) + r, column l%16
+    __device__ static __forceinline__ int row(int lane, int r) { return 4 * (lane >> 4) + r; }
+};
+
+template <class R, bool CX> struct ElemT;
+template <> struct ElemT<float, false> { typedef float type; };
+template <> struct ElemT<double, false> { typedef double type; };
+template <> struct ElemT<float, true> { typedef float2 type; };
+template <> struct ElemT<double, true> { typedef double2 type; };
+
+
+
+}  // namespace gemm
+}  // namespace tfh

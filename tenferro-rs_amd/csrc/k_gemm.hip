@@ -24,66 +24,13 @@
 #include <cstring>
 #include <mutex>
 
+#include "gemm128.hpp"
 #include "internal.hpp"
 
 namespace tfh {
 namespace {
 
-constexpr int THREADS = 256;
-
-typedef double d4 __attribute__((ext_vector_type(4)));
-typedef float f4 __attribute__((ext_vector_type(4)));
-
-struct OffFn {
-    const int64_t* tab;  // offsets per fused index, or null
-    int64_t stride;      // used when tab == null
-};
-__device__ __forceinline__ int64_t off_of(const OffFn& f, int64_t i) { return f.tab ? f.tab[i] : i * f.stride; }
-
-struct GroupProblem {   // one problem of a grouped launch (plain strided matrices)
-    const void* A;
-    const void* B;
-    void* C;
-    int64_t M, N, K;
-    int64_t sam, sak, sbk, sbn, scm, scn;
-};
-
-struct GemmArgs {
-    const void* A;
-    const void* B;
-    void* C;
-    int64_t M, N, K, nbatch;
-    OffFn am, ak, bk, bn, cm, cn, ab, bb, cb;
-    int32_t a_kfast, b_kfast, conj_a, conj_b;
-    int32_t nsplit, use_beta;
-    int64_t k_per_split;
-    void* partial;
-    int32_t tiles_m, tiles_n;
-    double alpha_re, alpha_im, beta_re, beta_im;
-    const GroupProblem* problems;  // grouped launch when non-null
-    const int4* tile_map;          // per block: (problem, tile_m, tile_n, 0)
-};
-
-template <class R> struct Mfma;
-template <> struct Mfma<double> {
-    typedef d4 acc_t;
-    __device__ static __forceinline__ d4 run(double a, double b, d4 c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
-    // accumulator register r of lane l holds row (l/16) + 4r, column l%16
-    __device__ static __forceinline__ int row(int lane, int r) { return (lane >> 4) + 4 * r; }
-};
-template <> struct Mfma<float> {
-    typedef f4 acc_t;
-    __device__ static __forceinline__ f4 run(float a, float b, f4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
-    // accumulator register r of lane l holds row 4*(l/16) + r, column l%16
-    __device__ static __forceinline__ int row(int lane, int r) { return 4 * (lane >> 4) + r; }
-};
-
-template <class R, bool CX> struct ElemT;
-template <> struct ElemT<float, false> { typedef float type; };
-template <> struct ElemT<double, false> { typedef double type; };
-template <> struct ElemT<float, true> { typedef float2 type; };
-template <> struct ElemT<double, true> { typedef double2 type; };
-
+using namespace gemm;
 
 template <class R, bool CX, int BM, int BN>
 struct Cfg {
@@ -92,19 +39,22 @@ struct Cfg {
     static constexpr int PAD = 16 / sizeof(R);
     static constexpr int PITCH = BKR + PAD;
     static constexpr int BNE = CX ? BN / 2 : BN;          // element columns per tile
-    static constexpr int WM = BM / 2, WN = BN / 2;        // wave tile
+    // 128x128: 8 waves as 4x2, wave tile 32x64.  64x64: 4 waves as 2x2, wave tile 32x32.
+    static constexpr int WAVES_M = BM / 32, WAVES_N = 2;
+    static constexpr int NT = 64 * WAVES_M * WAVES_N;     // threads per block
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int TM = WM / 16, TN = WN / 16;
-    static constexpr int NUA = BM * BKE / THREADS, NUB = BNE * BKE / THREADS;   // elements per thread per stage
+    static constexpr int NUA = BM * BKE / NT, NUB = BNE * BKE / NT;   // elements per thread per stage
     static constexpr size_t TILE_BYTES = (size_t)2 * (BM + BN) * PITCH * sizeof(R);
     static constexpr size_t LDS_BYTES = TILE_BYTES + (size_t)(BM + BNE) * sizeof(int64_t);
-    static_assert(BM * BKE % THREADS == 0 && BNE * BKE % THREADS == 0, "tile must divide over the block");
-    static_assert(THREADS % BKE == 0 && THREADS % BM == 0 && THREADS % BNE == 0, "thread mapping");
+    static_assert(BM * BKE % NT == 0 && BNE * BKE % NT == 0, "tile must divide over the block");
+    static_assert(NT % BKE == 0 && NT % BM == 0 && NT % BNE == 0, "thread mapping");
 };
 
 // Loads this thread's share of one operand tile (ROWS x BKE elements) into registers.  Every address is
 // valid (row and k indices are clamped); `kmask` bit u tells whether element u lies inside the k range,
 // rows outside the matrix are zeroed when the tile is written to LDS.
-template <class E, int ROWS, int BKE, int NU>
+template <class E, int ROWS, int BKE, int NU, int NT>
 __device__ __forceinline__ void load_tile(E (&v)[NU], uint32_t& kmask, const E* __restrict__ base, const int64_t* rowoff_lds,
                                           int64_t rowoff_fixed, bool kfast, const OffFn& fk, int64_t k0, int64_t kend) {
     const int t = threadIdx.x;
@@ -114,14 +64,14 @@ __device__ __forceinline__ void load_tile(E (&v)[NU], uint32_t& kmask, const E* 
         const int64_t ko = off_of(fk, kok ? k0 + kk : k0);
         kmask = kok ? 0xffffffffu : 0u;
 #pragma unroll
-        for (int u = 0; u < NU; ++u) v[u] = base[rowoff_lds[t / BKE + u * (THREADS / BKE)] + ko];
+        for (int u = 0; u < NU; ++u) v[u] = base[rowoff_lds[t / BKE + u * (NT / BKE)] + ko];
     } else {
         kmask = 0;
         int64_t ko[NU];
         if (fk.tab) {
 #pragma unroll
             for (int u = 0; u < NU; ++u) {
-                const int64_t kidx = k0 + t / ROWS + u * (THREADS / ROWS);
+                const int64_t kidx = k0 + t / ROWS + u * (NT / ROWS);
                 const bool kok = kidx < kend;
                 kmask |= (kok ? 1u : 0u) << u;
                 ko[u] = fk.tab[kok ? kidx : k0];
@@ -129,7 +79,7 @@ __device__ __forceinline__ void load_tile(E (&v)[NU], uint32_t& kmask, const E* 
         } else {
 #pragma unroll
             for (int u = 0; u < NU; ++u) {
-                const int64_t kidx = k0 + t / ROWS + u * (THREADS / ROWS);
+                const int64_t kidx = k0 + t / ROWS + u * (NT / ROWS);
                 const bool kok = kidx < kend;
                 kmask |= (kok ? 1u : 0u) << u;
                 ko[u] = (kok ? kidx : k0) * fk.stride;
@@ -141,12 +91,12 @@ __device__ __forceinline__ void load_tile(E (&v)[NU], uint32_t& kmask, const E* 
 }
 
 template <class R, bool CX, int BM, int BN>
-__global__ void __launch_bounds__(THREADS, 2) gemm_kernel(GemmArgs g) {
+__global__ void __launch_bounds__((Cfg<R, CX, BM, BN>::NT), 2) gemm_kernel(GemmArgs g) {
     typedef Cfg<R, CX, BM, BN> C_;
     typedef typename ElemT<R, CX>::type E;
     typedef typename Mfma<R>::acc_t acc_t;
     constexpr int BKR = C_::BKR, BKE = C_::BKE, PITCH = C_::PITCH, BNE = C_::BNE, TM = C_::TM, TN = C_::TN;
-    constexpr int NUA = C_::NUA, NUB = C_::NUB;
+    constexpr int NUA = C_::NUA, NUB = C_::NUB, NT = C_::NT;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     R* As = reinterpret_cast<R*>(smem_raw);                 // [2][BM][PITCH]
     R* Bs = As + 2 * BM * PITCH;                            // [2][BN][PITCH]
@@ -184,14 +134,14 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_kernel(GemmArgs g) {
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // row offsets of the tile (clamped to the last valid row so that every load address is valid)
-    for (int r = tid; r < BM; r += THREADS) rowA[r] = off_of(am, m0 + (r < rowsA ? r : rowsA - 1));
-    for (int r = tid; r < BNE; r += THREADS) rowB[r] = off_of(bn, n0 + (r < rowsB ? r : rowsB - 1));
+    for (int r = tid; r < BM; r += NT) rowA[r] = off_of(am, m0 + (r < rowsA ? r : rowsA - 1));
+    for (int r = tid; r < BNE; r += NT) rowB[r] = off_of(bn, n0 + (r < rowsB ? r : rowsB - 1));
     __syncthreads();
     const E* baseA = reinterpret_cast<const E*>(Ap) + (g.problems ? 0 : off_of(g.ab, batch));
     const E* baseB = reinterpret_cast<const E*>(Bp) + (g.problems ? 0 : off_of(g.bb, batch));
     const int64_t fixedA = rowA[tid % BM], fixedB = rowB[tid % BNE];
 
-    const int wm0 = (wave >> 1) * C_::WM, wn0 = (wave & 1) * C_::WN;
+    const int wm0 = (wave / C_::WAVES_N) * C_::WM, wn0 = (wave % C_::WAVES_N) * C_::WN;
     const int lrow = lane & 15, lgrp = lane >> 4;
 
     acc_t acc[TM][TN];
@@ -208,8 +158,8 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_kernel(GemmArgs g) {
         R* bs = Bs + buf * BN * PITCH;
 #pragma unroll
         for (int u = 0; u < NUA; ++u) {
-            const int row = a_kfast ? tid / BKE + u * (THREADS / BKE) : tid % BM;
-            const int kk = a_kfast ? tid % BKE : tid / BM + u * (THREADS / BM);
+            const int row = a_kfast ? tid / BKE + u * (NT / BKE) : tid % BM;
+            const int kk = a_kfast ? tid % BKE : tid / BM + u * (NT / BM);
             const bool ok = row < rowsA && ((maskA >> u) & 1u);
             E x = va[u];
             if constexpr (CX) {
@@ -222,8 +172,8 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_kernel(GemmArgs g) {
         }
 #pragma unroll
         for (int u = 0; u < NUB; ++u) {
-            const int row = b_kfast ? tid / BKE + u * (THREADS / BKE) : tid % BNE;
-            const int kk = b_kfast ? tid % BKE : tid / BNE + u * (THREADS / BNE);
+            const int row = b_kfast ? tid / BKE + u * (NT / BKE) : tid % BNE;
+            const int kk = b_kfast ? tid % BKE : tid / BNE + u * (NT / BNE);
             const bool ok = row < rowsB && ((maskB >> u) & 1u);
             E x = vb[u];
             if constexpr (CX) {
@@ -242,8 +192,8 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_kernel(GemmArgs g) {
 
     const int64_t nstage = kend > kbeg ? (kend - kbeg + BKE - 1) / BKE : 0;
     if (nstage > 0) {
-        load_tile<E, BM, BKE, NUA>(va, maskA, baseA, rowA, fixedA, a_kfast, ak, kbeg, kend);
-        load_tile<E, BNE, BKE, NUB>(vb, maskB, baseB, rowB, fixedB, b_kfast, bk, kbeg, kend);
+        load_tile<E, BM, BKE, NUA, NT>(va, maskA, baseA, rowA, fixedA, a_kfast, ak, kbeg, kend);
+        load_tile<E, BNE, BKE, NUB, NT>(vb, maskB, baseB, rowB, fixedB, b_kfast, bk, kbeg, kend);
         store_tiles(0);
     }
     __syncthreads();
@@ -252,8 +202,8 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_kernel(GemmArgs g) {
         const int buf = (int)(s & 1);
         const bool more = s + 1 < nstage;
         if (more) {
-            load_tile<E, BM, BKE, NUA>(va, maskA, baseA, rowA, fixedA, a_kfast, ak, kbeg + (s + 1) * BKE, kend);
-            load_tile<E, BNE, BKE, NUB>(vb, maskB, baseB, rowB, fixedB, b_kfast, bk, kbeg + (s + 1) * BKE, kend);
+            load_tile<E, BM, BKE, NUA, NT>(va, maskA, baseA, rowA, fixedA, a_kfast, ak, kbeg + (s + 1) * BKE, kend);
+            load_tile<E, BNE, BKE, NUB, NT>(vb, maskB, baseB, rowB, fixedB, b_kfast, bk, kbeg + (s + 1) * BKE, kend);
         }
         // lane l feeds A[row l%16][k = 4*step + l/16] and B[k = 4*step + l/16][col l%16]
         const R* as = As + buf * BM * PITCH + (wm0 + lrow) * PITCH + lgrp;
@@ -381,9 +331,10 @@ __global__ void __launch_bounds__(THREADS) splitk_finalize_kernel(GemmArgs g) {
 
 // Offsets of every fused index of an axis group (last axis fastest): tab[i] = sum_d idx_d * stride_d.
 struct TableJob {
-    int64_t* dst;
+    int64_t* dst;        // element offsets, or
+    uint32_t* dst32;     // byte offsets modulo 2^32 (when non-null)
     int64_t n;
-    int32_t naxes;
+    int32_t naxes, elem_bytes;
     int64_t dims[TFH_MAX_RANK], strides[TFH_MAX_RANK];
 };
 __global__ void __launch_bounds__(THREADS) build_table_kernel(TableJob j) {
@@ -395,7 +346,8 @@ __global__ void __launch_bounds__(THREADS) build_table_kernel(TableJob j) {
         off += (lin - q * j.dims[d]) * j.strides[d];
         lin = q;
     }
-    j.dst[i] = off;
+    if (j.dst32) j.dst32[i] = (uint32_t)(off * j.elem_bytes);
+    else j.dst[i] = off;
 }
 
 int64_t prod(const std::vector<Axis>& ax) {
@@ -428,21 +380,33 @@ void launch_tile(const GemmArgs& g, dim3 grid, hipStream_t st) {
         return true;
     }();
     (void)once;
-    hipLaunchKernelGGL((gemm_kernel<R, CX, BM, BN>), grid, dim3(THREADS), lds, st, g);
+    hipLaunchKernelGGL((gemm_kernel<R, CX, BM, BN>), grid, dim3(Cfg<R, CX, BM, BN>::NT), lds, st, g);
 }
 
-template <class R, bool CX>
-void launch_any_tile(const GemmArgs& g, dim3 grid, int bm, hipStream_t st) {
-    if (bm == 128) launch_tile<R, CX, 128, 128>(g, grid, st);
-    else launch_tile<R, CX, 64, 64>(g, grid, st);
-}
-
-void launch_dtype(int dtype, const GemmArgs& g, dim3 grid, int bm, hipStream_t st) {
+void launch_generic64(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st) {
     switch (dtype) {
-        case TFH_F32: launch_any_tile<float, false>(g, grid, bm, st); break;
-        case TFH_F64: launch_any_tile<double, false>(g, grid, bm, st); break;
-        case TFH_C64: launch_any_tile<float, true>(g, grid, bm, st); break;
-        default: launch_any_tile<double, true>(g, grid, bm, st); break;
+        case TFH_F32: launch_tile<float, false, 64, 64>(g, grid, st); break;
+        case TFH_F64: launch_tile<double, false, 64, 64>(g, grid, st); break;
+        case TFH_C64: launch_tile<float, true, 64, 64>(g, grid, st); break;
+        default: launch_tile<double, true, 64, 64>(g, grid, st); break;
+    }
+}
+void launch_128(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st) {
+    switch (dtype) {
+        case TFH_F32: launch_gemm128_f32(g, grid, g.a_kfast, g.b_kfast, st); break;
+        case TFH_F64: launch_gemm128_f64(g, grid, g.a_kfast, g.b_kfast, st); break;
+        case TFH_C64: launch_gemm128_c64(g, grid, g.a_kfast, g.b_kfast, st); break;
+        default: launch_gemm128_c128(g, grid, g.a_kfast, g.b_kfast, st); break;
+    }
+}
+
+// Lowest and highest element offset reachable through a set of axes (slot = operand).
+void reach(const std::vector<Axis>& ax, int slot, int64_t& lo, int64_t& hi) {
+    for (auto& a : ax) {
+        if (a.n <= 1) continue;
+        int64_t e = (a.n - 1) * a.s[slot];
+        if (e < 0) lo += e;
+        else hi += e;
     }
 }
 
@@ -526,6 +490,20 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         return set_error(TFH_ERR_INVALID_ARGUMENT, "contraction too large for one launch (tiles %lld, batch*split %lld)",
                          (long long)g.tiles_m * g.tiles_n, (long long)(nb * nsplit));
 
+    // The 128x128 kernel addresses each operand as a uniform base + 32-bit byte offset: usable when the
+    // bytes reachable inside one batch entry span less than 4 GiB (larger operands take the generic kernel).
+    bool use128 = bm == 128;
+    int64_t lo_a = 0, hi_a = 0, lo_b = 0, hi_b = 0;
+    reach(ax.M, 0, lo_a, hi_a); reach(ax.K, 0, lo_a, hi_a);
+    reach(ax.N, 1, lo_b, hi_b); reach(ax.K, 1, lo_b, hi_b);
+    if ((hi_a - lo_a + 1) * (int64_t)eb >= ((int64_t)1 << 32) || (hi_b - lo_b + 1) * (int64_t)eb >= ((int64_t)1 << 32)) use128 = false;
+    if (!use128 && bm == 128) {
+        bm = 64;
+        g.tiles_m = (int)((M + bm - 1) / bm);
+        g.tiles_n = (int)((NR + bm - 1) / bm);
+    }
+    const bool ktab32 = use128 && (ax.K.size() > 1);   // k tables for both operands or for none
+
     // workspace: offset tables for every multi-axis group, then the split-K partials
     struct Want { std::vector<Axis>* grp; int slot; OffFn* fn; int64_t n; };
     Want wants[9] = {{&ax.M, 0, &g.am, M}, {&ax.K, 0, &g.ak, K}, {&ax.K, 1, &g.bk, K}, {&ax.N, 1, &g.bn, N}, {&ax.M, 2, &g.cm, M},
@@ -533,6 +511,12 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     size_t table_bytes = 0;
     for (auto& w : wants)
         if (w.grp->size() > 1) table_bytes += ((size_t)w.n * sizeof(int64_t) + 255) & ~(size_t)255;
+    // 32-bit tables of the 128 kernel: rows of A and B when multi-axis, k of both when k is multi-axis
+    struct Want32 { std::vector<Axis>* grp; int slot; Off32* fn; int64_t n; bool force; };
+    Want32 wants32[4] = {{&ax.M, 0, &g.am32, M, false}, {&ax.K, 0, &g.ak32, K, ktab32}, {&ax.K, 1, &g.bk32, K, ktab32}, {&ax.N, 1, &g.bn32, N, false}};
+    if (use128)
+        for (auto& w : wants32)
+            if (w.grp->size() > 1 || w.force) table_bytes += ((size_t)w.n * sizeof(uint32_t) + 255) & ~(size_t)255;
     size_t partial_bytes = nsplit > 1 ? (size_t)nsplit * nb * M * NR * rb : 0;
     char* ws = nullptr;
     if (table_bytes + partial_bytes) {
@@ -561,10 +545,38 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         w.fn->stride = 0;
         cursor += ((size_t)w.n * sizeof(int64_t) + 255) & ~(size_t)255;
     }
+    if (use128) {
+        for (auto& w : wants32) {
+            if (w.grp->size() <= 1 && !w.force) {
+                w.fn->tab = nullptr;
+                w.fn->stride = w.grp->empty() ? 0u : (uint32_t)((*w.grp)[0].s[w.slot] * (int64_t)eb);
+                continue;
+            }
+            TableJob j;
+            std::memset(&j, 0, sizeof j);
+            j.dst32 = (uint32_t*)(ws + cursor);
+            j.n = w.n;
+            j.elem_bytes = (int32_t)eb;
+            j.naxes = (int)w.grp->size();
+            for (int d = 0; d < j.naxes; ++d) {
+                j.dims[d] = (*w.grp)[d].n;
+                j.strides[d] = (*w.grp)[d].s[w.slot];
+            }
+            hipLaunchKernelGGL(build_table_kernel, dim3((uint32_t)((w.n + THREADS - 1) / THREADS)), dim3(THREADS), 0, st, j);
+            w.fn->tab = j.dst32;
+            w.fn->stride = 0;
+            cursor += ((size_t)w.n * sizeof(uint32_t) + 255) & ~(size_t)255;
+        }
+        g.A32 = (const char*)a + lo_a * (int64_t)eb;
+        g.B32 = (const char*)b + lo_b * (int64_t)eb;
+        g.bias_a32 = (uint32_t)(-lo_a * (int64_t)eb);
+        g.bias_b32 = (uint32_t)(-lo_b * (int64_t)eb);
+    }
     if (nsplit > 1) g.partial = ws + cursor;
     dim3 grid((uint32_t)(g.tiles_m * g.tiles_n), 1, (uint32_t)(nb * nsplit));
     const int prof = prof_begin(PROF_CONTRACT, stream);
-    launch_dtype(dtype, g, grid, bm, st);
+    if (use128) launch_128(dtype, g, grid, st);
+    else launch_generic64(dtype, g, grid, st);
     prof_end(prof, stream);
     if (int32_t e = hip_check(hipGetLastError(), "contraction kernel launch")) return e;
     if (nsplit > 1) {
@@ -667,6 +679,7 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
     const int dtype = plan.dtype;
     const size_t eb = dtype_size(dtype);
     std::vector<GroupProblem> probs((size_t)plan.n_groups);
+    bool ok128 = true;
     for (int gi = 0; gi < plan.n_groups; ++gi) {
         const tfh_view& va = inputs[(size_t)gi * 2 + 0];
         const tfh_view& vb = inputs[(size_t)gi * 2 + 1];
@@ -700,7 +713,12 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
         p.sak = ax.K.empty() ? 0 : ax.K[0].s[0];
         p.sbk = ax.K.empty() ? 0 : ax.K[0].s[1];
         if ((p.M > 1 && p.scm == 0) || (p.N > 1 && p.scn == 0)) return set_error(TFH_ERR_STRIDED, "output view has stride 0");
+        if (p.sam < 0 || p.sak < 0 || p.sbk < 0 || p.sbn < 0) ok128 = false;
+        if (((p.M - 1) * p.sam + (p.K - 1) * p.sak + 1) * (int64_t)eb >= ((int64_t)1 << 32)) ok128 = false;
+        if (((p.N - 1) * p.sbn + (p.K - 1) * p.sbk + 1) * (int64_t)eb >= ((int64_t)1 << 32)) ok128 = false;
     }
+    if (gs->bm == 128 && !ok128)
+        return set_error(TFH_ERR_INVALID_ARGUMENT, "grouped contraction: an operand has a negative stride or spans 4 GiB or more");
     {
         std::lock_guard<std::mutex> lk(gs->mu);
         int dev = 0;
@@ -741,7 +759,8 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
     g.tile_map = gs->tile_map_dev;
     dim3 grid((uint32_t)gs->tile_map_host.size(), 1, 1);
     const int prof = prof_begin(PROF_CONTRACT, stream);
-    launch_dtype(dtype, g, grid, gs->bm, st);
+    if (gs->bm == 128) launch_128(dtype, g, grid, st);
+    else launch_generic64(dtype, g, grid, st);
     prof_end(prof, stream);
     return hip_check(hipGetLastError(), "grouped contraction launch");
 }

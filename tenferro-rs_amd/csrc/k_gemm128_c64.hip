@@ -1,0 +1,8 @@
+// k_gemm128_c64.hip -- instantiates the 128x128 contraction kernel for c64 (four operand layouts).
+#include "gemm128.hpp"
+
+namespace tfh {
+void launch_gemm128_c64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
+    gemm::launch_gemm128_any<float, true>(g, grid, akf, bkf, st);
+}
+}  // namespace tfh
