@@ -446,12 +446,59 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
             for (auto& x : *grp) std::swap(x.s[0], x.s[1]);
     }
     // loaders run their lanes along k when the operand is contiguous in k, along the row index otherwise
-    const bool a_kfast = min_stride(ax.K, 0) <= min_stride(ax.M, 0);
-    const bool b_kfast = min_stride(ax.K, 1) <= min_stride(ax.N, 1);
+    bool a_kfast = min_stride(ax.K, 0) <= min_stride(ax.M, 0);
+    bool b_kfast = min_stride(ax.K, 1) <= min_stride(ax.N, 1);
+    // the order of the k modes is free (it is a sum): follow the memory order of the larger k-contiguous operand
+    const bool k_by_b = b_kfast && (!a_kfast || N > M);
     order_by(ax.M, a_kfast ? 2 : 0);
     order_by(ax.N, 2);
-    order_by(ax.K, a_kfast ? 0 : (b_kfast ? 1 : 0));
+    order_by(ax.K, k_by_b ? 1 : 0);
     order_by(ax.batch, 2);
+
+    // An operand whose lanes would stride through memory (its contiguous mode is not the one the loader's lanes
+    // run along) is first packed into [batch][rows][k], k contiguous, by the tiled copy kernel: two passes over
+    // that operand instead of one 64-byte sector per element in every tile that re-reads it.
+    void* packed[2] = {nullptr, nullptr};
+    auto release_packed = [&]() {
+        for (void* p : packed) pool_free(stream, p);
+    };
+    for (int slot = 0; slot < 2; ++slot) {
+        std::vector<Axis>& rows = slot == 0 ? ax.M : ax.N;
+        const bool kfast = slot == 0 ? a_kfast : b_kfast;
+        const std::vector<Axis>& lanes = kfast ? ax.K : rows;
+        if (lanes.empty() || lanes.back().n == 1) continue;
+        const Axis& inner = lanes.back();
+        const int64_t run = std::llabs(inner.s[slot]) == 1 ? inner.n * (int64_t)eb : (int64_t)eb;
+        if (run >= 32) continue;
+        int64_t elems = 1;
+        for (auto* grp : {&ax.batch, &rows, &ax.K})
+            for (auto& x : *grp)
+                if (x.s[slot] != 0) elems *= x.n;
+        if (elems * (int64_t)eb > ((int64_t)2 << 30) || elems < 4096) continue;
+        void* buf = nullptr;
+        if (int32_t e = pool_alloc(stream, (size_t)elems * eb, &buf)) {
+            release_packed();
+            return e;
+        }
+        packed[slot] = buf;
+        std::vector<Axis> cp;
+        int64_t stride = 1;
+        std::vector<Axis>* order[3] = {&ax.K, &rows, &ax.batch};   // innermost group first
+        for (auto* grp : order)
+            for (int d = (int)grp->size() - 1; d >= 0; --d) {
+                Axis& x = (*grp)[d];
+                if (x.s[slot] == 0) continue;
+                cp.push_back(Axis{x.n, {x.s[slot], stride, 0}, x.label});
+                x.s[slot] = stride;
+                stride *= x.n;
+            }
+        if (int32_t e = launch_copy(dtype, slot == 0 ? a : b, buf, cp, Scalar{1, 0}, Scalar{0, 0}, false, stream)) {
+            release_packed();
+            return e;
+        }
+        if (slot == 0) { a = buf; a_kfast = true; }
+        else { b = buf; b_kfast = true; }
+    }
     fuse_axes(ax.M, 3);
     fuse_axes(ax.N, 3);
     fuse_axes(ax.K, 3);
@@ -486,9 +533,11 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     g.k_per_split = kps;
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((NR + bm - 1) / bm);
-    if ((int64_t)g.tiles_m * g.tiles_n > 0x7fffffffll || nb * nsplit > 65535)
+    if ((int64_t)g.tiles_m * g.tiles_n > 0x7fffffffll || nb * nsplit > 65535) {
+        release_packed();
         return set_error(TFH_ERR_INVALID_ARGUMENT, "contraction too large for one launch (tiles %lld, batch*split %lld)",
                          (long long)g.tiles_m * g.tiles_n, (long long)(nb * nsplit));
+    }
 
     // The 128x128 kernel addresses each operand as a uniform base + 32-bit byte offset: usable when the
     // bytes reachable inside one batch entry span less than 4 GiB (larger operands take the generic kernel).
@@ -521,7 +570,10 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     char* ws = nullptr;
     if (table_bytes + partial_bytes) {
         void* p = nullptr;
-        if (int32_t e = workspace(stream, table_bytes + partial_bytes, &p)) return e;
+        if (int32_t e = workspace(stream, table_bytes + partial_bytes, &p)) {
+            release_packed();
+            return e;
+        }
         ws = (char*)p;
     }
     size_t cursor = 0;
@@ -578,6 +630,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     if (use128) launch_128(dtype, g, grid, st);
     else launch_generic64(dtype, g, grid, st);
     prof_end(prof, stream);
+    release_packed();   // stream-ordered: the next user of these blocks is enqueued after this kernel
     if (int32_t e = hip_check(hipGetLastError(), "contraction kernel launch")) return e;
     if (nsplit > 1) {
         int64_t total = nb * M * N;
