@@ -29,6 +29,7 @@ struct CopyArgs {
     int32_t nt, ng;
     int32_t tile_elems;    // product of tile extents (power of two)
     int32_t pad_;
+    int64_t ntiles;        // tiles in the whole tensor (the copy kernel's blocks loop over them)
     // tile axes in read order (ascending input stride) and in write order (ascending output stride)
     int32_t r_shift[MAXT], r_mask[MAXT], r_id[MAXT];
     int64_t r_si[MAXT];
@@ -50,12 +51,11 @@ struct BlockOrigin {
     int64_t lim[MAXT];  // remaining extent of each tile axis at this block
 };
 
-__device__ __forceinline__ BlockOrigin block_origin(const CopyArgs& a) {
+__device__ __forceinline__ BlockOrigin block_origin(const CopyArgs& a, uint64_t bid) {
     BlockOrigin o;
     o.in = o.in2 = o.out = 0;
 #pragma unroll
     for (int t = 0; t < MAXT; ++t) o.lim[t] = t < a.nt ? a.t_n[t] : 1;
-    uint64_t bid = (uint64_t)blockIdx.x + (uint64_t)blockIdx.y * gridDim.x;
     for (int g = 0; g < a.ng; ++g) {
         uint64_t q = bid / (uint64_t)a.g_count[g];
         int64_t c = (int64_t)(bid - q * (uint64_t)a.g_count[g]);
@@ -111,68 +111,105 @@ struct ConjOp {  // bit-exact conj: flip the sign of the imaginary part
     }
 };
 
-template <class V, class Op, int EPT, bool READ_OLD>
+template <class V, int N>
+struct alignas(sizeof(V) * N) Pack {
+    V v[N];
+};
+
+__device__ __forceinline__ int64_t pick_lim(const BlockOrigin& o, int id) {
+    return id == 0 ? o.lim[0] : id == 1 ? o.lim[1] : id == 2 ? o.lim[2] : o.lim[3];
+}
+
+// Persistent blocks: block b moves tiles b, b + gridDim.x, ...  The next tile's global loads are issued
+// (into registers) before the current tile is written out, so loads stay in flight during the store phase.
+// VR / VW: elements per global access on the read / write side (16-byte accesses when the layout allows).
+template <class V, class Op, int EPT, int VR, int VW, bool READ_OLD>
 __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     V* lds = reinterpret_cast<V*>(smem_raw);
-    const BlockOrigin o = block_origin(a);
-    const V* in = reinterpret_cast<const V*>(a.in) + o.in;
-    V* out = reinterpret_cast<V*>(a.out) + o.out;
-    const int tid = threadIdx.x;
+    int tid = threadIdx.x;
     V regs[EPT];
+    auto load = [&](const BlockOrigin& o) {
+        // the index arithmetic below is invariant over the tile loop; recomputing it per tile is far cheaper
+        // than the ~100 registers it would occupy if hoisted, so hide the invariance from the optimiser
+        asm volatile("" : "+v"(tid));
+        const V* in = reinterpret_cast<const V*>(a.in) + o.in;
+#pragma clang loop unroll(full)
+        for (int u = 0; u < EPT / VR; ++u) {
+            const int r = (u * THREADS + tid) * VR;
+            bool ok = r < a.tile_elems;
+            int64_t off = 0;
 #pragma unroll
-    for (int u = 0; u < EPT; ++u) {
-        int r = u * THREADS + tid;
-        bool ok = r < a.tile_elems;
-        int64_t off = 0;
-#pragma unroll
-        for (int t = 0; t < MAXT; ++t) {
-            if (t < a.nt) {
-                int c = (r >> a.r_shift[t]) & a.r_mask[t];
+            for (int t = 0; t < MAXT; ++t) {   // unused axis slots are neutral: mask 0, stride 0, id 0
+                const int c = (r >> a.r_shift[t]) & a.r_mask[t];
                 off += (int64_t)c * a.r_si[t];
-                int id = a.r_id[t];
-                int64_t lim = id == 0 ? o.lim[0] : id == 1 ? o.lim[1] : id == 2 ? o.lim[2] : o.lim[3];
-                ok &= c < lim;
+                ok &= c < pick_lim(o, a.r_id[t]);
+            }
+            if (ok) {
+                const Pack<V, VR> p = *reinterpret_cast<const Pack<V, VR>*>(in + off);
+#pragma unroll
+                for (int j = 0; j < VR; ++j) regs[u * VR + j] = p.v[j];
             }
         }
-        if (ok) regs[u] = in[off];
-    }
+    };
+    uint64_t tile = blockIdx.x;
+    if (tile >= (uint64_t)a.ntiles) return;
+    BlockOrigin o = block_origin(a, tile);
+    load(o);
+    for (;;) {
+#pragma clang loop unroll(full)
+        for (int u = 0; u < EPT / VR; ++u) {
+            const int r = (u * THREADS + tid) * VR;
+            if (r < a.tile_elems) {
 #pragma unroll
-    for (int u = 0; u < EPT; ++u) {
-        int r = u * THREADS + tid;
-        if (r < a.tile_elems) lds[swz(r)] = regs[u];
-    }
-    __syncthreads();
+                for (int j = 0; j < VR; ++j) lds[swz(r) + j] = regs[u * VR + j];
+            }
+        }
+        __syncthreads();
+        const uint64_t next = tile + gridDim.x;
+        const bool more = next < (uint64_t)a.ntiles;
+        BlockOrigin o2 = o;
+        if (more) {
+            o2 = block_origin(a, next);
+            load(o2);
+        }
+        V* out = reinterpret_cast<V*>(a.out) + o.out;
+        asm volatile("" : "+v"(tid));
+#pragma clang loop unroll(full)
+        for (int u = 0; u < EPT / VW; ++u) {
+            const int w = (u * THREADS + tid) * VW;
+            bool ok = w < a.tile_elems;
+            int64_t off = 0;
+            int r = 0;
 #pragma unroll
-    for (int u = 0; u < EPT; ++u) {
-        int w = u * THREADS + tid;
-        bool ok = w < a.tile_elems;
-        int64_t off = 0;
-        int r = 0;
-#pragma unroll
-        for (int t = 0; t < MAXT; ++t) {
-            if (t < a.nt) {
-                int c = (w >> a.w_shift[t]) & a.w_mask[t];
+            for (int t = 0; t < MAXT; ++t) {
+                const int c = (w >> a.w_shift[t]) & a.w_mask[t];
                 off += (int64_t)c * a.w_so[t];
                 r += c * a.w_rpos[t];
-                int id = a.w_id[t];
-                int64_t lim = id == 0 ? o.lim[0] : id == 1 ? o.lim[1] : id == 2 ? o.lim[2] : o.lim[3];
-                ok &= c < lim;
+                ok &= c < pick_lim(o, a.w_id[t]);
+            }
+            if (ok) {
+                Pack<V, VW> x, old;
+#pragma unroll
+                for (int j = 0; j < VW; ++j) x.v[j] = lds[swz(r + j * a.w_rpos[0])];
+                old = x;
+                if (READ_OLD) old = *reinterpret_cast<const Pack<V, VW>*>(out + off);
+#pragma unroll
+                for (int j = 0; j < VW; ++j) x.v[j] = op(x.v[j], old.v[j], a);
+                *reinterpret_cast<Pack<V, VW>*>(out + off) = x;
             }
         }
-        if (ok) {
-            V x = lds[swz(r)];
-            V old = x;
-            if (READ_OLD) old = out[off];
-            out[off] = op(x, old, a);
-        }
+        if (!more) break;
+        __syncthreads();
+        tile = next;
+        o = o2;
     }
 }
 
 // Direct (no LDS) kernels in write order: fill and elementwise multiply.
 template <class V>
 __global__ void __launch_bounds__(THREADS) fill_kernel(CopyArgs a, V value, int ept) {
-    const BlockOrigin o = block_origin(a);
+    const BlockOrigin o = block_origin(a, (uint64_t)blockIdx.x + (uint64_t)blockIdx.y * gridDim.x);
     V* out = reinterpret_cast<V*>(a.out) + o.out;
     for (int u = 0; u < ept; ++u) {
         int w = u * THREADS + threadIdx.x;
@@ -181,7 +218,7 @@ __global__ void __launch_bounds__(THREADS) fill_kernel(CopyArgs a, V value, int 
         for (int t = 0; t < a.nt; ++t) {
             int c = (w >> a.w_shift[t]) & a.w_mask[t];
             off += (int64_t)c * a.w_so[t];
-            ok &= c < o.lim[a.w_id[t]];
+            ok &= c < pick_lim(o, a.w_id[t]);
         }
         if (ok) out[off] = value;
     }
@@ -190,7 +227,7 @@ __global__ void __launch_bounds__(THREADS) fill_kernel(CopyArgs a, V value, int 
 template <class R, bool CX>
 __global__ void __launch_bounds__(THREADS) emul_kernel(CopyArgs a, int ept) {
     constexpr int NC = CX ? 2 : 1;
-    const BlockOrigin o = block_origin(a);
+    const BlockOrigin o = block_origin(a, (uint64_t)blockIdx.x + (uint64_t)blockIdx.y * gridDim.x);
     const R* A = reinterpret_cast<const R*>(a.in) + o.in * NC;
     const R* B = reinterpret_cast<const R*>(a.in2) + o.in2 * NC;
     R* C = reinterpret_cast<R*>(a.out) + o.out * NC;
@@ -203,7 +240,7 @@ __global__ void __launch_bounds__(THREADS) emul_kernel(CopyArgs a, int ept) {
             oa += (int64_t)c * a.w_si[t];
             ob += (int64_t)c * a.w_si2[t];
             oc += (int64_t)c * a.w_so[t];
-            ok &= c < o.lim[a.w_id[t]];
+            ok &= c < pick_lim(o, a.w_id[t]);
         }
         if (!ok) continue;
         R ar = (R)a.alpha_re, ai = (R)a.alpha_im;
@@ -237,6 +274,8 @@ struct TilePlan {
     CopyArgs args;
     dim3 grid;
     int ept;
+    bool vec_in, vec_out;   // strides allow 16-byte accesses on the input / output side
+    uint32_t persistent;    // block count for the looping copy kernel
 };
 
 // axes: s[0] = input stride, s[1] = output stride, s[2] = second input stride (emul only).
@@ -335,22 +374,40 @@ int32_t plan_tiles(std::vector<Axis> axes, int elem_bytes, int max_tile_elems, b
         a.w_si2[t] = axes[i].s[2];
         sh += tl[i];
     }
-    // grid axes
+    // grid axes; the axes a tile covers only partly come first (fastest block index), so blocks that run at
+    // the same time complete each other's contiguous runs in DRAM
     a.ng = 0;
     uint64_t blocks = 1;
-    for (int i = 0; i < na; ++i) {
-        int64_t text = (int64_t)1 << tl[i];
-        int64_t cnt = (axes[i].n + text - 1) / text;
-        if (cnt <= 1) continue;
-        int g = a.ng++;
-        a.g_count[g] = cnt;
-        a.g_si[g] = axes[i].s[0] * text;
-        a.g_si2[g] = axes[i].s[2] * text;
-        a.g_so[g] = axes[i].s[1] * text;
-        a.g_tid[g] = tl[i] > 0 ? id_of(i) : -1;
-        a.g_text[g] = (int32_t)text;
-        blocks *= (uint64_t)cnt;
-    }
+    for (int pass = 0; pass < 2; ++pass)
+        for (int i = 0; i < na; ++i) {
+            int64_t text = (int64_t)1 << tl[i];
+            int64_t cnt = (axes[i].n + text - 1) / text;
+            if (cnt <= 1) continue;
+            if ((pass == 0) != (tl[i] > 0)) continue;
+            int g = a.ng++;
+            a.g_count[g] = cnt;
+            a.g_si[g] = axes[i].s[0] * text;
+            a.g_si2[g] = axes[i].s[2] * text;
+            a.g_so[g] = axes[i].s[1] * text;
+            a.g_tid[g] = tl[i] > 0 ? id_of(i) : -1;
+            a.g_text[g] = (int32_t)text;
+            blocks *= (uint64_t)cnt;
+        }
+    a.ntiles = (int64_t)blocks;
+    tp.persistent = (uint32_t)std::min<uint64_t>(blocks, 1024);
+    // 16-byte accesses: the side's fastest tile axis is contiguous, a multiple of the vector length, and every
+    // other stride keeps the vectors aligned
+    const int vec = 16 / elem_bytes;
+    auto side_ok = [&](int slot, const std::vector<int>& order_) {
+        if (vec <= 1 || order_.empty()) return false;
+        const int i0 = order_[0];
+        if (axes[i0].s[slot] != 1 || axes[i0].n % vec != 0 || (1 << tl[i0]) < vec) return false;
+        for (int i = 0; i < na; ++i)
+            if (i != i0 && axes[i].s[slot] % vec != 0) return false;
+        return true;
+    };
+    tp.vec_in = side_ok(0, rd);
+    tp.vec_out = side_ok(1, wr);
     if (blocks > (uint64_t)0x7fffffff * 65535ull) return set_error(TFH_ERR_INVALID_ARGUMENT, "tensor too large for one launch");
     uint32_t gx = (uint32_t)std::min<uint64_t>(blocks, 0x7fffffffull);
     uint32_t gy = (uint32_t)((blocks + gx - 1) / gx);
@@ -374,21 +431,38 @@ void set_scalars(CopyArgs& a, Scalar alpha, Scalar beta, bool conj) {
     a.use_beta = !beta.is_zero();
 }
 
-template <class V, class Op>
-int32_t run_copy(const TilePlan& tp, Op op, bool read_old, hipStream_t st) {
-    size_t lds = (size_t)(tp.args.tile_elems + tp.args.tile_elems / 32 + 1) * sizeof(V);
-    const int ept = tp.ept;
+template <class V, class Op, int EPT, int VR, int VW>
+void launch_copy_variant(const TilePlan& tp, Op op, bool read_old, size_t lds, hipStream_t st) {
+    const dim3 grid(tp.persistent), block(THREADS);
+    if (read_old) hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, true>), grid, block, lds, st, tp.args, op);
+    else hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, false>), grid, block, lds, st, tp.args, op);
+}
+
+// ALLVEC: also instantiate the mixed (vector on one side only) variants.
+template <class V, class Op, bool ALLVEC>
+int32_t run_copy(const TilePlan& tp, Op op, bool read_old, bool vin, bool vout, hipStream_t st) {
+    constexpr int VEC = 16 / sizeof(V);
+    constexpr int BIG = sizeof(V) >= 16 ? 8 : 16;
+    const size_t lds = (size_t)(tp.args.tile_elems + tp.args.tile_elems / 32 + 4) * sizeof(V);
     const int prof = prof_begin(PROF_COPY, st);
-#define TFH_LAUNCH(E)                                                                                     \
-    do {                                                                                                  \
-        if (read_old) hipLaunchKernelGGL((copy_kernel<V, Op, E, true>), tp.grid, dim3(THREADS), lds, st, tp.args, op);   \
-        else hipLaunchKernelGGL((copy_kernel<V, Op, E, false>), tp.grid, dim3(THREADS), lds, st, tp.args, op);           \
-    } while (0)
-    if (ept <= 1) TFH_LAUNCH(1);
-    else if (ept <= 4) TFH_LAUNCH(4);
-    else if (ept <= 8) TFH_LAUNCH(8);
-    else TFH_LAUNCH(16);
-#undef TFH_LAUNCH
+    const bool big = tp.ept > 4;
+    if constexpr (VEC == 1) {
+        if (big) launch_copy_variant<V, Op, BIG, 1, 1>(tp, op, read_old, lds, st);
+        else launch_copy_variant<V, Op, 4, 1, 1>(tp, op, read_old, lds, st);
+    } else {
+        if (!ALLVEC && !(vin && vout)) vin = vout = false;
+        if (big) {
+            if (vin && vout) launch_copy_variant<V, Op, BIG, VEC, VEC>(tp, op, read_old, lds, st);
+            else if constexpr (ALLVEC) {
+                if (vin) launch_copy_variant<V, Op, BIG, VEC, 1>(tp, op, read_old, lds, st);
+                else if (vout) launch_copy_variant<V, Op, BIG, 1, VEC>(tp, op, read_old, lds, st);
+                else launch_copy_variant<V, Op, BIG, 1, 1>(tp, op, read_old, lds, st);
+            } else launch_copy_variant<V, Op, BIG, 1, 1>(tp, op, read_old, lds, st);
+        } else {
+            if (vin && vout && tp.args.tile_elems >= THREADS * VEC) launch_copy_variant<V, Op, 4, VEC, VEC>(tp, op, read_old, lds, st);
+            else launch_copy_variant<V, Op, 4, 1, 1>(tp, op, read_old, lds, st);
+        }
+    }
     prof_end(prof, st);
     return hip_check(hipGetLastError(), "copy kernel launch");
 }
@@ -410,25 +484,26 @@ int32_t launch_copy(int dtype, const void* in, void* out, std::vector<Axis> axes
     tp.args.out = out;
     set_scalars(tp.args, alpha, beta, conj);
     hipStream_t st = (hipStream_t)stream;
+    const bool vin = tp.vec_in && aligned(in, 16), vout = tp.vec_out && aligned(out, 16);
     const bool cx = is_complex(dtype);
     const bool raw = alpha.is_one() && beta.is_zero() && !(conj && cx);
     if (raw) {
         switch (eb) {
-            case 4: return run_copy<uint32_t>(tp, RawOp<uint32_t>(), false, st);
-            case 8: return run_copy<uint64_t>(tp, RawOp<uint64_t>(), false, st);
-            default: return run_copy<double2>(tp, RawOp<double2>(), false, st);
+            case 4: return run_copy<uint32_t, RawOp<uint32_t>, true>(tp, RawOp<uint32_t>(), false, vin, vout, st);
+            case 8: return run_copy<uint64_t, RawOp<uint64_t>, true>(tp, RawOp<uint64_t>(), false, vin, vout, st);
+            default: return run_copy<double2, RawOp<double2>, false>(tp, RawOp<double2>(), false, vin, vout, st);
         }
     }
     const bool rb = !beta.is_zero();
     if (alpha.is_one() && beta.is_zero() && conj) {
-        if (dtype == TFH_C64) return run_copy<float2>(tp, ConjOp<float2>(), false, st);
-        return run_copy<double2>(tp, ConjOp<double2>(), false, st);
+        if (dtype == TFH_C64) return run_copy<float2, ConjOp<float2>, false>(tp, ConjOp<float2>(), false, vin, vout, st);
+        return run_copy<double2, ConjOp<double2>, false>(tp, ConjOp<double2>(), false, vin, vout, st);
     }
     switch (dtype) {
-        case TFH_F32: return run_copy<float>(tp, RealOp<float>(), rb, st);
-        case TFH_F64: return run_copy<double>(tp, RealOp<double>(), rb, st);
-        case TFH_C64: return run_copy<float2>(tp, CplxOp<float2, float>(), rb, st);
-        default: return run_copy<double2>(tp, CplxOp<double2, double>(), rb, st);
+        case TFH_F32: return run_copy<float, RealOp<float>, false>(tp, RealOp<float>(), rb, vin, vout, st);
+        case TFH_F64: return run_copy<double, RealOp<double>, false>(tp, RealOp<double>(), rb, vin, vout, st);
+        case TFH_C64: return run_copy<float2, CplxOp<float2, float>, false>(tp, CplxOp<float2, float>(), rb, vin, vout, st);
+        default: return run_copy<double2, CplxOp<double2, double>, false>(tp, CplxOp<double2, double>(), rb, vin, vout, st);
     }
 }
 
