@@ -30,6 +30,10 @@ struct CopyArgs {
     int32_t tile_elems;    // product of tile extents (power of two)
     int32_t pad_;
     int64_t ntiles;        // tiles in the whole tensor (the copy kernel's blocks loop over them)
+    // fast path: every in-tile offset, taken relative to the lowest address of the tile, fits 32-bit bytes
+    int32_t fast32, pad2_;
+    int64_t in_rebase, out_rebase;   // lowest in-tile element offset on each side (<= 0)
+    int32_t t_text[MAXT];            // tile extent per tile-axis id
     // tile axes in read order (ascending input stride) and in write order (ascending output stride)
     int32_t r_shift[MAXT], r_mask[MAXT], r_id[MAXT];
     int64_t r_si[MAXT];
@@ -51,6 +55,11 @@ struct BlockOrigin {
     int64_t lim[MAXT];  // remaining extent of each tile axis at this block
 };
 
+__device__ __forceinline__ int64_t uniform64(int64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 __device__ __forceinline__ BlockOrigin block_origin(const CopyArgs& a, uint64_t bid) {
     BlockOrigin o;
     o.in = o.in2 = o.out = 0;
@@ -70,6 +79,13 @@ __device__ __forceinline__ BlockOrigin block_origin(const CopyArgs& a, uint64_t 
                 if (k == t) o.lim[k] -= c * a.g_text[g];
         }
     }
+    // the tile index is uniform, but the division sequences above run on the vector unit: move the results to
+    // scalar registers so a tile origin costs no vector registers
+    o.in = uniform64(o.in);
+    o.in2 = uniform64(o.in2);
+    o.out = uniform64(o.out);
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) o.lim[t] = uniform64(o.lim[t]);
     return o;
 }
 
@@ -120,22 +136,84 @@ __device__ __forceinline__ int64_t pick_lim(const BlockOrigin& o, int id) {
     return id == 0 ? o.lim[0] : id == 1 ? o.lim[1] : id == 2 ? o.lim[2] : o.lim[3];
 }
 
+typedef const __attribute__((address_space(1))) char* gcptr;
+typedef __attribute__((address_space(1))) char* gmptr;
+template <int BYTES> struct RawBits;
+template <> struct RawBits<4> { typedef uint32_t type; };
+template <> struct RawBits<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <> struct RawBits<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+// Global load/store of a Pack through a uniform base and a 32-bit byte offset (scalar-base addressing).
+template <class P>
+__device__ __forceinline__ P gload_pack(gcptr base, uint32_t off) {
+    typedef typename RawBits<sizeof(P)>::type Raw;
+    const Raw r = *reinterpret_cast<const __attribute__((address_space(1))) Raw*>(base + off);
+    return __builtin_bit_cast(P, r);
+}
+template <class P>
+__device__ __forceinline__ void gstore_pack(gmptr base, uint32_t off, const P& p) {
+    typedef typename RawBits<sizeof(P)>::type Raw;
+    *reinterpret_cast<__attribute__((address_space(1))) Raw*>(base + off) = __builtin_bit_cast(Raw, p);
+}
+
 // Persistent blocks: block b moves tiles b, b + gridDim.x, ...  The next tile's global loads are issued
 // (into registers) before the current tile is written out, so loads stay in flight during the store phase.
 // VR / VW: elements per global access on the read / write side (16-byte accesses when the layout allows).
-template <class V, class Op, int EPT, int VR, int VW, bool READ_OLD>
+// Interior tiles take a fast path: the in-tile byte offsets and LDS positions of each thread's accesses are
+// computed once (32-bit) and reused for every tile against a uniform per-tile base; edge tiles and tensors
+// whose tiles span 4 GiB recompute coordinates with bounds checks.
+template <class V, class Op, int EPT, int VR, int VW, bool READ_OLD, bool FAST>
 __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     V* lds = reinterpret_cast<V*>(smem_raw);
+    constexpr int NR = EPT / VR, NW = EPT / VW;
     int tid = threadIdx.x;
     V regs[EPT];
+    uint32_t roff[FAST ? NR : 1], woff[FAST ? NW : 1];
+    int wl[FAST ? NW : 1];
+    uint32_t rmask = 0, wmask = 0;
+#pragma clang loop unroll(full)
+    for (int u = 0; u < (FAST ? NR : 0); ++u) {
+        const int r = (u * THREADS + tid) * VR;
+        int64_t off = 0;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t) off += (int64_t)((r >> a.r_shift[t]) & a.r_mask[t]) * a.r_si[t];
+        roff[u] = (uint32_t)((off - a.in_rebase) * (int64_t)sizeof(V));
+        rmask |= (r < a.tile_elems ? 1u : 0u) << u;
+    }
+#pragma clang loop unroll(full)
+    for (int u = 0; u < (FAST ? NW : 0); ++u) {
+        const int w = (u * THREADS + tid) * VW;
+        int64_t off = 0;
+        int r = 0;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t) {
+            const int c = (w >> a.w_shift[t]) & a.w_mask[t];
+            off += (int64_t)c * a.w_so[t];
+            r += c * a.w_rpos[t];
+        }
+        woff[u] = (uint32_t)((off - a.out_rebase) * (int64_t)sizeof(V));
+        wl[u] = r;
+        wmask |= (w < a.tile_elems ? 1u : 0u) << u;
+    }
+
     auto load = [&](const BlockOrigin& o) {
-        // the index arithmetic below is invariant over the tile loop; recomputing it per tile is far cheaper
-        // than the ~100 registers it would occupy if hoisted, so hide the invariance from the optimiser
+        if constexpr (FAST) {
+            const gcptr base = (gcptr)(uintptr_t)(reinterpret_cast<const V*>(a.in) + o.in + a.in_rebase);
+#pragma clang loop unroll(full)
+            for (int u = 0; u < NR; ++u) {
+                if ((rmask >> u) & 1u) {
+                    const Pack<V, VR> p = gload_pack<Pack<V, VR>>(base, roff[u]);
+#pragma unroll
+                    for (int j = 0; j < VR; ++j) regs[u * VR + j] = p.v[j];
+                }
+            }
+            return;
+        } else {
+        // hide the tile-invariance of this index arithmetic so that it is not hoisted into ~100 registers
         asm volatile("" : "+v"(tid));
         const V* in = reinterpret_cast<const V*>(a.in) + o.in;
 #pragma clang loop unroll(full)
-        for (int u = 0; u < EPT / VR; ++u) {
+        for (int u = 0; u < NR; ++u) {
             const int r = (u * THREADS + tid) * VR;
             bool ok = r < a.tile_elems;
             int64_t off = 0;
@@ -151,6 +229,7 @@ __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
                 for (int j = 0; j < VR; ++j) regs[u * VR + j] = p.v[j];
             }
         }
+        }
     };
     uint64_t tile = blockIdx.x;
     if (tile >= (uint64_t)a.ntiles) return;
@@ -158,9 +237,9 @@ __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
     load(o);
     for (;;) {
 #pragma clang loop unroll(full)
-        for (int u = 0; u < EPT / VR; ++u) {
+        for (int u = 0; u < NR; ++u) {
             const int r = (u * THREADS + tid) * VR;
-            if (r < a.tile_elems) {
+            if (FAST ? (bool)((rmask >> u) & 1u) : r < a.tile_elems) {
 #pragma unroll
                 for (int j = 0; j < VR; ++j) lds[swz(r) + j] = regs[u * VR + j];
             }
@@ -173,30 +252,47 @@ __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
             o2 = block_origin(a, next);
             load(o2);
         }
-        V* out = reinterpret_cast<V*>(a.out) + o.out;
-        asm volatile("" : "+v"(tid));
+        if constexpr (FAST) {
+            const gmptr base = (gmptr)(uintptr_t)(reinterpret_cast<V*>(a.out) + o.out + a.out_rebase);
 #pragma clang loop unroll(full)
-        for (int u = 0; u < EPT / VW; ++u) {
-            const int w = (u * THREADS + tid) * VW;
-            bool ok = w < a.tile_elems;
-            int64_t off = 0;
-            int r = 0;
+            for (int u = 0; u < NW; ++u) {
+                if ((wmask >> u) & 1u) {
+                    Pack<V, VW> x, old;
 #pragma unroll
-            for (int t = 0; t < MAXT; ++t) {
-                const int c = (w >> a.w_shift[t]) & a.w_mask[t];
-                off += (int64_t)c * a.w_so[t];
-                r += c * a.w_rpos[t];
-                ok &= c < pick_lim(o, a.w_id[t]);
+                    for (int j = 0; j < VW; ++j) x.v[j] = lds[swz(wl[u] + j * a.w_rpos[0])];
+                    old = x;
+                    if (READ_OLD) old = gload_pack<Pack<V, VW>>((gcptr)base, woff[u]);
+#pragma unroll
+                    for (int j = 0; j < VW; ++j) x.v[j] = op(x.v[j], old.v[j], a);
+                    gstore_pack<Pack<V, VW>>(base, woff[u], x);
+                }
             }
-            if (ok) {
-                Pack<V, VW> x, old;
+        } else {
+            V* out = reinterpret_cast<V*>(a.out) + o.out;
+            asm volatile("" : "+v"(tid));
+#pragma clang loop unroll(full)
+            for (int u = 0; u < NW; ++u) {
+                const int w = (u * THREADS + tid) * VW;
+                bool ok = w < a.tile_elems;
+                int64_t off = 0;
+                int r = 0;
 #pragma unroll
-                for (int j = 0; j < VW; ++j) x.v[j] = lds[swz(r + j * a.w_rpos[0])];
-                old = x;
-                if (READ_OLD) old = *reinterpret_cast<const Pack<V, VW>*>(out + off);
+                for (int t = 0; t < MAXT; ++t) {
+                    const int c = (w >> a.w_shift[t]) & a.w_mask[t];
+                    off += (int64_t)c * a.w_so[t];
+                    r += c * a.w_rpos[t];
+                    ok &= c < pick_lim(o, a.w_id[t]);
+                }
+                if (ok) {
+                    Pack<V, VW> x, old;
 #pragma unroll
-                for (int j = 0; j < VW; ++j) x.v[j] = op(x.v[j], old.v[j], a);
-                *reinterpret_cast<Pack<V, VW>*>(out + off) = x;
+                    for (int j = 0; j < VW; ++j) x.v[j] = lds[swz(r + j * a.w_rpos[0])];
+                    old = x;
+                    if (READ_OLD) old = *reinterpret_cast<const Pack<V, VW>*>(out + off);
+#pragma unroll
+                    for (int j = 0; j < VW; ++j) x.v[j] = op(x.v[j], old.v[j], a);
+                    *reinterpret_cast<Pack<V, VW>*>(out + off) = x;
+                }
             }
         }
         if (!more) break;
@@ -275,6 +371,7 @@ struct TilePlan {
     dim3 grid;
     int ept;
     bool vec_in, vec_out;   // strides allow 16-byte accesses on the input / output side
+    bool all_full;          // no partial tiles and 32-bit in-tile offsets: the kernel's fast path applies
     uint32_t persistent;    // block count for the looping copy kernel
 };
 
@@ -374,6 +471,24 @@ int32_t plan_tiles(std::vector<Axis> axes, int elem_bytes, int max_tile_elems, b
         a.w_si2[t] = axes[i].s[2];
         sh += tl[i];
     }
+    // fast path data: tile extents and the lowest in-tile offset per side; usable when the tile spans < 4 GiB
+    {
+        int64_t lo_in = 0, hi_in = 0, lo_out = 0, hi_out = 0;
+        for (int t = 0; t < MAXT; ++t) a.t_text[t] = 1;
+        for (int t = 0; t < a.nt; ++t) {
+            const int i = ids[t];
+            const int64_t ext = ((int64_t)1 << tl[i]) - 1;
+            a.t_text[t] = 1 << tl[i];
+            (axes[i].s[0] < 0 ? lo_in : hi_in) += ext * axes[i].s[0];
+            (axes[i].s[1] < 0 ? lo_out : hi_out) += ext * axes[i].s[1];
+        }
+        a.in_rebase = lo_in;
+        a.out_rebase = lo_out;
+        a.fast32 = (hi_in - lo_in + 1) * (int64_t)elem_bytes < ((int64_t)1 << 32) &&
+                   (hi_out - lo_out + 1) * (int64_t)elem_bytes < ((int64_t)1 << 32);
+        tp.all_full = a.fast32 != 0;
+        for (int t = 0; t < a.nt; ++t) tp.all_full &= axes[ids[t]].n % ((int64_t)1 << tl[ids[t]]) == 0;
+    }
     // grid axes; the axes a tile covers only partly come first (fastest block index), so blocks that run at
     // the same time complete each other's contiguous runs in DRAM
     a.ng = 0;
@@ -434,8 +549,14 @@ void set_scalars(CopyArgs& a, Scalar alpha, Scalar beta, bool conj) {
 template <class V, class Op, int EPT, int VR, int VW>
 void launch_copy_variant(const TilePlan& tp, Op op, bool read_old, size_t lds, hipStream_t st) {
     const dim3 grid(tp.persistent), block(THREADS);
-    if (read_old) hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, true>), grid, block, lds, st, tp.args, op);
-    else hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, false>), grid, block, lds, st, tp.args, op);
+    // FAST: every tile is full (each tiled extent is a multiple of its tile extent) and spans < 4 GiB
+    if (tp.all_full) {
+        if (read_old) hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, true, true>), grid, block, lds, st, tp.args, op);
+        else hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, false, true>), grid, block, lds, st, tp.args, op);
+    } else {
+        if (read_old) hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, true, false>), grid, block, lds, st, tp.args, op);
+        else hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, false, false>), grid, block, lds, st, tp.args, op);
+    }
 }
 
 // ALLVEC: also instantiate the mixed (vector on one side only) variants.
