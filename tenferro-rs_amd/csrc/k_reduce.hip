@@ -272,12 +272,287 @@ __global__ void __launch_bounds__(THREADS) reduce_finalize_kernel(ReduceArgs a) 
     }
 }
 
+// ---- fast path ------------------------------------------------------------------------------------------------
+// Used when no tile is partial (every tiled extent is a multiple of its tile extent), the thread tile is exactly
+// 256 lanes and there are enough outputs to fill the chip.  Per load the vector unit does one 64-bit add: the
+// thread's in-tile offset is computed once, the block origin is scalar, and the offsets of the serial reduced
+// indices come from a small LDS table built at block start.  VEC elements per load along A's contiguous axis
+// (16 bytes); KV: that axis is kept (VEC outputs per lane) rather than reduced (summed in registers).
+// KS: consecutive outer kept indices handled by one block, each with its own accumulators, so that short
+// reductions still give every thread >= 8 independent loads and one LDS tree serves them all.
+constexpr int FAST_MAX_RTAB = 1024;
+struct FastReduceArgs {
+    const void* in;
+    void* out;
+    int32_t nt, ng, nr, op;
+    int32_t red_bits, use_beta;
+    int32_t t_shift[MAXT], t_mask[MAXT], t_red[MAXT];
+    int64_t t_sa[MAXT], t_sc[MAXT];
+    int64_t g_count[MAXG], g_sa[MAXG], g_sc[MAXG];
+    int64_t r_count[MAXR], r_sa[MAXR];
+    int32_t r_total, pad_;
+    int64_t ks_sa, ks_sc;     // strides of the block-serial kept axis
+    int64_t vc_stride;        // C stride between the VEC outputs of one lane (KV)
+    double alpha, beta;
+};
+
+template <class R, int N>
+struct alignas(sizeof(R) * N) RVec {
+    R v[N];
+};
+
+template <class R, int VEC, bool KV, int KS>
+__global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) {
+    constexpr int NV = KV ? VEC : 1;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    int64_t* rtab = reinterpret_cast<int64_t*>(smem_raw);                               // [r_total]
+    double* lds = reinterpret_cast<double*>(smem_raw + FAST_MAX_RTAB * sizeof(int64_t)); // [KS*NV][THREADS]
+    const int tid = threadIdx.x;
+    for (int i = tid; i < a.r_total; i += THREADS) {
+        int64_t lin = i, off = 0;
+#pragma unroll
+        for (int r = 0; r < MAXR; ++r)
+            if (r < a.nr) {
+                int64_t q = lin / a.r_count[r];
+                off += (lin - q * a.r_count[r]) * a.r_sa[r];
+                lin = q;
+            }
+        rtab[i] = off;
+    }
+    // block origin (uniform) and this thread's offsets inside the tile
+    int64_t org_in = 0, org_out = 0;
+    {
+        uint64_t bid = blockIdx.x;
+        for (int g = 0; g < a.ng; ++g) {
+            uint64_t q = bid / (uint64_t)a.g_count[g];
+            int64_t c = (int64_t)(bid - q * (uint64_t)a.g_count[g]);
+            bid = q;
+            org_in += c * a.g_sa[g];
+            org_out += c * a.g_sc[g];
+        }
+    }
+    int64_t toff_in = 0, toff_out = 0;
+    bool writer = true;
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) {   // unused slots are neutral (mask 0)
+        const int c = (tid >> a.t_shift[t]) & a.t_mask[t];
+        toff_in += (int64_t)c * a.t_sa[t];
+        if (a.t_red[t]) writer &= c == 0;
+        else toff_out += (int64_t)c * a.t_sc[t];
+    }
+    const R* A = reinterpret_cast<const R*>(a.in) + org_in + toff_in;
+    const int op = a.op;
+    double acc[KS][NV];
+#pragma unroll
+    for (int k = 0; k < KS; ++k)
+#pragma unroll
+        for (int j = 0; j < NV; ++j) acc[k][j] = identity(op);
+    __syncthreads();
+    constexpr int U = KS >= 8 ? 2 : 8;
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+        const R* Ak = A + k * a.ks_sa;
+        for (int it = 0; it < a.r_total; it += U) {
+            RVec<R, VEC> v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (it + u < a.r_total) v[u] = *reinterpret_cast<const RVec<R, VEC>*>(Ak + rtab[it + u]);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (it + u < a.r_total) {
+                    if (KV) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) acc[k][j] = combine(acc[k][j], (double)v[u].v[j], op);
+                    } else {
+                        double s = (double)v[u].v[0];
+#pragma unroll
+                        for (int j = 1; j < VEC; ++j) s = combine(s, (double)v[u].v[j], op);
+                        acc[k][0] = combine(acc[k][0], s, op);
+                    }
+                }
+        }
+    }
+    // lanes that share outputs fold through LDS over the reduced thread-id bits
+    if (a.red_bits) {
+#pragma unroll
+        for (int k = 0; k < KS; ++k)
+#pragma unroll
+            for (int j = 0; j < NV; ++j) lds[(k * NV + j) * THREADS + tid] = acc[k][j];
+        __syncthreads();
+        for (int b = 7; b >= 0; --b) {
+            const int bit = 1 << b;
+            if (a.red_bits & bit) {
+                if (!(tid & bit)) {
+#pragma unroll
+                    for (int q = 0; q < KS * NV; ++q) lds[q * THREADS + tid] = combine(lds[q * THREADS + tid], lds[q * THREADS + (tid | bit)], op);
+                }
+                __syncthreads();
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < KS; ++k)
+#pragma unroll
+            for (int j = 0; j < NV; ++j) acc[k][j] = lds[(k * NV + j) * THREADS + tid];
+    }
+    if (!writer) return;
+    R* C = reinterpret_cast<R*>(a.out) + org_out + toff_out;
+#pragma unroll
+    for (int k = 0; k < KS; ++k)
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            R* dst = C + k * a.ks_sc + j * a.vc_stride;
+            double r = a.alpha * acc[k][j];
+            if (a.use_beta) r += a.beta * (double)*dst;
+            *dst = (R)r;
+        }
+}
+
+template <class R, int VEC, bool KV>
+void launch_fast_ks(const FastReduceArgs& fa, dim3 grid, int ks, hipStream_t st) {
+    const int nv = KV ? VEC : 1;
+    if (ks == 8) {
+        size_t lds = FAST_MAX_RTAB * sizeof(int64_t) + (size_t)8 * nv * THREADS * sizeof(double);
+        hipLaunchKernelGGL((reduce_fast_kernel<R, VEC, KV, 8>), grid, dim3(THREADS), lds, st, fa);
+    } else {
+        size_t lds = FAST_MAX_RTAB * sizeof(int64_t) + (size_t)nv * THREADS * sizeof(double);
+        hipLaunchKernelGGL((reduce_fast_kernel<R, VEC, KV, 1>), grid, dim3(THREADS), lds, st, fa);
+    }
+}
+template <class R>
+void launch_fast(const FastReduceArgs& fa, dim3 grid, int vec, bool kv, int ks, hipStream_t st) {
+    constexpr int V = 16 / sizeof(R);
+    if (vec > 1) {
+        if (kv) launch_fast_ks<R, V, true>(fa, grid, ks, st);
+        else launch_fast_ks<R, V, false>(fa, grid, ks, st);
+    } else
+        launch_fast_ks<R, 1, true>(fa, grid, ks, st);
+}
+
 int ceil_log2(int64_t n) {
     int l = 0;
     while (((int64_t)1 << l) < n) ++l;
     return l;
 }
 
+}  // namespace
+
+namespace {
+// Returns true when the fast kernel was launched.
+bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, std::vector<Axis> red, int reduce_op,
+                     Scalar alpha, Scalar beta, void* stream, int32_t& status) {
+    status = TFH_OK;
+    const bool cx = is_complex(dtype);
+    if (cx && (reduce_op != TFH_REDUCE_SUM || alpha.im != 0 || beta.im != 0)) return false;
+    const int rbytes = is_double(dtype) ? 8 : 4;
+    if (cx) {   // complex sum = real sum over the interleaved layout with an extra kept axis (re, im)
+        for (auto& x : kept) { x.s[0] *= 2; x.s[1] *= 2; }
+        for (auto& x : red) x.s[0] *= 2;
+        kept.push_back(Axis{2, {1, 1, 0}, 0xffffffffu});
+    }
+    std::stable_sort(kept.begin(), kept.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[1]) > std::llabs(y.s[1]); });
+    for (auto& x : kept) x.s[2] = 0;
+    fuse_axes(kept, 2);
+    for (auto& x : red) x.s[1] = x.s[2] = 0;
+    std::stable_sort(red.begin(), red.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[0]) > std::llabs(y.s[0]); });
+    fuse_axes(red, 1);
+    for (auto& x : kept)
+        if (x.s[1] == 0 || x.s[0] == 0) return false;
+    for (auto& x : red)
+        if (x.s[0] == 0) return false;
+    struct Ax { Axis a; bool red; int tl; int64_t neff; };
+    std::vector<Ax> all;
+    for (auto& x : kept) all.push_back({x, false, 0, x.n});
+    for (auto& x : red) all.push_back({x, true, 0, x.n});
+    if (all.empty() || (int)all.size() > MAXG) return false;
+    std::stable_sort(all.begin(), all.end(), [](const Ax& x, const Ax& y) { return std::llabs(x.a.s[0]) < std::llabs(y.a.s[0]); });
+    // vector loads along A's contiguous axis
+    int vec = 16 / rbytes;
+    {
+        Ax& f = all[0];
+        bool ok = f.a.s[0] == 1 && f.a.n % vec == 0 && ((uintptr_t)a % 16) == 0;
+        for (size_t i = 1; i < all.size(); ++i) ok &= all[i].a.s[0] % vec == 0;
+        if (!ok) vec = 1;
+    }
+    const bool kv = !all[0].red;
+    all[0].neff = all[0].a.n / vec;
+    FastReduceArgs fa;
+    std::memset(&fa, 0, sizeof fa);
+    int bits = 8, shift = 0;
+    for (size_t i = 0; i < all.size(); ++i) {
+        Ax& x = all[i];
+        if (bits == 0) break;
+        int t = std::min(ceil_log2(x.neff), bits);
+        while (t > 0 && x.neff % ((int64_t)1 << t) != 0) --t;   // no partial tiles
+        if (t == 0) {
+            if (x.neff == 1) continue;
+            break;   // an odd extent blocks the tile: not a fast-path shape
+        }
+        if (fa.nt == MAXT) break;
+        x.tl = t;
+        const int id = fa.nt++;
+        const int64_t mul = i == 0 ? vec : 1;
+        fa.t_shift[id] = shift;
+        fa.t_mask[id] = (1 << t) - 1;
+        fa.t_red[id] = x.red;
+        fa.t_sa[id] = x.a.s[0] * mul;
+        fa.t_sc[id] = x.a.s[1] * mul;
+        if (x.red) fa.red_bits |= fa.t_mask[id] << shift;
+        shift += t;
+        bits -= t;
+    }
+    if (bits != 0) return false;
+    int64_t blocks = 1, r_total = 1;
+    for (size_t i = 0; i < all.size(); ++i) {
+        const Ax& x = all[i];
+        const int64_t text = (int64_t)1 << x.tl;
+        const int64_t cnt = x.neff / text;
+        if (cnt <= 1) continue;
+        const int64_t mul = (i == 0 ? vec : 1) * text;
+        if (x.red) {
+            if (fa.nr == MAXR) return false;
+            fa.r_count[fa.nr] = cnt;
+            fa.r_sa[fa.nr] = x.a.s[0] * mul;
+            ++fa.nr;
+            r_total *= cnt;
+        } else {
+            fa.g_count[fa.ng] = cnt;
+            fa.g_sa[fa.ng] = x.a.s[0] * mul;
+            fa.g_sc[fa.ng] = x.a.s[1] * mul;
+            ++fa.ng;
+            blocks *= cnt;
+        }
+    }
+    if (r_total > FAST_MAX_RTAB || blocks > 0x7fffffffll) return false;
+    // block-serial kept indices when the serial reduction alone gives a thread too few loads
+    int ks = 1;
+    const int nv = kv ? vec : 1;
+    if (r_total < 8 && fa.ng > 0 && fa.g_count[0] % 8 == 0 && blocks / 8 >= 512 && nv <= 2) {   // nv <= 2: LDS stays under 48 KB
+        ks = 8;
+        fa.ks_sa = fa.g_sa[0];
+        fa.ks_sc = fa.g_sc[0];
+        fa.g_count[0] /= 8;
+        fa.g_sa[0] *= 8;
+        fa.g_sc[0] *= 8;
+        blocks /= 8;
+    }
+    if (blocks < 256 && r_total >= 64) return false;   // few outputs, long reduction: the split kernel handles it
+    fa.r_total = (int32_t)r_total;
+    fa.in = a;
+    fa.out = c;
+    fa.op = reduce_op;
+    fa.alpha = alpha.re;
+    fa.beta = beta.re;
+    fa.use_beta = !beta.is_zero();
+    fa.vc_stride = all[0].a.s[1];
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid((uint32_t)blocks);
+    const int prof = prof_begin(PROF_REDUCE, stream);
+    if (rbytes == 8) launch_fast<double>(fa, grid, vec, kv, ks, st);
+    else launch_fast<float>(fa, grid, vec, kv, ks, st);
+    prof_end(prof, stream);
+    status = hip_check(hipGetLastError(), "reduce kernel launch");
+    return true;
+}
 }  // namespace
 
 int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, std::vector<Axis> red, int reduce_op,
@@ -297,6 +572,10 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
         for (auto& x : kept) ax.push_back(Axis{x.n, {x.s[1], x.s[1], 0}, x.label});
         if (beta.is_zero()) return launch_fill(dtype, c, ax, Scalar{0, 0}, stream);
         return launch_copy(dtype, c, c, ax, beta, Scalar{0, 0}, false, stream);
+    }
+    {
+        int32_t st_fast = TFH_OK;
+        if (try_fast_reduce(dtype, a, c, kept, red, reduce_op, alpha, beta, stream, st_fast)) return st_fast;
     }
     // merge axes (kept and reduced separately; slot 0 = A, slot 1 = C)
     std::stable_sort(kept.begin(), kept.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[1]) > std::llabs(y.s[1]); });
