@@ -65,7 +65,7 @@ struct ThreadPos {
     bool writer;          // reduced bits all zero
 };
 
-__device__ __forceinline__ ThreadPos thread_pos(const ReduceArgs& a) {
+__device__ __forceinline__ ThreadPos thread_pos(const ReduceArgs& a, int tid) {
     ThreadPos p;
     p.in = p.out = 0;
 #pragma unroll
@@ -82,7 +82,6 @@ __device__ __forceinline__ ThreadPos thread_pos(const ReduceArgs& a) {
         for (int k = 0; k < MAXT; ++k)
             if (k == t) p.lim[k] -= c * a.g_text[g];
     }
-    const int tid = threadIdx.x;
     p.ok = tid < a.tile_elems;
     p.writer = true;
     p.red_ok = true;
@@ -113,7 +112,7 @@ template <class R, bool CX>
 __global__ void __launch_bounds__(THREADS) reduce_kernel(ReduceArgs a) {
     constexpr int NC = CX ? 2 : 1;
     __shared__ double lds[THREADS * NC];
-    const ThreadPos p = thread_pos(a);
+    const ThreadPos p = thread_pos(a, threadIdx.x);
     const R* A = reinterpret_cast<const R*>(a.in) + p.in * NC;
     const int op = a.op;
     double acc_re = identity(op), acc_im = 0.0;
@@ -242,19 +241,47 @@ __global__ void __launch_bounds__(THREADS) reduce_kernel(ReduceArgs a) {
     }
 }
 
-// Second pass of a split reduction: fold the partials of every chunk, in chunk order.
+// Second pass of a split reduction: one block per block of the first pass.  The block's kept lanes (thread
+// ids whose reduced bits are zero) each own one output; the other threads help: thread (kept lane l, part p)
+// folds chunks p, p+P, ... and the parts meet in an LDS tree, so the order of the fold is fixed.
 template <class R, bool CX>
 __global__ void __launch_bounds__(THREADS) reduce_finalize_kernel(ReduceArgs a) {
     constexpr int NC = CX ? 2 : 1;
-    const ThreadPos p = thread_pos(a);
-    if (!(p.writer && p.ok)) return;
+    __shared__ double lds[THREADS * NC];
+    const int keep_mask = 255 & ~a.red_bits;
+    const int kl = 1 << __popc(keep_mask);   // kept lanes per block
+    const int P = THREADS / kl;              // helper parts per kept lane
+    const int lane = threadIdx.x % kl, part = threadIdx.x / kl;
+    // the thread id of kept lane `lane` in the first pass: deposit its bits into the kept bit positions
+    int tid0 = 0;
+    for (int b = 0, src = 0; b < 8; ++b)
+        if (keep_mask >> b & 1) {
+            tid0 |= ((lane >> src) & 1) << b;
+            ++src;
+        }
+    const ThreadPos p = thread_pos(a, tid0);
     const int op = a.op;
     double acc_re = identity(op), acc_im = 0.0;
-    for (int ch = 0; ch < a.nchunks; ++ch) {
-        int64_t slot = ((int64_t)ch * a.kept_slots + (int64_t)blockIdx.x * THREADS + p.kept_lane) * NC;
-        acc_re = combine(acc_re, a.partial[slot], op);
-        if (CX) acc_im += a.partial[slot + 1];
+    if (p.ok)
+        for (int ch = part; ch < a.nchunks; ch += P) {
+            int64_t slot = ((int64_t)ch * a.kept_slots + (int64_t)blockIdx.x * THREADS + p.kept_lane) * NC;
+            acc_re = combine(acc_re, a.partial[slot], op);
+            if (CX) acc_im += a.partial[slot + 1];
+        }
+    lds[threadIdx.x * NC] = acc_re;
+    if (CX) lds[threadIdx.x * NC + 1] = acc_im;
+    __syncthreads();
+    for (int step = P >> 1; step > 0; step >>= 1) {
+        if (part < step) {
+            const int other = (part + step) * kl + lane;
+            lds[threadIdx.x * NC] = combine(lds[threadIdx.x * NC], lds[other * NC], op);
+            if (CX) lds[threadIdx.x * NC + 1] += lds[other * NC + 1];
+        }
+        __syncthreads();
     }
+    if (part != 0 || !p.ok) return;
+    acc_re = lds[threadIdx.x * NC];
+    if (CX) acc_im = lds[threadIdx.x * NC + 1];
     R* C = reinterpret_cast<R*>(a.out) + p.out * NC;
     if (CX) {
         double rr = a.alpha_re * acc_re - a.alpha_im * acc_im, ri = a.alpha_re * acc_im + a.alpha_im * acc_re;
@@ -348,7 +375,7 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
 #pragma unroll
         for (int j = 0; j < NV; ++j) acc[k][j] = identity(op);
     __syncthreads();
-    constexpr int U = KS >= 8 ? 2 : 8;
+    constexpr int U = KS >= 8 ? 2 : 16;
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
         const R* Ak = A + k * a.ks_sa;

@@ -494,3 +494,159 @@ def test_execute_errors(tf):
     assert [str(d) for d in tf.preferred_compute_devices(tf.GpuMemory(0), tf.OpKind.Contract)] == ["hip:0"]
     with pytest.raises(tf.NoCompatibleComputeDevice):
         tf.preferred_compute_devices(tf.GpuMemory(99), tf.OpKind.Contract)
+
+
+# ------------------------------------------------------------------------------------------------ kernel-variant coverage
+def _permute_check(tf, oracle, a, perm, alpha=1.0, beta=0.0, b0=None):
+    shape = [a.shape[p] for p in perm]
+    modes = list(range(a.ndim))
+    ref = np.zeros(shape, a.dtype) if b0 is None else b0.copy()
+    oracle.permute(a, modes, ref, list(perm), alpha=alpha, beta=beta)
+    out = dev(tf, np.zeros(shape, a.dtype) if b0 is None else b0)
+    plan = tf.HipBackend.plan(a.dtype, tf.PrimDescriptor.Permute(modes, list(perm)), [a.shape, shape])
+    tf.HipBackend.execute(plan, alpha, [dev(tf, a)], beta, out)
+    return out.to_numpy(), ref
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_permute_power_of_two_shapes_take_the_vector_path(tf, oracle, dtype):
+    # every tile full, contiguous fastest axes on both sides: 16-byte accesses, no bounds checks
+    rng = np.random.default_rng(41)
+    a = rand(rng, (32, 8, 64, 16), dtype)
+    for perm in [(3, 1, 0, 2), (0, 1, 2, 3), (2, 3, 0, 1), (1, 0, 3, 2)]:
+        got, ref = _permute_check(tf, oracle, a, perm)
+        assert got.tobytes() == ref.tobytes(), perm
+    b0 = rand(rng, (16, 8, 32, 64), dtype)
+    alpha, beta = (0.5 - 2j, 1.5 + 1j) if np.issubdtype(dtype, np.complexfloating) else (0.5, -1.5)
+    got, ref = _permute_check(tf, oracle, a, (3, 1, 0, 2), alpha, beta, b0)
+    assert relerr(got, ref) < TOL[dtype]
+
+
+def test_permute_misaligned_base_and_odd_inner_extent(tf, oracle):
+    # a view that starts one element into its buffer is only 8-byte aligned: the scalar path must be used
+    rng = np.random.default_rng(42)
+    big = rng.standard_normal(64 * 64 * 16 + 1)
+    a = big[1:].reshape(64, 64, 16)
+    got, ref = _permute_check(tf, oracle, a, (2, 0, 1))
+    assert got.tobytes() == ref.tobytes()
+    b = rng.standard_normal((64, 30, 17))            # partial tiles on every axis
+    got, ref = _permute_check(tf, oracle, b, (2, 1, 0))
+    assert got.tobytes() == ref.tobytes()
+
+
+def _reduce_check(tf, oracle, a, modes_a, modes_c, op_tf, op_or, alpha=1.0, beta=0.0, c0=None):
+    ext = dict(zip(modes_a, a.shape))
+    shape = [ext[m] for m in modes_c]
+    ref = np.zeros(shape, a.dtype) if c0 is None else c0.copy()
+    oracle.reduce(a, modes_a, ref, modes_c, op=op_or, alpha=alpha, beta=beta)
+    out = dev(tf, np.full(shape, np.nan, a.dtype) if c0 is None else c0)
+    plan = tf.HipBackend.plan(a.dtype, tf.PrimDescriptor.Reduce(list(modes_a), list(modes_c), op_tf), [a.shape, shape])
+    tf.HipBackend.execute(plan, alpha, [dev(tf, a)], beta, out)
+    return out.to_numpy(), ref
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_reduce_fast_path_variants(tf, oracle, dtype):
+    rng = np.random.default_rng(43)
+    a = rand(rng, (8, 16, 4, 16, 32), dtype)
+    m = [0, 1, 2, 3, 4]
+    cases = [[0, 1, 2, 3],          # contiguous axis reduced, few addends: block-serial kept indices
+             [0, 2, 4],             # contiguous axis kept, two reduced axes
+             [4, 0],                # output order differs from input order
+             [1, 2, 3, 4],          # slowest axis reduced
+             [3]]
+    for mc in cases:
+        got, ref = _reduce_check(tf, oracle, a, m, mc, tf.ReduceOp.Sum, oracle.SUM)
+        assert relerr(got, ref) < TOL[dtype], mc
+    c0 = rand(rng, (8, 4, 32), dtype)
+    got, ref = _reduce_check(tf, oracle, a, m, [0, 2, 4], tf.ReduceOp.Sum, oracle.SUM, alpha=2.0, beta=-0.5, c0=c0)
+    assert relerr(got, ref) < TOL[dtype]
+    if np.issubdtype(dtype, np.complexfloating):
+        got, ref = _reduce_check(tf, oracle, a, m, [0, 2, 4], tf.ReduceOp.Sum, oracle.SUM, alpha=0.5 - 1j, beta=0.25j, c0=c0)
+        assert relerr(got, ref) < TOL[dtype]          # complex alpha/beta: general kernel
+    else:
+        for op_tf, op_or in [(tf.ReduceOp.Max, oracle.MAX), (tf.ReduceOp.Min, oracle.MIN)]:
+            got, ref = _reduce_check(tf, oracle, a, m, [0, 2, 4], op_tf, op_or)
+            assert np.array_equal(got, ref)
+
+
+def test_reduce_misaligned_base_and_split_reductions(tf, oracle):
+    rng = np.random.default_rng(44)
+    big = rng.standard_normal(16 * 16 * 64 + 1)
+    a = big[1:].reshape(16, 16, 64)                   # 8-byte aligned only
+    got, ref = _reduce_check(tf, oracle, a, [0, 1, 2], [0, 2], tf.ReduceOp.Sum, oracle.SUM)
+    assert relerr(got, ref) < 1e-12
+    # few outputs, long reductions: split over blocks + second pass, every dtype of accumulator layout
+    b = rng.standard_normal((5, 300000))
+    got, ref = _reduce_check(tf, oracle, b, [0, 1], [0], tf.ReduceOp.Sum, oracle.SUM)
+    assert relerr(got, ref) < 1e-12
+    got, ref = _reduce_check(tf, oracle, b, [0, 1], [0], tf.ReduceOp.Max, oracle.MAX)
+    assert np.array_equal(got, ref)
+    z = (rng.standard_normal(1 << 20) + 1j * rng.standard_normal(1 << 20))
+    got, ref = _reduce_check(tf, oracle, z, [0], [], tf.ReduceOp.Sum, oracle.SUM, alpha=1 - 2j)
+    assert relerr(got, ref) < 1e-12
+    c = rng.standard_normal((4096, 48))
+    got, ref = _reduce_check(tf, oracle, c, [0, 1], [1], tf.ReduceOp.Sum, oracle.SUM)
+    assert relerr(got, ref) < 1e-12
+
+
+BIG_CASES = [
+    ("ajbk,kcj->abc", dict(a=16, j=8, b=16, k=12, c=160)),      # 128x128 tiles, two-mode k through offset tables, packed B
+    ("mk,kn->mn", dict(m=300, k=203, n=260)),                    # ragged edges and a k tail in the 128x128 kernel
+    ("km,nk->mn", dict(m=256, k=100, n=384)),
+    ("mk,nk->nm", dict(m=200, k=64, n=130)),                     # operands swap
+    ("bmk,kbn->bmn", dict(b=3, m=130, k=40, n=140)),             # batch + 128 tiles
+]
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("case", BIG_CASES, ids=[c[0] for c in BIG_CASES])
+def test_contract_128_tile_kernel(tf, oracle, dtype, case):
+    pattern, ext = case
+    ins, mc = pattern.split("->")
+    ma, mb = ins.split(",")
+    rng = np.random.default_rng(45)
+    a = rand(rng, [ext[l] for l in ma], dtype)
+    b = rand(rng, [ext[l] for l in mb], dtype)
+    cshape = [ext[l] for l in mc]
+    alpha, beta = (0.7 - 1.1j, -0.3 + 0.2j) if np.issubdtype(dtype, np.complexfloating) else (0.7, -0.3)
+    c0 = rand(rng, cshape, dtype)
+    ref = c0.copy()
+    oracle.contract(a, lab(ma), b, lab(mb), ref, lab(mc), alpha=alpha, beta=beta)
+    out = dev(tf, c0)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [a.shape, b.shape, cshape])
+    tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, out)
+    assert relerr(out.to_numpy(), ref) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.complex128])
+def test_contract_128_tile_negative_strides_and_offsets(tf, oracle, dtype):
+    # reversed views: the kernel rebases each operand to its lowest address
+    rng = np.random.default_rng(46)
+    abig, bbig = rand(rng, (400, 310), dtype), rand(rng, (310, 280), dtype)
+    av, bv = abig[::-2, ::-1][:, 5:], bbig[::-1, ::-2][5:, :]      # 200 x 305, 305 x 140
+    ref = np.empty((200, 140), dtype)
+    oracle.contract(av, lab("mk"), bv, lab("kn"), ref, lab("mn"))
+    out = tf.Tensor.empty([200, 140], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("mk"), lab("kn"), lab("mn")), [av.shape, bv.shape, [200, 140]])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, av), dev(tf, bv)], 0.0, out)
+    assert relerr(out.to_numpy(), ref) < TOL[dtype]
+
+
+def test_config3_full_size_complex128(tf, oracle):
+    # "awc,asx,wstv,cty->xvy", chi=1024, D=16, d=2: the optimiser's tree on the GPU against the oracle along the same tree
+    from tenferro_rs_amd import inputs
+    chi, D, d = 1024, 16, 2
+    sig = 1.0 / np.sqrt(chi)
+    L = inputs.complex_normal(1003, 0, (chi, D, chi), sig)
+    A = inputs.complex_normal(1003, 1, (chi, d, chi), sig)
+    W = inputs.complex_normal(1003, 2, (D, d, d, D), sig)
+    host = [L, A, W, np.conj(A)]
+    terms, out = ["awc", "asx", "wstv", "cty"], "xvy"
+    subs = tf.Subscripts.parse(",".join(terms) + "->" + out)
+    tree = tf.ContractionTree.optimize(subs, [x.shape for x in host])
+    assert abs(8 * tree.mac_count - 558.3e9) < 0.1e9
+    res = tf.einsum_with_plan(tree, [dev(tf, x) for x in host])
+    ref = np.empty((chi, D, chi), np.complex128)
+    oracle.einsum_pairs(host, [lab(t) for t in terms], ref, lab(out), tree.steps)
+    assert relerr(res.to_numpy(), ref) < 1e-12
