@@ -130,7 +130,7 @@ def run_c1(h):
         "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
         "roofline": {"bound": "mfma", "achieved": flops / (kms * 1e-3) / 1e12, "peak": PEAK["f32"], "unit": "TFLOP/s",
                      "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f32"], "traffic": None,
-                     "kernel": "gemm_kernel<float,false,128,128>", "kernel_ms": kms, "launches_per_step": per_step},
+                     "kernel": "gemm128_kernel<float, false, true, true> (split-K)", "kernel_ms": kms, "launches_per_step": per_step},
     }
     if h.cpu:
         ref = np.empty((a, b, c), np.float32)
@@ -169,10 +169,10 @@ def run_c2(h):
         "dtype": "f64", "ms_per_step": ms, "value": (pbytes + rbytes) / (ms * 1e-3) / 1e9, "unit": "GB/s",
         "permute": {"roofline": {"bound": "hbm", "achieved": pbytes / (pms * 1e-3) / 1e9, "peak": PEAK["hbm"], "unit": "GB/s",
                                  "frac": pbytes / (pms * 1e-3) / 1e9 / PEAK["hbm"], "traffic": None,
-                                 "kernel": "copy_kernel<u64>", "kernel_ms": pms}, "algorithmic_bytes": pbytes},
+                                 "kernel": "copy_kernel<u64, OpCopy, 16, 2, 2, false, true>", "kernel_ms": pms}, "algorithmic_bytes": pbytes},
         "reduce": {"roofline": {"bound": "hbm", "achieved": rbytes / (rms * 1e-3) / 1e9, "peak": PEAK["hbm"], "unit": "GB/s",
                                 "frac": rbytes / (rms * 1e-3) / 1e9 / PEAK["hbm"], "traffic": None,
-                                "kernel": "reduce_kernel<double>", "kernel_ms": rms}, "algorithmic_bytes": rbytes},
+                                "kernel": "reduce_fast_kernel<double, 2, true, 1>", "kernel_ms": rms}, "algorithmic_bytes": rbytes},
     }
     if h.cpu:
         P = np.empty(shape)
@@ -213,7 +213,7 @@ def run_c3(h):
         "peak_intermediate_bytes": tree.peak_intermediate * 16,
         "roofline": {"bound": "mfma", "achieved": flops / (total_kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
                      "frac": flops / (total_kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": None,
-                     "kernel": "gemm_kernel<double,true,...> x3 (the three pairwise contractions of the tree)",
+                     "kernel": "gemm128_kernel<double, true, ...> x2 + gemm_kernel<double, true, 64, 64> x1 (the three pairwise contractions of the tree)",
                      "kernel_ms": total_kms, "launches_per_step": per_step},
     }
     if h.cpu:
@@ -246,7 +246,7 @@ def run_c4(h):
         "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
         "roofline": {"bound": "mfma", "achieved": flops / (kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
                      "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": None,
-                     "kernel": "gemm_kernel<double,false,128,128> (grouped)", "kernel_ms": kms, "launches_per_step": per_step},
+                     "kernel": "gemm128_kernel<double, false, true, true> (grouped)", "kernel_ms": kms, "launches_per_step": per_step},
     }
     if h.cpu:
         refs = [np.empty((i, k)) for i, j, k in dims]

@@ -1,13 +1,24 @@
 // gemm128.hpp -- the 128x128 MFMA contraction kernel (see k_gemm.hip for the algorithm overview).
 //
-// 512 threads = 8 waves as 4x2, wave tile 32x64, two blocks per CU (<= 128 VGPRs, 76 KB LDS each) so that
-// the MFMA phase of one block overlaps the load/store phase of the other.  All operand addressing is a
-// uniform 64-bit base plus a per-thread 32-bit byte offset that is constant over the k loop; the base
-// advances by one stage per iteration on the scalar unit (single-stride k) or a per-stage table entry is
-// added (multi-mode k).  Rows past the matrix edge are read from a clamped (valid) address and never
-// stored; only the last, partial k stage is masked to zero.
+// 256 threads = 4 waves as 2x2, wave tile 64x64 (4x4 MFMA blocks), two blocks per CU so that the MFMA
+// phase of one block overlaps the load/store phase of the other.  All operand addressing is a uniform
+// 64-bit base plus a per-thread 32-bit byte offset that is constant over the k loop; the base advances by
+// one stage per iteration on the scalar unit (single-stride k) or a per-stage table entry is added
+// (multi-mode k).  Rows past the matrix edge are read from a clamped (valid) address and never stored;
+// only the last, partial k stage is masked to zero.
+//
+// A stage of an operand is ROWS x 128 bytes of k in LDS: eight 16-byte chunks per row, the chunk index
+// XOR-ed with bits 4..5 of the row so that the stores of both loader shapes and the fragment reads are free
+// of bank conflicts.  A loader moves V elements per access (V = 16 bytes / element when the operand's
+// contiguous direction allows it, else 1):
+//   k-contiguous operand  : one global load of V consecutive k of one row, one LDS store;
+//   row-contiguous operand: V loads (V consecutive k) of V consecutive rows each, transposed in registers
+//                           into V LDS stores of V consecutive k.
+// A lane reads its fragments as whole chunks (two 16-byte LDS reads per 16-row block and stage) and feeds
+// MFMA number (h, c) with k = (2*(lane/16) + h)*CH + c -- a permutation of k applied to A and B alike.
+//
 // f64 accumulators must stay in VGPRs: with AGPR accumulators v_mfma_f64_16x16x4_f64 issues every 130
-// cycles instead of 64 on gfx950 (measured), so the kernel is bounded to 128 registers and uses no AGPRs.
+// cycles instead of 64 on gfx950 (measured), so the kernel is sized to 256 VGPRs and uses no AGPRs.
 #pragma once
 #include "gemm_common.hpp"
 
@@ -24,64 +35,157 @@ __device__ __forceinline__ gptr uniform_ptr(gptr p) {
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return (gptr)(((uint64_t)hi << 32) | lo);
 }
-template <class E> struct RawOf { typedef E type; };
-template <> struct RawOf<float2> { typedef float type __attribute__((ext_vector_type(2))); };
-template <> struct RawOf<double2> { typedef double type __attribute__((ext_vector_type(2))); };
-template <class E>
-__device__ __forceinline__ E gload(gptr base, uint32_t off) {
-    typedef typename RawOf<E>::type Raw;
+template <class R, int N> struct RawVec { typedef R type __attribute__((ext_vector_type(N))); };
+template <class R> struct RawVec<R, 1> { typedef R type; };
+template <class R, int N> struct alignas(sizeof(R) * N) Pack { R v[N]; };
+template <class R, int N>
+__device__ __forceinline__ Pack<R, N> gload_pack(gptr base, uint32_t off) {
+    typedef typename RawVec<R, N>::type Raw;
     const Raw r = *reinterpret_cast<const __attribute__((address_space(1))) Raw*>(base + off);
-    return __builtin_bit_cast(E, r);
+    return __builtin_bit_cast(Pack<R, N>, r);
+}
+template <class R, int N>
+__device__ __forceinline__ void lds_store_pack(R* p, const R (&x)[N]) {
+    typedef typename RawVec<R, N>::type Raw;
+    Pack<R, N> t;
+#pragma unroll
+    for (int i = 0; i < N; ++i) t.v[i] = x[i];
+    *reinterpret_cast<Raw*>(p) = __builtin_bit_cast(Raw, t);
 }
 
 template <class R, bool CX>
 struct Cfg128 {
     static constexpr int BM = 128, BN = 128;
-    static constexpr int BKR = sizeof(R) == 8 ? 16 : 32;  // real k per stage
-    static constexpr int BKE = CX ? BKR / 2 : BKR;        // elements of k per stage
-    static constexpr int PAD = 16 / sizeof(R);
+    static constexpr int BKR = 128 / sizeof(R);           // real k per stage: 128 bytes per row
+    static constexpr int EC = CX ? 2 : 1;                 // reals per element
+    static constexpr int BKE = BKR / EC;                  // elements of k per stage
+    static constexpr int CH = 16 / sizeof(R);             // reals per 16-byte chunk
+    static constexpr int VMAX = CH / EC;                  // elements per 16-byte chunk
+    static constexpr int PAD = CH;
     static constexpr int PITCH = BKR + PAD;
-    static constexpr int BNE = CX ? BN / 2 : BN;          // element columns per tile
+    static constexpr int BNE = BN / EC;                   // element columns per tile
     static constexpr int WAVES_M = 2, WAVES_N = 2, NT = 64 * WAVES_M * WAVES_N;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 16, TN = WN / 16;
     static constexpr int MIN_WAVES = 2;   // waves per SIMD the register budget is sized for
-    static constexpr int NUA = BM * BKE / NT, NUB = BNE * BKE / NT;
     static constexpr size_t LDS_BYTES = (size_t)2 * (BM + BN) * PITCH * sizeof(R);
+    static_assert(TM == 4 && TN == 4, "the chunk swizzle assumes four 16-row blocks per wave tile");
+    // LDS index of real k `rk` in real row `rr`
+    __device__ static __forceinline__ int lds_idx(int rr, int rk) { return rr * PITCH + (((rk / CH) ^ ((rr >> 4) & 3)) * CH) + rk % CH; }
 };
 
-// Per-thread, loop-invariant description of one operand's share of a stage.  Element u of the thread sits
-// at LDS index lds0 + u*LDS_STEP and k index kk0 + u*KK_STEP (compile-time steps).
-template <class R, bool CX, int ROWS, int NU, bool KFAST, int RM>
-struct TileMap {
+// Per-thread, loop-invariant description of one operand's share of a stage (ROWS element rows x BKE k).
+//   KFAST : load l covers row rq + l*RP, k elements kq .. kq+V-1
+//   else  : load l = p*V + j covers rows rq .. rq+V-1 at k element (p*KP + kq)*V + j
+template <class R, bool CX, int ROWS, bool KFAST, int V, int RM>
+struct OperandMap {
     typedef Cfg128<R, CX> C_;
-    static constexpr int KK_STEP = KFAST ? 0 : C_::NT / ROWS;
-    static constexpr int LDS_STEP = KFAST ? (C_::NT / C_::BKE) * C_::PITCH * RM : KK_STEP * (CX ? 2 : 1);
-    uint32_t voff[NU];   // byte offset of element u relative to the (advancing) base
-    int lds0, kk0;
-    __device__ __forceinline__ int kk(int u) const { return kk0 + u * KK_STEP; }
-    __device__ __forceinline__ int lds(int u) const { return lds0 + u * LDS_STEP; }
+    static constexpr int EC = C_::EC, PN = V * EC;
+    static constexpr int KV = C_::BKE / V;             // KFAST: loads per row
+    static constexpr int RP = C_::NT / KV;             // KFAST: rows per pass
+    static constexpr int RVN = ROWS / V;               // row-contiguous: row groups per k
+    static constexpr int KP = C_::NT / RVN;            // row-contiguous: k patches per pass
+    static constexpr int NP = KFAST ? ROWS / RP : C_::BKE / (KP * V);
+    static constexpr int NL = KFAST ? NP : NP * V;     // loads per thread and stage
+    static_assert(NP >= 1 && (KFAST ? NP * RP == ROWS : NP * KP * V == C_::BKE), "operand tile must divide over the block");
+    typedef Pack<R, PN> P;
+    uint32_t voff[NL];   // byte offset of load l relative to the (advancing) base
+    int kq, rq;
+    __device__ __forceinline__ int kk(int l) const { return KFAST ? kq : ((l / V) * KP + kq) * V + (l % V); }
     __device__ __forceinline__ void init(const Off32& frow, const Off32& fk, int64_t row0, int rows_valid) {
-        constexpr int BKE = C_::BKE, NT = C_::NT, PITCH = C_::PITCH;
         const int t = threadIdx.x;
-        const int r0 = KFAST ? t / BKE : t % ROWS;
-        kk0 = KFAST ? t % BKE : t / ROWS;
-        lds0 = r0 * RM * PITCH + (CX ? 2 * kk0 : kk0);   // RM real rows per element row (2 for a complex B)
+        if (KFAST) { kq = (t % KV) * V; rq = t / KV; }
+        else { rq = (t % RVN) * V; kq = t / RVN; }
 #pragma unroll
-        for (int u = 0; u < NU; ++u) {
-            const int row = KFAST ? r0 + u * (NT / BKE) : r0;
-            const int rc = row < rows_valid ? row : rows_valid - 1;
-            voff[u] = off32_of(frow, row0 + rc) + (fk.tab ? 0u : (uint32_t)kk(u) * fk.stride);
+        for (int l = 0; l < NL; ++l) {
+            const int row = KFAST ? rq + l * RP : rq;
+            // a load past the edge is redirected to the last valid one (V divides rows_valid when rows carry the vector)
+            const int rc = row < rows_valid ? row : rows_valid - (KFAST ? 1 : V);
+            voff[l] = off32_of(frow, row0 + rc) + (fk.tab ? 0u : (uint32_t)kk(l) * fk.stride);
         }
+    }
+    // single-stride k, full stage
+    __device__ __forceinline__ void load_fast(P (&x)[NL], gptr base) const {
+#pragma unroll
+        for (int l = 0; l < NL; ++l) x[l] = gload_pack<R, PN>(base, voff[l]);
+    }
+    // single-stride k, last stage with `rem` valid k: k redirected into the range (masked to zero when stored)
+    __device__ __forceinline__ void load_tail(P (&x)[NL], gptr base, int rem, uint32_t kstride) const {
+#pragma unroll
+        for (int l = 0; l < NL; ++l) {
+            const int last = KFAST ? rem - V : rem - 1;
+            const int d = kk(l) > last ? last - kk(l) : 0;
+            x[l] = gload_pack<R, PN>(base, voff[l] + (uint32_t)d * kstride);
+        }
+    }
+    // multi-mode k: per-stage offsets from the table (k redirected to the last valid index); KFAST needs one entry
+    static constexpr int NKO = KFAST ? 1 : NL;
+    __device__ __forceinline__ void fetch_tab(uint32_t (&ko)[NKO], const uint32_t* tab, int64_t k0, int64_t kend) const {
+#pragma unroll
+        for (int l = 0; l < NKO; ++l) {
+            const int64_t ki = k0 + kk(l), last = kend - (KFAST ? V : 1);
+            ko[l] = tab[ki < last ? ki : last];
+        }
+    }
+    __device__ __forceinline__ void load_tab(P (&x)[NL], gptr base, const uint32_t* tab, int64_t k0, int64_t kend) const {
+        uint32_t ko[NKO];
+        fetch_tab(ko, tab, k0, kend);
+#pragma unroll
+        for (int l = 0; l < NL; ++l) x[l] = gload_pack<R, PN>(base, voff[l] + ko[KFAST ? 0 : l]);
+    }
+    // one load of a full stage (l is a compile-time constant at every call site)
+    __device__ __forceinline__ void load_one(P (&x)[NL], int l, gptr base, const uint32_t (&ko)[NKO], bool tab) const {
+        x[l] = gload_pack<R, PN>(base, voff[l] + (tab ? ko[KFAST ? 0 : l] : 0u));
+    }
+    // registers -> LDS tile [ROWS*RM][PITCH]; k past `rem` is zeroed when mask_tail.  A complex B (RM == 2) is
+    // expanded to B'[2n][2k] = br, B'[2n][2k+1] = -bi, B'[2n+1][2k] = bi, B'[2n+1][2k+1] = br.
+    static constexpr int VV = KFAST ? 1 : V;     // LDS stores per pass
+    static constexpr int NSU = NP * VV;          // store units per thread and stage
+    __device__ __forceinline__ void store(R* tile, const P (&x)[NL], bool mask_tail, int rem, bool conj) const {
+#pragma unroll
+        for (int u = 0; u < NSU; ++u) store_unit(tile, x, u, mask_tail, rem, conj);
+    }
+    // store unit u = (pass p, row v of the patch): one 16-byte (V > 1) or one-element LDS store (two for a complex B)
+    __device__ __forceinline__ void store_unit(R* tile, const P (&x)[NL], int u, bool mask_tail, int rem, bool conj) const {
+        constexpr int PITCH = C_::PITCH;
+        const int p = u / VV, v = u % VV;
+        // the LDS index is recomputed at every use (a few VALU operations): kept out of the loop-invariant set, it
+        // does not occupy a register during the MFMA phase
+        int rq_ = rq, kq_ = kq;
+        asm volatile("" : "+v"(rq_), "+v"(kq_));
+        const int row = KFAST ? rq_ + p * RP : rq_ + v;
+        const int kel0 = KFAST ? kq_ : (p * KP + kq_) * V;
+        R out0[PN], out1[PN];
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            const P& src = x[KFAST ? p : p * V + j];
+            const int e = KFAST ? j : v;
+            const bool ok = !mask_tail || kel0 + j < rem;
+            if constexpr (CX) {
+                const R re = ok ? src.v[2 * e] : R(0);
+                const R im = ok ? (conj ? -src.v[2 * e + 1] : src.v[2 * e + 1]) : R(0);
+                if constexpr (RM == 2) {
+                    out0[2 * j] = re; out0[2 * j + 1] = -im;
+                    out1[2 * j] = im; out1[2 * j + 1] = re;
+                } else {
+                    out0[2 * j] = re; out0[2 * j + 1] = im;
+                }
+            } else {
+                out0[j] = ok ? src.v[e] : R(0);
+            }
+        }
+        const int idx = C_::lds_idx(row * RM, kel0 * EC);
+        lds_store_pack<R, PN>(tile + idx, out0);
+        if constexpr (RM == 2) lds_store_pack<R, PN>(tile + idx + PITCH, out1);
     }
 };
 
-template <class R, bool CX, bool AKF, bool BKF>
+template <class R, bool CX, bool AKF, bool BKF, int VA, int VB>
 __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES)) gemm128_kernel(GemmArgs g) {
     typedef Cfg128<R, CX> C_;
     typedef typename ElemT<R, CX>::type E;
     typedef typename Mfma<R>::acc_t acc_t;
-    constexpr int BM = C_::BM, BN = C_::BN, BKR = C_::BKR, BKE = C_::BKE, PITCH = C_::PITCH, BNE = C_::BNE;
-    constexpr int TM = C_::TM, TN = C_::TN, NUA = C_::NUA, NUB = C_::NUB;
+    constexpr int BM = C_::BM, BN = C_::BN, BKE = C_::BKE, PITCH = C_::PITCH, BNE = C_::BNE, CH = C_::CH;
+    constexpr int TM = C_::TM, TN = C_::TN;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     R* As = reinterpret_cast<R*>(smem_raw);   // [2][BM][PITCH]
     R* Bs = As + 2 * BM * PITCH;              // [2][BN][PITCH]
@@ -106,10 +210,11 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
         tile_m = tm.y;
         tile_n = tm.z;
     } else {
-        tile_n = blockIdx.x % g.tiles_n;
-        tile_m = blockIdx.x / g.tiles_n;
-        split = blockIdx.z % g.nsplit;
-        batch = blockIdx.z / g.nsplit;
+        const uint64_t lb = logical_block((uint64_t)blockIdx.z * gridDim.x + blockIdx.x, (uint64_t)gridDim.x * gridDim.z);
+        const uint32_t lz = (uint32_t)(lb / gridDim.x);
+        tile_of((uint32_t)(lb % gridDim.x), g.tiles_m, g.tiles_n, tile_m, tile_n);
+        split = (int)(lz % (uint32_t)g.nsplit);
+        batch = lz / (uint32_t)g.nsplit;
         Ap += off_of(g.ab, batch) * (int64_t)sizeof(E);
         Bp += off_of(g.bb, batch) * (int64_t)sizeof(E);
     }
@@ -119,14 +224,16 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
     const int rowsA = (int)(M - m0 < BM ? M - m0 : BM), rowsB = (int)(N - n0 < BNE ? N - n0 : BNE);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    TileMap<R, CX, BM, NUA, AKF, 1> ma;
-    TileMap<R, CX, BNE, NUB, BKF, (CX ? 2 : 1)> mb;
+    typedef OperandMap<R, CX, BM, AKF, VA, 1> MapA;
+    typedef OperandMap<R, CX, BNE, BKF, VB, (CX ? 2 : 1)> MapB;
+    MapA ma;
+    MapB mb;
     ma.init(am, ak, m0, rowsA);
 #pragma unroll
-    for (int u = 0; u < NUA; ++u) ma.voff[u] += g.problems ? 0u : g.bias_a32;
+    for (int l = 0; l < MapA::NL; ++l) ma.voff[l] += g.problems ? 0u : g.bias_a32;
     mb.init(bn, bk, n0, rowsB);
 #pragma unroll
-    for (int u = 0; u < NUB; ++u) mb.voff[u] += g.problems ? 0u : g.bias_b32;
+    for (int l = 0; l < MapB::NL; ++l) mb.voff[l] += g.problems ? 0u : g.bias_b32;
     // uniform bases; single-stride k advances them by one stage per iteration
     gptr sa = Ap + (ak.tab ? 0 : (int64_t)(int32_t)ak.stride * kbeg);
     gptr sb = Bp + (bk.tab ? 0 : (int64_t)(int32_t)bk.stride * kbeg);
@@ -142,156 +249,155 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = acc_t{0, 0, 0, 0};
 
-    E va[NUA], vb[NUB];
+    typename MapA::P va[MapA::NL];
+    typename MapB::P vb[MapB::NL];
     const int64_t klen = kend > kbeg ? kend - kbeg : 0;
     const int64_t nstage = (klen + BKE - 1) / BKE;
     const int rem = (int)(klen - (nstage - 1) * BKE);   // k elements in the last stage (1..BKE)
     const bool ktab = ak.tab != nullptr;               // the host builds k tables for both operands or for none
 
-    // ---- stage loaders ---------------------------------------------------------------------------------------
-    // single-stride k, full stage: the invariant offsets against the advancing uniform base
     auto load_fast = [&]() {
         sa = uniform_ptr(sa);
         sb = uniform_ptr(sb);
-#pragma unroll
-        for (int u = 0; u < NUA; ++u) va[u] = gload<E>(sa, ma.voff[u]);
-#pragma unroll
-        for (int u = 0; u < NUB; ++u) vb[u] = gload<E>(sb, mb.voff[u]);
+        ma.load_fast(va, sa);
+        mb.load_fast(vb, sb);
         sa += stepA;
         sb += stepB;
     };
-    // single-stride k, last stage: k clamped into the range (masked to zero when stored)
     auto load_tail = [&]() {
-#pragma unroll
-        for (int u = 0; u < NUA; ++u) {
-            const int d = ma.kk(u) >= rem ? rem - 1 - ma.kk(u) : 0;
-            va[u] = gload<E>(sa, ma.voff[u] + (uint32_t)d * ak.stride);
-        }
-#pragma unroll
-        for (int u = 0; u < NUB; ++u) {
-            const int d = mb.kk(u) >= rem ? rem - 1 - mb.kk(u) : 0;
-            vb[u] = gload<E>(sb, mb.voff[u] + (uint32_t)d * bk.stride);
-        }
+        ma.load_tail(va, sa, rem, ak.stride);
+        mb.load_tail(vb, sb, rem, bk.stride);
     };
-    // multi-mode k: per-stage offsets from the tables (k clamped to the last valid index)
     auto load_tab = [&](int64_t s) {
-        const int64_t k0 = kbeg + s * BKE;
-        uint32_t ka[NUA], kb[NUB];
-#pragma unroll
-        for (int u = 0; u < NUA; ++u) {
-            if (AKF && u > 0) { ka[u] = ka[0]; continue; }
-            const int64_t ki = k0 + ma.kk(u);
-            ka[u] = ak.tab[ki < kend ? ki : kend - 1];
-        }
-#pragma unroll
-        for (int u = 0; u < NUB; ++u) {
-            if (BKF && u > 0) { kb[u] = kb[0]; continue; }
-            const int64_t ki = k0 + mb.kk(u);
-            kb[u] = bk.tab[ki < kend ? ki : kend - 1];
-        }
-#pragma unroll
-        for (int u = 0; u < NUA; ++u) va[u] = gload<E>(sa, ma.voff[u] + ka[u]);
-#pragma unroll
-        for (int u = 0; u < NUB; ++u) vb[u] = gload<E>(sb, mb.voff[u] + kb[u]);
+        ma.load_tab(va, sa, ak.tab, kbeg + s * BKE, kend);
+        mb.load_tab(vb, sb, bk.tab, kbeg + s * BKE, kend);
     };
-
     auto store_stage = [&](int buf, bool mask_tail) {
-        R* as = As + buf * BM * PITCH;
-        R* bs = Bs + buf * BN * PITCH;
+        ma.store(As + buf * BM * PITCH, va, mask_tail, rem, g.conj_a != 0);
+        mb.store(Bs + buf * BN * PITCH, vb, mask_tail, rem, g.conj_b != 0);
+    };
+
+    typedef typename RawVec<R, CH>::type Chunk;
+    auto compute = [&](int buf) {
+        const R* as = As + buf * BM * PITCH + (wm0 + lrow) * PITCH;
+        const R* bs = Bs + buf * BN * PITCH + (wn0 + lrow) * PITCH;
 #pragma unroll
-        for (int u = 0; u < NUA; ++u) {
-            E x = va[u];
-            const bool ok = !mask_tail || ma.kk(u) < rem;
-            if constexpr (CX) {
-                x.x = ok ? x.x : R(0);
-                x.y = ok ? (g.conj_a ? -x.y : x.y) : R(0);
-                *reinterpret_cast<E*>(as + ma.lds(u)) = x;
-            } else {
-                as[ma.lds(u)] = ok ? x : R(0);
-            }
-        }
+        for (int h = 0; h < 2; ++h) {
+            Chunk a[TM], b[TN];
 #pragma unroll
-        for (int u = 0; u < NUB; ++u) {
-            E x = vb[u];
-            const bool ok = !mask_tail || mb.kk(u) < rem;
-            if constexpr (CX) {
-                const R xr = ok ? x.x : R(0);
-                const R xi = ok ? (g.conj_b ? -x.y : x.y) : R(0);
-                E r0, r1;   // B'[2k][2n] = br, B'[2k+1][2n] = -bi ; B'[2k][2n+1] = bi, B'[2k+1][2n+1] = br
-                r0.x = xr; r0.y = -xi;
-                r1.x = xi; r1.y = xr;
-                *reinterpret_cast<E*>(bs + mb.lds(u)) = r0;            // real row 2n
-                *reinterpret_cast<E*>(bs + mb.lds(u) + PITCH) = r1;    // real row 2n+1
-            } else {
-                bs[mb.lds(u)] = ok ? x : R(0);
-            }
+            for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const Chunk*>(as + i * 16 * PITCH + ((2 * lgrp + h) ^ i) * CH);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const Chunk*>(bs + j * 16 * PITCH + ((2 * lgrp + h) ^ j) * CH);
+#pragma unroll
+            for (int c = 0; c < CH; ++c)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<R>::run(a[i][c], b[j][c], acc[i][j]);
         }
     };
 
-    constexpr int NS = BKR / 4;   // MFMA k-steps per stage
-    auto compute = [&](int buf) {
-        // lane l feeds A[row l%16][k = 4*step + l/16] and B[k = 4*step + l/16][col l%16]
-        const R* as = As + buf * BM * PITCH + (wm0 + lrow) * PITCH + lgrp;
-        const R* bs = Bs + buf * BN * PITCH + (wn0 + lrow) * PITCH + lgrp;
+    // One full iteration of the main loop with everything else issued in the shadow of the MFMAs: the global loads
+    // of stage s+1 go out between the MFMAs of the first half of stage s, the LDS stores of stage s+1 (into the other
+    // buffer, which nobody reads during this iteration) between those of the second half.  An MFMA occupies the matrix core for 32 or 64 cycles after it issues, so the instructions placed
+    // between two of them cost nothing as long as they take less than that to issue.  sched_barrier pins the
+    // order against the compiler.  With multi-mode k the table entries of stage s+2 are fetched one iteration
+    // ahead, so no load waits for its offset.
+    constexpr int HALF = TM * TN * CH;                        // MFMAs per half stage
+    constexpr int NLD = MapA::NL + MapB::NL, NST = MapA::NSU + MapB::NSU;
+    // spread evenly over the half stage (measured: better than bunching the loads early and the stores late)
+    constexpr int LD_EVERY = HALF / (NLD + 1) > 0 ? HALF / (NLD + 1) : 1;
+    constexpr int ST_EVERY = HALF / (NST + 1) > 0 ? HALF / (NST + 1) : 1;
+    constexpr int ST_FIRST = 0;
+    static_assert(LD_EVERY * NLD <= HALF && ST_FIRST >= 0, "one half stage must take all loads / stores");
+    uint32_t ka[MapA::NKO], kb[MapB::NKO];   // multi-mode k: table entries of the stage whose loads are issued next
+    auto stage_interleaved = [&](int buf, bool tab, int64_t k0_after_next) {
+        const R* as = As + buf * BM * PITCH + (wm0 + lrow) * PITCH;
+        const R* bs = Bs + buf * BN * PITCH + (wn0 + lrow) * PITCH;
+        R* as_next = As + (buf ^ 1) * BM * PITCH;
+        R* bs_next = Bs + (buf ^ 1) * BN * PITCH;
+        Chunk a[2][TM], b[2][TN];
 #pragma unroll
-        for (int st = 0; st < NS; ++st) {
-            R a[TM], b[TN];
+        for (int h = 0; h < 2; ++h) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i) a[i] = as[i * 16 * PITCH + 4 * st];
+            for (int i = 0; i < TM; ++i) a[h][i] = *reinterpret_cast<const Chunk*>(as + i * 16 * PITCH + ((2 * lgrp + h) ^ i) * CH);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) b[j] = bs[j * 16 * PITCH + 4 * st];
+            for (int j = 0; j < TN; ++j) b[h][j] = *reinterpret_cast<const Chunk*>(bs + j * 16 * PITCH + ((2 * lgrp + h) ^ j) * CH);
+        }
+        if (!tab) {
+            sa = uniform_ptr(sa);
+            sb = uniform_ptr(sb);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<R>::run(a[i], b[j], acc[i][j]);
+                for (int j = 0; j < TN; ++j) {
+                    acc[i][j] = Mfma<R>::run(a[0][i][c], b[0][j][c], acc[i][j]);
+                    const int m = (c * TM + i) * TN + j;
+                    if (m % LD_EVERY == LD_EVERY - 1 && m / LD_EVERY < NLD) {
+                        const int l = m / LD_EVERY;
+                        if (l < MapA::NL) ma.load_one(va, l, sa, ka, tab);
+                        else mb.load_one(vb, l - MapA::NL, sb, kb, tab);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+        if (tab) {
+            ma.fetch_tab(ka, ak.tab, k0_after_next, kend);
+            mb.fetch_tab(kb, bk.tab, k0_after_next, kend);
+        } else {
+            sa += stepA;
+            sb += stepB;
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    acc[i][j] = Mfma<R>::run(a[1][i][c], b[1][j][c], acc[i][j]);
+                    const int m = (c * TM + i) * TN + j;
+                    if (m >= ST_FIRST && (m - ST_FIRST) % ST_EVERY == ST_EVERY - 1) {
+                        const int u = (m - ST_FIRST) / ST_EVERY;
+                        if (u < MapA::NSU) ma.store_unit(as_next, va, u, false, rem, g.conj_a != 0);
+                        else mb.store_unit(bs_next, vb, u - MapA::NSU, false, rem, g.conj_b != 0);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
     };
 
     if (nstage > 0) {
-        if (ktab) {
-            load_tab(0);
-            store_stage(0, nstage == 1);
-            __syncthreads();
-            int64_t s = 0;
-            for (; s + 2 < nstage; ++s) {
-                load_tab(s + 1);
-                __builtin_amdgcn_sched_barrier(0);
-                compute((int)(s & 1));
-                __builtin_amdgcn_sched_barrier(0);
-                store_stage((int)((s + 1) & 1), false);
-                __syncthreads();
-            }
-            if (s + 1 < nstage) {
-                load_tab(s + 1);
-                compute((int)(s & 1));
-                store_stage((int)((s + 1) & 1), true);
-                __syncthreads();
-                ++s;
-            }
-            compute((int)(s & 1));
+        // prologue: stage 0 into buffer 0 and, when a full stage follows, its loads into the registers
+        if (nstage == 1) {
+            if (ktab) load_tab(0);
+            else load_tail();
         } else {
-            if (nstage == 1) load_tail();
+            if (ktab) load_tab(0);
             else load_fast();
-            store_stage(0, nstage == 1);
-            __syncthreads();
-            int64_t s = 0;
-            for (; s + 2 < nstage; ++s) {
-                load_fast();
-                __builtin_amdgcn_sched_barrier(0);
-                compute((int)(s & 1));
-                __builtin_amdgcn_sched_barrier(0);
-                store_stage((int)((s + 1) & 1), false);
-                __syncthreads();
-            }
-            if (s + 1 < nstage) {
-                load_tail();
-                compute((int)(s & 1));
-                store_stage((int)((s + 1) & 1), true);
-                __syncthreads();
-                ++s;
-            }
-            compute((int)(s & 1));
         }
+        store_stage(0, nstage == 1);
+        if (ktab) {
+            ma.fetch_tab(ka, ak.tab, kbeg + BKE, kend);
+            mb.fetch_tab(kb, bk.tab, kbeg + BKE, kend);
+        }
+        __syncthreads();
+        int64_t s = 0;
+        for (; s + 2 < nstage; ++s) {
+            stage_interleaved((int)(s & 1), ktab, kbeg + (s + 2) * BKE);
+            __syncthreads();
+        }
+        if (s + 1 < nstage) {
+            if (ktab) load_tab(s + 1);
+            else load_tail();
+            compute((int)(s & 1));
+            store_stage((int)((s + 1) & 1), true);
+            __syncthreads();
+            ++s;
+        }
+        compute((int)(s & 1));
     }
 
     // ---- epilogue: real column wn0 + 16 j + lrow; for complex, column 2n+p is part p of element n ----------
@@ -358,10 +464,10 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
         }
 }
 
-template <class R, bool CX, bool AKF, bool BKF>
+template <class R, bool CX, bool AKF, bool BKF, int VA, int VB>
 inline void launch_gemm128_variant(const GemmArgs& g, dim3 grid, hipStream_t st) {
     static bool once = [] {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm128_kernel<R, CX, AKF, BKF>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm128_kernel<R, CX, AKF, BKF, VA, VB>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg128<R, CX>::LDS_BYTES);
         return true;
     }();
@@ -369,18 +475,31 @@ inline void launch_gemm128_variant(const GemmArgs& g, dim3 grid, hipStream_t st)
     typedef Cfg128<R, CX> C_;
     const size_t lds = C_::LDS_BYTES;
     const dim3 block(C_::NT);
-    hipLaunchKernelGGL((gemm128_kernel<R, CX, AKF, BKF>), grid, block, lds, st, g);
+    hipLaunchKernelGGL((gemm128_kernel<R, CX, AKF, BKF, VA, VB>), grid, block, lds, st, g);
 }
 
+template <class R, bool CX, int V>
+inline void launch_gemm128_layout(const GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
+    if (akf) {
+        if (bkf) launch_gemm128_variant<R, CX, true, true, V, V>(g, grid, st);
+        else launch_gemm128_variant<R, CX, true, false, V, V>(g, grid, st);
+    } else {
+        if (bkf) launch_gemm128_variant<R, CX, false, true, V, V>(g, grid, st);
+        else launch_gemm128_variant<R, CX, false, false, V, V>(g, grid, st);
+    }
+}
+
+// g.vec: both operands satisfy the alignment and divisibility rules of 16-byte accesses
 template <class R, bool CX>
 inline void launch_gemm128_any(const GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
-    if (akf) {
-        if (bkf) launch_gemm128_variant<R, CX, true, true>(g, grid, st);
-        else launch_gemm128_variant<R, CX, true, false>(g, grid, st);
-    } else {
-        if (bkf) launch_gemm128_variant<R, CX, false, true>(g, grid, st);
-        else launch_gemm128_variant<R, CX, false, false>(g, grid, st);
+    constexpr int VMAX = Cfg128<R, CX>::VMAX;
+    if constexpr (VMAX > 1) {
+        if (g.vec) {
+            launch_gemm128_layout<R, CX, VMAX>(g, grid, akf, bkf, st);
+            return;
+        }
     }
+    launch_gemm128_layout<R, CX, 1>(g, grid, akf, bkf, st);
 }
 
 }  // namespace gemm

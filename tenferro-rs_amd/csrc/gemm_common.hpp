@@ -51,9 +51,27 @@ struct GemmArgs {
     const char* B32;
     Off32 am32, ak32, bk32, bn32;
     uint32_t bias_a32, bias_b32;   // byte distance from the rebased base back to element 0
+    int32_t vec;                   // both operands allow 16-byte accesses along their contiguous direction
     const GroupProblem* problems;  // grouped launch when non-null
     const int4* tile_map;          // per block: (problem, tile_m, tile_n, 0)
 };
+
+// Workgroups are handed to the eight XCDs (each with its own L2) round-robin in launch order.  logical_block()
+// maps a launch position to a logical position such that every XCD works through one contiguous range of
+// logical positions; tile_of() walks the tiles of one matrix eight tile rows at a time (tile row fastest), so
+// that the ~64 blocks resident on an XCD form a compact patch that shares its A rows and B columns in that L2.
+constexpr int XCDS = 8;
+__host__ __device__ __forceinline__ uint64_t logical_block(uint64_t flat, uint64_t total) {
+    const uint64_t per = total / XCDS, rem = total % XCDS, xcd = flat % XCDS, pos = flat / XCDS;
+    return (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + pos;
+}
+__device__ __forceinline__ void tile_of(uint32_t x, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+    constexpr uint32_t GM = 8;
+    const uint32_t span = GM * (uint32_t)tiles_n, first = (x / span) * GM, r = x % span;
+    const uint32_t gsz = (uint32_t)tiles_m - first < GM ? (uint32_t)tiles_m - first : GM;
+    tile_m = (int)(first + r % gsz);
+    tile_n = (int)(r / gsz);
+}
 
 template <class R> struct Mfma;
 template <> struct Mfma<double> {

@@ -509,8 +509,8 @@ int32_t plan_tiles(std::vector<Axis> axes, int elem_bytes, int max_tile_elems, b
             blocks *= (uint64_t)cnt;
         }
     a.ntiles = (int64_t)blocks;
-    static const int tune_blocks = getenv("TFH_COPY_BLOCKS") ? atoi(getenv("TFH_COPY_BLOCKS")) : 1024;
-    tp.persistent = (uint32_t)std::min<uint64_t>(blocks, (uint64_t)tune_blocks);
+    // 4 resident blocks per CU on 256 CUs; block counts from 512 to 4096 measure within 2% of each other
+    tp.persistent = (uint32_t)std::min<uint64_t>(blocks, 1024);
     // 16-byte accesses: the side's fastest tile axis is contiguous, a multiple of the vector length, and every
     // other stride keeps the vectors aligned
     const int vec = 16 / elem_bytes;
@@ -599,8 +599,7 @@ int32_t launch_copy(int dtype, const void* in, void* out, std::vector<Axis> axes
     if (!aligned(in, eb) || !aligned(out, eb)) return set_error(TFH_ERR_STRIDED, "view base is not aligned to the element size (%d bytes)", eb);
     for (auto& x : axes) x.s[2] = 0;
     TilePlan tp;
-    static const int tune_tile = getenv("TFH_COPY_TILE") ? atoi(getenv("TFH_COPY_TILE")) : 0;
-    const int max_tile = tune_tile ? tune_tile : (eb >= 16 ? 2048 : 4096);
+    const int max_tile = eb >= 16 ? 2048 : 4096;   // 32 KB of LDS per tile
     if (int32_t e = plan_tiles(axes, eb, max_tile, true, tp)) return e;
     if (tp.grid.x == 0) return TFH_OK;
     tp.args.in = in;

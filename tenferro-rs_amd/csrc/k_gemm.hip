@@ -121,10 +121,11 @@ __global__ void __launch_bounds__((Cfg<R, CX, BM, BN>::NT), 2) gemm_kernel(GemmA
         tile_m = tm.y;
         tile_n = tm.z;
     } else {
-        tile_n = blockIdx.x % g.tiles_n;
-        tile_m = blockIdx.x / g.tiles_n;
-        split = blockIdx.z % g.nsplit;
-        batch = blockIdx.z / g.nsplit;
+        const uint64_t lb = logical_block((uint64_t)blockIdx.z * gridDim.x + blockIdx.x, (uint64_t)gridDim.x * gridDim.z);
+        const uint32_t lz = (uint32_t)(lb / gridDim.x);
+        tile_of((uint32_t)(lb % gridDim.x), g.tiles_m, g.tiles_n, tile_m, tile_n);
+        split = (int)(lz % (uint32_t)g.nsplit);
+        batch = lz / (uint32_t)g.nsplit;
     }
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BNE;
     const int64_t kbeg = (int64_t)split * g.k_per_split;
@@ -329,25 +330,29 @@ __global__ void __launch_bounds__(THREADS) splitk_finalize_kernel(GemmArgs g) {
     }
 }
 
-// Offsets of every fused index of an axis group (last axis fastest): tab[i] = sum_d idx_d * stride_d.
-struct TableJob {
-    int64_t* dst;        // element offsets, or
-    uint32_t* dst32;     // byte offsets modulo 2^32 (when non-null)
-    int64_t n;
-    int32_t naxes, elem_bytes;
-    int64_t dims[TFH_MAX_RANK], strides[TFH_MAX_RANK];
+// Offsets of every fused index of an axis group (last axis fastest): tab[i] = sum_d idx_d * stride_d.  All
+// tables of one contraction are built by one launch (blockIdx.y = table).
+constexpr int MAX_TABLES = 13, MAX_TABLE_AXES = 96;
+struct TableJobs {
+    struct Job {
+        void* dst;            // int64 element offsets, or uint32 byte offsets modulo 2^32 when elem_bytes != 0
+        int64_t n;
+        int32_t first_axis, naxes, elem_bytes, pad;
+    } job[MAX_TABLES];
+    int64_t dims[MAX_TABLE_AXES], strides[MAX_TABLE_AXES];
 };
-__global__ void __launch_bounds__(THREADS) build_table_kernel(TableJob j) {
-    int64_t i = (int64_t)blockIdx.x * THREADS + threadIdx.x;
+__global__ void __launch_bounds__(THREADS) build_tables_kernel(TableJobs J) {
+    const TableJobs::Job& j = J.job[blockIdx.y];
+    const int64_t i = (int64_t)blockIdx.x * THREADS + threadIdx.x;
     if (i >= j.n) return;
     int64_t lin = i, off = 0;
-    for (int d = j.naxes - 1; d >= 0; --d) {
-        int64_t q = lin / j.dims[d];
-        off += (lin - q * j.dims[d]) * j.strides[d];
+    for (int d = j.first_axis + j.naxes - 1; d >= j.first_axis; --d) {
+        const int64_t q = lin / J.dims[d];
+        off += (lin - q * J.dims[d]) * J.strides[d];
         lin = q;
     }
-    if (j.dst32) j.dst32[i] = (uint32_t)(off * j.elem_bytes);
-    else j.dst[i] = off;
+    if (j.elem_bytes) reinterpret_cast<uint32_t*>(j.dst)[i] = (uint32_t)(off * j.elem_bytes);
+    else reinterpret_cast<int64_t*>(j.dst)[i] = off;
 }
 
 int64_t prod(const std::vector<Axis>& ax) {
@@ -408,6 +413,21 @@ void reach(const std::vector<Axis>& ax, int slot, int64_t& lo, int64_t& hi) {
         if (e < 0) lo += e;
         else hi += e;
     }
+}
+
+// 16-byte accesses along an operand's contiguous direction (`lanes`, innermost axis last): that axis has stride 1
+// and an extent divisible by the vector length, every other stride of the operand is a multiple of it, and the
+// base is 16-byte aligned.
+bool vec_ok(const void* base, int dtype, const std::vector<Axis>& lanes, std::initializer_list<const std::vector<Axis>*> groups, int slot) {
+    const int64_t V = 16 / (int64_t)dtype_size(dtype);
+    if (V <= 1) return false;
+    if ((uintptr_t)base % 16 || lanes.empty()) return false;
+    const Axis* inner = &lanes.back();
+    if (inner->s[slot] != 1 || inner->n % V) return false;
+    for (auto* grp : groups)
+        for (auto& x : *grp)
+            if (&x != inner && x.s[slot] % V) return false;
+    return true;
 }
 
 int bke_of(int dtype) {
@@ -552,20 +572,25 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         g.tiles_n = (int)((NR + bm - 1) / bm);
     }
     const bool ktab32 = use128 && (ax.K.size() > 1);   // k tables for both operands or for none
+    g.vec = use128 && vec_ok(a, dtype, a_kfast ? ax.K : ax.M, {&ax.batch, &ax.M, &ax.K}, 0) &&
+            vec_ok(b, dtype, b_kfast ? ax.K : ax.N, {&ax.batch, &ax.N, &ax.K}, 1);
 
-    // workspace: offset tables for every multi-axis group, then the split-K partials
-    struct Want { std::vector<Axis>* grp; int slot; OffFn* fn; int64_t n; };
-    Want wants[9] = {{&ax.M, 0, &g.am, M}, {&ax.K, 0, &g.ak, K}, {&ax.K, 1, &g.bk, K}, {&ax.N, 1, &g.bn, N}, {&ax.M, 2, &g.cm, M},
-                     {&ax.N, 2, &g.cn, N}, {&ax.batch, 0, &g.ab, nb}, {&ax.batch, 1, &g.bb, nb}, {&ax.batch, 2, &g.cb, nb}};
-    size_t table_bytes = 0;
-    for (auto& w : wants)
-        if (w.grp->size() > 1) table_bytes += ((size_t)w.n * sizeof(int64_t) + 255) & ~(size_t)255;
-    // 32-bit tables of the 128 kernel: rows of A and B when multi-axis, k of both when k is multi-axis
+    // workspace: offset tables for every multi-axis group, then the split-K partials.  The 128 kernel reads the
+    // operands through 32-bit byte tables (rows of A and B when multi-axis, k of both when k is multi-axis) and
+    // only C and the batch offsets through 64-bit element tables.
+    struct Want { std::vector<Axis>* grp; int slot; OffFn* fn; int64_t n; bool operand; };
+    Want wants[9] = {{&ax.M, 0, &g.am, M, true}, {&ax.K, 0, &g.ak, K, true}, {&ax.K, 1, &g.bk, K, true}, {&ax.N, 1, &g.bn, N, true},
+                     {&ax.M, 2, &g.cm, M, false}, {&ax.N, 2, &g.cn, N, false}, {&ax.batch, 0, &g.ab, nb, false},
+                     {&ax.batch, 1, &g.bb, nb, false}, {&ax.batch, 2, &g.cb, nb, false}};
     struct Want32 { std::vector<Axis>* grp; int slot; Off32* fn; int64_t n; bool force; };
     Want32 wants32[4] = {{&ax.M, 0, &g.am32, M, false}, {&ax.K, 0, &g.ak32, K, ktab32}, {&ax.K, 1, &g.bk32, K, ktab32}, {&ax.N, 1, &g.bn32, N, false}};
-    if (use128)
-        for (auto& w : wants32)
-            if (w.grp->size() > 1 || w.force) table_bytes += ((size_t)w.n * sizeof(uint32_t) + 255) & ~(size_t)255;
+    auto need64 = [&](const Want& w) { return w.grp->size() > 1 && !(use128 && w.operand); };
+    auto need32 = [&](const Want32& w) { return use128 && (w.grp->size() > 1 || w.force); };
+    size_t table_bytes = 0;
+    for (auto& w : wants)
+        if (need64(w)) table_bytes += ((size_t)w.n * sizeof(int64_t) + 255) & ~(size_t)255;
+    for (auto& w : wants32)
+        if (need32(w)) table_bytes += ((size_t)w.n * sizeof(uint32_t) + 255) & ~(size_t)255;
     size_t partial_bytes = nsplit > 1 ? (size_t)nsplit * nb * M * NR * rb : 0;
     char* ws = nullptr;
     if (table_bytes + partial_bytes) {
@@ -577,48 +602,47 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         ws = (char*)p;
     }
     size_t cursor = 0;
+    TableJobs jobs;
+    std::memset(&jobs, 0, sizeof jobs);
+    int njobs = 0, naxes = 0;
+    int64_t longest = 0;
+    auto add_job = [&](const std::vector<Axis>& grp, int slot, int64_t n, int elem_bytes, size_t entry) {
+        TableJobs::Job& j = jobs.job[njobs++];
+        j.dst = ws + cursor;
+        j.n = n;
+        j.first_axis = naxes;
+        j.naxes = (int32_t)grp.size();
+        j.elem_bytes = elem_bytes;
+        j.pad = 0;
+        for (auto& x : grp) {
+            jobs.dims[naxes] = x.n;
+            jobs.strides[naxes++] = x.s[slot];
+        }
+        longest = std::max(longest, n);
+        cursor += ((size_t)n * entry + 255) & ~(size_t)255;
+        return j.dst;
+    };
     for (auto& w : wants) {
-        if (w.grp->size() <= 1) {
-            w.fn->tab = nullptr;
-            w.fn->stride = w.grp->empty() ? 0 : (*w.grp)[0].s[w.slot];
-            continue;
-        }
-        TableJob j;
-        std::memset(&j, 0, sizeof j);
-        j.dst = (int64_t*)(ws + cursor);
-        j.n = w.n;
-        j.naxes = (int)w.grp->size();
-        for (int d = 0; d < j.naxes; ++d) {
-            j.dims[d] = (*w.grp)[d].n;
-            j.strides[d] = (*w.grp)[d].s[w.slot];
-        }
-        hipLaunchKernelGGL(build_table_kernel, dim3((uint32_t)((w.n + THREADS - 1) / THREADS)), dim3(THREADS), 0, st, j);
-        w.fn->tab = j.dst;
-        w.fn->stride = 0;
-        cursor += ((size_t)w.n * sizeof(int64_t) + 255) & ~(size_t)255;
-    }
-    if (use128) {
-        for (auto& w : wants32) {
-            if (w.grp->size() <= 1 && !w.force) {
-                w.fn->tab = nullptr;
-                w.fn->stride = w.grp->empty() ? 0u : (uint32_t)((*w.grp)[0].s[w.slot] * (int64_t)eb);
-                continue;
-            }
-            TableJob j;
-            std::memset(&j, 0, sizeof j);
-            j.dst32 = (uint32_t*)(ws + cursor);
-            j.n = w.n;
-            j.elem_bytes = (int32_t)eb;
-            j.naxes = (int)w.grp->size();
-            for (int d = 0; d < j.naxes; ++d) {
-                j.dims[d] = (*w.grp)[d].n;
-                j.strides[d] = (*w.grp)[d].s[w.slot];
-            }
-            hipLaunchKernelGGL(build_table_kernel, dim3((uint32_t)((w.n + THREADS - 1) / THREADS)), dim3(THREADS), 0, st, j);
-            w.fn->tab = j.dst32;
+        if (need64(w)) {
+            w.fn->tab = (const int64_t*)add_job(*w.grp, w.slot, w.n, 0, sizeof(int64_t));
             w.fn->stride = 0;
-            cursor += ((size_t)w.n * sizeof(uint32_t) + 255) & ~(size_t)255;
+        } else {
+            w.fn->tab = nullptr;
+            w.fn->stride = w.grp->size() == 1 ? (*w.grp)[0].s[w.slot] : 0;
         }
+    }
+    for (auto& w : wants32) {
+        if (need32(w)) {
+            w.fn->tab = (const uint32_t*)add_job(*w.grp, w.slot, w.n, (int)eb, sizeof(uint32_t));
+            w.fn->stride = 0;
+        } else {
+            w.fn->tab = nullptr;
+            w.fn->stride = w.grp->size() == 1 ? (uint32_t)((*w.grp)[0].s[w.slot] * (int64_t)eb) : 0u;
+        }
+    }
+    if (njobs)
+        hipLaunchKernelGGL(build_tables_kernel, dim3((uint32_t)((longest + THREADS - 1) / THREADS), (uint32_t)njobs), dim3(THREADS), 0, st, jobs);
+    if (use128) {
         g.A32 = (const char*)a + lo_a * (int64_t)eb;
         g.B32 = (const char*)b + lo_b * (int64_t)eb;
         g.bias_a32 = (uint32_t)(-lo_a * (int64_t)eb);
@@ -706,6 +730,7 @@ int32_t grouped_plan_init(tfh_plan& plan) {
             for (int64_t tn = 0; tn * gs->bm < NR; ++tn) tiles.push_back({gi, (int)tm, (int)tn, K});
     }
     std::stable_sort(tiles.begin(), tiles.end(), [](const T& x, const T& y) { return x.k > y.k; });
+    // launch order = sorted order: the XCDs take the tiles round-robin, so each gets an equal share of the heavy ones
     for (auto& t : tiles) gs->tile_map_host.push_back(make_int4(t.p, t.tm, t.tn, 0));
     plan.grouped = gs;
     return TFH_OK;
@@ -732,7 +757,8 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
     const int dtype = plan.dtype;
     const size_t eb = dtype_size(dtype);
     std::vector<GroupProblem> probs((size_t)plan.n_groups);
-    bool ok128 = true;
+    bool ok128 = true, vec = true;
+    const int64_t V = 16 / (int64_t)eb;
     for (int gi = 0; gi < plan.n_groups; ++gi) {
         const tfh_view& va = inputs[(size_t)gi * 2 + 0];
         const tfh_view& vb = inputs[(size_t)gi * 2 + 1];
@@ -806,6 +832,17 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
     // pick the mapping from the first problem's strides
     g.a_kfast = std::llabs(probs[0].sak) <= std::llabs(probs[0].sam) || probs[0].M == 1;
     g.b_kfast = std::llabs(probs[0].sbk) <= std::llabs(probs[0].sbn) || probs[0].N == 1;
+    // 16-byte accesses: every problem is contiguous along the direction the mapping names, with an extent divisible
+    // by the vector length there, an aligned stride in the other direction and an aligned base
+    auto vec_side = [&](const void* base, int64_t s_lane, int64_t n_lane, int64_t s_other, int64_t n_other) {
+        return (uintptr_t)base % 16 == 0 && s_lane == 1 && n_lane % V == 0 && (s_other % V == 0 || n_other == 1);
+    };
+    for (auto& p : probs) {
+        if (V <= 1) vec = false;
+        else if (!(g.a_kfast ? vec_side(p.A, p.sak, p.K, p.sam, p.M) : vec_side(p.A, p.sam, p.M, p.sak, p.K))) vec = false;
+        else if (!(g.b_kfast ? vec_side(p.B, p.sbk, p.K, p.sbn, p.N) : vec_side(p.B, p.sbn, p.N, p.sbk, p.K))) vec = false;
+    }
+    g.vec = gs->bm == 128 && vec;
     g.alpha_re = alpha.re; g.alpha_im = alpha.im; g.beta_re = beta.re; g.beta_im = beta.im;
     g.use_beta = !beta.is_zero();
     g.problems = gs->problems_dev;
