@@ -130,7 +130,7 @@ def run_c1(h):
         "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
         "roofline": {"bound": "mfma", "achieved": flops / (kms * 1e-3) / 1e12, "peak": PEAK["f32"], "unit": "TFLOP/s",
                      "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f32"], "traffic": None,
-                     "kernel": "gemm128_kernel<float, false, true, true> (split-K)", "kernel_ms": kms, "launches_per_step": per_step},
+                     "kernel": "gemm128_kernel<float, false, true, true, 4, 4> (split-K 8)", "kernel_ms": kms, "launches_per_step": per_step},
     }
     if h.cpu:
         ref = np.empty((a, b, c), np.float32)
@@ -213,7 +213,7 @@ def run_c3(h):
         "peak_intermediate_bytes": tree.peak_intermediate * 16,
         "roofline": {"bound": "mfma", "achieved": flops / (total_kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
                      "frac": flops / (total_kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": None,
-                     "kernel": "gemm128_kernel<double, true, ...> x2 + gemm_kernel<double, true, 64, 64> x1 (the three pairwise contractions of the tree)",
+                     "kernel": "gemm128_kernel<double, true, ..., 1, 1> x2 + gemm_kernel<double, true, 64, 64> x1 (the three pairwise contractions of the tree)",
                      "kernel_ms": total_kms, "launches_per_step": per_step},
     }
     if h.cpu:
@@ -246,7 +246,7 @@ def run_c4(h):
         "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
         "roofline": {"bound": "mfma", "achieved": flops / (kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
                      "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": None,
-                     "kernel": "gemm128_kernel<double, false, true, true> (grouped)", "kernel_ms": kms, "launches_per_step": per_step},
+                     "kernel": "gemm128_kernel<double, false, true, false, 2, 2> (grouped)", "kernel_ms": kms, "launches_per_step": per_step},
     }
     if h.cpu:
         refs = [np.empty((i, k)) for i, j, k in dims]
@@ -271,11 +271,21 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--configs", default="c1,c2,c3,c4")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also launch three plain 1 GiB device-to-device copies (torch's elementwise copy kernel): under "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE their readings give the counter's scale for known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus %d is not supported\n" % args.gpus)
         sys.exit(2)
     h = Harness(args.steps, args.warmup, not args.no_cpu)
+    if args.pmc_calibration:
+        src = h.torch.ones(1 << 28, dtype=h.torch.float32, device="cuda")
+        dst = h.torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        h.torch.cuda.synchronize()
+        del src, dst
     wanted = [c.strip() for c in args.configs.split(",") if c.strip()]
     if "c1" not in wanted:
         wanted.insert(0, "c1")

@@ -21,6 +21,7 @@
 // cycles instead of 64 on gfx950 (measured), so the kernel is sized to 256 VGPRs and uses no AGPRs.
 #pragma once
 #include "gemm_common.hpp"
+#include "launch.hpp"
 
 namespace tfh {
 namespace gemm {
@@ -475,7 +476,7 @@ inline void launch_gemm128_variant(const GemmArgs& g, dim3 grid, hipStream_t st)
     typedef Cfg128<R, CX> C_;
     const size_t lds = C_::LDS_BYTES;
     const dim3 block(C_::NT);
-    hipLaunchKernelGGL((gemm128_kernel<R, CX, AKF, BKF, VA, VB>), grid, block, lds, st, g);
+    TFH_LAUNCH_TIMED((gemm128_kernel<R, CX, AKF, BKF, VA, VB>), grid, block, lds, st, g);
 }
 
 template <class R, bool CX, int V>

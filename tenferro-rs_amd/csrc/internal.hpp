@@ -126,6 +126,14 @@ int32_t hip_check(int err, const char* what);
 enum { PROF_CONTRACT = 0, PROF_COPY = 1, PROF_REDUCE = 2 };
 int prof_begin(int kind, void* stream);
 void prof_end(int token, void* stream);
+// The dominant kernel's launch takes the pair of events prof_begin() prepared on this thread (null when profiling is
+// off): launched with them, the events carry the dispatch's own begin and end timestamps, so their difference is the
+// kernel's duration as a kernel trace reports it, without the launch overhead two recorded events would add.
+struct ProfEvents {
+    void* start = nullptr;
+    void* stop = nullptr;
+};
+ProfEvents prof_take();
 
 // Byte pointer of a view's element 0.
 inline char* view_ptr(const tfh_view& v, int dtype) { return (char*)v.base + v.offset * (int64_t)dtype_size(dtype); }

@@ -14,6 +14,7 @@
 #include <cstring>
 
 #include "internal.hpp"
+#include "launch.hpp"
 
 namespace tfh {
 namespace {
@@ -552,11 +553,11 @@ void launch_copy_variant(const TilePlan& tp, Op op, bool read_old, size_t lds, h
     const dim3 grid(tp.persistent), block(THREADS);
     // FAST: every tile is full (each tiled extent is a multiple of its tile extent) and spans < 4 GiB
     if (tp.all_full) {
-        if (read_old) hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, true, true>), grid, block, lds, st, tp.args, op);
-        else hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, false, true>), grid, block, lds, st, tp.args, op);
+        if (read_old) TFH_LAUNCH_TIMED((copy_kernel<V, Op, EPT, VR, VW, true, true>), grid, block, lds, st, tp.args, op);
+        else TFH_LAUNCH_TIMED((copy_kernel<V, Op, EPT, VR, VW, false, true>), grid, block, lds, st, tp.args, op);
     } else {
-        if (read_old) hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, true, false>), grid, block, lds, st, tp.args, op);
-        else hipLaunchKernelGGL((copy_kernel<V, Op, EPT, VR, VW, false, false>), grid, block, lds, st, tp.args, op);
+        if (read_old) TFH_LAUNCH_TIMED((copy_kernel<V, Op, EPT, VR, VW, true, false>), grid, block, lds, st, tp.args, op);
+        else TFH_LAUNCH_TIMED((copy_kernel<V, Op, EPT, VR, VW, false, false>), grid, block, lds, st, tp.args, op);
     }
 }
 

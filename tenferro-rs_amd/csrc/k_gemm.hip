@@ -385,7 +385,7 @@ void launch_tile(const GemmArgs& g, dim3 grid, hipStream_t st) {
         return true;
     }();
     (void)once;
-    hipLaunchKernelGGL((gemm_kernel<R, CX, BM, BN>), grid, dim3(Cfg<R, CX, BM, BN>::NT), lds, st, g);
+    TFH_LAUNCH_TIMED((gemm_kernel<R, CX, BM, BN>), grid, dim3(Cfg<R, CX, BM, BN>::NT), lds, st, g);
 }
 
 void launch_generic64(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st) {
@@ -729,8 +729,10 @@ int32_t grouped_plan_init(tfh_plan& plan) {
         for (int64_t tm = 0; tm * gs->bm < M; ++tm)
             for (int64_t tn = 0; tn * gs->bm < NR; ++tn) tiles.push_back({gi, (int)tm, (int)tn, K});
     }
+    // Heaviest tiles (largest K) first so that the tail of the launch is short.  The XCDs take the list round-robin,
+    // so each gets an equal share of every problem; giving whole problems to one XCD for L2 locality measured 10%
+    // slower (the balance is worth more than the operand re-use).
     std::stable_sort(tiles.begin(), tiles.end(), [](const T& x, const T& y) { return x.k > y.k; });
-    // launch order = sorted order: the XCDs take the tiles round-robin, so each gets an equal share of the heavy ones
     for (auto& t : tiles) gs->tile_map_host.push_back(make_int4(t.p, t.tm, t.tn, 0));
     plan.grouped = gs;
     return TFH_OK;

@@ -15,6 +15,7 @@
 #include <cstring>
 
 #include "internal.hpp"
+#include "launch.hpp"
 
 namespace tfh {
 namespace {
@@ -439,10 +440,10 @@ void launch_fast_ks(const FastReduceArgs& fa, dim3 grid, int ks, hipStream_t st)
     const int nv = KV ? VEC : 1;
     if (ks == 8) {
         size_t lds = FAST_MAX_RTAB * sizeof(int64_t) + (size_t)8 * nv * THREADS * sizeof(double);
-        hipLaunchKernelGGL((reduce_fast_kernel<R, VEC, KV, 8>), grid, dim3(THREADS), lds, st, fa);
+        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 8>), grid, dim3(THREADS), lds, st, fa);
     } else {
         size_t lds = FAST_MAX_RTAB * sizeof(int64_t) + (size_t)nv * THREADS * sizeof(double);
-        hipLaunchKernelGGL((reduce_fast_kernel<R, VEC, KV, 1>), grid, dim3(THREADS), lds, st, fa);
+        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 1>), grid, dim3(THREADS), lds, st, fa);
     }
 }
 template <class R>
@@ -713,10 +714,10 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
     dim3 grid((uint32_t)blocks, (uint32_t)nchunks, 1), block(THREADS);
     const int prof = prof_begin(PROF_REDUCE, stream);
     switch (dtype) {
-        case TFH_F32: hipLaunchKernelGGL((reduce_kernel<float, false>), grid, block, 0, st, ra); break;
-        case TFH_F64: hipLaunchKernelGGL((reduce_kernel<double, false>), grid, block, 0, st, ra); break;
-        case TFH_C64: hipLaunchKernelGGL((reduce_kernel<float, true>), grid, block, 0, st, ra); break;
-        default: hipLaunchKernelGGL((reduce_kernel<double, true>), grid, block, 0, st, ra); break;
+        case TFH_F32: TFH_LAUNCH_TIMED((reduce_kernel<float, false>), grid, block, 0, st, ra); break;
+        case TFH_F64: TFH_LAUNCH_TIMED((reduce_kernel<double, false>), grid, block, 0, st, ra); break;
+        case TFH_C64: TFH_LAUNCH_TIMED((reduce_kernel<float, true>), grid, block, 0, st, ra); break;
+        default: TFH_LAUNCH_TIMED((reduce_kernel<double, true>), grid, block, 0, st, ra); break;
     }
     prof_end(prof, stream);
     if (int32_t e = hip_check(hipGetLastError(), "reduce kernel launch")) return e;

@@ -109,19 +109,33 @@ hipEvent_t prof_event() {
 }
 }  // namespace
 
+namespace {
+thread_local ProfEvents t_pending;
+}
 int prof_begin(int kind, void* stream) {
+    (void)stream;
     if (!g_prof_on) return -1;
     std::lock_guard<std::mutex> lk(g_prof_mu);
     ProfRec r{kind, prof_event(), prof_event()};
     if (!r.a || !r.b) return -1;
-    (void)hipEventRecord(r.a, (hipStream_t)stream);
+    t_pending.start = r.a;
+    t_pending.stop = r.b;
     g_prof.push_back(r);
     return (int)g_prof.size() - 1;
 }
+ProfEvents prof_take() {
+    ProfEvents e = t_pending;
+    t_pending = ProfEvents{};
+    return e;
+}
 void prof_end(int token, void* stream) {
     if (token < 0) return;
-    std::lock_guard<std::mutex> lk(g_prof_mu);
-    if (token < (int)g_prof.size()) (void)hipEventRecord(g_prof[(size_t)token].b, (hipStream_t)stream);
+    // no kernel took the events (the call returned before its launch): record them so that the pair is complete
+    ProfEvents e = prof_take();
+    if (e.start) {
+        (void)hipEventRecord((hipEvent_t)e.start, (hipStream_t)stream);
+        (void)hipEventRecord((hipEvent_t)e.stop, (hipStream_t)stream);
+    }
 }
 
 }  // namespace tfh
