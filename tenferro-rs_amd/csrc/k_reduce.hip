@@ -350,10 +350,10 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
     // block origin (uniform) and this thread's offsets inside the tile
     int64_t org_in = 0, org_out = 0;
     {
-        uint64_t bid = blockIdx.x;
+        uint32_t bid = blockIdx.x;   // the grid (and so every count) is below 2^31
         for (int g = 0; g < a.ng; ++g) {
-            uint64_t q = bid / (uint64_t)a.g_count[g];
-            int64_t c = (int64_t)(bid - q * (uint64_t)a.g_count[g]);
+            const uint32_t n = (uint32_t)a.g_count[g], q = bid / n;
+            const int64_t c = (int64_t)(bid - q * n);
             bid = q;
             org_in += c * a.g_sa[g];
             org_out += c * a.g_sc[g];
@@ -368,46 +368,59 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
         if (a.t_red[t]) writer &= c == 0;
         else toff_out += (int64_t)c * a.t_sc[t];
     }
-    const R* A = reinterpret_cast<const R*>(a.in) + org_in + toff_in;
     const int op = a.op;
+    __syncthreads();
+    const R* A = reinterpret_cast<const R*>(a.in) + org_in + toff_in;
     double acc[KS][NV];
 #pragma unroll
     for (int k = 0; k < KS; ++k)
 #pragma unroll
         for (int j = 0; j < NV; ++j) acc[k][j] = identity(op);
-    __syncthreads();
-    constexpr int U = KS >= 8 ? 2 : 16;
+    constexpr int U = KS >= 8 ? 2 : 8;
+    // a rolling window of U loads per thread: the load of step it+U is issued as soon as the value of step it has
+    // been taken, so the memory pipeline never drains between batches
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
         const R* Ak = A + k * a.ks_sa;
+        RVec<R, VEC> v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < a.r_total) v[u] = *reinterpret_cast<const RVec<R, VEC>*>(Ak + rtab[u]);
         for (int it = 0; it < a.r_total; it += U) {
-            RVec<R, VEC> v[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (it + u < a.r_total) v[u] = *reinterpret_cast<const RVec<R, VEC>*>(Ak + rtab[it + u]);
+            for (int u = 0; u < U; ++u) {
+                if (it + u >= a.r_total) break;
+                const RVec<R, VEC> x = v[u];
+                if (it + U + u < a.r_total) v[u] = *reinterpret_cast<const RVec<R, VEC>*>(Ak + rtab[it + U + u]);
+                if (KV) {
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (it + u < a.r_total) {
-                    if (KV) {
+                    for (int j = 0; j < VEC; ++j) acc[k][j] = combine(acc[k][j], (double)x.v[j], op);
+                } else {
+                    double s = (double)x.v[0];
 #pragma unroll
-                        for (int j = 0; j < VEC; ++j) acc[k][j] = combine(acc[k][j], (double)v[u].v[j], op);
-                    } else {
-                        double s = (double)v[u].v[0];
-#pragma unroll
-                        for (int j = 1; j < VEC; ++j) s = combine(s, (double)v[u].v[j], op);
-                        acc[k][0] = combine(acc[k][0], s, op);
-                    }
+                    for (int j = 1; j < VEC; ++j) s = combine(s, (double)x.v[j], op);
+                    acc[k][0] = combine(acc[k][0], s, op);
                 }
+            }
         }
     }
-    // lanes that share outputs fold through LDS over the reduced thread-id bits
-    if (a.red_bits) {
+    // lanes that share outputs fold over the reduced thread-id bits: inside a wave with lane exchanges, across
+    // waves (bits 6 and 7) through LDS
+#pragma unroll
+    for (int b = 0; b < 6; ++b)
+        if (a.red_bits & (1 << b)) {
+#pragma unroll
+            for (int k = 0; k < KS; ++k)
+#pragma unroll
+                for (int j = 0; j < NV; ++j) acc[k][j] = combine(acc[k][j], __shfl_xor(acc[k][j], 1 << b), op);
+        }
+    if (a.red_bits & 0xc0) {
 #pragma unroll
         for (int k = 0; k < KS; ++k)
 #pragma unroll
             for (int j = 0; j < NV; ++j) lds[(k * NV + j) * THREADS + tid] = acc[k][j];
         __syncthreads();
-        for (int b = 7; b >= 0; --b) {
+        for (int b = 7; b >= 6; --b) {
             const int bit = 1 << b;
             if (a.red_bits & bit) {
                 if (!(tid & bit)) {
@@ -422,17 +435,18 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
 #pragma unroll
             for (int j = 0; j < NV; ++j) acc[k][j] = lds[(k * NV + j) * THREADS + tid];
     }
-    if (!writer) return;
-    R* C = reinterpret_cast<R*>(a.out) + org_out + toff_out;
+    if (writer) {
+        R* C = reinterpret_cast<R*>(a.out) + org_out + toff_out;
 #pragma unroll
-    for (int k = 0; k < KS; ++k)
+        for (int k = 0; k < KS; ++k)
 #pragma unroll
-        for (int j = 0; j < NV; ++j) {
-            R* dst = C + k * a.ks_sc + j * a.vc_stride;
-            double r = a.alpha * acc[k][j];
-            if (a.use_beta) r += a.beta * (double)*dst;
-            *dst = (R)r;
-        }
+            for (int j = 0; j < NV; ++j) {
+                R* dst = C + k * a.ks_sc + j * a.vc_stride;
+                double r = a.alpha * acc[k][j];
+                if (a.use_beta) r += a.beta * (double)*dst;
+                *dst = (R)r;
+            }
+    }
 }
 
 template <class R, int VEC, bool KV>
@@ -564,6 +578,7 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
         blocks /= 8;
     }
     if (blocks < 256 && r_total >= 64) return false;   // few outputs, long reduction: the split kernel handles it
+
     fa.r_total = (int32_t)r_total;
     fa.in = a;
     fa.out = c;
