@@ -28,6 +28,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK = {"hbm": 8000.0, "f32": 157.3, "f64": 78.6}   # GB/s, TFLOP/s (MI355X published peaks)
+# HBM bytes per launch of each configuration's dominant kernel, from the two rocprofv3 --pmc passes (FETCH_SIZE, then
+# WRITE_SIZE) summarised in profiles/bench_hbm_traffic_pmc.txt, each scaled by what the same counter read for plain
+# 1 GiB device copies in the same run (x2.0 and x1.0).  A profiler cannot run inside this script; these are that run's
+# figures for exactly these workloads.
+TRAFFIC = {"c1": 223.5e6 + 33.6e6, "c2_permute": 134.3e6 + 134.2e6, "c2_reduce": 134.4e6 + 0.5e6,
+           "c3": 2 * (2636.2e6 + 402.7e6) + 554.0e6 + 536.9e6, "c4": 2729.6e6 + 323.2e6}
 METRIC = "contraction TFLOP/s & % MFMA peak (f64/f32); permute/reduce GB/s & % HBM peak"
 
 
@@ -129,7 +135,8 @@ def run_c1(h):
         "dtype": "f32", "ms_per_step": ms, "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
         "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
         "roofline": {"bound": "mfma", "achieved": flops / (kms * 1e-3) / 1e12, "peak": PEAK["f32"], "unit": "TFLOP/s",
-                     "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f32"], "traffic": None,
+                     "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f32"], "traffic": TRAFFIC["c1"],
+                     "traffic_unit": "HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, calibrated)",
                      "kernel": "gemm128_kernel<float, false, true, true, 4, 4> (split-K 8)", "kernel_ms": kms, "launches_per_step": per_step},
     }
     if h.cpu:
@@ -168,10 +175,10 @@ def run_c2(h):
         "workload": "f64 16^6 tensor: permute to (5,2,0,4,1,3), then sum over output axes 1 and 4",
         "dtype": "f64", "ms_per_step": ms, "value": (pbytes + rbytes) / (ms * 1e-3) / 1e9, "unit": "GB/s",
         "permute": {"roofline": {"bound": "hbm", "achieved": pbytes / (pms * 1e-3) / 1e9, "peak": PEAK["hbm"], "unit": "GB/s",
-                                 "frac": pbytes / (pms * 1e-3) / 1e9 / PEAK["hbm"], "traffic": None,
+                                 "frac": pbytes / (pms * 1e-3) / 1e9 / PEAK["hbm"], "traffic": TRAFFIC["c2_permute"],
                                  "kernel": "copy_kernel<u64, OpCopy, 16, 2, 2, false, true>", "kernel_ms": pms}, "algorithmic_bytes": pbytes},
         "reduce": {"roofline": {"bound": "hbm", "achieved": rbytes / (rms * 1e-3) / 1e9, "peak": PEAK["hbm"], "unit": "GB/s",
-                                "frac": rbytes / (rms * 1e-3) / 1e9 / PEAK["hbm"], "traffic": None,
+                                "frac": rbytes / (rms * 1e-3) / 1e9 / PEAK["hbm"], "traffic": TRAFFIC["c2_reduce"],
                                 "kernel": "reduce_fast_kernel<double, 2, true, 1>", "kernel_ms": rms}, "algorithmic_bytes": rbytes},
     }
     if h.cpu:
@@ -212,7 +219,7 @@ def run_c3(h):
         "flops_per_step": flops, "tree_steps": tree.steps, "min_flop_tree": bool(abs(flops - 558.3e9) < 0.1e9),
         "peak_intermediate_bytes": tree.peak_intermediate * 16,
         "roofline": {"bound": "mfma", "achieved": flops / (total_kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
-                     "frac": flops / (total_kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": None,
+                     "frac": flops / (total_kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": TRAFFIC["c3"],
                      "kernel": "gemm128_kernel<double, true, ..., 1, 1> x2 + gemm_kernel<double, true, 64, 64> x1 (the three pairwise contractions of the tree)",
                      "kernel_ms": total_kms, "launches_per_step": per_step},
     }
@@ -245,7 +252,7 @@ def run_c4(h):
         "dtype": "f64", "ms_per_step": ms, "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
         "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
         "roofline": {"bound": "mfma", "achieved": flops / (kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
-                     "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": None,
+                     "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": TRAFFIC["c4"],
                      "kernel": "gemm128_kernel<double, false, true, false, 2, 2> (grouped)", "kernel_ms": kms, "launches_per_step": per_step},
     }
     if h.cpu:
