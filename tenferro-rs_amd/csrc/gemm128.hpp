@@ -39,11 +39,21 @@ __device__ __forceinline__ gptr uniform_ptr(gptr p) {
 template <class R, int N> struct RawVec { typedef R type __attribute__((ext_vector_type(N))); };
 template <class R> struct RawVec<R, 1> { typedef R type; };
 template <class R, int N> struct alignas(sizeof(R) * N) Pack { R v[N]; };
+// Global loads promise only element alignment (gfx950 executes an under-aligned global_load_dwordx4), so an operand
+// whose rows start at odd element offsets still takes the 16-byte path.
+template <class R, int N> struct RawVecU { typedef R type __attribute__((ext_vector_type(N), aligned(sizeof(R)))); };
+template <class R> struct RawVecU<R, 1> { typedef R type; };
 template <class R, int N>
 __device__ __forceinline__ Pack<R, N> gload_pack(gptr base, uint32_t off) {
-    typedef typename RawVec<R, N>::type Raw;
+    typedef typename RawVecU<R, N>::type Raw;
     const Raw r = *reinterpret_cast<const __attribute__((address_space(1))) Raw*>(base + off);
-    return __builtin_bit_cast(Pack<R, N>, r);
+    Pack<R, N> out;
+    if constexpr (N == 1) out.v[0] = r;
+    else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) out.v[i] = r[i];
+    }
+    return out;
 }
 template <class R, int N>
 __device__ __forceinline__ void lds_store_pack(R* p, const R (&x)[N]) {
@@ -91,15 +101,22 @@ struct OperandMap {
     typedef Pack<R, PN> P;
     uint32_t voff[NL];   // byte offset of load l relative to the (advancing) base
     int kq, rq;
+    // Last stage only.  A vector that straddles the end of its contiguous direction (k past `rem` for a k-contiguous
+    // operand, rows past the matrix edge for a row-contiguous one) is loaded from a window moved back to end exactly
+    // at the boundary -- nothing is read past the operand -- and its elements are moved up by the same amount when
+    // they are stored.  Full stages need none of this: there such a vector only over-reads into the operand's next
+    // column, which exists.
+    int row_shift;
     __device__ __forceinline__ int kk(int l) const { return KFAST ? kq : ((l / V) * KP + kq) * V + (l % V); }
     __device__ __forceinline__ void init(const Off32& frow, const Off32& fk, int64_t row0, int rows_valid) {
         const int t = threadIdx.x;
         if (KFAST) { kq = (t % KV) * V; rq = t / KV; }
         else { rq = (t % RVN) * V; kq = t / RVN; }
+        row_shift = (!KFAST && rq < rows_valid && rq + V > rows_valid) ? rq + V - rows_valid : 0;
 #pragma unroll
         for (int l = 0; l < NL; ++l) {
             const int row = KFAST ? rq + l * RP : rq;
-            // a load past the edge is redirected to the last valid one (V divides rows_valid when rows carry the vector)
+            // a load wholly past the edge is redirected to the last valid one
             const int rc = row < rows_valid ? row : rows_valid - (KFAST ? 1 : V);
             voff[l] = off32_of(frow, row0 + rc) + (fk.tab ? 0u : (uint32_t)kk(l) * fk.stride);
         }
@@ -110,12 +127,13 @@ struct OperandMap {
         for (int l = 0; l < NL; ++l) x[l] = gload_pack<R, PN>(base, voff[l]);
     }
     // single-stride k, last stage with `rem` valid k: k redirected into the range (masked to zero when stored)
-    __device__ __forceinline__ void load_tail(P (&x)[NL], gptr base, int rem, uint32_t kstride) const {
+    __device__ __forceinline__ void load_tail(P (&x)[NL], gptr base, int rem, uint32_t kstride, uint32_t rowstride) const {
+        const uint32_t back = (uint32_t)(-row_shift) * rowstride;
 #pragma unroll
         for (int l = 0; l < NL; ++l) {
             const int last = KFAST ? rem - V : rem - 1;
             const int d = kk(l) > last ? last - kk(l) : 0;
-            x[l] = gload_pack<R, PN>(base, voff[l] + (uint32_t)d * kstride);
+            x[l] = gload_pack<R, PN>(base, voff[l] + (uint32_t)d * kstride + back);
         }
     }
     // multi-mode k: per-stage offsets from the table (k redirected to the last valid index); KFAST needs one entry
@@ -133,6 +151,7 @@ struct OperandMap {
 #pragma unroll
         for (int l = 0; l < NL; ++l) x[l] = gload_pack<R, PN>(base, voff[l] + ko[KFAST ? 0 : l]);
     }
+    static_assert(V >= 1, "");
     // one load of a full stage (l is a compile-time constant at every call site)
     __device__ __forceinline__ void load_one(P (&x)[NL], int l, gptr base, const uint32_t (&ko)[NKO], bool tab) const {
         x[l] = gload_pack<R, PN>(base, voff[l] + (tab ? ko[KFAST ? 0 : l] : 0u));
@@ -145,6 +164,16 @@ struct OperandMap {
 #pragma unroll
         for (int u = 0; u < NSU; ++u) store_unit(tile, x, u, mask_tail, rem, conj);
     }
+    // element e (possibly a run-time index, last stage only) of a load
+    __device__ static __forceinline__ void pick(const P& src, int e, R& re, R& im) {
+        re = src.v[0];
+        im = EC == 2 ? src.v[EC - 1] : R(0);
+#pragma unroll
+        for (int i = 1; i < V; ++i) {
+            re = e == i ? src.v[i * EC] : re;
+            if (EC == 2) im = e == i ? src.v[i * EC + EC - 1] : im;
+        }
+    }
     // store unit u = (pass p, row v of the patch): one 16-byte (V > 1) or one-element LDS store (two for a complex B)
     __device__ __forceinline__ void store_unit(R* tile, const P (&x)[NL], int u, bool mask_tail, int rem, bool conj) const {
         constexpr int PITCH = C_::PITCH;
@@ -156,14 +185,23 @@ struct OperandMap {
         const int row = KFAST ? rq_ + p * RP : rq_ + v;
         const int kel0 = KFAST ? kq_ : (p * KP + kq_) * V;
         R out0[PN], out1[PN];
+        // last stage: the window of a straddling vector was moved back by this many elements
+        const int kshift = (mask_tail && KFAST && kel0 < rem && kel0 + V > rem) ? kel0 + V - rem : 0;
 #pragma unroll
         for (int j = 0; j < V; ++j) {
             const P& src = x[KFAST ? p : p * V + j];
             const int e = KFAST ? j : v;
             const bool ok = !mask_tail || kel0 + j < rem;
+            R sre, sim;
+            if (mask_tail && V > 1) {
+                pick(src, KFAST ? j + kshift : v + row_shift, sre, sim);   // indices past V-1 belong to masked k / rows outside the matrix
+            } else {
+                sre = src.v[EC * e];
+                sim = EC == 2 ? src.v[EC * e + EC - 1] : R(0);
+            }
             if constexpr (CX) {
-                const R re = ok ? src.v[2 * e] : R(0);
-                const R im = ok ? (conj ? -src.v[2 * e + 1] : src.v[2 * e + 1]) : R(0);
+                const R re = ok ? sre : R(0);
+                const R im = ok ? (conj ? -sim : sim) : R(0);
                 if constexpr (RM == 2) {
                     out0[2 * j] = re; out0[2 * j + 1] = -im;
                     out1[2 * j] = im; out1[2 * j + 1] = re;
@@ -171,7 +209,7 @@ struct OperandMap {
                     out0[2 * j] = re; out0[2 * j + 1] = im;
                 }
             } else {
-                out0[j] = ok ? src.v[e] : R(0);
+                out0[j] = ok ? sre : R(0);
             }
         }
         const int idx = C_::lds_idx(row * RM, kel0 * EC);
@@ -266,8 +304,8 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
         sb += stepB;
     };
     auto load_tail = [&]() {
-        ma.load_tail(va, sa, rem, ak.stride);
-        mb.load_tail(vb, sb, rem, bk.stride);
+        ma.load_tail(va, sa, rem, ak.stride, am.stride);
+        mb.load_tail(vb, sb, rem, bk.stride, bn.stride);
     };
     auto load_tab = [&](int64_t s) {
         ma.load_tab(va, sa, ak.tab, kbeg + s * BKE, kend);

@@ -415,19 +415,20 @@ void reach(const std::vector<Axis>& ax, int slot, int64_t& lo, int64_t& hi) {
     }
 }
 
-// 16-byte accesses along an operand's contiguous direction (`lanes`, innermost axis last): that axis has stride 1
-// and an extent divisible by the vector length, every other stride of the operand is a multiple of it, and the
-// base is 16-byte aligned.
-bool vec_ok(const void* base, int dtype, const std::vector<Axis>& lanes, std::initializer_list<const std::vector<Axis>*> groups, int slot) {
+// 16-byte accesses along an operand's contiguous direction (`lanes`, innermost axis last; `other` is the group the
+// lanes do not run along): the innermost axis has stride 1 and either an extent divisible by the vector length, or
+// the direction is a single axis of at least one vector -- then the kernel handles the vector that straddles the
+// end in its last stage; a row-contiguous operand additionally needs the next k column to lie above the current
+// one, because full stages over-read into it.  No alignment beyond the element's is required.
+bool vec_ok(int dtype, const std::vector<Axis>& lanes, const std::vector<Axis>& other, bool lanes_are_k, int slot) {
     const int64_t V = 16 / (int64_t)dtype_size(dtype);
-    if (V <= 1) return false;
-    if ((uintptr_t)base % 16 || lanes.empty()) return false;
-    const Axis* inner = &lanes.back();
-    if (inner->s[slot] != 1 || inner->n % V) return false;
-    for (auto* grp : groups)
-        for (auto& x : *grp)
-            if (&x != inner && x.s[slot] % V) return false;
-    return true;
+    if (V <= 1 || lanes.empty()) return false;
+    const Axis& inner = lanes.back();
+    if (inner.s[slot] != 1) return false;
+    if (inner.n % V == 0) return true;
+    if (lanes.size() != 1 || inner.n < V) return false;
+    if (lanes_are_k) return true;
+    return other.empty() || (other.size() == 1 && (other[0].n == 1 || other[0].s[slot] >= V));
 }
 
 int bke_of(int dtype) {
@@ -572,8 +573,8 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         g.tiles_n = (int)((NR + bm - 1) / bm);
     }
     const bool ktab32 = use128 && (ax.K.size() > 1);   // k tables for both operands or for none
-    g.vec = use128 && vec_ok(a, dtype, a_kfast ? ax.K : ax.M, {&ax.batch, &ax.M, &ax.K}, 0) &&
-            vec_ok(b, dtype, b_kfast ? ax.K : ax.N, {&ax.batch, &ax.N, &ax.K}, 1);
+    g.vec = use128 && vec_ok(dtype, a_kfast ? ax.K : ax.M, a_kfast ? ax.M : ax.K, a_kfast, 0) &&
+            vec_ok(dtype, b_kfast ? ax.K : ax.N, b_kfast ? ax.N : ax.K, b_kfast, 1);
 
     // workspace: offset tables for every multi-axis group, then the split-K partials.  The 128 kernel reads the
     // operands through 32-bit byte tables (rows of A and B when multi-axis, k of both when k is multi-axis) and
@@ -834,15 +835,19 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
     // pick the mapping from the first problem's strides
     g.a_kfast = std::llabs(probs[0].sak) <= std::llabs(probs[0].sam) || probs[0].M == 1;
     g.b_kfast = std::llabs(probs[0].sbk) <= std::llabs(probs[0].sbn) || probs[0].N == 1;
-    // 16-byte accesses: every problem is contiguous along the direction the mapping names, with an extent divisible
-    // by the vector length there, an aligned stride in the other direction and an aligned base
-    auto vec_side = [&](const void* base, int64_t s_lane, int64_t n_lane, int64_t s_other, int64_t n_other) {
-        return (uintptr_t)base % 16 == 0 && s_lane == 1 && n_lane % V == 0 && (s_other % V == 0 || n_other == 1);
+    // 16-byte accesses: every problem is contiguous along the direction the mapping names, with an extent there that
+    // is divisible by the vector length or at least one vector long (the kernel's last stage handles the straddle; a
+    // row-contiguous operand then needs its next k column above the current one)
+    auto vec_side = [&](bool kfast, int64_t s_lane, int64_t n_lane, int64_t s_other, int64_t n_other) {
+        if (s_lane != 1) return false;
+        if (n_lane % V == 0) return true;
+        if (n_lane < V) return false;
+        return kfast || n_other == 1 || s_other >= V;
     };
     for (auto& p : probs) {
         if (V <= 1) vec = false;
-        else if (!(g.a_kfast ? vec_side(p.A, p.sak, p.K, p.sam, p.M) : vec_side(p.A, p.sam, p.M, p.sak, p.K))) vec = false;
-        else if (!(g.b_kfast ? vec_side(p.B, p.sbk, p.K, p.sbn, p.N) : vec_side(p.B, p.sbn, p.N, p.sbk, p.K))) vec = false;
+        else if (!(g.a_kfast ? vec_side(true, p.sak, p.K, p.sam, p.M) : vec_side(false, p.sam, p.M, p.sak, p.K))) vec = false;
+        else if (!(g.b_kfast ? vec_side(true, p.sbk, p.K, p.sbn, p.N) : vec_side(false, p.sbn, p.N, p.sbk, p.K))) vec = false;
     }
     g.vec = gs->bm == 128 && vec;
     g.alpha_re = alpha.re; g.alpha_im = alpha.im; g.beta_re = beta.re; g.beta_im = beta.im;

@@ -650,3 +650,42 @@ def test_config3_full_size_complex128(tf, oracle):
     ref = np.empty((chi, D, chi), np.complex128)
     oracle.einsum_pairs(host, [lab(t) for t in terms], ref, lab(out), tree.steps)
     assert relerr(res.to_numpy(), ref) < 1e-12
+
+
+ODD_SIZES = [(129, 131, 133), (255, 77, 257), (131, 5, 129), (130, 3, 131), (257, 4, 130), (193, 34, 97)]
+LAYOUTS = [("mk", "kn"), ("mk", "nk"), ("km", "kn"), ("km", "nk")]
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("layout", LAYOUTS, ids=["NN", "NT", "TN", "TT"])
+def test_contract_odd_extents_take_the_straddling_vector_path(tf, oracle, dtype, layout):
+    # extents that are not multiples of the 16-byte vector length: the last vector of a row or column straddles the
+    # end of the operand and is loaded from a window moved back inside it (k smaller than one vector: scalar path)
+    ma, mb = layout
+    rng = np.random.default_rng(47)
+    for m, k, n in ODD_SIZES:
+        ext = dict(m=m, k=k, n=n)
+        a = rand(rng, [ext[l] for l in ma], dtype)
+        b = rand(rng, [ext[l] for l in mb], dtype)
+        ref = np.empty((m, n), dtype)
+        oracle.contract(a, lab(ma), b, lab(mb), ref, lab("mn"))
+        out = dev(tf, np.full((m, n), np.nan, dtype))
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab("mn")), [a.shape, b.shape, [m, n]])
+        tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
+        assert relerr(out.to_numpy(), ref) < TOL[dtype], (m, k, n)
+
+
+def test_contract_operand_ending_at_the_end_of_its_allocation(tf, oracle):
+    # the operands are the tail of exactly-sized device buffers: a read past the last element would leave the buffer
+    rng = np.random.default_rng(48)
+    for dtype, m, k, n in [(np.float32, 131, 133, 129), (np.float64, 129, 67, 131)]:
+        for ma, mb in LAYOUTS:
+            ext = dict(m=m, k=k, n=n)
+            a = rand(rng, [ext[l] for l in ma], dtype)
+            b = rand(rng, [ext[l] for l in mb], dtype)
+            ref = np.empty((m, n), dtype)
+            oracle.contract(a, lab(ma), b, lab(mb), ref, lab("mn"))
+            out = dev(tf, np.zeros((m, n), dtype))
+            plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab("mn")), [a.shape, b.shape, [m, n]])
+            tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
+            assert relerr(out.to_numpy(), ref) < TOL[dtype], (dtype, ma, mb)
