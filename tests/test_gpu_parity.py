@@ -689,3 +689,42 @@ def test_contract_operand_ending_at_the_end_of_its_allocation(tf, oracle):
             plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab("mn")), [a.shape, b.shape, [m, n]])
             tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
             assert relerr(out.to_numpy(), ref) < TOL[dtype], (dtype, ma, mb)
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_permute_extents_with_divisor_tiles(tf, oracle, dtype):
+    # extents that are not powers of two but have useful divisors (15, 50, 60, 250): tiled without partial tiles
+    rng = np.random.default_rng(49)
+    for shape, perm in [((15, 15, 15, 15), (3, 1, 0, 2)), ((60, 50, 70), (2, 0, 1)), ((250, 130), (1, 0)), ((6, 250, 9, 20), (1, 3, 0, 2)),
+                        ((33, 257), (1, 0)), ((12, 100, 35), (0, 2, 1))]:
+        a = rand(rng, shape, dtype)
+        got, ref = _permute_check(tf, oracle, a, perm)
+        assert got.tobytes() == ref.tobytes(), (shape, perm)
+    a = rand(rng, (60, 50, 70), dtype)
+    b0 = rand(rng, (70, 60, 50), dtype)
+    alpha, beta = (0.5 - 2j, 1.5 + 1j) if np.issubdtype(dtype, np.complexfloating) else (0.5, -1.5)
+    got, ref = _permute_check(tf, oracle, a, (2, 0, 1), alpha, beta, b0)
+    assert relerr(got, ref) < TOL[dtype]
+    # a view whose rows start at odd element offsets: 16-byte accesses that are only element-aligned
+    big = rand(rng, (64, 131), dtype)
+    got, ref = _permute_check(tf, oracle, big[:, 1:129], (1, 0))
+    assert got.tobytes() == ref.tobytes()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex128])
+def test_permute_large_ragged_tensors_split_into_interior_and_border(tf, oracle, dtype):
+    # more than 2^20 elements with extents just off the tile grid: whole tiles go through the fast path, the border
+    # slabs are copied separately; every element must be written exactly once
+    rng = np.random.default_rng(50)
+    for shape, perm in [((1030, 1100), (1, 0)), ((101, 103, 107), (2, 0, 1)), ((65, 129, 131), (1, 2, 0)), ((3, 1025, 515), (2, 1, 0))]:
+        a = rand(rng, shape, dtype)
+        got, ref = _permute_check(tf, oracle, a, perm)
+        assert got.tobytes() == ref.tobytes(), (shape, perm)
+    a = rand(rng, (1030, 1100), dtype)
+    b0 = rand(rng, (1100, 1030), dtype)
+    alpha, beta = (0.5 - 2j, 1.5 + 1j) if np.issubdtype(dtype, np.complexfloating) else (0.5, -1.5)
+    got, ref = _permute_check(tf, oracle, a, (1, 0), alpha, beta, b0)
+    assert relerr(got, ref) < TOL[dtype]
+    v = rand(rng, (1200, 1300), dtype)[7:1037, 3:1103]          # strided view in, strided view out is covered by dev()
+    got, ref = _permute_check(tf, oracle, v, (1, 0))
+    assert got.tobytes() == ref.tobytes()
