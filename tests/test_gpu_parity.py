@@ -728,3 +728,97 @@ def test_permute_large_ragged_tensors_split_into_interior_and_border(tf, oracle,
     v = rand(rng, (1200, 1300), dtype)[7:1037, 3:1103]          # strided view in, strided view out is covered by dev()
     got, ref = _permute_check(tf, oracle, v, (1, 0))
     assert got.tobytes() == ref.tobytes()
+
+
+def _random_contraction(rng, big):
+    """Random binary contraction: labels split into batch / free-A / free-B / contracted groups, random extents,
+    operands stored in a random axis order and seen through random strided (possibly reversed) views."""
+    labels = list("abcdefgh")
+    rng.shuffle(labels)
+    nb, nm, nn, nk = rng.integers(0, 2), rng.integers(0, 3), rng.integers(0, 3), rng.integers(0, 3)
+    groups, pos = [], 0
+    for cnt in (nb, nm, nn, nk):
+        groups.append(labels[pos:pos + cnt])
+        pos += cnt
+    batch, fm, fn, kk = groups
+    top = 150 if big else 12
+    ext = {l: int(rng.integers(1, top + 1)) for l in labels[:pos]}
+    if big:   # keep the work bounded: at most two large extents per group product
+        for grp in (batch, fm, fn, kk):
+            for l in grp[1:]:
+                ext[l] = int(rng.integers(1, 7))
+        for l in batch:
+            ext[l] = int(rng.integers(1, 4))
+    ma = batch + fm + kk
+    mb = batch + kk + fn
+    mc = batch + fm + fn
+    rng.shuffle(ma); rng.shuffle(mb); rng.shuffle(mc)
+    return "".join(ma), "".join(mb), "".join(mc), ext
+
+
+def _random_view(rng, shape, dtype):
+    """A tensor of the given shape seen through a random view of a larger buffer (steps 1, 2 or -1, offsets)."""
+    steps = [int(rng.choice([1, 1, 1, 2, -1])) for _ in shape]
+    pads = [int(rng.integers(0, 3)) for _ in shape]
+    big_shape = [n * abs(st) + p for n, st, p in zip(shape, steps, pads)]
+    big = rand(rng, big_shape, dtype)
+    idx = []
+    for n, st, p in zip(shape, steps, pads):
+        lo = int(rng.integers(0, p + 1))
+        if st > 0:
+            idx.append(slice(lo, lo + n * st, st))
+        else:
+            idx.append(slice(lo + n - 1, lo - 1 if lo > 0 else None, -1))
+    v = big[tuple(idx)]
+    assert list(v.shape) == list(shape)
+    return v
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("big", [False, True], ids=["small", "large"])
+def test_contract_random_label_patterns_and_views(tf, oracle, dtype, big):
+    rng = np.random.default_rng(51 + (7 if big else 0))
+    for case in range(25 if big else 40):
+        ma, mb, mc, ext = _random_contraction(rng, big)
+        while not ma or not mb:   # rank-0 operands are not views of anything
+            ma, mb, mc, ext = _random_contraction(rng, big)
+        a = _random_view(rng, [ext[l] for l in ma], dtype)
+        b = _random_view(rng, [ext[l] for l in mb], dtype)
+        cshape = [ext[l] for l in mc]
+        use_beta = bool(rng.integers(0, 2)) and len(cshape) > 0
+        alpha, beta = (0.7 - 1.1j, (-0.3 + 0.2j) if use_beta else 0.0) if np.issubdtype(dtype, np.complexfloating) else (0.7, -0.3 if use_beta else 0.0)
+        c0 = rand(rng, cshape, dtype) if use_beta else np.full(cshape, np.nan, dtype)
+        ref = c0.copy()
+        oracle.contract(a, lab(ma), b, lab(mb), ref, lab(mc), alpha=alpha, beta=beta)
+        out = dev(tf, c0) if cshape else tf.Tensor.empty([], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [a.shape, b.shape, cshape])
+        tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, out)
+        err = relerr(out.to_numpy(), ref)
+        assert err < TOL[dtype], (case, ma, mb, mc, ext, err)
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_permute_and_reduce_random_shapes_and_views(tf, oracle, dtype):
+    rng = np.random.default_rng(52)
+    for case in range(30):
+        rank = int(rng.integers(1, 6))
+        shape = [int(rng.integers(1, 24)) for _ in range(rank)]
+        if case % 5 == 0:
+            shape[int(rng.integers(0, rank))] = int(rng.integers(100, 400))
+        a = _random_view(rng, shape, dtype)
+        modes = list(range(rank))
+        perm = [int(p) for p in rng.permutation(rank)]
+        ref = np.empty([shape[p] for p in perm], dtype)
+        oracle.permute(a, modes, ref, perm)
+        out = tf.Tensor.empty([shape[p] for p in perm], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Permute(modes, perm), [shape, [shape[p] for p in perm]])
+        tf.HipBackend.execute(plan, 1.0, [dev(tf, a)], 0.0, out)
+        assert out.to_numpy().tobytes() == ref.tobytes(), (case, shape, perm)
+        keep = [m for m in perm if rng.integers(0, 2)]
+        kshape = [shape[m] for m in keep]
+        rref = np.empty(kshape, dtype)
+        oracle.reduce(a, modes, rref, keep)
+        rout = tf.Tensor.empty(kshape, tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        rplan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Reduce(modes, keep, tf.ReduceOp.Sum), [shape, kshape])
+        tf.HipBackend.execute(rplan, 1.0, [dev(tf, a)], 0.0, rout)
+        assert relerr(rout.to_numpy(), rref) < 20 * TOL[dtype], (case, shape, keep)
