@@ -822,3 +822,68 @@ def test_permute_and_reduce_random_shapes_and_views(tf, oracle, dtype):
         rplan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Reduce(modes, keep, tf.ReduceOp.Sum), [shape, kshape])
         tf.HipBackend.execute(rplan, 1.0, [dev(tf, a)], 0.0, rout)
         assert relerr(rout.to_numpy(), rref) < 20 * TOL[dtype], (case, shape, keep)
+
+
+def test_calls_are_capturable_in_a_hip_graph_and_replay_correctly(tf, oracle):
+    # After one eager pass on the capture stream (which sizes the per-stream workspace and the intermediate pool), the
+    # calls allocate nothing and synchronise nothing: a contraction with operand packing, offset tables and split-K, a
+    # permute, a reduction and a three-operand einsum are captured into one graph and replayed on new input contents,
+    # with eager work and synchronisation between the replays; every replay must equal the eager result.
+    import torch
+    rng = np.random.default_rng(53)
+    ext = dict(a=8, j=32, b=16, k=48, c=64)
+    A = rand(rng, [ext[l] for l in "ajbk"], np.float64)
+    B = rand(rng, [ext[l] for l in "kcj"], np.float64)
+    X = rand(rng, (16, 12, 20, 8), np.float64)
+    E1, E2, E3 = rand(rng, (24, 30), np.complex128), rand(rng, (30, 18), np.complex128), rand(rng, (18, 40), np.complex128)
+    tA, tB, tX = (torch.from_numpy(x).cuda() for x in (A, B, X))
+    tE = [torch.from_numpy(x).cuda() for x in (E1, E2, E3)]
+    dA, dB, dX = tf.Tensor.from_torch(tA), tf.Tensor.from_torch(tB), tf.Tensor.from_torch(tX)
+    dE = [tf.Tensor.from_torch(t) for t in tE]
+    gpu0 = tf.GpuMemory(0)
+    oC = tf.Tensor.empty([8, 16, 64], gpu0, tf.MemoryOrder.RowMajor, np.float64)
+    oP = tf.Tensor.empty([8, 16, 20, 12], gpu0, tf.MemoryOrder.RowMajor, np.float64)
+    oR = tf.Tensor.empty([12, 8], gpu0, tf.MemoryOrder.RowMajor, np.float64)
+    oE = tf.Tensor.empty([24, 40], gpu0, tf.MemoryOrder.RowMajor, np.complex128)
+    pc = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Contract(lab("ajbk"), lab("kcj"), lab("abc")), [A.shape, B.shape, [8, 16, 64]])
+    pp = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute([0, 1, 2, 3], [3, 0, 2, 1]), [X.shape, [8, 16, 20, 12]])
+    pr = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Reduce([0, 1, 2, 3], [1, 3], tf.ReduceOp.Sum), [X.shape, [12, 8]])
+    subs = tf.Subscripts.parse("ij,jk,kl->il")
+    tree = tf.ContractionTree.optimize(subs, [E1.shape, E2.shape, E3.shape])
+
+    def work():
+        tf.HipBackend.execute(pc, 1.0, [dA, dB], 0.0, oC)
+        tf.HipBackend.execute(pp, 1.0, [dX], 0.0, oP)
+        tf.HipBackend.execute(pr, 1.0, [dX], 0.0, oR)
+        tf.einsum_with_plan_into(tree, dE, 1.0, 0.0, oE)
+
+    def expected():
+        c = np.empty((8, 16, 64)); oracle.contract(tA.cpu().numpy(), lab("ajbk"), tB.cpu().numpy(), lab("kcj"), c, lab("abc"))
+        x = tX.cpu().numpy()
+        p = np.empty((8, 16, 20, 12)); oracle.permute(x, [0, 1, 2, 3], p, [3, 0, 2, 1])
+        r = np.empty((12, 8)); oracle.reduce(x, [0, 1, 2, 3], r, [1, 3])
+        e = np.empty((24, 40), np.complex128)
+        oracle.einsum_pairs([t.cpu().numpy() for t in tE], [lab("ij"), lab("jk"), lab("kl")], e, lab("il"), tree.steps)
+        return c, p, r, e
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()                                    # eager pass on the capture stream
+    side.synchronize()
+    for t in (oC, oP, oR, oE):
+        t.event = None                            # completed; an event recorded outside the capture must not be waited on inside it
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        work()
+    for replay in range(3):
+        for t in [tA, tB, tX] + tE:               # new contents, same buffers
+            t.mul_(-0.5).add_(0.25 * (replay + 1))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        c, p, r, e = expected()
+        assert relerr(oC.to_numpy(), c) < 1e-12, replay
+        assert oP.to_numpy().tobytes() == p.tobytes(), replay
+        assert relerr(oR.to_numpy(), r) < 1e-12, replay
+        assert relerr(oE.to_numpy(), e) < 1e-12, replay
