@@ -93,6 +93,8 @@ static void host_checks() {
     CHECK(a.reshape({6, 4}).strides() == (std::vector<ptrdiff_t>{4, 1}));
     CHECK(raises(Error::Kind::ShapeMismatch, [&] { a.reshape({5, 5}); }));
     CHECK(raises(Error::Kind::InvalidArgument, [&] { ap.reshape({24}); }));
+    // column-major from_slice([1..6], [2,3]) is [[1,3,5],[2,4,6]] (tenferro-tensor/src/lib.rs:34-39)
+    CHECK(Tensor<double>::from_slice({1, 2, 3, 4, 5, 6}, {2, 3}, MemoryOrder::ColumnMajor).to_vec() == (std::vector<double>{1, 3, 5, 2, 4, 6}));
     auto col = Tensor<double>::from_slice(data, {2, 3, 4}, MemoryOrder::ColumnMajor);
     CHECK(col.strides() == (std::vector<ptrdiff_t>{1, 2, 6}) && col.is_contiguous());
     auto sq = Tensor<double>::from_slice(std::vector<double>(data.begin(), data.begin() + 9), {3, 3}, MemoryOrder::RowMajor);
