@@ -425,6 +425,16 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
         __syncthreads();
         int64_t s = 0;
         for (; s + 2 < nstage; ++s) {
+            // Two blocks share a CU.  The arbiter favours the older wave, so one block runs ahead and the other is
+            // left to finish alone; lowering a block's issue priority as it progresses keeps the one that is behind
+            // ahead in the arbitration, and the two finish together (a launch of exactly one wave of blocks gains ~2%).
+            if ((s & 3) == 0) {
+                const int q = (int)((4 * s) / nstage);
+                if (q == 0) __builtin_amdgcn_s_setprio(3);
+                else if (q == 1) __builtin_amdgcn_s_setprio(2);
+                else if (q == 2) __builtin_amdgcn_s_setprio(1);
+                else __builtin_amdgcn_s_setprio(0);
+            }
             stage_interleaved((int)(s & 1), ktab, kbeg + (s + 2) * BKE);
             __syncthreads();
         }
