@@ -290,6 +290,8 @@ public:
         return preferred_compute_devices(space_, op);
     }
     ptrdiff_t offset() const { return offset_; }
+    // true when no other tensor (a permute/broadcast/diagonal view, a copy) shares this tensor's buffer
+    bool sole_owner() const { return buf_ && buf_.use_count() == 1; }
 
     // ---- views (:445-460): device views; waits for a pending transfer first
     StridedView<T> view() const {
@@ -626,8 +628,10 @@ Tensor<T> einsum_with_plan_owned(const ContractionTree& tree, std::vector<Tensor
     auto ptrs = detail::pointers(operands);
     const LogicalMemorySpace s = detail::common_space(ptrs);
     Tensor<T> out = Tensor<T>::uninit(tree.output_dims(), s, MemoryOrder::RowMajor);
-    const uint64_t all = operands.size() >= 64 ? ~0ull : ((1ull << operands.size()) - 1);
-    detail::run_tree(tree, ptrs, T(1), T(0), out, all);
+    uint64_t donate = 0;   // only buffers nobody else can see may be overwritten
+    for (size_t i = 0; i < operands.size() && i < 64; ++i)
+        if (operands[i].sole_owner()) donate |= 1ull << i;
+    detail::run_tree(tree, ptrs, T(1), T(0), out, donate);
     out.wait();   // the operands are released when this function returns
     return out;
 }

@@ -208,7 +208,9 @@ double tfh_tree_peak_intermediate(const tfh_tree* t);
  * `stream`; intermediates stay in device memory; the host never waits.  The allocating and
  * string/subscript variants (:393-498, :541-582) are this call behind tfh_subscripts_parse,
  * tfh_tree_optimize and an output buffer sized with tfh_tree_output_dims.
- * donate_mask: bit i set = operand i's buffer may be overwritten (the *_owned variants, :436-498). */
+ * donate_mask: bit i set = operand i's buffer may be overwritten (the *_owned variants, :436-498):
+ * a dense operand that overlaps no other operand nor the output may hold an intermediate of a
+ * step later than the one that reads it.  Its contents after the call are unspecified. */
 int32_t tfh_einsum_execute(int32_t dtype, const tfh_tree* tree,
                            const tfh_view* operands, int32_t n_operands,
                            const void* alpha, const void* beta, tfh_view* output,

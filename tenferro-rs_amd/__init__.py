@@ -581,6 +581,12 @@ class Tensor:
         self._buf, self._dims, self._strides, self._offset = buffer, list(dims), list(strides), int(offset)
         self.logical_memory_space_, self.dtype, self.event = space, dtype, event
         self.preferred_compute_device_ = preferred
+        self._lib_alloc = False     # the buffer was allocated by this module (not wrapped from the caller's tensor)
+
+    def _sole_owner(self):
+        """No other Tensor (a permute/broadcast/diagonal view) and no caller-held object shares the buffer."""
+        import sys
+        return self._lib_alloc and sys.getrefcount(self._buf) <= 2      # the attribute + getrefcount's argument
 
     # ---- constructors (:336-371)
     @classmethod
@@ -595,6 +601,7 @@ class Tensor:
         tdt = {F32: torch.float32, F64: torch.float64, C64: torch.complex64, C128: torch.complex128}[dt]
         buf = torch.empty(max(n, 1), dtype=tdt, device=f"cuda:{space.space_id}")
         t = cls(buf, dims, _contig_strides(dims, order), 0, space, dt)
+        t._lib_alloc = True
         if fill is not None:
             v = t._view()
             st = current_stream()
@@ -664,8 +671,10 @@ class Tensor:
 
     # ---- views (:502-542): metadata only, shared buffer
     def _like(self, dims, strides, offset=None):
-        return Tensor(self._buf, dims, strides, self._offset if offset is None else offset, self.logical_memory_space_,
-                      self.dtype, self.event, self.preferred_compute_device_)
+        t = Tensor(self._buf, dims, strides, self._offset if offset is None else offset, self.logical_memory_space_,
+                   self.dtype, self.event, self.preferred_compute_device_)
+        t._lib_alloc = self._lib_alloc
+        return t
 
     def permute(self, perm):
         if sorted(perm) != list(range(self.ndim())):
@@ -767,7 +776,9 @@ class Tensor:
         import torch
         if target.kind == 1:
             buf = torch.from_numpy(np.ascontiguousarray(self._buf)).to(f"cuda:{target.space_id}", non_blocking=True)
-            return Tensor(buf, self._dims, self._strides, self._offset, target, self.dtype, CompletionEvent(current_stream()))
+            t = Tensor(buf, self._dims, self._strides, self._offset, target, self.dtype, CompletionEvent(current_stream()))
+            t._lib_alloc = True
+            return t
         self.wait()
         return Tensor(self._buf.cpu().numpy(), self._dims, self._strides, self._offset, target, self.dtype)
 
@@ -822,11 +833,11 @@ def einsum_with_plan_into(tree, operands, alpha, beta, output, stream=None, _don
     output.event = CompletionEvent(st)
 
 
-def einsum_with_plan(tree, operands, stream=None):
+def einsum_with_plan(tree, operands, stream=None, _donate=0):
     """:412-430"""
     space = _dispatch_check(operands)
     out = Tensor.empty(tree.output_dims, space, MemoryOrder.ColumnMajor, operands[0].dtype)
-    einsum_with_plan_into(tree, operands, 1.0, 0.0, out, stream)
+    einsum_with_plan_into(tree, operands, 1.0, 0.0, out, stream, _donate)
     return out
 
 
@@ -854,8 +865,10 @@ def einsum_into(subscripts, operands, alpha, beta, output, stream=None):
 
 
 def einsum_with_plan_owned(tree, operands, stream=None):
-    """:493-498: operands are consumed; their buffers are released once the kernels are enqueued."""
-    out = einsum_with_plan(tree, operands, stream)
+    """:493-498: operands are consumed: the executor may keep intermediates in the buffers that no other tensor
+    shares, and they are released once the kernels are enqueued."""
+    donate = sum(1 << i for i, t in enumerate(operands[:64]) if t._sole_owner())
+    out = einsum_with_plan(tree, operands, stream, donate)
     operands.clear() if isinstance(operands, list) else None
     return out
 

@@ -608,7 +608,6 @@ int32_t reduce_or_copy(int dtype, const Operand& src, const Operand& dst, Scalar
 
 int32_t tfh_einsum_execute(int32_t dtype, const tfh_tree* tree, const tfh_view* operands, int32_t n_operands,
                            const void* alpha, const void* beta, tfh_view* output, uint64_t donate_mask, tfh_stream stream) {
-    (void)donate_mask;   // operands are never overwritten; owned variants simply release their buffers afterwards
     if (!tree || !alpha || !beta || !output || (n_operands > 0 && !operands)) return set_error(TFH_ERR_INVALID_ARGUMENT, "null argument");
     if (dtype < TFH_F32 || dtype > TFH_C128) return set_error(TFH_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
     const tfh_tree& t = *tree;
@@ -680,6 +679,58 @@ int32_t tfh_einsum_execute(int32_t dtype, const tfh_tree* tree, const tfh_view* 
         return e;
     }
     const int ns = (int)t.steps.size();
+    // Donated operands (the *_owned variants, tenferro-einsum/src/lib.rs:436-498): once the step that consumes one
+    // has been enqueued, its buffer is dead and may hold a later intermediate.  Only a dense view qualifies (its
+    // elements occupy one contiguous block), and the kernels that read it precede the writer on the same stream.
+    struct Donated { char* ptr; size_t bytes; int consumed_at; bool used; };
+    std::vector<Donated> donated;
+    for (int i = 0; i < n_operands && i < 64; ++i) {
+        if (!((donate_mask >> i) & 1)) continue;
+        const tfh_view& v = operands[i];
+        std::vector<std::pair<int64_t, int64_t>> ax;   // (|stride|, extent) of the non-trivial axes
+        bool dense = true;
+        int64_t count = 1;
+        for (int d = 0; d < v.rank; ++d) {
+            count *= v.dims[d];
+            if (v.dims[d] > 1) {
+                if (v.strides[d] <= 0) dense = false;
+                ax.emplace_back(v.strides[d], v.dims[d]);
+            }
+        }
+        std::sort(ax.begin(), ax.end());
+        int64_t expect = 1;
+        for (auto& a : ax) {
+            if (a.first != expect) dense = false;
+            expect *= a.second;
+        }
+        if (!dense || count == 0) continue;
+        int consumed = -1;
+        for (int s = 0; s < ns; ++s)
+            if (t.steps[s].lhs == i || t.steps[s].rhs == i) consumed = s;
+        if (consumed < 0) continue;
+        // the block must be this operand's alone: no other operand and not the output may reach into it
+        auto range = [&](const tfh_view& w, const char*& lo, const char*& hi) {
+            int64_t a = 0, b = 0;
+            for (int d = 0; d < w.rank; ++d) {
+                if (w.dims[d] <= 1) continue;
+                const int64_t e = (w.dims[d] - 1) * w.strides[d];
+                (e < 0 ? a : b) += e;
+            }
+            lo = view_ptr(w, dtype) + a * (int64_t)eb;
+            hi = view_ptr(w, dtype) + (b + 1) * (int64_t)eb;
+        };
+        const char* lo = view_ptr(v, dtype);
+        const char* hi = lo + (size_t)count * eb;
+        bool alone = true;
+        for (int j = 0; j <= n_operands && alone; ++j) {
+            if (j == i) continue;
+            const char *l2, *h2;
+            range(j < n_operands ? operands[j] : *output, l2, h2);
+            if (l2 < hi && lo < h2) alone = false;
+        }
+        if (!alone) continue;
+        donated.push_back(Donated{view_ptr(v, dtype), (size_t)count * eb, consumed, false});
+    }
     for (int s = 0; s < ns; ++s) {
         const bool last = s == ns - 1;
         const Operand& A = nodes[t.steps[s].lhs];
@@ -697,13 +748,22 @@ int32_t tfh_einsum_execute(int32_t dtype, const tfh_tree* tree, const tfh_view* 
                 C.strides[d] = n;
                 n *= C.dims[d];
             }
-            void* p = nullptr;
-            if (int32_t e = pool_alloc(stream, (size_t)std::max<int64_t>(n, 1) * eb, &p)) {
-                release_all();
-                return e;
+            const size_t need = (size_t)std::max<int64_t>(n, 1) * eb;
+            Donated* reuse = nullptr;
+            for (auto& dn : donated)   // smallest donated buffer that fits and whose reader is already enqueued
+                if (!dn.used && dn.consumed_at < s && dn.bytes >= need && (!reuse || dn.bytes < reuse->bytes)) reuse = &dn;
+            if (reuse) {
+                reuse->used = true;
+                C.ptr = reuse->ptr;
+            } else {
+                void* p = nullptr;
+                if (int32_t e = pool_alloc(stream, need, &p)) {
+                    release_all();
+                    return e;
+                }
+                C.ptr = (char*)p;
+                C.owned = p;
             }
-            C.ptr = (char*)p;
-            C.owned = p;
         }
         ContractAxes ax;
         int32_t e = classify_contract(A.labels, A.dims.data(), A.strides.data(), B.labels, B.dims.data(), B.strides.data(), C.labels,

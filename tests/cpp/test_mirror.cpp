@@ -142,6 +142,29 @@ static void gpu_checks() {
     CHECK(rel_frobenius(einsum_with_plan<double>(tree, {&A, &B}).to_vec(), ref) < 1e-12);
     CHECK(rel_frobenius(einsum_with_subscripts<double>(subs, {&A, &B}).to_vec(), ref) < 1e-12);
     CHECK(rel_frobenius(einsum_owned<double>("ij,jk->ik", {A, B}).to_vec(), ref) < 1e-12);
+    // the copies handed over above share A's and B's buffers, so nothing was donated and both are intact
+    CHECK(A.to_vec() == ha && B.to_vec() == hb);
+    {   // a chain whose operands are moved in: each is the sole owner of its buffer, which may then hold an intermediate
+        auto mm = [n](const std::vector<double>& x, const std::vector<double>& y) {
+            std::vector<double> z(n * n, 0.0);
+            for (size_t i = 0; i < n; ++i)
+                for (size_t k = 0; k < n; ++k)
+                    for (size_t j = 0; j < n; ++j) z[i * n + j] += x[i * n + k] * y[k * n + j];
+            return z;
+        };
+        std::vector<Tensor<double>> ops;
+        for (int r = 0; r < 4; ++r)
+            ops.push_back(Tensor<double>::from_slice(r % 2 ? hb : ha, {n, n}, MemoryOrder::RowMajor).to_memory_space_async(gpu));
+        CHECK(ops[0].sole_owner() && ops[3].sole_owner());
+        auto keep = ops[1].permute({1, 0});          // shares operand 1's buffer: that one must survive
+        CHECK(!ops[1].sole_owner());
+        auto chain = einsum_owned<double>("ij,jk,kl,lm->im", std::move(ops));
+        CHECK(rel_frobenius(chain.to_vec(), mm(mm(mm(ha, hb), ha), hb)) < 1e-12);
+        std::vector<double> hbt(n * n);
+        for (size_t i = 0; i < n; ++i)
+            for (size_t j = 0; j < n; ++j) hbt[j * n + i] = hb[i * n + j];
+        CHECK(keep.to_vec() == hbt);
+    }
 
     // three operands with an explicit pairwise order, complex128, one operand conjugated (Tensor::conj, :622-651)
     {

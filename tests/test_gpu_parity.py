@@ -887,3 +887,61 @@ def test_calls_are_capturable_in_a_hip_graph_and_replay_correctly(tf, oracle):
         assert oP.to_numpy().tobytes() == p.tobytes(), replay
         assert relerr(oR.to_numpy(), r) < 1e-12, replay
         assert relerr(oE.to_numpy(), e) < 1e-12, replay
+
+
+def test_owned_variant_keeps_intermediates_in_donated_operand_buffers(tf, oracle):
+    # einsum_with_plan_owned (tenferro-einsum/src/lib.rs:493-498): the operands are consumed, so an intermediate that fits
+    # may live in the buffer of an operand whose step is already enqueued.  The result is unchanged; a donated buffer
+    # ends up overwritten; the borrowing variant leaves its operands intact; a buffer that another tensor shares, or
+    # that the caller wrapped from their own torch tensor, is never written.
+    import torch
+    rng = np.random.default_rng(54)
+    host = [rand(rng, (64, 64), np.float64) for _ in range(4)]
+    subs = tf.Subscripts.parse("ij,jk,kl,lm->im")
+    tree = tf.ContractionTree.from_pairs(subs, [h.shape for h in host], [(0, 1), (4, 2), (5, 3)])
+    ref = np.empty((64, 64))
+    oracle.einsum_pairs(host, [lab(t) for t in ("ij", "jk", "kl", "lm")], ref, lab("im"), tree.steps)
+
+    def upload():
+        return [tf.Tensor.from_slice(h, h.shape, tf.MemoryOrder.RowMajor).to_memory_space_async(tf.GpuMemory(0)) for h in host]
+
+    ops = upload()
+    out = tf.einsum_with_plan(tree, ops)
+    assert relerr(out.to_numpy(), ref) < 1e-12
+    assert all(np.array_equal(o.to_numpy(), h) for o, h in zip(ops, host))               # borrowed: untouched
+
+    # the test's own window onto the memory: the raw device addresses (the blocks stay mapped in torch's caching
+    # allocator after the tensors are dropped)
+    addrs = [o._buf.data_ptr() for o in ops]
+    assert all(o._sole_owner() for o in ops)
+    out2 = tf.einsum_with_plan_owned(tree, ops)
+    assert ops == []                                                                     # consumed
+    assert relerr(out2.to_numpy(), ref) < 1e-12
+    torch.cuda.synchronize()
+    after = [np.empty_like(h) for h in host]
+    for a, dst in zip(addrs, after):
+        assert tf.lib().tfh_memcpy_d2h(dst.ctypes.data, a, dst.nbytes, None) == 0
+    torch.cuda.synchronize()
+    assert any(not np.array_equal(a, h) for a, h in zip(after, host))                    # one holds an intermediate
+
+    # shared buffers: a permuted view of operand 0 is alive, so operand 0 is not donated; the others still are
+    ops = upload()
+    keep = ops[0].permute([1, 0])
+    assert not ops[0]._sole_owner() and ops[1]._sole_owner()
+    out3 = tf.einsum_with_plan_owned(tree, ops)
+    assert relerr(out3.to_numpy(), ref) < 1e-12
+    assert np.array_equal(keep.to_numpy(), host[0].T)
+
+    # caller-owned torch memory is never donated
+    bufs = [torch.from_numpy(h).cuda() for h in host]
+    out4 = tf.einsum_with_plan_owned(tree, [tf.Tensor.from_torch(b) for b in bufs])
+    assert relerr(out4.to_numpy(), ref) < 1e-12
+    assert all(np.array_equal(b.cpu().numpy(), h) for b, h in zip(bufs, host))
+
+    # the raw C entry point with every bit set and one buffer given as all four operands: overlap is detected
+    sq = torch.from_numpy(host[0]).cuda()
+    same = [tf.Tensor.from_torch(sq)] * 4
+    ref4 = host[0] @ host[0] @ host[0] @ host[0]
+    out5 = tf.einsum_with_plan(tree, same, None, 0xF)
+    assert relerr(out5.to_numpy(), ref4) < 1e-12
+    assert np.array_equal(sq.cpu().numpy(), host[0])
