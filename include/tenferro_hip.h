@@ -264,7 +264,7 @@ int32_t tfh_stream_wait_event(tfh_stream s, tfh_event e);  /* chaining without a
 int32_t tfh_profile_enable(int32_t on);
 int32_t tfh_profile_collect(int32_t kind, double* total_ms, int32_t* launches);
 
-/* Releases the cached workspace and intermediate buffers of every stream (after a synchronize). */
+/* Releases the cached workspace, intermediate buffers and offset tables of every stream (after a synchronize). */
 int32_t tfh_release_workspaces(void);
 
 #ifdef __cplusplus

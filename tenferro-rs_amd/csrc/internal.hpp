@@ -117,6 +117,12 @@ void grouped_state_destroy(GroupedState* g);
 // Workspace: one growing buffer per stream; kernels on a stream are ordered, so successive calls
 // reuse it.  Valid until the next workspace() call on the same stream.
 int32_t workspace(void* stream, size_t bytes, void** out);
+// Offset tables of a contraction depend only on the fused dims and strides (`key`): the first call on a stream
+// builds them with a kernel into a block that later calls on that stream reuse without a launch (stream order
+// makes them ready).  *tables == nullptr: no cached block (cache full, stream being captured, entry being built by
+// another thread) -- build them in the workspace.  *fresh: the caller fills the block, then calls commit.
+int32_t table_cache_get(void* stream, const std::string& key, size_t bytes, void** tables, bool* fresh);
+void table_cache_commit(void* stream, const std::string& key);
 // Intermediates of an einsum tree: stream-ordered cached allocations (free returns the block to the
 // stream's cache; reuse on the same stream needs no synchronisation).
 int32_t pool_alloc(void* stream, size_t bytes, void** out);

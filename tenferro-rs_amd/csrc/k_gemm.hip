@@ -593,63 +593,91 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     for (auto& w : wants32)
         if (need32(w)) table_bytes += ((size_t)w.n * sizeof(uint32_t) + 255) & ~(size_t)255;
     size_t partial_bytes = nsplit > 1 ? (size_t)nsplit * nb * M * NR * rb : 0;
-    char* ws = nullptr;
-    if (table_bytes + partial_bytes) {
-        void* p = nullptr;
-        if (int32_t e = workspace(stream, table_bytes + partial_bytes, &p)) {
-            release_packed();
-            return e;
-        }
-        ws = (char*)p;
-    }
+    // The jobs first, with offsets in place of addresses: their dims and strides are the key under which the finished
+    // tables are kept for later calls on this stream.
     size_t cursor = 0;
     TableJobs jobs;
     std::memset(&jobs, 0, sizeof jobs);
     int njobs = 0, naxes = 0;
     int64_t longest = 0;
+    std::string key;
     auto add_job = [&](const std::vector<Axis>& grp, int slot, int64_t n, int elem_bytes, size_t entry) {
         TableJobs::Job& j = jobs.job[njobs++];
-        j.dst = ws + cursor;
+        const size_t at = cursor;
         j.n = n;
         j.first_axis = naxes;
         j.naxes = (int32_t)grp.size();
         j.elem_bytes = elem_bytes;
         j.pad = 0;
+        const int64_t head[3] = {n, (int64_t)grp.size(), elem_bytes};
+        key.append((const char*)head, sizeof head);
         for (auto& x : grp) {
             jobs.dims[naxes] = x.n;
             jobs.strides[naxes++] = x.s[slot];
+            const int64_t ds[2] = {x.n, x.s[slot]};
+            key.append((const char*)ds, sizeof ds);
         }
         longest = std::max(longest, n);
         cursor += ((size_t)n * entry + 255) & ~(size_t)255;
-        return j.dst;
+        return at;
     };
-    for (auto& w : wants) {
+    size_t at64[9], at32[4];
+    for (int i = 0; i < 9; ++i)
+        if (need64(wants[i])) at64[i] = add_job(*wants[i].grp, wants[i].slot, wants[i].n, 0, sizeof(int64_t));
+    for (int i = 0; i < 4; ++i)
+        if (need32(wants32[i])) at32[i] = add_job(*wants32[i].grp, wants32[i].slot, wants32[i].n, (int)eb, sizeof(uint32_t));
+    void* cached = nullptr;
+    bool fresh = false;
+    if (njobs)
+        if (int32_t e = table_cache_get(stream, key, table_bytes, &cached, &fresh)) {
+            release_packed();
+            return e;
+        }
+    char* ws = nullptr;
+    const size_t ws_bytes = (cached ? 0 : table_bytes) + partial_bytes;
+    if (ws_bytes) {
+        void* p = nullptr;
+        if (int32_t e = workspace(stream, ws_bytes, &p)) {
+            release_packed();
+            return e;
+        }
+        ws = (char*)p;
+    }
+    char* tables = cached ? (char*)cached : ws;
+    int jn = 0;
+    for (int i = 0; i < 9; ++i) {
+        Want& w = wants[i];
         if (need64(w)) {
-            w.fn->tab = (const int64_t*)add_job(*w.grp, w.slot, w.n, 0, sizeof(int64_t));
+            jobs.job[jn++].dst = tables + at64[i];
+            w.fn->tab = (const int64_t*)(tables + at64[i]);
             w.fn->stride = 0;
         } else {
             w.fn->tab = nullptr;
             w.fn->stride = w.grp->size() == 1 ? (*w.grp)[0].s[w.slot] : 0;
         }
     }
-    for (auto& w : wants32) {
+    for (int i = 0; i < 4; ++i) {
+        Want32& w = wants32[i];
         if (need32(w)) {
-            w.fn->tab = (const uint32_t*)add_job(*w.grp, w.slot, w.n, (int)eb, sizeof(uint32_t));
+            jobs.job[jn++].dst = tables + at32[i];
+            w.fn->tab = (const uint32_t*)(tables + at32[i]);
             w.fn->stride = 0;
         } else {
             w.fn->tab = nullptr;
             w.fn->stride = w.grp->size() == 1 ? (uint32_t)((*w.grp)[0].s[w.slot] * (int64_t)eb) : 0u;
         }
     }
-    if (njobs)
+    if (njobs && (!cached || fresh)) {
         hipLaunchKernelGGL(build_tables_kernel, dim3((uint32_t)((longest + THREADS - 1) / THREADS), (uint32_t)njobs), dim3(THREADS), 0, st, jobs);
+        if (fresh) table_cache_commit(stream, key);
+    }
     if (use128) {
         g.A32 = (const char*)a + lo_a * (int64_t)eb;
         g.B32 = (const char*)b + lo_b * (int64_t)eb;
         g.bias_a32 = (uint32_t)(-lo_a * (int64_t)eb);
         g.bias_b32 = (uint32_t)(-lo_b * (int64_t)eb);
     }
-    if (nsplit > 1) g.partial = ws + cursor;
+    if (nsplit > 1) g.partial = ws + (cached ? 0 : table_bytes);
     dim3 grid((uint32_t)(g.tiles_m * g.tiles_n), 1, (uint32_t)(nb * nsplit));
     const int prof = prof_begin(PROF_CONTRACT, stream);
     if (use128) launch_128(dtype, g, grid, st);

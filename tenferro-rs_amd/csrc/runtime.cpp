@@ -5,6 +5,7 @@
 
 #include <map>
 #include <mutex>
+#include <string>
 #include <vector>
 
 #include "internal.hpp"
@@ -22,7 +23,13 @@ struct StreamScratch {
     size_t ws_bytes = 0;
     std::multimap<size_t, void*> free_blocks;   // cached intermediates by size
     std::map<void*, size_t> live;
+    // offset tables of contractions already run on this stream, by the dims and strides they were built from
+    struct Tables { void* dev; size_t bytes; bool filled; };
+    std::map<std::string, Tables> tables;
+    size_t table_bytes = 0;
 };
+constexpr size_t TABLE_CACHE_BYTES = (size_t)64 << 20;   // per stream; beyond it tables go to the workspace again
+constexpr size_t TABLE_CACHE_ENTRIES = 256;
 std::mutex g_mu;
 std::map<std::pair<int, void*>, StreamScratch> g_scratch;   // (device, stream)
 
@@ -53,6 +60,47 @@ int32_t workspace(void* stream, size_t bytes, void** out) {
     }
     *out = s->ws;
     return TFH_OK;
+}
+
+int32_t table_cache_get(void* stream, const std::string& key, size_t bytes, void** tables, bool* fresh) {
+    *tables = nullptr;
+    *fresh = false;
+    std::lock_guard<std::mutex> lk(g_mu);
+    int32_t err;
+    StreamScratch* s = scratch_for(stream, &err);
+    if (!s) return err;
+    auto it = s->tables.find(key);
+    if (it != s->tables.end()) {
+        if (it->second.filled && it->second.bytes == bytes) *tables = it->second.dev;
+        return TFH_OK;
+    }
+    if (s->tables.size() >= TABLE_CACHE_ENTRIES || s->table_bytes + bytes > TABLE_CACHE_BYTES) return TFH_OK;
+    // no allocation while the stream is being captured into a graph: the call then builds its tables in the workspace
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess) {
+        (void)hipGetLastError();
+        return TFH_OK;
+    }
+    if (cs != hipStreamCaptureStatusNone) return TFH_OK;
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        (void)hipGetLastError();   // out of memory for the cache is not an error of the call
+        return TFH_OK;
+    }
+    s->tables[key] = StreamScratch::Tables{p, bytes, false};
+    s->table_bytes += bytes;
+    *tables = p;
+    *fresh = true;
+    return TFH_OK;
+}
+
+void table_cache_commit(void* stream, const std::string& key) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    int32_t err;
+    StreamScratch* s = scratch_for(stream, &err);
+    if (!s) return;
+    auto it = s->tables.find(key);
+    if (it != s->tables.end()) it->second.filled = true;
 }
 
 int32_t pool_alloc(void* stream, size_t bytes, void** out) {
@@ -191,6 +239,9 @@ int32_t tfh_release_workspaces(void) {
         kv.second.ws_bytes = 0;
         for (auto& b : kv.second.free_blocks) (void)hipFree(b.second);
         kv.second.free_blocks.clear();
+        for (auto& t : kv.second.tables) (void)hipFree(t.second.dev);
+        kv.second.tables.clear();
+        kv.second.table_bytes = 0;
     }
     return TFH_OK;
 }

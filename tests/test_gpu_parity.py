@@ -945,3 +945,29 @@ def test_owned_variant_keeps_intermediates_in_donated_operand_buffers(tf, oracle
     out5 = tf.einsum_with_plan(tree, same, None, 0xF)
     assert relerr(out5.to_numpy(), ref4) < 1e-12
     assert np.array_equal(sq.cpu().numpy(), host[0])
+
+
+def test_offset_tables_are_kept_per_layout_and_survive_a_release(tf, oracle):
+    # The offset tables of a multi-mode contraction are built once per (dims, strides) and stream and reused by later
+    # calls.  Two layouts of the same shapes alternate through one plan: each call must use its own layout's tables;
+    # releasing the library's scratch memory in between drops them and the next call builds them again.
+    rng = np.random.default_rng(77)
+    sa, sb, sc = (16, 40, 8, 24), (24, 130, 40), (16, 8, 130)                  # "ajbk,kcj->abc": 128x128 tiles
+    a1, b1 = rand(rng, sa, np.float64), rand(rng, sb, np.float64)
+    a2 = np.ascontiguousarray(rand(rng, (24, 8, 40, 16), np.float64)).transpose(3, 2, 1, 0)      # same dims, reversed strides
+    b2 = np.ascontiguousarray(rand(rng, (40, 130, 24), np.float64)).transpose(2, 1, 0)
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Contract(lab("ajbk"), lab("kcj"), lab("abc")), [sa, sb, sc])
+    pairs = [(a1, b1), (a2, b2), (a1, b2), (a2, b1)]
+    refs = []
+    for a, b in pairs:
+        r = np.empty(sc)
+        oracle.contract(a, lab("ajbk"), b, lab("kcj"), r, lab("abc"))
+        refs.append(r)
+    devs = [(dev(tf, a), dev(tf, b)) for a, b in pairs]
+    out = tf.Tensor.empty(list(sc), tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+    for rnd in range(3):
+        for (da, db), r in zip(devs, refs):
+            tf.HipBackend.execute(plan, 1.0, [da, db], 0.0, out)
+            assert relerr(out.to_numpy(), r) < 1e-12
+        if rnd == 1:
+            assert tf.lib().tfh_release_workspaces() == 0
