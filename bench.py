@@ -230,7 +230,7 @@ def run_c3(h):
         "peak_intermediate_bytes": tree.peak_intermediate * 16,
         "roofline": {"bound": "mfma", "achieved": flops / (total_kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
                      "frac": flops / (total_kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": TRAFFIC["c3"],
-                     "kernel": "gemm128_kernel<double, true, ..., 1, 1> x2 + gemm_kernel<double, true, 64, 64> x1 (the three pairwise contractions of the tree)",
+                     "kernel": "gemm128_kernel<double, true, ..., 1, 1> x2 + gemm_skinny_kernel<true> x1 (the three pairwise contractions of the tree)",
                      "kernel_ms": total_kms, "launches_per_step": per_step},
     }
     if h.cpu:

@@ -1,0 +1,34 @@
+// gemm_skinny.hpp -- argument block of the contraction kernel for a small left operand (k_gemm_skinny.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "gemm_common.hpp"
+
+namespace tfh {
+namespace gemm {
+
+constexpr int SKINNY_UNIT = 16;        // consecutive n (rows of B, columns of C) per work unit
+constexpr int SKINNY_MAX_M = 32;       // rows of A
+constexpr int SKINNY_MAX_KR = 64;      // real k per row of B (64 doubles = 32 chunks of 16 bytes)
+
+struct SkinnyArgs {
+    const void* A;
+    const void* B;
+    void* C;
+    int32_t M, K;            // rows of A, elements of k
+    int32_t kc;              // 16-byte chunks per row of B: K for complex128, K/2 for f64
+    int32_t conj_a, conj_b, use_beta, plain;   // plain: alpha == 1 and beta == 0
+    int64_t units;           // N / SKINNY_UNIT
+    OffFn am, ak, cm;        // element offsets of A's rows and k, of C's rows
+    OffFn bu, cu;            // element offset of a unit's first n in B and in C
+    int32_t b_in, c_in;      // element stride between consecutive n inside a unit, in B and in C
+    double alpha_re, alpha_im, beta_re, beta_im;
+};
+
+}  // namespace gemm
+
+// dtype is TFH_F64 or TFH_C128
+void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st);
+}  // namespace tfh

@@ -25,6 +25,7 @@
 #include <mutex>
 
 #include "gemm128.hpp"
+#include "gemm_skinny.hpp"
 #include "internal.hpp"
 
 namespace tfh {
@@ -525,6 +526,39 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     fuse_axes(ax.K, 3);
     fuse_axes(ax.batch, 3);
 
+    // A small left operand against a long n whose rows of B are contiguous in k: the streaming kernel of
+    // k_gemm_skinny.hip (work units of SKINNY_UNIT consecutive n; the n tables then hold one entry per unit).
+    const bool cxd = dtype == TFH_C128;
+    bool skinny = (dtype == TFH_F64 || cxd) && nb == 1 && M <= SKINNY_MAX_M && K * (cxd ? 2 : 1) <= SKINNY_MAX_KR && N >= 4096 &&
+                  b_kfast && !ax.K.empty() && k_by_b && !ax.N.empty() &&
+                  ax.N.back().n % SKINNY_UNIT == 0 && ax.N.back().s[2] == 1;
+    if (skinny) {   // a row of B is one contiguous run of k (A's k order is free: it goes through the k table)
+        int64_t expect = 1;
+        for (int d = (int)ax.K.size() - 1; d >= 0; --d) {
+            if (ax.K[d].n > 1 && ax.K[d].s[1] != expect) skinny = false;
+            expect *= ax.K[d].n;
+        }
+    }
+    if (skinny && !cxd) {   // 16-byte chunks of two f64: rows of B must start on 16-byte boundaries and hold whole chunks
+        skinny = K % 2 == 0 && (uintptr_t)b % 16 == 0;
+        for (auto& x : ax.N) skinny = skinny && x.s[1] % 2 == 0;
+    }
+    int64_t inner_b = 0, inner_c = 0;
+    if (skinny) {
+        int64_t lo = 0, hi = 0;
+        reach(ax.M, 2, lo, hi);
+        if (std::max(-lo, hi) * (cxd ? 2 : 1) >= ((int64_t)1 << 31)) skinny = false;
+        if (std::llabs(ax.N.back().s[1]) * SKINNY_UNIT * (int64_t)eb >= ((int64_t)1 << 31)) skinny = false;
+    }
+    if (skinny) {
+        Axis& x = ax.N.back();
+        inner_b = x.s[1];
+        inner_c = x.s[2];
+        x.n /= SKINNY_UNIT;
+        for (int slot = 0; slot < 3; ++slot) x.s[slot] *= SKINNY_UNIT;
+    }
+    const int64_t Ntab = skinny ? N / SKINNY_UNIT : N;   // entries of the n tables
+
     GemmArgs g;
     std::memset(&g, 0, sizeof g);
     g.A = a; g.B = b; g.C = c;
@@ -548,6 +582,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         nsplit = (int)std::min<int64_t>((512 + tiles - 1) / tiles, kstages / 8);
         nsplit = std::max(1, std::min(nsplit, 64));
     }
+    if (skinny) nsplit = 1;
     int64_t kps = ((kstages + nsplit - 1) / nsplit) * bke;
     nsplit = (int)((K + kps - 1) / kps);
     g.nsplit = nsplit;
@@ -562,7 +597,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
 
     // The 128x128 kernel addresses each operand as a uniform base + 32-bit byte offset: usable when the
     // bytes reachable inside one batch entry span less than 4 GiB (larger operands take the generic kernel).
-    bool use128 = bm == 128;
+    bool use128 = bm == 128 && !skinny;
     int64_t lo_a = 0, hi_a = 0, lo_b = 0, hi_b = 0;
     reach(ax.M, 0, lo_a, hi_a); reach(ax.K, 0, lo_a, hi_a);
     reach(ax.N, 1, lo_b, hi_b); reach(ax.K, 1, lo_b, hi_b);
@@ -580,11 +615,11 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     // operands through 32-bit byte tables (rows of A and B when multi-axis, k of both when k is multi-axis) and
     // only C and the batch offsets through 64-bit element tables.
     struct Want { std::vector<Axis>* grp; int slot; OffFn* fn; int64_t n; bool operand; };
-    Want wants[9] = {{&ax.M, 0, &g.am, M, true}, {&ax.K, 0, &g.ak, K, true}, {&ax.K, 1, &g.bk, K, true}, {&ax.N, 1, &g.bn, N, true},
-                     {&ax.M, 2, &g.cm, M, false}, {&ax.N, 2, &g.cn, N, false}, {&ax.batch, 0, &g.ab, nb, false},
+    Want wants[9] = {{&ax.M, 0, &g.am, M, true}, {&ax.K, 0, &g.ak, K, true}, {&ax.K, 1, &g.bk, K, true}, {&ax.N, 1, &g.bn, Ntab, true},
+                     {&ax.M, 2, &g.cm, M, false}, {&ax.N, 2, &g.cn, Ntab, false}, {&ax.batch, 0, &g.ab, nb, false},
                      {&ax.batch, 1, &g.bb, nb, false}, {&ax.batch, 2, &g.cb, nb, false}};
     struct Want32 { std::vector<Axis>* grp; int slot; Off32* fn; int64_t n; bool force; };
-    Want32 wants32[4] = {{&ax.M, 0, &g.am32, M, false}, {&ax.K, 0, &g.ak32, K, ktab32}, {&ax.K, 1, &g.bk32, K, ktab32}, {&ax.N, 1, &g.bn32, N, false}};
+    Want32 wants32[4] = {{&ax.M, 0, &g.am32, M, false}, {&ax.K, 0, &g.ak32, K, ktab32}, {&ax.K, 1, &g.bk32, K, ktab32}, {&ax.N, 1, &g.bn32, Ntab, false}};
     auto need64 = [&](const Want& w) { return w.grp->size() > 1 && !(use128 && w.operand); };
     auto need32 = [&](const Want32& w) { return use128 && (w.grp->size() > 1 || w.force); };
     size_t table_bytes = 0;
@@ -680,7 +715,20 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     if (nsplit > 1) g.partial = ws + (cached ? 0 : table_bytes);
     dim3 grid((uint32_t)(g.tiles_m * g.tiles_n), 1, (uint32_t)(nb * nsplit));
     const int prof = prof_begin(PROF_CONTRACT, stream);
-    if (use128) launch_128(dtype, g, grid, st);
+    if (skinny) {
+        SkinnyArgs sk;
+        std::memset(&sk, 0, sizeof sk);
+        sk.A = a; sk.B = b; sk.C = c;
+        sk.M = (int32_t)M; sk.K = (int32_t)K;
+        sk.kc = (int32_t)(cxd ? K : K / 2);
+        sk.use_beta = g.use_beta;
+        sk.plain = alpha.re == 1.0 && alpha.im == 0.0 && beta.is_zero();
+        sk.units = Ntab;
+        sk.am = g.am; sk.ak = g.ak; sk.cm = g.cm; sk.bu = g.bn; sk.cu = g.cn;
+        sk.b_in = (int32_t)inner_b; sk.c_in = (int32_t)inner_c;
+        sk.alpha_re = alpha.re; sk.alpha_im = alpha.im; sk.beta_re = beta.re; sk.beta_im = beta.im;
+        launch_gemm_skinny(dtype, sk, st);
+    } else if (use128) launch_128(dtype, g, grid, st);
     else launch_generic64(dtype, g, grid, st);
     prof_end(prof, stream);
     release_packed();   // stream-ordered: the next user of these blocks is enqueued after this kernel

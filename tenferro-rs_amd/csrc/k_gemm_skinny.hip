@@ -1,0 +1,213 @@
+// k_gemm_skinny.hip -- contraction with a small left operand: C[m, n] = alpha * sum_k A[m, k] * B[n, k] + beta * C
+// with at most 32 rows m, at most 64 real k, and a long n (the "apply a small operator to every fibre of a large
+// tensor" step of a tensor-network contraction, PrimDescriptor::Contract, tenferro-prims/src/lib.rs:227-239).
+//
+// Such a product is bound by HBM (B is read once, C written once, a few flops per byte), and a tiled GEMM kernel
+// spends it in per-tile latency: with so little k there is no main loop to hide the loads and the stores behind.
+// Here A lives in registers, already laid out as MFMA operands, for the whole kernel, and every wave streams B on
+// its own: a work unit is 16 consecutive n; the wave loads the unit's rows of B (k contiguous) with 16-byte
+// accesses into registers, parks them in its private LDS region, has the next unit's loads in flight while the
+// MFMAs of the current one run, and writes the unit's columns of C from the accumulators.  Waves never wait for
+// each other (no block barrier).
+//
+// v_mfma_f64_16x16x4_f64: lane l = 16 g + j feeds A'[row j][k' = 4 step + g] and B'[k' = 4 step + g][col j] and
+// receives C'[row g + 4 r][col j] in accumulator register r.  One 16-byte chunk of B serves two steps:
+//   complex128: chunk c of row n is the element B[n][k = c] = (br, bi).  Real form of the product: A'[m][2k + q] =
+//     (re, im)[q] of A[m][k]; B'[2k][2n] = br, B'[2k+1][2n] = -bi, B'[2k][2n+1] = bi, B'[2k+1][2n+1] = br; C'[m][2n + p]
+//     is the interleaved complex C.  Column j is (n = j / 2, p = j % 2): the lane turns its chunk into the operands
+//     (p ? bi : br) for q = 0 and (p ? br : -bi) for q = 1.  Two column blocks (16 n) per unit.
+//   f64: chunk c of row n holds B[n][2c], B[n][2c+1], the operands of q = 0, 1.  Column j is n.  One column block.
+// Pair i of steps (2i, 2i+1) uses chunk 4i + g in lane group g: a permutation of k shared by A' and B', harmless
+// under the sum.  HBM-bound: algorithmic bytes = sizeof(B) + sizeof(C) (+ C again when beta != 0).
+#include <hip/hip_runtime.h>
+
+#include "gemm_skinny.hpp"
+#include "launch.hpp"
+
+namespace tfh {
+namespace {
+
+using namespace gemm;
+
+typedef double d2 __attribute__((ext_vector_type(2)));
+
+constexpr int MAX_KC = SKINNY_MAX_KR / 2;          // 16-byte chunks per row of B at most
+constexpr int PITCH = MAX_KC * 16 + 64;            // bytes per LDS row: rows 0..3 start 16 banks apart
+constexpr int WAVE_LDS = SKINNY_UNIT * PITCH;      // each wave parks one unit
+constexpr int LOADS = SKINNY_UNIT * MAX_KC / 64;   // 16-byte loads per lane and unit at most
+constexpr int PAIRS = MAX_KC / 4;
+
+// Orders the LDS accesses of one wave: lanes read what other lanes of the same wave wrote.  The LDS executes a wave's
+// instructions in order, so only the compiler has to be kept from moving accesses across this point.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <bool CX>
+__global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
+    constexpr int NBLK = CX ? 2 : 1;   // column blocks (16 real columns each) per unit
+    constexpr int NC = CX ? 2 : 1;     // doubles per element
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    unsigned char* lds = smem + wave * WAVE_LDS;
+    const int g = lane >> 4, j = lane & 15, p = j & 1;
+    const int kc = s.kc, npair = (kc + 3) >> 2, nmb = s.M > 16 ? 2 : 1;
+
+    // ---- A as MFMA operands: a[mb][i][q] = A'[j + 16 mb][2 (4i + g) + q], zero outside the matrix
+    double a[2][PAIRS][2];
+    {
+        const double* Ad = reinterpret_cast<const double*>(s.A);
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int i = 0; i < PAIRS; ++i) {
+                const int m = j + 16 * mb, c = 4 * i + g;
+                double x0 = 0, x1 = 0;
+                if (m < s.M) {
+                    if constexpr (CX) {
+                        if (c < s.K) {
+                            const double* q = Ad + 2 * (off_of(s.am, m) + off_of(s.ak, c));
+                            x0 = q[0];
+                            x1 = s.conj_a ? -q[1] : q[1];
+                        }
+                    } else {
+                        if (2 * c < s.K) x0 = Ad[off_of(s.am, m) + off_of(s.ak, 2 * c)];
+                        if (2 * c + 1 < s.K) x1 = Ad[off_of(s.am, m) + off_of(s.ak, 2 * c + 1)];
+                    }
+                }
+                a[mb][i][0] = x0;
+                a[mb][i][1] = x1;
+            }
+    }
+
+    // ---- this lane's share of a unit of B: chunk id = lane + 64 u -> (row, chunk of the row)
+    int32_t goff[LOADS], loff[LOADS];
+    uint32_t have = 0;
+#pragma unroll
+    for (int u = 0; u < LOADS; ++u) {
+        const int id = lane + 64 * u, row = id / kc, col = id - row * kc;
+        const bool ok = id < SKINNY_UNIT * kc;
+        have |= (ok ? 1u : 0u) << u;
+        goff[u] = ok ? row * s.b_in * (8 * NC) + col * 16 : 0;
+        loff[u] = ok ? row * PITCH + col * 16 : 0;
+    }
+    // ---- where this lane reads its operands and writes its results
+    int32_t roff[NBLK], ccol[NBLK], crow[2][4];
+#pragma unroll
+    for (int nb = 0; nb < NBLK; ++nb) {
+        const int nloc = CX ? 8 * nb + (j >> 1) : j;
+        roff[nb] = nloc * PITCH + g * 16;
+        ccol[nb] = nloc * s.c_in * NC + (CX ? p : 0);
+    }
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = Mfma<double>::row(lane, r) + 16 * mb;
+            crow[mb][r] = m < s.M ? (int32_t)(off_of(s.cm, m) * NC) : 0;
+        }
+    const double ar = s.alpha_re, ai = s.alpha_im, br = s.beta_re, bi = s.beta_im;
+
+    const int64_t nwaves = (int64_t)gridDim.x * (THREADS / 64);
+    int64_t unit = (int64_t)blockIdx.x * (THREADS / 64) + wave;
+    d2 stage[LOADS];
+    auto issue = [&](int64_t un) {
+        const unsigned char* Bu = reinterpret_cast<const unsigned char*>(s.B) + off_of(s.bu, un) * (8 * NC);
+#pragma unroll
+        for (int u = 0; u < LOADS; ++u)
+            if ((have >> u) & 1u) stage[u] = __builtin_nontemporal_load(reinterpret_cast<const d2*>(Bu + goff[u]));
+    };
+    if (unit < s.units) issue(unit);
+    while (unit < s.units) {
+#pragma unroll
+        for (int u = 0; u < LOADS; ++u)
+            if ((have >> u) & 1u) *reinterpret_cast<d2*>(lds + loff[u]) = stage[u];
+        const int64_t next = unit + nwaves;
+        if (next < s.units) issue(next);
+        wave_sync();
+
+        d4 acc[2][NBLK];
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int nb = 0; nb < NBLK; ++nb) acc[mb][nb] = d4{0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < PAIRS; ++i) {
+            if (i < npair) {
+                const bool kok = 4 * i + g < kc;
+#pragma unroll
+                for (int nb = 0; nb < NBLK; ++nb) {
+                    const d2 ch = *reinterpret_cast<const d2*>(lds + roff[nb] + i * 64);
+                    double b0, b1;
+                    if constexpr (CX) {
+                        const double im = s.conj_b ? -ch.y : ch.y;
+                        b0 = p ? im : ch.x;
+                        b1 = p ? ch.x : -im;
+                    } else {
+                        b0 = ch.x;
+                        b1 = ch.y;
+                    }
+                    b0 = kok ? b0 : 0.0;   // a row of B may be shorter than the LDS row: never multiply what was not loaded
+                    b1 = kok ? b1 : 0.0;
+                    acc[0][nb] = Mfma<double>::run(a[0][i][0], b0, acc[0][nb]);
+                    acc[0][nb] = Mfma<double>::run(a[0][i][1], b1, acc[0][nb]);
+                    if (nmb > 1) {
+                        acc[1][nb] = Mfma<double>::run(a[1][i][0], b0, acc[1][nb]);
+                        acc[1][nb] = Mfma<double>::run(a[1][i][1], b1, acc[1][nb]);
+                    }
+                }
+            }
+        }
+        wave_sync();   // the next unit is parked over these rows
+
+        // ---- results: lane (g, j) holds rows g + 4r (+16), column j of each column block
+        double* Cu = reinterpret_cast<double*>(s.C) + off_of(s.cu, unit) * NC;
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+            if (mb < nmb) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const bool ok = Mfma<double>::row(lane, r) + 16 * mb < s.M;
+#pragma unroll
+                    for (int nb = 0; nb < NBLK; ++nb) {
+                        double* dst = Cu + crow[mb][r] + ccol[nb];
+                        double v = acc[mb][nb][r];
+                        if (!s.plain) {
+                            if constexpr (CX) {
+                                // even lanes hold re, odd lanes im of one element: exchange with the neighbour
+                                const double other = __shfl_xor(v, 1);
+                                const double re_v = p ? other : v, im_v = p ? v : other;
+                                v = p ? (ar * im_v + ai * re_v) : (ar * re_v - ai * im_v);
+                                if (s.use_beta) {
+                                    const double old = ok ? *dst : 0.0;
+                                    const double old_other = __shfl_xor(old, 1);
+                                    const double re_o = p ? old_other : old, im_o = p ? old : old_other;
+                                    v += p ? (br * im_o + bi * re_o) : (br * re_o - bi * im_o);
+                                }
+                            } else {
+                                v *= ar;
+                                if (s.use_beta && ok) v += br * *dst;
+                            }
+                        }
+                        if (ok) __builtin_nontemporal_store(v, dst);
+                    }
+                }
+            }
+        }
+        unit = next;
+    }
+}
+
+}  // namespace
+
+void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
+    const int64_t blocks_wanted = (s.units + THREADS / 64 - 1) / (THREADS / 64);
+    const dim3 grid((uint32_t)std::min<int64_t>(blocks_wanted, 512)), block(THREADS);
+    const size_t lds = (size_t)(THREADS / 64) * WAVE_LDS;
+    if (dtype == TFH_C128) TFH_LAUNCH_TIMED((gemm_skinny_kernel<true>), grid, block, lds, st, s);
+    else TFH_LAUNCH_TIMED((gemm_skinny_kernel<false>), grid, block, lds, st, s);
+}
+
+}  // namespace tfh

@@ -971,3 +971,37 @@ def test_offset_tables_are_kept_per_layout_and_survive_a_release(tf, oracle):
             assert relerr(out.to_numpy(), r) < 1e-12
         if rnd == 1:
             assert tf.lib().tfh_release_workspaces() == 0
+
+
+@pytest.mark.parametrize("dtype", [np.complex128, np.float64])
+@pytest.mark.parametrize("m,k,x,c", [(32, 32, 8, 1024), (20, 13, 64, 80), (16, 32, 1, 4096), (7, 6, 16, 512), (32, 2, 32, 160)])
+def test_contract_small_operator_applied_to_a_long_tensor(tf, oracle, dtype, m, k, x, c):
+    # T[x, c, k] . W[k, m] -> out[x, m, c]: few rows, little k, a long n = (x, c) whose fastest output axis is c -- the
+    # shape of an operator applied to every fibre of a large tensor, which takes the streaming kernel.  Odd m and k,
+    # general alpha/beta, and a W that is a strided view are covered; f64 needs an even k for that kernel and falls
+    # back to the tiled one otherwise (k = 13).
+    rng = np.random.default_rng(91)
+    t = rand(rng, (x, c, k), dtype)
+    w = rand(rng, (k, 2 * m), dtype)[:, ::2]
+    ref = rand(rng, (x, m, c), dtype)
+    out0 = ref.copy()
+    cplx = np.iscomplexobj(t)
+    for alpha, beta in [(1.0, 0.0), ((0.5 - 2j, 1.5 + 1j) if cplx else (0.5, -1.5))]:
+        ref = out0.copy()
+        oracle.contract(t, lab("xck"), w, lab("km"), ref, lab("xmc"), alpha=alpha, beta=beta)
+        dout = dev(tf, out0)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab("xmc")), [t.shape, w.shape, ref.shape])
+        tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
+        assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
+
+
+def test_contract_small_operator_exact_on_integer_inputs(tf):
+    # small integers: every product and sum is exact, so the streaming kernel must agree with numpy to the bit, and a
+    # wrong sign in the complex expansion or a misplaced k would show
+    rng = np.random.default_rng(92)
+    t = (rng.integers(-4, 5, (4, 1024, 32)) + 1j * rng.integers(-4, 5, (4, 1024, 32))).astype(np.complex128)
+    w = (rng.integers(-4, 5, (32, 32)) + 1j * rng.integers(-4, 5, (32, 32))).astype(np.complex128)
+    out = tf.Tensor.empty([4, 32, 1024], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.complex128)
+    plan = tf.HipBackend.plan(np.complex128, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab("xmc")), [t.shape, w.shape, [4, 32, 1024]])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, t), dev(tf, w)], 0.0, out)
+    assert np.array_equal(out.to_numpy(), np.einsum("xck,km->xmc", t, w))
