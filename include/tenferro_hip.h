@@ -264,6 +264,11 @@ int32_t tfh_stream_wait_event(tfh_stream s, tfh_event e);  /* chaining without a
 int32_t tfh_profile_enable(int32_t on);
 int32_t tfh_profile_collect(int32_t kind, double* total_ms, int32_t* launches);
 
+/* Diagnostic, no counterpart in the reference: the source-level name (template arguments as written in the
+ * library) of the dominant kernel most recently launched by the calling thread, "" before the first one.
+ * Tests use it to check which kernel a call was routed to. */
+const char* tfh_last_kernel(void);
+
 /* Releases the cached workspace, intermediate buffers and offset tables of every stream (after a synchronize). */
 int32_t tfh_release_workspaces(void);
 

@@ -105,6 +105,8 @@ def lib():
         L.tfh_has_extension.argtypes = [C.c_int32, C.c_int32]
         L.tfh_profile_enable.argtypes = [C.c_int32]
         L.tfh_profile_collect.argtypes = [C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_int32)]
+        L.tfh_last_kernel.restype = C.c_char_p
+        L.tfh_last_kernel.argtypes = []
         L.tfh_subscripts_labels.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]
         L.tfh_subscripts_nesting.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t]
         L.tfh_plan_describe.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t]
@@ -891,6 +893,11 @@ PROF_CONTRACT, PROF_COPY, PROF_REDUCE = 0, 1, 2
 def profile_enable(on=True):
     """Bracket the dominant kernel of every launch with HIP events on its stream (tfh_profile_enable)."""
     _check(lib().tfh_profile_enable(1 if on else 0))
+
+
+def last_kernel():
+    """Name of the dominant kernel the calling thread launched last (diagnostic)."""
+    return lib().tfh_last_kernel().decode()
 
 
 def profile_collect(kind):

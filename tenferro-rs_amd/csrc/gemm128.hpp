@@ -127,12 +127,17 @@ struct OperandMap {
         for (int l = 0; l < NL; ++l) x[l] = gload_pack<R, PN>(base, voff[l]);
     }
     // single-stride k, last stage with `rem` valid k: k redirected into the range (masked to zero when stored)
+    // The 32-bit offsets are unsigned distances from `base`.  With fewer than V valid k the window of a k-contiguous
+    // operand starts before this stage (inside the previous one): the base itself is moved back by that much, so
+    // that no offset goes below zero.
     __device__ __forceinline__ void load_tail(P (&x)[NL], gptr base, int rem, uint32_t kstride, uint32_t rowstride) const {
         const uint32_t back = (uint32_t)(-row_shift) * rowstride;
+        const int before = KFAST && rem < V ? V - rem : 0;
+        base -= (int64_t)(int32_t)kstride * before;
 #pragma unroll
         for (int l = 0; l < NL; ++l) {
             const int last = KFAST ? rem - V : rem - 1;
-            const int d = kk(l) > last ? last - kk(l) : 0;
+            const int d = (kk(l) > last ? last - kk(l) : 0) + before;
             x[l] = gload_pack<R, PN>(base, voff[l] + (uint32_t)d * kstride + back);
         }
     }

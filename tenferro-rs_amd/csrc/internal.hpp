@@ -131,6 +131,8 @@ int32_t hip_check(int err, const char* what);
 // Event bracket around a dominant kernel while profiling is enabled (runtime.cpp); -1 when disabled.
 enum { PROF_CONTRACT = 0, PROF_COPY = 1, PROF_REDUCE = 2 };
 int prof_begin(int kind, void* stream);
+// Remembers, per host thread, the source-level name of the dominant kernel launched last (tfh_last_kernel).
+void note_kernel(const char* name);
 void prof_end(int token, void* stream);
 // The dominant kernel's launch takes the pair of events prof_begin() prepared on this thread (null when profiling is
 // off): launched with them, the events carry the dispatch's own begin and end timestamps, so their difference is the

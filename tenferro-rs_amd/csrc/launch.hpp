@@ -7,6 +7,7 @@
 
 #define TFH_LAUNCH_TIMED(kernel, grid, block, lds, st, ...)                                                          \
     do {                                                                                                             \
+        tfh::note_kernel(#kernel);                                                                                   \
         const tfh::ProfEvents pe_ = tfh::prof_take();                                                                \
         if (pe_.start)                                                                                               \
             hipExtLaunchKernelGGL(kernel, grid, block, lds, st, (hipEvent_t)pe_.start, (hipEvent_t)pe_.stop, 0, __VA_ARGS__); \

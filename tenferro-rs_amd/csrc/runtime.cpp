@@ -159,7 +159,10 @@ hipEvent_t prof_event() {
 
 namespace {
 thread_local ProfEvents t_pending;
+thread_local const char* t_last_kernel = "";
 }
+void note_kernel(const char* name) { t_last_kernel = name; }
+const char* last_kernel() { return t_last_kernel; }
 int prof_begin(int kind, void* stream) {
     (void)stream;
     if (!g_prof_on) return -1;
@@ -229,6 +232,8 @@ int32_t tfh_profile_collect(int32_t kind, double* total_ms, int32_t* launches) {
     *launches = n;
     return TFH_OK;
 }
+
+const char* tfh_last_kernel(void) { return tfh::last_kernel(); }
 
 int32_t tfh_release_workspaces(void) {
     std::lock_guard<std::mutex> lk(tfh::g_mu);

@@ -515,6 +515,7 @@ def test_permute_power_of_two_shapes_take_the_vector_path(tf, oracle, dtype):
     a = rand(rng, (32, 8, 64, 16), dtype)
     for perm in [(3, 1, 0, 2), (0, 1, 2, 3), (2, 3, 0, 1), (1, 0, 3, 2)]:
         got, ref = _permute_check(tf, oracle, a, perm)
+        assert tf.last_kernel().startswith("(copy_kernel") and tf.last_kernel().endswith("true>)"), tf.last_kernel()   # FAST
         assert got.tobytes() == ref.tobytes(), perm
     b0 = rand(rng, (16, 8, 32, 64), dtype)
     alpha, beta = (0.5 - 2j, 1.5 + 1j) if np.issubdtype(dtype, np.complexfloating) else (0.5, -1.5)
@@ -531,6 +532,7 @@ def test_permute_misaligned_base_and_odd_inner_extent(tf, oracle):
     assert got.tobytes() == ref.tobytes()
     b = rng.standard_normal((64, 30, 17))            # partial tiles on every axis
     got, ref = _permute_check(tf, oracle, b, (2, 1, 0))
+    assert tf.last_kernel().startswith("(copy_kernel") and tf.last_kernel().endswith("false>)"), tf.last_kernel()      # bounds-checked
     assert got.tobytes() == ref.tobytes()
 
 
@@ -557,6 +559,11 @@ def test_reduce_fast_path_variants(tf, oracle, dtype):
              [3]]
     for mc in cases:
         got, ref = _reduce_check(tf, oracle, a, m, mc, tf.ReduceOp.Sum, oracle.SUM)
+        # the first two and the fourth must take the tiled fast path for every dtype; 16 outputs ([3]) are too few for it
+        if mc in ([0, 1, 2, 3], [0, 2, 4], [1, 2, 3, 4]):
+            assert "reduce_fast_kernel" in tf.last_kernel(), (mc, tf.last_kernel())
+        if mc == [3]:
+            assert "reduce_fast_kernel" not in tf.last_kernel()
         assert relerr(got, ref) < TOL[dtype], mc
     c0 = rand(rng, (8, 4, 32), dtype)
     got, ref = _reduce_check(tf, oracle, a, m, [0, 2, 4], tf.ReduceOp.Sum, oracle.SUM, alpha=2.0, beta=-0.5, c0=c0)
@@ -591,11 +598,12 @@ def test_reduce_misaligned_base_and_split_reductions(tf, oracle):
 
 
 BIG_CASES = [
-    ("ajbk,kcj->abc", dict(a=16, j=8, b=16, k=12, c=160)),      # 128x128 tiles, two-mode k through offset tables, packed B
-    ("mk,kn->mn", dict(m=300, k=203, n=260)),                    # ragged edges and a k tail in the 128x128 kernel
-    ("km,nk->mn", dict(m=256, k=100, n=384)),
-    ("mk,nk->nm", dict(m=200, k=64, n=130)),                     # operands swap
-    ("bmk,kbn->bmn", dict(b=3, m=130, k=40, n=140)),             # batch + 128 tiles
+    # k long enough (>= 32 stages) that the few 128x128 tiles are preferred to 64x64 ones and split over k
+    ("ajbk,kcj->abc", dict(a=16, j=24, b=16, k=48, c=160)),     # two-mode k through offset tables, packed B
+    ("mk,kn->mn", dict(m=300, k=1103, n=260)),                   # ragged edges and a k tail
+    ("km,nk->mn", dict(m=256, k=1040, n=384)),
+    ("mk,nk->nm", dict(m=200, k=1030, n=130)),                   # operands swap
+    ("bmk,kbn->bmn", dict(b=3, m=130, k=1050, n=140)),           # batch
 ]
 
 
@@ -616,6 +624,7 @@ def test_contract_128_tile_kernel(tf, oracle, dtype, case):
     out = dev(tf, c0)
     plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [a.shape, b.shape, cshape])
     tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, out)
+    assert "gemm128_kernel" in tf.last_kernel(), tf.last_kernel()
     assert relerr(out.to_numpy(), ref) < TOL[dtype]
 
 
@@ -652,7 +661,11 @@ def test_config3_full_size_complex128(tf, oracle):
     assert relerr(res.to_numpy(), ref) < 1e-12
 
 
-ODD_SIZES = [(129, 131, 133), (255, 77, 257), (131, 5, 129), (130, 3, 131), (257, 4, 130), (193, 34, 97)]
+# sizes that the launcher gives to the 128x128 kernel: a long k (>= 32 stages) over few tiles, or many tiles over a k
+# shorter than one vector
+# (the last three leave fewer k than one vector in the final stage: its window then starts inside the previous stage)
+ODD_SIZES = [(129, 1031, 133), (255, 1077, 257), (1801, 5, 1795), (1810, 3, 1811), (1793, 4, 1800), (193, 1058, 97),
+             (257, 1025, 129), (130, 1027, 131), (1801, 66, 1795)]
 LAYOUTS = [("mk", "kn"), ("mk", "nk"), ("km", "kn"), ("km", "nk")]
 
 
@@ -672,13 +685,14 @@ def test_contract_odd_extents_take_the_straddling_vector_path(tf, oracle, dtype,
         out = dev(tf, np.full((m, n), np.nan, dtype))
         plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab("mn")), [a.shape, b.shape, [m, n]])
         tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
+        assert "gemm128_kernel" in tf.last_kernel(), (m, k, n, tf.last_kernel())
         assert relerr(out.to_numpy(), ref) < TOL[dtype], (m, k, n)
 
 
 def test_contract_operand_ending_at_the_end_of_its_allocation(tf, oracle):
     # the operands are the tail of exactly-sized device buffers: a read past the last element would leave the buffer
     rng = np.random.default_rng(48)
-    for dtype, m, k, n in [(np.float32, 131, 133, 129), (np.float64, 129, 67, 131)]:
+    for dtype, m, k, n in [(np.float32, 131, 1033, 129), (np.float64, 129, 523, 131)]:
         for ma, mb in LAYOUTS:
             ext = dict(m=m, k=k, n=n)
             a = rand(rng, [ext[l] for l in ma], dtype)
@@ -688,6 +702,7 @@ def test_contract_operand_ending_at_the_end_of_its_allocation(tf, oracle):
             out = dev(tf, np.zeros((m, n), dtype))
             plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab("mn")), [a.shape, b.shape, [m, n]])
             tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
+            assert "gemm128_kernel" in tf.last_kernel(), tf.last_kernel()
             assert relerr(out.to_numpy(), ref) < TOL[dtype], (dtype, ma, mb)
 
 
@@ -992,6 +1007,8 @@ def test_contract_small_operator_applied_to_a_long_tensor(tf, oracle, dtype, m, 
         dout = dev(tf, out0)
         plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab("xmc")), [t.shape, w.shape, ref.shape])
         tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
+        streamed = cplx or k % 2 == 0
+        assert ("gemm_skinny_kernel" in tf.last_kernel()) == streamed, tf.last_kernel()
         assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
 
 
@@ -1004,4 +1021,34 @@ def test_contract_small_operator_exact_on_integer_inputs(tf):
     out = tf.Tensor.empty([4, 32, 1024], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.complex128)
     plan = tf.HipBackend.plan(np.complex128, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab("xmc")), [t.shape, w.shape, [4, 32, 1024]])
     tf.HipBackend.execute(plan, 1.0, [dev(tf, t), dev(tf, w)], 0.0, out)
+    assert "gemm_skinny_kernel" in tf.last_kernel()
     assert np.array_equal(out.to_numpy(), np.einsum("xck,km->xmc", t, w))
+
+
+@pytest.mark.parametrize("dtype", [np.complex128, np.float64])
+def test_contract_small_operator_strided_rows_and_split_k_order(tf, oracle, dtype):
+    # the streaming kernel's addressing: rows of the long operand reversed along c and padded (a view of a larger buffer),
+    # its k split over two modes that the small operand holds in the opposite order (its k goes through the offset table),
+    # the small operand's rows split over two modes of the output
+    rng = np.random.default_rng(93)
+    x, c, s_, w_, t_, v_ = 16, 320, 2, 8, 2, 7
+    t1 = rand(rng, (x, c, s_, w_), dtype)[:, ::-1]                                        # contiguous k per row, rows reversed
+    wop = rand(rng, (w_, s_, t_, v_), dtype)
+    ref = np.empty((x, v_, t_, c), dtype)
+    oracle.contract(t1, lab("xcsw"), wop, lab("wstv"), ref, lab("xvtc"))
+    out = tf.Tensor.empty([x, v_, t_, c], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xcsw"), lab("wstv"), lab("xvtc")), [t1.shape, wop.shape, ref.shape])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, t1), dev(tf, wop)], 0.0, out)
+    assert "gemm_skinny_kernel" in tf.last_kernel()
+    assert relerr(out.to_numpy(), ref) < 1e-12
+    # padded rows: each (x, c) row is the first 16 elements of a 24-element row of a larger buffer
+    bigk = rand(rng, (x, c, 24), dtype)
+    t2 = bigk[:, :, :16]
+    w2 = rand(rng, (16, 20), dtype)
+    ref2 = np.empty((x, 20, c), dtype)
+    oracle.contract(t2, lab("xck"), w2, lab("km"), ref2, lab("xmc"))
+    out2 = tf.Tensor.empty([x, 20, c], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    plan2 = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab("xmc")), [t2.shape, w2.shape, ref2.shape])
+    tf.HipBackend.execute(plan2, 1.0, [dev(tf, t2), dev(tf, w2)], 0.0, out2)
+    assert "gemm_skinny_kernel" in tf.last_kernel()
+    assert relerr(out2.to_numpy(), ref2) < 1e-12
