@@ -813,6 +813,46 @@ def test_contract_random_label_patterns_and_views(tf, oracle, dtype, big):
 
 
 @pytest.mark.parametrize("dtype", ALL)
+def test_contract_random_layouts_on_the_128_tile_kernel(tf, oracle, dtype):
+    # random shapes sized for the 128x128 kernel (both free products >= 97, k of a thousand or more, so >= 32 stages):
+    # one or two modes per group, random axis orders, random strided / reversed / offset views, odd extents.  Most
+    # cases are contiguous along some operand direction (16-byte loads with their tail handling), the stepped views are not.
+    rng = np.random.default_rng(58)
+    on128 = 0
+    for case in range(14):
+        labels = list("abcdefgh")
+        rng.shuffle(labels)
+        nb, nm, nn, nk = int(rng.integers(0, 2)), int(rng.integers(1, 3)), int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        batch, fm, fn, kk = labels[:nb], labels[nb:nb + nm], labels[nb + nm:nb + nm + nn], labels[nb + nm + nn:nb + nm + nn + nk]
+        ext = {}
+        for grp, lo, hi in ((fm, 97, 300), (fn, 97, 300), (kk, 1000, 1100)):
+            ext[grp[0]] = int(rng.integers(lo, hi + 1))
+            for l in grp[1:]:
+                ext[l] = int(rng.integers(1, 4))
+        for l in batch:
+            ext[l] = int(rng.integers(1, 3))
+        ma, mb, mc = batch + fm + kk, batch + kk + fn, batch + fm + fn
+        rng.shuffle(ma); rng.shuffle(mb); rng.shuffle(mc)
+        plain = case % 2 == 0            # every other case: dense operands (the vector paths); else random views
+        mk = (lambda shape: rand(rng, shape, dtype)) if plain else (lambda shape: _random_view(rng, shape, dtype))
+        a, b = mk([ext[l] for l in ma]), mk([ext[l] for l in mb])
+        cshape = [ext[l] for l in mc]
+        use_beta = bool(rng.integers(0, 2))
+        alpha, beta = (0.7 - 1.1j, (-0.3 + 0.2j) if use_beta else 0.0) if np.issubdtype(dtype, np.complexfloating) else (0.7, -0.3 if use_beta else 0.0)
+        c0 = rand(rng, cshape, dtype) if use_beta else np.full(cshape, np.nan, dtype)
+        ref = c0.copy()
+        oracle.contract(a, lab(ma), b, lab(mb), ref, lab(mc), alpha=alpha, beta=beta)
+        out = dev(tf, c0)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [a.shape, b.shape, cshape])
+        print("case", case, "".join(ma), "".join(mb), "".join(mc), ext, "plain" if plain else "views", flush=True)
+        tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, out)
+        on128 += "gemm128_kernel" in tf.last_kernel()
+        err = relerr(out.to_numpy(), ref)
+        assert err < TOL[dtype], (case, ma, mb, mc, ext, err)
+    assert on128 >= 12, on128
+
+
+@pytest.mark.parametrize("dtype", ALL)
 def test_permute_and_reduce_random_shapes_and_views(tf, oracle, dtype):
     rng = np.random.default_rng(52)
     for case in range(30):
