@@ -343,6 +343,15 @@ def test_grouped_small_ragged(tf, oracle):
     assert _grouped_case(tf, oracle, dims, np.float64, 77) < 1e-12
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_grouped_odd_extents_on_128_tiles(tf, oracle, dtype):
+    # one grouped launch over problems whose extents are not multiples of the tile, the stage or the vector length
+    # (k tails of 1, 2, 5, 6 and 7 elements; edges of 1 and 3 rows), all large enough for 128x128 tiles
+    dims = [(129, 1031, 133), (255, 66, 257), (193, 1058, 97), (300, 5, 310), (131, 130, 129), (257, 1025, 129), (300, 6, 310)]
+    assert _grouped_case(tf, oracle, dims, dtype, 78) < TOL[dtype]
+    assert "gemm128_kernel" in tf.last_kernel(), tf.last_kernel()
+
+
 def test_config4_grouped_full_size(tf, oracle):
     # 128 blocks, i,j,k iid from {64,...,1024}: every block <= 1e-12 against the oracle, one launch
     from tenferro_rs_amd import inputs
