@@ -60,6 +60,9 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise RuntimeError(f"{LIB_PATH} is missing: build it with `python tenferro-rs_amd/build.py`")
+        # GpuMemory tensors of this module live in torch CUDA tensors, so torch's HIP runtime must be the one in the
+        # process: loaded after the system runtime that the library would otherwise pull in, torch finds no device.
+        import torch  # noqa: F401
         L = C.CDLL(LIB_PATH)
         L.tfh_status_name.restype = C.c_char_p
         L.tfh_version.restype = C.c_char_p
