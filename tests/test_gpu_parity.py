@@ -468,6 +468,50 @@ def test_einsum_every_tree_of_a_small_network_agrees(tf, oracle, dtype):
     assert relerr(dc.to_numpy(), 3 * ref - c0) < 1e-12
 
 
+def _random_network(rng):
+    """A random einsum of 2-5 operands over a pool of labels: repeated labels inside an operand (diagonals), labels
+    held by one operand only and absent from the output (summed), labels shared by three operands, a random output
+    order, sometimes a repeated output label or an empty output."""
+    pool = list("abcdefg")
+    ext = {l: int(rng.integers(1, 7)) for l in pool}
+    n = int(rng.integers(2, 6))
+    terms = []
+    for _ in range(n):
+        r = int(rng.integers(1, 4))
+        t = [str(rng.choice(pool)) for _ in range(r)] if rng.integers(0, 4) == 0 else [str(x) for x in rng.choice(pool, r, replace=False)]
+        terms.append("".join(t))
+    used = sorted(set("".join(terms)))
+    k = int(rng.integers(0, min(4, len(used)) + 1))
+    out = [str(x) for x in rng.choice(used, k, replace=False)]
+    if out and rng.integers(0, 6) == 0:
+        out.append(out[0])
+    rng.shuffle(out)
+    return terms, "".join(out), ext
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.complex128, np.float32])
+def test_einsum_random_networks(tf, oracle, dtype):
+    # the executor end to end (parser, optimiser, layouts of intermediates, diagonal views, reductions, output
+    # diagonals, alpha/beta into a strided output) against the oracle's single-loop-nest einsum
+    rng = np.random.default_rng(59)
+    for case in range(60):
+        terms, out, ext = _random_network(rng)
+        ops = [_random_view(rng, [ext[l] for l in t], dtype) for t in terms]
+        oshape = [ext[l] for l in out]
+        pattern = ",".join(terms) + "->" + out
+        ref = np.empty(oshape, dtype)
+        oracle.einsum_naive(ops, [lab(t) for t in terms], ref, lab(out))
+        dops = [dev(tf, o) for o in ops]
+        res = tf.einsum(pattern, dops)
+        assert res.dims() == oshape, pattern
+        assert relerr(res.to_numpy(), ref) < 10 * TOL[dtype], (case, pattern, ext)
+        if oshape and case % 3 == 0:
+            c0 = _random_view(rng, oshape, dtype)
+            dc = dev(tf, c0)
+            tf.einsum_into(pattern, dops, 0.5, -2.0, dc)
+            assert relerr(dc.to_numpy(), 0.5 * ref - 2.0 * c0) < 10 * TOL[dtype], (case, pattern, ext, "into")
+
+
 def test_einsum_async_chaining(tf):
     # tenferro-einsum/src/lib.rs:158-177: the second call chains on the first result's event
     rng = np.random.default_rng(34)
