@@ -353,7 +353,7 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
     constexpr int LD_EVERY = HALF / (NLD + 1) > 0 ? HALF / (NLD + 1) : 1;
     constexpr int ST_EVERY = HALF / (NST + 1) > 0 ? HALF / (NST + 1) : 1;
     constexpr int ST_FIRST = 0;
-    static_assert(LD_EVERY * NLD <= HALF && ST_FIRST >= 0, "one half stage must take all loads / stores");
+    static_assert(LD_EVERY * NLD <= HALF && ST_FIRST + ST_EVERY * NST <= HALF, "one half stage must take all loads / stores");
     uint32_t ka[MapA::NKO], kb[MapB::NKO];   // multi-mode k: table entries of the stage whose loads are issued next
     auto stage_interleaved = [&](int buf, bool tab, int64_t k0_after_next) {
         const R* as = As + buf * BM * PITCH + (wm0 + lrow) * PITCH;
@@ -404,7 +404,7 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
                 for (int j = 0; j < TN; ++j) {
                     acc[i][j] = Mfma<R>::run(a[1][i][c], b[1][j][c], acc[i][j]);
                     const int m = (c * TM + i) * TN + j;
-                    if (m >= ST_FIRST && (m - ST_FIRST) % ST_EVERY == ST_EVERY - 1) {
+                    if (m >= ST_FIRST && (m - ST_FIRST) % ST_EVERY == ST_EVERY - 1 && (m - ST_FIRST) / ST_EVERY < NST) {
                         const int u = (m - ST_FIRST) / ST_EVERY;
                         if (u < MapA::NSU) ma.store_unit(as_next, va, u, false, rem, g.conj_a != 0);
                         else mb.store_unit(bs_next, vb, u - MapA::NSU, false, rem, g.conj_b != 0);
