@@ -331,6 +331,41 @@ __global__ void __launch_bounds__(THREADS) splitk_finalize_kernel(GemmArgs g) {
     }
 }
 
+// The same fold with 16-byte accesses, for a C that is contiguous along n: one thread per 16 bytes of a row of C.
+template <class R, bool CX>
+__global__ void __launch_bounds__(THREADS) splitk_finalize_vec_kernel(GemmArgs g) {
+    constexpr int VEC = 16 / sizeof(R), NC = CX ? 2 : 1;
+    typedef R Vec __attribute__((ext_vector_type(VEC)));
+    const int64_t NR = g.N * NC, nv = NR / VEC;
+    const int64_t idx = (int64_t)blockIdx.x * THREADS + threadIdx.x;
+    if (idx >= g.nbatch * g.M * nv) return;
+    const int64_t v = idx % nv, t = idx / nv, m = t % g.M, b = t / g.M;
+    const int64_t plane = g.nbatch * g.M * NR;
+    const R* p = reinterpret_cast<const R*>(g.partial) + (b * g.M + m) * NR + v * VEC;
+    Vec sum = __builtin_nontemporal_load(reinterpret_cast<const Vec*>(p));
+    for (int s = 1; s < g.nsplit; ++s) sum += __builtin_nontemporal_load(reinterpret_cast<const Vec*>(p + s * plane));
+    Vec* dst = reinterpret_cast<Vec*>(reinterpret_cast<R*>(g.C) + (off_of(g.cb, b) + off_of(g.cm, m)) * NC + v * VEC);
+    const R ar = (R)g.alpha_re, ai = (R)g.alpha_im, br = (R)g.beta_re, bi = (R)g.beta_im;
+    Vec out;
+    if constexpr (CX) {
+        Vec old = sum;
+        if (g.use_beta) old = *dst;
+#pragma unroll
+        for (int e = 0; e < VEC; e += 2) {
+            out[e] = ar * sum[e] - ai * sum[e + 1];
+            out[e + 1] = ar * sum[e + 1] + ai * sum[e];
+            if (g.use_beta) {
+                out[e] += br * old[e] - bi * old[e + 1];
+                out[e + 1] += br * old[e + 1] + bi * old[e];
+            }
+        }
+    } else {
+        out = sum * ar;
+        if (g.use_beta) out += *dst * br;
+    }
+    *dst = out;
+}
+
 // Offsets of every fused index of an axis group (last axis fastest): tab[i] = sum_d idx_d * stride_d.  All
 // tables of one contraction are built by one launch (blockIdx.y = table).
 constexpr int MAX_TABLES = 13, MAX_TABLE_AXES = 96;
@@ -734,6 +769,22 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     release_packed();   // stream-ordered: the next user of these blocks is enqueued after this kernel
     if (int32_t e = hip_check(hipGetLastError(), "contraction kernel launch")) return e;
     if (nsplit > 1) {
+        // 16-byte fold: C contiguous along n, whole vectors per row, every row of C on a 16-byte boundary
+        const int64_t vec = 16 / rb, ncx = cx ? 2 : 1;
+        bool fold_vec = !g.cn.tab && g.cn.stride == 1 && NR % vec == 0 && (uintptr_t)c % 16 == 0;
+        for (auto* grp : {&ax.M, &ax.batch})
+            for (auto& x : *grp) fold_vec = fold_vec && (x.n == 1 || (x.s[2] * ncx) % vec == 0);
+        if (fold_vec) {
+            const int64_t total = nb * M * (NR / vec);
+            dim3 g2((uint32_t)((total + THREADS - 1) / THREADS));
+            switch (dtype) {
+                case TFH_F32: hipLaunchKernelGGL((splitk_finalize_vec_kernel<float, false>), g2, dim3(THREADS), 0, st, g); break;
+                case TFH_F64: hipLaunchKernelGGL((splitk_finalize_vec_kernel<double, false>), g2, dim3(THREADS), 0, st, g); break;
+                case TFH_C64: hipLaunchKernelGGL((splitk_finalize_vec_kernel<float, true>), g2, dim3(THREADS), 0, st, g); break;
+                default: hipLaunchKernelGGL((splitk_finalize_vec_kernel<double, true>), g2, dim3(THREADS), 0, st, g); break;
+            }
+            return hip_check(hipGetLastError(), "split-K finalize launch");
+        }
         int64_t total = nb * M * N;
         dim3 g2((uint32_t)((total + THREADS - 1) / THREADS));
         switch (dtype) {
