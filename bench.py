@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs c1,c2,c3,c4] [--no-cpu]
 
-Prints ONE JSON line.  The headline (`value`) is configuration 1 of BASELINE.json -- the f32 einsum
+Prints ONE JSON line.  The headline (`value`) is configuration 1 of the benchmark definition -- the f32 einsum
 "ajbk,kcj->abc" (a=64, j=128, b=64, k=96, c=256) -- as whole-step TFLOP/s with inputs resident in
 HBM; `all_configs` carries the same measurements for configurations 2 (permute + reduce of a 16^6
 f64 tensor), 3 (complex128 MPS-MPO environment update, four operands) and 4 (128-block grouped f64
