@@ -564,9 +564,38 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     // A small left operand against a long n whose rows of B are contiguous in k: the streaming kernel of
     // k_gemm_skinny.hip (work units of SKINNY_UNIT consecutive n; the n tables then hold one entry per unit).
     const bool cxd = dtype == TFH_C128;
+    // The same product seen from the other side -- the long operand is A and C is contiguous along the few columns
+    // of B (C[m][n], n = 0..N-1 adjacent): exchange the operands; the kernel then writes C through a transposing
+    // LDS tile ("out_rows").
+    bool out_rows = false;
+    if ((dtype == TFH_F64 || cxd) && nb == 1 && N <= SKINNY_MAX_M && M >= 4096 && K * (cxd ? 2 : 1) <= SKINNY_MAX_KR && a_kfast &&
+        !k_by_b && !ax.K.empty() && ax.N.size() == 1 && ax.N[0].s[2] == 1 && !ax.M.empty() && ax.M.back().n % SKINNY_UNIT == 0 &&
+        (cxd || (N % 2 == 0 && K % 2 == 0 && (uintptr_t)c % 16 == 0 && (uintptr_t)a % 16 == 0))) {
+        bool ok = true;
+        int64_t expect = 1;
+        for (int d = (int)ax.K.size() - 1; d >= 0; --d) {   // a row of A is one contiguous run of k
+            if (ax.K[d].n > 1 && ax.K[d].s[0] != expect) ok = false;
+            expect *= ax.K[d].n;
+        }
+        if (!cxd)
+            for (auto& x : ax.M) ok = ok && x.s[2] % 2 == 0 && x.s[0] % 2 == 0;
+        const Axis& in = ax.M.back();
+        ok = ok && std::llabs(in.s[0]) * SKINNY_UNIT * (int64_t)eb < ((int64_t)1 << 31) &&
+             std::llabs(in.s[2]) * SKINNY_UNIT * (int64_t)eb < ((int64_t)1 << 31);
+        if (ok) {
+            std::swap(a, b);
+            std::swap(ax.M, ax.N);
+            std::swap(M, N);
+            std::swap(a_kfast, b_kfast);
+            for (auto* grp : {&ax.batch, &ax.M, &ax.N, &ax.K})
+                for (auto& x : *grp) std::swap(x.s[0], x.s[1]);
+            out_rows = true;
+        }
+    }
+    const bool k_rows_b = out_rows || k_by_b;   // the k modes are in the memory order of the (possibly exchanged) B
     bool skinny = (dtype == TFH_F64 || cxd) && nb == 1 && M <= SKINNY_MAX_M && K * (cxd ? 2 : 1) <= SKINNY_MAX_KR && N >= 4096 &&
-                  b_kfast && !ax.K.empty() && k_by_b && !ax.N.empty() &&
-                  ax.N.back().n % SKINNY_UNIT == 0 && ax.N.back().s[2] == 1;
+                  b_kfast && !ax.K.empty() && k_rows_b && !ax.N.empty() &&
+                  ax.N.back().n % SKINNY_UNIT == 0 && (out_rows || ax.N.back().s[2] == 1);
     if (skinny) {   // a row of B is one contiguous run of k (A's k order is free: it goes through the k table)
         int64_t expect = 1;
         for (int d = (int)ax.K.size() - 1; d >= 0; --d) {
@@ -757,6 +786,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         sk.M = (int32_t)M; sk.K = (int32_t)K;
         sk.kc = (int32_t)(cxd ? K : K / 2);
         sk.use_beta = g.use_beta;
+        sk.out_rows = out_rows;
         sk.plain = alpha.re == 1.0 && alpha.im == 0.0 && beta.is_zero();
         sk.units = Ntab;
         sk.am = g.am; sk.ak = g.ak; sk.cm = g.cm; sk.bu = g.bn; sk.cu = g.cn;

@@ -19,6 +19,10 @@
 //   f64: chunk c of row n holds B[n][2c], B[n][2c+1], the operands of q = 0, 1.  Column j is n.  One column block.
 // Pair i of steps (2i, 2i+1) uses chunk 4i + g in lane group g: a permutation of k shared by A' and B', harmless
 // under the sum.  HBM-bound: algorithmic bytes = sizeof(B) + sizeof(C) (+ C again when beta != 0).
+//
+// C may be contiguous along n (each lane stores its accumulators: 128-byte segments per row of C) or along m (the
+// other orientation of the same product, C[n][m]): then the unit's 16 x M results are transposed through the wave's
+// LDS region and leave as 16-byte stores along m.
 #include <hip/hip_runtime.h>
 
 #include "gemm_skinny.hpp"
@@ -36,6 +40,8 @@ constexpr int PITCH = MAX_KC * 16 + 64;            // bytes per LDS row: rows 0.
 constexpr int WAVE_LDS = SKINNY_UNIT * PITCH;      // each wave parks one unit
 constexpr int LOADS = SKINNY_UNIT * MAX_KC / 64;   // 16-byte loads per lane and unit at most
 constexpr int PAIRS = MAX_KC / 4;
+constexpr int OUT_PITCH = 2 * SKINNY_MAX_M + 2;   // doubles per row of the transposed result tile (complex: 32 x 2, +2 against bank conflicts)
+static_assert(SKINNY_UNIT * OUT_PITCH * 8 <= WAVE_LDS, "the result tile reuses the wave's LDS region");
 
 // Orders the LDS accesses of one wave: lanes read what other lanes of the same wave wrote.  The LDS executes a wave's
 // instructions in order, so only the compiler has to be kept from moving accesses across this point.
@@ -109,6 +115,20 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
             crow[mb][r] = m < s.M ? (int32_t)(off_of(s.cm, m) * NC) : 0;
         }
     const double ar = s.alpha_re, ai = s.alpha_im, br = s.beta_re, bi = s.beta_im;
+    // C contiguous along m: 16-byte piece id = lane + 64 u of the unit's result tile -> (n of the unit, piece of its row)
+    int32_t ogoff[LOADS], oloff[LOADS];
+    uint32_t ohave = 0;
+    if (s.out_rows) {
+        const int cpr = s.M * NC / 2;   // 16-byte pieces per row of C
+#pragma unroll
+        for (int u = 0; u < LOADS; ++u) {
+            const int id = lane + 64 * u, row = id / cpr, col = id - row * cpr;
+            const bool ok = id < SKINNY_UNIT * cpr;
+            ohave |= (ok ? 1u : 0u) << u;
+            ogoff[u] = ok ? (row * s.c_in * NC + col * 2) * 8 : 0;
+            oloff[u] = ok ? (row * OUT_PITCH + col * 2) * 8 : 0;
+        }
+    }
 
     const int64_t nwaves = (int64_t)gridDim.x * (THREADS / 64);
     int64_t unit = (int64_t)blockIdx.x * (THREADS / 64) + wave;
@@ -164,6 +184,48 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
 
         // ---- results: lane (g, j) holds rows g + 4r (+16), column j of each column block
         double* Cu = reinterpret_cast<double*>(s.C) + off_of(s.cu, unit) * NC;
+        if (s.out_rows) {
+            // tile[n of the unit][m][part] in LDS, then whole rows out: C[n][m] is contiguous along m
+            double* tile = reinterpret_cast<double*>(lds);
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+                if (mb < nmb) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+#pragma unroll
+                        for (int nb = 0; nb < NBLK; ++nb) {
+                            const int m = Mfma<double>::row(lane, r) + 16 * mb, nloc = CX ? 8 * nb + (j >> 1) : j;
+                            tile[nloc * OUT_PITCH + m * NC + (CX ? p : 0)] = acc[mb][nb][r];
+                        }
+                }
+            wave_sync();
+#pragma unroll
+            for (int u = 0; u < LOADS; ++u)
+                if ((ohave >> u) & 1u) {
+                    d2 v = *reinterpret_cast<const d2*>(lds + oloff[u]);
+                    d2* dst = reinterpret_cast<d2*>(reinterpret_cast<unsigned char*>(Cu) + ogoff[u]);
+                    if (!s.plain) {
+                        d2 o;
+                        if constexpr (CX) {
+                            o.x = ar * v.x - ai * v.y;
+                            o.y = ar * v.y + ai * v.x;
+                            if (s.use_beta) {
+                                const d2 old = *dst;
+                                o.x += br * old.x - bi * old.y;
+                                o.y += br * old.y + bi * old.x;
+                            }
+                        } else {
+                            o = v * ar;
+                            if (s.use_beta) o += *dst * br;
+                        }
+                        v = o;
+                    }
+                    __builtin_nontemporal_store(v, dst);
+                }
+            wave_sync();   // the next unit is parked over the tile
+            unit = next;
+            continue;
+        }
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb) {
             if (mb < nmb) {

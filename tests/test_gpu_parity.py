@@ -1145,3 +1145,38 @@ def test_contract_small_operator_strided_rows_and_split_k_order(tf, oracle, dtyp
     tf.HipBackend.execute(plan2, 1.0, [dev(tf, t2), dev(tf, w2)], 0.0, out2)
     assert "gemm_skinny_kernel" in tf.last_kernel()
     assert relerr(out2.to_numpy(), ref2) < 1e-12
+
+
+@pytest.mark.parametrize("dtype", [np.complex128, np.float64])
+@pytest.mark.parametrize("m,k,x,c", [(32, 32, 8, 1024), (20, 13, 64, 80), (16, 32, 1, 4096), (7, 6, 16, 512), (32, 2, 32, 160), (2, 64, 4, 2048)])
+def test_contract_small_operator_with_the_result_contiguous_along_its_columns(tf, oracle, dtype, m, k, x, c):
+    # the other orientation of the same product: T[x, c, k] . W[k, m] -> out[x, c, m], the few columns m adjacent in the
+    # output.  The streaming kernel then transposes each unit's results through LDS.  f64 needs even m and k for it.
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    if k > 32 and cplx:
+        k = 32
+    rng = np.random.default_rng(94)
+    t = rand(rng, (x, c, k), dtype)
+    w = rand(rng, (k, m), dtype)
+    out0 = rand(rng, (x, c, m), dtype)
+    for alpha, beta in [(1.0, 0.0), ((0.5 - 2j, 1.5 + 1j) if cplx else (0.5, -1.5))]:
+        ref = out0.copy()
+        oracle.contract(t, lab("xck"), w, lab("km"), ref, lab("xcm"), alpha=alpha, beta=beta)
+        dout = dev(tf, out0)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab("xcm")), [t.shape, w.shape, ref.shape])
+        tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
+        streamed = cplx or (k % 2 == 0 and m % 2 == 0)
+        assert ("gemm_skinny_kernel" in tf.last_kernel()) == streamed, tf.last_kernel()
+        assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
+    # the same with the output rows padded (a view of a wider buffer) and the long operand's rows reversed
+    wide = rand(rng, (x, c, m + 2), dtype)
+    view = wide[:, :, :m]
+    ref = view.copy()
+    tr = t[:, ::-1]
+    oracle.contract(tr, lab("xck"), w, lab("km"), ref, lab("xcm"), alpha=1.0, beta=0.0)
+    dwide = dev(tf, wide)
+    dview = tf.Tensor(dwide._buf, [x, c, m], dwide.strides(), 0, tf.GpuMemory(0), tf.dtype_code(dtype))
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, tr), dev(tf, w)], 0.0, dview)
+    got = dwide.to_numpy()
+    assert relerr(got[:, :, :m], ref) < 1e-12
+    assert np.array_equal(got[:, :, m:], wide[:, :, m:])          # the padding is untouched
