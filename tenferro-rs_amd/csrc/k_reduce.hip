@@ -320,6 +320,8 @@ struct FastReduceArgs {
     int64_t r_count[MAXR], r_sa[MAXR];
     int32_t r_total, pad_;
     int64_t ks_sa, ks_sc;     // strides of the block-serial kept axis
+    int32_t bf_bit[3];        // BF: the three lowest reduced thread-id bits inside a wave
+    int32_t pad2_;
     int64_t vc_stride;        // C stride between the VEC outputs of one lane (KV)
     double alpha, beta;
 };
@@ -338,7 +340,7 @@ __device__ __forceinline__ RVec<R, N> load_stream(const R* p) {
     return __builtin_bit_cast(RVec<R, N>, __builtin_nontemporal_load(reinterpret_cast<const Raw*>(p)));
 }
 
-template <class R, int VEC, bool KV, int KS>
+template <class R, int VEC, bool KV, int KS, bool BF>
 __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) {
     constexpr int NV = KV ? VEC : 1;
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -413,6 +415,69 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
             }
         }
     }
+    if constexpr (BF) {
+        // Eight accumulators per lane, every lane of a group holding a partial sum of each: a transposing butterfly.
+        // Across reduced bit b0 a lane keeps the four accumulators whose index has its own bit value in place 0 and
+        // hands the other four to its partner, then the same with two across b1 and one across b2 -- seven exchanges
+        // instead of twenty-four, after which the lane owns the output with index (its bits b0, b1, b2) and only
+        // that one value goes through the rest of the fold.
+        static_assert(KS == 8, "the butterfly folds eight block-serial outputs");
+        const int m0 = (tid >> a.bf_bit[0]) & 1, m1 = (tid >> a.bf_bit[1]) & 1, m2 = (tid >> a.bf_bit[2]) & 1;
+        const int x0 = 1 << a.bf_bit[0], x1 = 1 << a.bf_bit[1], x2 = 1 << a.bf_bit[2];
+        double one[NV];
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            double a4[4], a2[2];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const double keep = m0 ? acc[2 * q + 1][j] : acc[2 * q][j], send = m0 ? acc[2 * q][j] : acc[2 * q + 1][j];
+                a4[q] = combine(keep, __shfl_xor(send, x0), op);
+            }
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const double keep = m1 ? a4[2 * q + 1] : a4[2 * q], send = m1 ? a4[2 * q] : a4[2 * q + 1];
+                a2[q] = combine(keep, __shfl_xor(send, x1), op);
+            }
+            const double keep = m2 ? a2[1] : a2[0], send = m2 ? a2[0] : a2[1];
+            one[j] = combine(keep, __shfl_xor(send, x2), op);
+        }
+        const int rest = a.red_bits & ~(x0 | x1 | x2);
+#pragma unroll
+        for (int b = 0; b < 6; ++b)
+            if (rest & (1 << b)) {
+#pragma unroll
+                for (int j = 0; j < NV; ++j) one[j] = combine(one[j], __shfl_xor(one[j], 1 << b), op);
+            }
+        if (rest & 0xc0) {
+#pragma unroll
+            for (int j = 0; j < NV; ++j) lds[j * THREADS + tid] = one[j];
+            __syncthreads();
+            for (int b = 7; b >= 6; --b) {
+                const int bit = 1 << b;
+                if (rest & bit) {
+                    if (!(tid & bit)) {
+#pragma unroll
+                        for (int j = 0; j < NV; ++j) lds[j * THREADS + tid] = combine(lds[j * THREADS + tid], lds[j * THREADS + (tid | bit)], op);
+                    }
+                    __syncthreads();
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NV; ++j) one[j] = lds[j * THREADS + tid];
+        }
+        if ((tid & rest) == 0) {
+            const int k = m0 + 2 * m1 + 4 * m2;
+            R* C = reinterpret_cast<R*>(a.out) + org_out + toff_out + k * a.ks_sc;
+#pragma unroll
+            for (int j = 0; j < NV; ++j) {
+                R* dst = C + j * a.vc_stride;
+                double r = a.alpha * one[j];
+                if (a.use_beta) r += a.beta * (double)*dst;
+                *dst = (R)r;
+            }
+        }
+        return;
+    }
     // lanes that share outputs fold over the reduced thread-id bits: inside a wave with lane exchanges, across
     // waves (bits 6 and 7) through LDS
 #pragma unroll
@@ -459,24 +524,27 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
 }
 
 template <class R, int VEC, bool KV>
-void launch_fast_ks(const FastReduceArgs& fa, dim3 grid, int ks, hipStream_t st) {
+void launch_fast_ks(const FastReduceArgs& fa, dim3 grid, int ks, bool bf, hipStream_t st) {
     const int nv = KV ? VEC : 1;
-    if (ks == 8) {
+    if (ks == 8 && bf) {
+        size_t lds = FAST_MAX_RTAB * sizeof(int64_t) + (size_t)nv * THREADS * sizeof(double);
+        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 8, true>), grid, dim3(THREADS), lds, st, fa);
+    } else if (ks == 8) {
         size_t lds = FAST_MAX_RTAB * sizeof(int64_t) + (size_t)8 * nv * THREADS * sizeof(double);
-        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 8>), grid, dim3(THREADS), lds, st, fa);
+        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 8, false>), grid, dim3(THREADS), lds, st, fa);
     } else {
         size_t lds = FAST_MAX_RTAB * sizeof(int64_t) + (size_t)nv * THREADS * sizeof(double);
-        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 1>), grid, dim3(THREADS), lds, st, fa);
+        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 1, false>), grid, dim3(THREADS), lds, st, fa);
     }
 }
 template <class R>
-void launch_fast(const FastReduceArgs& fa, dim3 grid, int vec, bool kv, int ks, hipStream_t st) {
+void launch_fast(const FastReduceArgs& fa, dim3 grid, int vec, bool kv, int ks, bool bf, hipStream_t st) {
     constexpr int V = 16 / sizeof(R);
     if (vec > 1) {
-        if (kv) launch_fast_ks<R, V, true>(fa, grid, ks, st);
-        else launch_fast_ks<R, V, false>(fa, grid, ks, st);
+        if (kv) launch_fast_ks<R, V, true>(fa, grid, ks, bf, st);
+        else launch_fast_ks<R, V, false>(fa, grid, ks, bf, st);
     } else
-        launch_fast_ks<R, 1, true>(fa, grid, ks, st);
+        launch_fast_ks<R, 1, true>(fa, grid, ks, bf, st);
 }
 
 int ceil_log2(int64_t n) {
@@ -599,8 +667,16 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((uint32_t)blocks);
     const int prof = prof_begin(PROF_REDUCE, stream);
-    if (rbytes == 8) launch_fast<double>(fa, grid, vec, kv, ks, st);
-    else launch_fast<float>(fa, grid, vec, kv, ks, st);
+    // eight block-serial outputs and at least three reduced lane bits inside a wave: the transposing butterfly
+    bool bf = false;
+    if (ks == 8) {
+        int found = 0;
+        for (int b = 0; b < 6 && found < 3; ++b)
+            if (fa.red_bits & (1 << b)) fa.bf_bit[found++] = b;
+        bf = found == 3;
+    }
+    if (rbytes == 8) launch_fast<double>(fa, grid, vec, kv, ks, bf, st);
+    else launch_fast<float>(fa, grid, vec, kv, ks, bf, st);
     prof_end(prof, stream);
     status = hip_check(hipGetLastError(), "reduce kernel launch");
     return true;

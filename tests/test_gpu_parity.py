@@ -1180,3 +1180,34 @@ def test_contract_small_operator_with_the_result_contiguous_along_its_columns(tf
     got = dwide.to_numpy()
     assert relerr(got[:, :, :m], ref) < 1e-12
     assert np.array_equal(got[:, :, m:], wide[:, :, m:])          # the padding is untouched
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_reduce_rows_and_inner_axes_take_the_butterfly_fold(tf, oracle, dtype):
+    # sums over the contiguous axis (row sums) and over an inner axis next to a short kept one: nothing is left to loop
+    # over, so a block handles eight outputs per lane group and folds them with the transposing butterfly.  Exact
+    # integer inputs make a misrouted accumulator visible; max/min and alpha/beta go the same way.
+    rng = np.random.default_rng(95)
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    def ints(shape):
+        x = rng.integers(-9, 10, shape).astype(np.float64)
+        return (x + 1j * rng.integers(-9, 10, shape)).astype(dtype) if cplx else x.astype(dtype)
+    cases = [((32768, 256), [0, 1], [0]),                      # row sums, 128 lanes per row
+             ((16, 16, 16, 16, 16, 16), list(range(6)), [0, 1, 2, 3, 5]),   # inner axis of 16 next to a kept axis of 16
+             ((65536, 64), [0, 1], [0]),                       # two rows per wave
+             ((512, 8, 32, 16), [0, 1, 2, 3], [0, 1, 3])]
+    for shape, ma, mc in cases:
+        a = ints(shape)
+        got, ref = _reduce_check(tf, oracle, a, ma, mc, tf.ReduceOp.Sum, oracle.SUM)
+        if dtype == np.float64:      # (the other element sizes tile these shapes differently; they are checked for their results)
+            assert "8, true>" in tf.last_kernel(), (shape, tf.last_kernel())
+        assert np.array_equal(got, ref), shape
+    a = rand(rng, (32768, 256), dtype)
+    c0 = rand(rng, (32768,), dtype)
+    got, ref = _reduce_check(tf, oracle, a, [0, 1], [0], tf.ReduceOp.Sum, oracle.SUM, alpha=2.0, beta=-0.5, c0=c0)
+    assert relerr(got, ref) < TOL[dtype]
+    if not cplx:
+        for op_tf, op_or in [(tf.ReduceOp.Max, oracle.MAX), (tf.ReduceOp.Min, oracle.MIN)]:
+            got, ref = _reduce_check(tf, oracle, a, [0, 1], [0], op_tf, op_or)
+            assert dtype != np.float64 or "8, true>" in tf.last_kernel()
+            assert np.array_equal(got, ref)
