@@ -321,7 +321,11 @@ struct FastReduceArgs {
     int32_t r_total, pad_;
     int64_t ks_sa, ks_sc;     // strides of the block-serial kept axis
     int32_t bf_bit[3];        // BF: the three lowest reduced thread-id bits inside a wave
-    int32_t pad2_;
+    // few outputs, long serial range: blockIdx.y takes `rps` serial indices and writes raw partial results (mode 1),
+    // a second launch folds the nchunks partials of every output in a fixed order (mode 2); mode 0: no split
+    int32_t mode;
+    int32_t nchunks, rps, nblocks;
+    double* partial;          // [nchunks][nblocks][THREADS][NV]
     int64_t vc_stride;        // C stride between the VEC outputs of one lane (KV)
     double alpha, beta;
 };
@@ -347,8 +351,10 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
     int64_t* rtab = reinterpret_cast<int64_t*>(smem_raw);                               // [r_total]
     double* lds = reinterpret_cast<double*>(smem_raw + FAST_MAX_RTAB * sizeof(int64_t)); // [KS*NV][THREADS]
     const int tid = threadIdx.x;
-    for (int i = tid; i < a.r_total; i += THREADS) {
-        int64_t lin = i, off = 0;
+    const int r_begin = a.mode == 1 ? (int)blockIdx.y * a.rps : 0;
+    const int r_count = a.mode == 2 ? 0 : (a.mode == 1 ? (a.r_total - r_begin < a.rps ? a.r_total - r_begin : a.rps) : a.r_total);
+    for (int i = tid; i < r_count; i += THREADS) {
+        int64_t lin = r_begin + i, off = 0;
 #pragma unroll
         for (int r = 0; r < MAXR; ++r)
             if (r < a.nr) {
@@ -396,13 +402,13 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
         RVec<R, VEC> v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            if (u < a.r_total) v[u] = load_stream<R, VEC>(Ak + rtab[u]);
-        for (int it = 0; it < a.r_total; it += U) {
+            if (u < r_count) v[u] = load_stream<R, VEC>(Ak + rtab[u]);
+        for (int it = 0; it < r_count; it += U) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (it + u >= a.r_total) break;
+                if (it + u >= r_count) break;
                 const RVec<R, VEC> x = v[u];
-                if (it + U + u < a.r_total) v[u] = load_stream<R, VEC>(Ak + rtab[it + U + u]);
+                if (it + U + u < r_count) v[u] = load_stream<R, VEC>(Ak + rtab[it + U + u]);
                 if (KV) {
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) acc[k][j] = combine(acc[k][j], (double)x.v[j], op);
@@ -413,6 +419,22 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
                     acc[k][0] = combine(acc[k][0], s, op);
                 }
             }
+        }
+    }
+    if (KS == 1 && a.mode == 2) {
+        // second launch of a split reduction: the lanes that share an output take the partials of the chunks in turn
+        // (chunk = the lane's reduced bits, compressed, then every P-th) and the ordinary fold below adds them up
+        int part = 0, P = 1;
+        for (int b = 0; b < 8; ++b)
+            if (a.red_bits & (1 << b)) {
+                part |= ((tid >> b) & 1) * P;
+                P <<= 1;
+            }
+        const int wl = tid & ~a.red_bits;
+        for (int ch = part; ch < a.nchunks; ch += P) {
+            const double* src = a.partial + (((int64_t)ch * a.nblocks + blockIdx.x) * THREADS + wl) * NV;
+#pragma unroll
+            for (int j = 0; j < NV; ++j) acc[0][j] = combine(acc[0][j], src[j], op);
         }
     }
     if constexpr (BF) {
@@ -508,6 +530,12 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
         for (int k = 0; k < KS; ++k)
 #pragma unroll
             for (int j = 0; j < NV; ++j) acc[k][j] = lds[(k * NV + j) * THREADS + tid];
+    }
+    if (writer && KS == 1 && a.mode == 1) {
+        double* dst = a.partial + (((int64_t)blockIdx.y * a.nblocks + blockIdx.x) * THREADS + tid) * NV;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) dst[j] = acc[0][j];
+        return;
     }
     if (writer) {
         R* C = reinterpret_cast<R*>(a.out) + org_out + toff_out;
@@ -641,11 +669,24 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
             blocks *= cnt;
         }
     }
-    if (r_total > FAST_MAX_RTAB || blocks > 0x7fffffffll) return false;
+    if (blocks > 0x7fffffffll) return false;
+    // Few outputs and a long serial range: split the range over blockIdx.y (raw partials, then a second launch folds
+    // them) so that the chip is filled; this also lifts the limit of the serial-offset table, which then holds one
+    // chunk.
+    int64_t nchunks = 1, rps = r_total;
+    if (blocks < 512 && r_total >= 64) {
+        nchunks = std::max<int64_t>(1, std::min<int64_t>((2048 + blocks - 1) / blocks, r_total / 16));
+        rps = (r_total + nchunks - 1) / nchunks;
+        if (rps > FAST_MAX_RTAB) rps = FAST_MAX_RTAB;
+        nchunks = (r_total + rps - 1) / rps;
+        if (nchunks > 65535) return false;
+    } else if (r_total > FAST_MAX_RTAB) {
+        return false;
+    }
     // block-serial kept indices when the serial reduction alone gives a thread too few loads
     int ks = 1;
     const int nv = kv ? vec : 1;
-    if (r_total < 8 && fa.ng > 0 && fa.g_count[0] % 8 == 0 && blocks / 8 >= 512 && nv <= 2) {   // nv <= 2: LDS stays under 48 KB
+    if (nchunks == 1 && r_total < 8 && fa.ng > 0 && fa.g_count[0] % 8 == 0 && blocks / 8 >= 512 && nv <= 2) {   // nv <= 2: LDS stays under 48 KB
         ks = 8;
         fa.ks_sa = fa.g_sa[0];
         fa.ks_sc = fa.g_sc[0];
@@ -654,7 +695,6 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
         fa.g_sc[0] *= 8;
         blocks /= 8;
     }
-    if (blocks < 256 && r_total >= 64) return false;   // few outputs, long reduction: the split kernel handles it
 
     fa.r_total = (int32_t)r_total;
     fa.in = a;
@@ -665,7 +705,19 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
     fa.use_beta = !beta.is_zero();
     fa.vc_stride = all[0].a.s[1];
     hipStream_t st = (hipStream_t)stream;
-    dim3 grid((uint32_t)blocks);
+    dim3 grid((uint32_t)blocks, (uint32_t)nchunks);
+    if (nchunks > 1) {
+        void* ws = nullptr;
+        if (int32_t e = workspace(stream, (size_t)nchunks * (size_t)blocks * THREADS * nv * sizeof(double), &ws)) {
+            status = e;
+            return true;
+        }
+        fa.mode = 1;
+        fa.nchunks = (int32_t)nchunks;
+        fa.rps = (int32_t)rps;
+        fa.nblocks = (int32_t)blocks;
+        fa.partial = (double*)ws;
+    }
     const int prof = prof_begin(PROF_REDUCE, stream);
     // eight block-serial outputs and at least three reduced lane bits inside a wave: the transposing butterfly
     bool bf = false;
@@ -678,6 +730,11 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
     if (rbytes == 8) launch_fast<double>(fa, grid, vec, kv, ks, bf, st);
     else launch_fast<float>(fa, grid, vec, kv, ks, bf, st);
     prof_end(prof, stream);
+    if (nchunks > 1) {
+        fa.mode = 2;
+        if (rbytes == 8) launch_fast<double>(fa, dim3((uint32_t)blocks), vec, kv, ks, bf, st);
+        else launch_fast<float>(fa, dim3((uint32_t)blocks), vec, kv, ks, bf, st);
+    }
     status = hip_check(hipGetLastError(), "reduce kernel launch");
     return true;
 }

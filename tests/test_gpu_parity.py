@@ -612,11 +612,10 @@ def test_reduce_fast_path_variants(tf, oracle, dtype):
              [3]]
     for mc in cases:
         got, ref = _reduce_check(tf, oracle, a, m, mc, tf.ReduceOp.Sum, oracle.SUM)
-        # the first two and the fourth must take the tiled fast path for every dtype; 16 outputs ([3]) are too few for it
-        if mc in ([0, 1, 2, 3], [0, 2, 4], [1, 2, 3, 4]):
+        # the first two and the fourth must take the tiled fast path for every dtype, and so must the 16-output case
+        # ([3]: the serial range is split over blocks and folded by a second launch)
+        if mc in ([0, 1, 2, 3], [0, 2, 4], [1, 2, 3, 4], [3]):
             assert "reduce_fast_kernel" in tf.last_kernel(), (mc, tf.last_kernel())
-        if mc == [3]:
-            assert "reduce_fast_kernel" not in tf.last_kernel()
         assert relerr(got, ref) < TOL[dtype], mc
     c0 = rand(rng, (8, 4, 32), dtype)
     got, ref = _reduce_check(tf, oracle, a, m, [0, 2, 4], tf.ReduceOp.Sum, oracle.SUM, alpha=2.0, beta=-0.5, c0=c0)
@@ -1210,4 +1209,36 @@ def test_reduce_rows_and_inner_axes_take_the_butterfly_fold(tf, oracle, dtype):
         for op_tf, op_or in [(tf.ReduceOp.Max, oracle.MAX), (tf.ReduceOp.Min, oracle.MIN)]:
             got, ref = _reduce_check(tf, oracle, a, [0, 1], [0], op_tf, op_or)
             assert dtype != np.float64 or "8, true>" in tf.last_kernel()
+            assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_reduce_few_outputs_split_over_blocks(tf, oracle, dtype):
+    # few outputs and a long reduction: the serial range is split over blocks (raw partials) and a second launch folds
+    # the partials in a fixed order.  Exact integer inputs: any lost or doubled chunk changes the sum.
+    rng = np.random.default_rng(96)
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    def ints(shape):
+        x = rng.integers(-9, 10, shape).astype(np.float64)
+        return (x + 1j * rng.integers(-9, 10, shape)).astype(dtype) if cplx else x.astype(dtype)
+    cases = [((1 << 21,), [0], []),                                   # full sum, one output
+             ((2048, 512), [0, 1], [1]),                              # column sums
+             ((32, 64, 64, 32), [0, 1, 2, 3], [0, 3]),                # two middle axes
+             ((3, 1 << 19), [0, 1], [0])]                             # three long rows
+    for shape, ma, mc in cases:
+        a = ints(shape)
+        got, ref = _reduce_check(tf, oracle, a, ma, mc, tf.ReduceOp.Sum, oracle.SUM)
+        assert "reduce_fast_kernel" in tf.last_kernel(), (shape, tf.last_kernel())
+        assert np.array_equal(got, ref), shape
+        got2, _ = _reduce_check(tf, oracle, a, ma, mc, tf.ReduceOp.Sum, oracle.SUM)
+        assert np.array_equal(got, got2)                              # same bits on every run
+    a = rand(rng, (2048, 512), dtype)
+    c0 = rand(rng, (512,), dtype)
+    got, ref = _reduce_check(tf, oracle, a, [0, 1], [1], tf.ReduceOp.Sum, oracle.SUM, alpha=2.0, beta=-0.5, c0=c0)
+    assert relerr(got, ref) < TOL[dtype]
+    if not cplx:
+        for op_tf, op_or in [(tf.ReduceOp.Max, oracle.MAX), (tf.ReduceOp.Min, oracle.MIN)]:
+            got, ref = _reduce_check(tf, oracle, a, [0, 1], [1], op_tf, op_or)
+            assert np.array_equal(got, ref)
+            got, ref = _reduce_check(tf, oracle, a.reshape(-1), [0], [], op_tf, op_or)
             assert np.array_equal(got, ref)
