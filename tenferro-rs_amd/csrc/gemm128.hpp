@@ -254,9 +254,11 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
         tile_m = tm.y;
         tile_n = tm.z;
     } else {
-        const uint64_t lb = logical_block((uint64_t)blockIdx.z * gridDim.x + blockIdx.x, (uint64_t)gridDim.x * gridDim.z);
-        const uint32_t lz = (uint32_t)(lb / gridDim.x);
-        tile_of((uint32_t)(lb % gridDim.x), g.tiles_m, g.tiles_n, tile_m, tile_n);
+        // one-dimensional grid: tiles of one (batch, split) pair are adjacent logical positions
+        const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n;
+        const uint64_t lb = logical_block(blockIdx.x, gridDim.x);
+        const uint32_t lz = (uint32_t)(lb / tiles);
+        tile_of((uint32_t)(lb % tiles), g.tiles_m, g.tiles_n, tile_m, tile_n);
         split = (int)(lz % (uint32_t)g.nsplit);
         batch = lz / (uint32_t)g.nsplit;
         Ap += off_of(g.ab, batch) * (int64_t)sizeof(E);

@@ -122,9 +122,11 @@ __global__ void __launch_bounds__((Cfg<R, CX, BM, BN>::NT), 2) gemm_kernel(GemmA
         tile_m = tm.y;
         tile_n = tm.z;
     } else {
-        const uint64_t lb = logical_block((uint64_t)blockIdx.z * gridDim.x + blockIdx.x, (uint64_t)gridDim.x * gridDim.z);
-        const uint32_t lz = (uint32_t)(lb / gridDim.x);
-        tile_of((uint32_t)(lb % gridDim.x), g.tiles_m, g.tiles_n, tile_m, tile_n);
+        // one-dimensional grid: tiles of one (batch, split) pair are adjacent logical positions
+        const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n;
+        const uint64_t lb = logical_block(blockIdx.x, gridDim.x);
+        const uint32_t lz = (uint32_t)(lb / tiles);
+        tile_of((uint32_t)(lb % tiles), g.tiles_m, g.tiles_n, tile_m, tile_n);
         split = (int)(lz % (uint32_t)g.nsplit);
         batch = lz / (uint32_t)g.nsplit;
     }
@@ -324,6 +326,55 @@ __global__ void __launch_bounds__(THREADS) splitk_finalize_kernel(GemmArgs g) {
         }
         dst[0] = rr;
         dst[1] = ri;
+    } else {
+        R r = ar * sr;
+        if (g.use_beta) r += br * dst[0];
+        dst[0] = r;
+    }
+}
+
+// Many splits over few outputs (one tile with a very long k): sixteen lanes share an output, lane y adds the partials
+// of splits y, y + 16, ... in increasing order and lane 0 adds the sixteen sums in order -- a fixed order, so the
+// result does not depend on scheduling.
+template <class R, bool CX>
+__global__ void __launch_bounds__(THREADS) splitk_finalize_deep_kernel(GemmArgs g) {
+    constexpr int SL = 16, OUT = THREADS / SL, NC = CX ? 2 : 1;
+    __shared__ R part[SL][OUT][NC];
+    const int tx = threadIdx.x % OUT, ty = threadIdx.x / OUT;
+    const int64_t total = g.nbatch * g.M * g.N;
+    const int64_t idx = (int64_t)blockIdx.x * OUT + tx;
+    const bool ok = idx < total;
+    const int64_t plane = total * NC;
+    R sr = 0, si = 0;
+    if (ok) {
+        const R* p = reinterpret_cast<const R*>(g.partial) + idx * NC;
+        for (int s = ty; s < g.nsplit; s += SL) {
+            sr += p[s * plane];
+            if (CX) si += p[s * plane + 1];
+        }
+    }
+    part[ty][tx][0] = sr;
+    if (CX) part[ty][tx][NC - 1] = si;
+    __syncthreads();
+    if (ty != 0 || !ok) return;
+    sr = 0;
+    si = 0;
+    for (int y = 0; y < SL; ++y) {
+        sr += part[y][tx][0];
+        if (CX) si += part[y][tx][NC - 1];
+    }
+    const int64_t n = idx % g.N, t = idx / g.N, m = t % g.M, b = t / g.M;
+    R* dst = reinterpret_cast<R*>(g.C) + (off_of(g.cb, b) + off_of(g.cm, m) + off_of(g.cn, n)) * NC;
+    const R ar = (R)g.alpha_re, ai = (R)g.alpha_im, br = (R)g.beta_re, bi = (R)g.beta_im;
+    if (CX) {
+        R rr = ar * sr - ai * si, ri = ar * si + ai * sr;
+        if (g.use_beta) {
+            R cr = dst[0], ci = dst[NC - 1];
+            rr += br * cr - bi * ci;
+            ri += br * ci + bi * cr;
+        }
+        dst[0] = rr;
+        dst[NC - 1] = ri;
     } else {
         R r = ar * sr;
         if (g.use_beta) r += br * dst[0];
@@ -644,7 +695,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     int nsplit = 1;
     if (tiles < 256 && kstages >= 16) {
         nsplit = (int)std::min<int64_t>((512 + tiles - 1) / tiles, kstages / 8);
-        nsplit = std::max(1, std::min(nsplit, 64));
+        nsplit = std::max(1, std::min(nsplit, 512));   // a single tile with a very long k still fills the chip
     }
     if (skinny) nsplit = 1;
     int64_t kps = ((kstages + nsplit - 1) / nsplit) * bke;
@@ -653,7 +704,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     g.k_per_split = kps;
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((NR + bm - 1) / bm);
-    if ((int64_t)g.tiles_m * g.tiles_n > 0x7fffffffll || nb * nsplit > 65535) {
+    if ((double)g.tiles_m * (double)g.tiles_n * (double)nb * (double)nsplit > 2147483647.0) {
         release_packed();
         return set_error(TFH_ERR_INVALID_ARGUMENT, "contraction too large for one launch (tiles %lld, batch*split %lld)",
                          (long long)g.tiles_m * g.tiles_n, (long long)(nb * nsplit));
@@ -777,7 +828,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         g.bias_b32 = (uint32_t)(-lo_b * (int64_t)eb);
     }
     if (nsplit > 1) g.partial = ws + (cached ? 0 : table_bytes);
-    dim3 grid((uint32_t)(g.tiles_m * g.tiles_n), 1, (uint32_t)(nb * nsplit));
+    dim3 grid((uint32_t)((int64_t)g.tiles_m * g.tiles_n * nb * nsplit), 1, 1);
     const int prof = prof_begin(PROF_CONTRACT, stream);
     if (skinny) {
         SkinnyArgs sk;
@@ -798,6 +849,17 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     prof_end(prof, stream);
     release_packed();   // stream-ordered: the next user of these blocks is enqueued after this kernel
     if (int32_t e = hip_check(hipGetLastError(), "contraction kernel launch")) return e;
+    if (nsplit > 32) {
+        const int64_t total = nb * M * N;
+        dim3 g2((uint32_t)((total + 15) / 16));
+        switch (dtype) {
+            case TFH_F32: hipLaunchKernelGGL((splitk_finalize_deep_kernel<float, false>), g2, dim3(THREADS), 0, st, g); break;
+            case TFH_F64: hipLaunchKernelGGL((splitk_finalize_deep_kernel<double, false>), g2, dim3(THREADS), 0, st, g); break;
+            case TFH_C64: hipLaunchKernelGGL((splitk_finalize_deep_kernel<float, true>), g2, dim3(THREADS), 0, st, g); break;
+            default: hipLaunchKernelGGL((splitk_finalize_deep_kernel<double, true>), g2, dim3(THREADS), 0, st, g); break;
+        }
+        return hip_check(hipGetLastError(), "split-K finalize launch");
+    }
     if (nsplit > 1) {
         // 16-byte fold: C contiguous along n, whole vectors per row, every row of C on a 16-byte boundary
         const int64_t vec = 16 / rb, ncx = cx ? 2 : 1;

@@ -1242,3 +1242,39 @@ def test_reduce_few_outputs_split_over_blocks(tf, oracle, dtype):
             assert np.array_equal(got, ref)
             got, ref = _reduce_check(tf, oracle, a.reshape(-1), [0], [], op_tf, op_or)
             assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_contract_one_tile_with_a_very_long_k_and_many_batches(tf, oracle, dtype):
+    # a single output tile under a k of several hundred thousand: the range is split hundreds of ways and the partials
+    # are folded by the many-splits kernel (fixed order: two runs give the same bits); and a batch count above 65535
+    # (more (batch, split) pairs than one grid dimension holds)
+    rng = np.random.default_rng(97)
+    m, n, k = 40, 24, 300000
+    a, b = rand(rng, (m, k), dtype), rand(rng, (n, k), dtype)
+    ref = np.empty((m, n), dtype)
+    oracle.contract(a, lab("mk"), b, lab("nk"), ref, lab("mn"))
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("mk"), lab("nk"), lab("mn")), [a.shape, b.shape, [m, n]])
+    da, db = dev(tf, a), dev(tf, b)
+    runs = []
+    for _ in range(2):
+        out = tf.Tensor.empty([m, n], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        tf.HipBackend.execute(plan, 1.0, [da, db], 0.0, out)
+        runs.append(out.to_numpy())
+    assert relerr(runs[0], ref) < 10 * TOL[dtype]
+    assert runs[0].tobytes() == runs[1].tobytes()
+    c0 = rand(rng, (m, n), dtype)
+    ref2 = c0.copy()
+    oracle.contract(a, lab("mk"), b, lab("nk"), ref2, lab("mn"), alpha=0.5, beta=-1.0)
+    dc = dev(tf, c0)
+    tf.HipBackend.execute(plan, 0.5, [da, db], -1.0, dc)
+    assert relerr(dc.to_numpy(), ref2) < 10 * TOL[dtype]
+    # 70000 batches of a 3 x 5 x 4 product
+    nb = 70000
+    x, y = rand(rng, (nb, 3, 5), dtype), rand(rng, (nb, 5, 4), dtype)
+    ref3 = np.empty((nb, 3, 4), dtype)
+    oracle.contract(x, lab("bik"), y, lab("bkj"), ref3, lab("bij"))
+    out3 = tf.Tensor.empty([nb, 3, 4], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    plan3 = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("bik"), lab("bkj"), lab("bij")), [x.shape, y.shape, [nb, 3, 4]])
+    tf.HipBackend.execute(plan3, 1.0, [dev(tf, x), dev(tf, y)], 0.0, out3)
+    assert relerr(out3.to_numpy(), ref3) < TOL[dtype]
