@@ -108,6 +108,10 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
 // C = alpha*A*B + beta*C over classified axes
 int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes axes, Scalar alpha,
                         Scalar beta, void* stream);
+// Matrix-vector-like contractions (one free group empty): the streaming product-reduction kernel of k_dot.hip.  Returns
+// false when the shape is not one it tiles; true when it launched (status holds the outcome).  Axis strides: A, B, C.
+bool try_dot(int dtype, const void* a, const void* b, void* c, std::vector<Axis> kept, std::vector<Axis> red, Scalar alpha,
+             Scalar beta, void* stream, int32_t& status);
 int32_t grouped_plan_init(tfh_plan& plan);
 int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* inputs, Scalar beta, tfh_view* outputs,
                        void* stream);

@@ -545,6 +545,15 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         if (beta.is_zero()) return launch_fill(dtype, c, out, Scalar{0, 0}, stream);
         return launch_copy(dtype, c, c, out, beta, Scalar{0, 0}, false, stream);
     }
+    // One free group empty (matrix-vector, vector-matrix, dot and batched dot products): there is nothing for a tile
+    // of MFMAs to reuse -- a reduction of the elementwise product, bound by HBM (k_dot.hip)
+    if (M == 1 || N == 1) {
+        std::vector<Axis> kept, red = ax.K;
+        for (auto* grp : {&ax.batch, &ax.M, &ax.N})
+            for (auto& x : *grp) kept.push_back(x);
+        int32_t st_dot = TFH_OK;
+        if (try_dot(dtype, a, b, c, kept, red, alpha, beta, stream, st_dot)) return st_dot;
+    }
     // lanes of the epilogue run along n: put C's fastest axis in the N group (swap operands if needed)
     if (min_stride(ax.M, 2) < min_stride(ax.N, 2)) {
         std::swap(a, b);

@@ -1278,3 +1278,66 @@ def test_contract_one_tile_with_a_very_long_k_and_many_batches(tf, oracle, dtype
     plan3 = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("bik"), lab("bkj"), lab("bij")), [x.shape, y.shape, [nb, 3, 4]])
     tf.HipBackend.execute(plan3, 1.0, [dev(tf, x), dev(tf, y)], 0.0, out3)
     assert relerr(out3.to_numpy(), ref3) < TOL[dtype]
+
+
+DOT_CASES = [
+    ("mk,k->m", dict(m=512, k=1024)),                 # matrix-vector, rows contiguous in k
+    ("km,k->m", dict(m=512, k=1024)),                 # ... columns: lanes along m, the vector element broadcast
+    ("k,kn->n", dict(n=2048, k=256)),                 # vector-matrix
+    ("k,k->", dict(k=1 << 18)),                       # dot product: one output, the range split over blocks
+    ("bi,bi->b", dict(b=4096, i=256)),                # batched dot
+    ("bmk,bk->bm", dict(b=16, m=64, k=512)),          # batched matrix-vector
+    ("abk,kb->ab", dict(a=32, b=64, k=128)),          # the second operand holds the modes in another order
+    ("mk,k->m", dict(m=100, k=36)),                   # extents that do not tile: the tiled kernels take it
+]
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("case", DOT_CASES, ids=[c[0] + "-" + "x".join(str(v) for v in c[1].values()) for c in DOT_CASES])
+def test_contract_with_an_empty_free_group_takes_the_product_reduction_kernel(tf, oracle, dtype, case):
+    pattern, ext = case
+    ins, mc = pattern.split("->")
+    ma, mb = ins.split(",")
+    rng = np.random.default_rng(98)
+    a = rand(rng, [ext[l] for l in ma], dtype)
+    b = rand(rng, [ext[l] for l in mb], dtype)
+    cshape = [ext[l] for l in mc]
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    tol = 10 * TOL[dtype]
+    for alpha, beta in [(1.0, 0.0), ((0.7 - 1.1j, -0.3 + 0.2j) if cplx else (0.7, -0.3))]:
+        c0 = rand(rng, cshape, dtype) if cshape else np.array(rng.standard_normal(), dtype)
+        ref = c0.copy()
+        oracle.contract(a, lab(ma), b, lab(mb), ref, lab(mc), alpha=alpha, beta=beta)
+        out = dev(tf, c0) if cshape else tf.Tensor.zeros([], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        if not cshape:
+            ref = np.empty([], dtype)
+            oracle.contract(a, lab(ma), b, lab(mb), ref, lab(mc), alpha=alpha, beta=0.0)
+            beta = 0.0
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [a.shape, b.shape, cshape])
+        tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, out)
+        tiled = "dot_fast_kernel" in tf.last_kernel()
+        assert tiled == (ext.get("k", 0) != 36), tf.last_kernel()
+        assert relerr(out.to_numpy(), ref) < tol, (alpha, beta)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.complex128, np.float32])
+def test_product_reduction_on_strided_and_reversed_views(tf, oracle, dtype):
+    # operands seen through stepped, reversed and offset views: scalar loads, negative strides
+    rng = np.random.default_rng(99)
+    big = rand(rng, (256, 2 * 512 + 3), dtype)
+    a = big[::-1, 1:1025:2]                       # [256, 512], rows reversed, every other column
+    x = rand(rng, (3 * 512,), dtype)[::3]
+    ref = np.empty((256,), dtype)
+    oracle.contract(a, lab("mk"), x, lab("k"), ref, lab("m"))
+    out = tf.Tensor.empty([256], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("mk"), lab("k"), lab("m")), [a.shape, x.shape, [256]])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, x)], 0.0, out)
+    assert "dot_fast_kernel" in tf.last_kernel()
+    assert relerr(out.to_numpy(), ref) < 10 * TOL[dtype]
+    # integer inputs: exact, and a mode of the vector that the matrix lacks is summed too ("mk,kj->m")
+    ai = rng.integers(-5, 6, (128, 256)).astype(dtype)
+    bi = rng.integers(-5, 6, (256, 4)).astype(dtype)
+    out2 = tf.Tensor.empty([128], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    plan2 = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("mk"), lab("kj"), lab("m")), [ai.shape, bi.shape, [128]])
+    tf.HipBackend.execute(plan2, 1.0, [dev(tf, ai), dev(tf, bi)], 0.0, out2)
+    assert np.array_equal(out2.to_numpy(), np.einsum("mk,kj->m", ai, bi))
