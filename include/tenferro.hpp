@@ -605,11 +605,11 @@ template <class T>
 void einsum_into(const std::string& notation, const std::vector<const Tensor<T>*>& operands, T alpha, T beta, Tensor<T>& output) {   // :500-543
     einsum_with_subscripts_into(Subscripts::parse(notation), operands, alpha, beta, output);
 }
-// allocating variants (:393-434): the result is row-major in the operands' memory space
+// allocating variants (:393-434): the result is column-major (the order of the reference's examples) in the operands' memory space
 template <class T>
 Tensor<T> einsum_with_plan(const ContractionTree& tree, const std::vector<const Tensor<T>*>& operands) {
     const LogicalMemorySpace s = detail::common_space(operands);
-    Tensor<T> out = Tensor<T>::uninit(tree.output_dims(), s, MemoryOrder::RowMajor);
+    Tensor<T> out = Tensor<T>::uninit(tree.output_dims(), s, MemoryOrder::ColumnMajor);
     detail::run_tree(tree, operands, T(1), T(0), out, 0);
     return out;
 }
@@ -627,7 +627,7 @@ template <class T>
 Tensor<T> einsum_with_plan_owned(const ContractionTree& tree, std::vector<Tensor<T>> operands) {
     auto ptrs = detail::pointers(operands);
     const LogicalMemorySpace s = detail::common_space(ptrs);
-    Tensor<T> out = Tensor<T>::uninit(tree.output_dims(), s, MemoryOrder::RowMajor);
+    Tensor<T> out = Tensor<T>::uninit(tree.output_dims(), s, MemoryOrder::ColumnMajor);
     uint64_t donate = 0;   // only buffers nobody else can see may be overwritten
     for (size_t i = 0; i < operands.size() && i < 64; ++i)
         if (operands[i].sole_owner()) donate |= 1ull << i;
