@@ -357,14 +357,12 @@ bool try_dot(int dtype, const void* a, const void* b, void* c, std::vector<Axis>
     }
     if (blocks > 0x7fffffffll || r_total > 0x7fffffffll) return false;
     int64_t nchunks = 1, rps = r_total;
-    if (blocks < 512 && r_total >= 64) {
+    if ((blocks < 512 && r_total >= 64) || r_total > MAX_RTAB) {   // (a serial range longer than the offset table is split as well)
         nchunks = std::max<int64_t>(1, std::min<int64_t>((2048 + blocks - 1) / blocks, r_total / 16));
         rps = (r_total + nchunks - 1) / nchunks;
         if (rps > MAX_RTAB) rps = MAX_RTAB;
         nchunks = (r_total + rps - 1) / rps;
         if (nchunks > 65535) return false;
-    } else if (r_total > MAX_RTAB) {
-        return false;
     }
     const int nv = cx ? 2 : (kv ? vec : 1);
     da.r_total = (int32_t)r_total;

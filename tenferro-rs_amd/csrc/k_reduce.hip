@@ -674,14 +674,12 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
     // them) so that the chip is filled; this also lifts the limit of the serial-offset table, which then holds one
     // chunk.
     int64_t nchunks = 1, rps = r_total;
-    if (blocks < 512 && r_total >= 64) {
+    if ((blocks < 512 && r_total >= 64) || r_total > FAST_MAX_RTAB) {   // (a serial range longer than the offset table is split as well)
         nchunks = std::max<int64_t>(1, std::min<int64_t>((2048 + blocks - 1) / blocks, r_total / 16));
         rps = (r_total + nchunks - 1) / nchunks;
         if (rps > FAST_MAX_RTAB) rps = FAST_MAX_RTAB;
         nchunks = (r_total + rps - 1) / rps;
         if (nchunks > 65535) return false;
-    } else if (r_total > FAST_MAX_RTAB) {
-        return false;
     }
     // block-serial kept indices when the serial reduction alone gives a thread too few loads
     int ks = 1;
