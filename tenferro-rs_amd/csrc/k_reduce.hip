@@ -786,6 +786,14 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
     for (auto& x : all) {
         if (bits == 0 || nt == MAXT) break;
         int t = std::min(ceil_log2(x.a.n), bits);
+        if (x.red && x.a.n >= 64) {
+            // leave a thread at least eight serial steps along a reduced axis: a short row spread over all 256 lanes
+            // would be one load per thread and a full fold per row (rows of 300 f64: 0.6 TB/s).  Extents below 64
+            // keep their lanes (as serial axes they would count against the limit on serial reduced axes).
+            int cap = 0;
+            while (((int64_t)16 << cap) <= x.a.n) ++cap;
+            t = std::min(t, cap);
+        }
         if (t == 0) continue;
         x.tl = t;
         bits -= t;
