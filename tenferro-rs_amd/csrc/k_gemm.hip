@@ -702,7 +702,31 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     if (bm == 128 && tiles_for(128) < 192 && kstages < 32 && tiles_for(64) >= 2 * tiles_for(128)) bm = 64;
     const int64_t tiles = tiles_for(bm);
     int nsplit = 1;
-    if (tiles < 256 && kstages >= 16) {
+    if (bm == 128 && tiles >= 32 && kstages >= 16) {
+        // 128x128 tiles: 512 blocks are resident at a time (two per CU).  Estimated time of a split count s, in us, from
+        // what the kernel measures on this device: a block-stage takes 1.95 us of a CU's matrix cores, a block costs
+        // about eight more stages of prologue and epilogue, two blocks sharing a CU overlap fully, one alone leaves
+        // latency exposed (x1.25), and the fold moves the partials twice.  Picks the s with the least estimate: it
+        // trades the idle tail of a partly filled last round against per-block overhead and partial traffic.
+        auto estimate = [&](int s_) {
+            const double per_block = ((double)((kstages + s_ - 1) / s_) + 8.0) * 1.95;
+            const int64_t blocks = tiles * s_, full = blocks / 512, rem = blocks % 512;
+            double t = (double)full * 2.0 * per_block;
+            if (rem > 256) t += 2.0 * per_block;
+            else if (rem > 0) t += 1.25 * per_block;
+            if (s_ > 1) t += 3.0 + (double)s_ * (double)(nb * M * NR * rb) * 2.0 / 10e6;
+            return t;
+        };
+        const int smax = (int)std::min<int64_t>(16, kstages / 8);
+        double best = estimate(1);
+        for (int s_ = 2; s_ <= smax; ++s_) {
+            const double t = estimate(s_);
+            if (t < best * 0.97) {   // a split has to pay for itself clearly
+                best = t;
+                nsplit = s_;
+            }
+        }
+    } else if (tiles < 256 && kstages >= 16) {
         nsplit = (int)std::min<int64_t>((512 + tiles - 1) / tiles, kstages / 8);
         nsplit = std::max(1, std::min(nsplit, 512));   // a single tile with a very long k still fills the chip
     }
