@@ -189,7 +189,7 @@ def run_c2(h):
                                  "kernel": "copy_kernel<u64, OpCopy, 16, 2, 2, false, true>", "kernel_ms": pms}, "algorithmic_bytes": pbytes},
         "reduce": {"roofline": {"bound": "hbm", "achieved": rbytes / (rms * 1e-3) / 1e9, "peak": PEAK["hbm"], "unit": "GB/s",
                                 "frac": rbytes / (rms * 1e-3) / 1e9 / PEAK["hbm"], "traffic": TRAFFIC["c2_reduce"],
-                                "kernel": "reduce_fast_kernel<double, 2, true, 1>", "kernel_ms": rms}, "algorithmic_bytes": rbytes},
+                                "kernel": "reduce_fast_kernel<double, 2, true, 1, false>", "kernel_ms": rms}, "algorithmic_bytes": rbytes},
     }
     if h.cpu:
         P = np.empty(shape)
