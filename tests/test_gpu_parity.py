@@ -1341,3 +1341,91 @@ def test_product_reduction_on_strided_and_reversed_views(tf, oracle, dtype):
     plan2 = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("mk"), lab("kj"), lab("m")), [ai.shape, bi.shape, [128]])
     tf.HipBackend.execute(plan2, 1.0, [dev(tf, ai), dev(tf, bi)], 0.0, out2)
     assert np.array_equal(out2.to_numpy(), np.einsum("mk,kj->m", ai, bi))
+
+
+def _pow2_extent(rng, big):
+    """Extents that tile without partial tiles: a power of two, sometimes times 3 or 5 on a large one."""
+    e = int(2 ** rng.integers(0, 8 if big else 4))
+    if big and e >= 16 and rng.integers(0, 3) == 0:
+        e *= int(rng.choice([3, 5]))
+    return e
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_product_reduction_random_shapes(tf, oracle, dtype):
+    # random contractions with one free group empty, over extents the product-reduction kernel tiles: random mode
+    # structure (batch modes, modes only one operand has, several contracted modes), random axis orders, dense or
+    # stepped / reversed views, alpha/beta.  Most cases must reach that kernel.
+    rng = np.random.default_rng(101)
+    hits = 0
+    ncase = 40
+    for case in range(ncase):
+        labels = list("abcdefgh")
+        rng.shuffle(labels)
+        nb, nfree, nk = int(rng.integers(0, 3)), int(rng.integers(0, 3)), int(rng.integers(1, 4))
+        batch, free, kk = labels[:nb], labels[nb:nb + nfree], labels[nb + nfree:nb + nfree + nk]
+        ext = {l: _pow2_extent(rng, True) for l in batch + free + kk}
+        while np.prod([ext[l] for l in batch + free + kk], dtype=np.float64) > 4e6:
+            l = max(ext, key=ext.get)
+            ext[l] = max(1, ext[l] // 4)
+        # the free modes belong to the first operand; the second holds batch and contracted modes (and sometimes lacks one)
+        ma, mb, mc = batch + free + kk, batch + kk, batch + free
+        if len(kk) > 1 and rng.integers(0, 4) == 0:
+            mb = batch + kk[:-1]                      # a contracted mode only the first operand has: summed over it
+        if rng.integers(0, 2):
+            ma, mb = mb, ma
+        ma, mb, mc = list(ma), list(mb), list(mc)
+        rng.shuffle(ma); rng.shuffle(mb); rng.shuffle(mc)
+        if not ma or not mb:
+            continue
+        plain = case % 3 != 0
+        mk = (lambda shape: rand(rng, shape, dtype)) if plain else (lambda shape: _random_view(rng, shape, dtype))
+        a, b = mk([ext[l] for l in ma]), mk([ext[l] for l in mb])
+        cshape = [ext[l] for l in mc]
+        cplx = np.issubdtype(dtype, np.complexfloating)
+        use_beta = bool(rng.integers(0, 2)) and len(cshape) > 0
+        alpha, beta = ((0.7 - 1.1j, (-0.3 + 0.2j) if use_beta else 0.0) if cplx else (0.7, -0.3 if use_beta else 0.0))
+        c0 = rand(rng, cshape, dtype) if use_beta else np.full(cshape, np.nan, dtype)
+        ref = c0.copy()
+        oracle.contract(a, lab(ma), b, lab(mb), ref, lab(mc), alpha=alpha, beta=beta)
+        out = dev(tf, c0) if cshape else tf.Tensor.empty([], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [a.shape, b.shape, cshape])
+        print("case", case, "".join(ma), "".join(mb), "".join(mc), ext, "plain" if plain else "views", flush=True)
+        tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, out)
+        hits += "dot_fast_kernel" in tf.last_kernel()
+        err = relerr(out.to_numpy(), ref)
+        assert err < 10 * TOL[dtype], (case, ma, mb, mc, ext, err, tf.last_kernel())
+    assert hits >= ncase // 2, hits
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_reduce_random_shapes_that_tile(tf, oracle, dtype):
+    # random reductions over power-of-two-friendly extents: every variant of the fast kernel (vector / scalar loads,
+    # contiguous axis kept or reduced, eight block-serial outputs with the butterfly fold, the serial range split over
+    # blocks) is reached by some case; sums, max/min, alpha/beta, dense and strided views
+    rng = np.random.default_rng(102)
+    kernels = set()
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    for case in range(60):
+        rank = int(rng.integers(1, 6))
+        shape = [_pow2_extent(rng, True) for _ in range(rank)]
+        while np.prod(shape, dtype=np.float64) > 4e6:
+            shape[int(np.argmax(shape))] //= 4
+        keep = [d for d in range(rank) if rng.integers(0, 2)]
+        rng.shuffle(keep)
+        a = rand(rng, shape, dtype) if case % 3 else _random_view(rng, shape, dtype)
+        op_tf, op_or = (tf.ReduceOp.Sum, oracle.SUM)
+        if not cplx and case % 5 == 0:
+            op_tf, op_or = [(tf.ReduceOp.Max, oracle.MAX), (tf.ReduceOp.Min, oracle.MIN)][case % 2]
+        oshape = [shape[d] for d in keep]
+        use_beta = case % 4 == 0 and op_or == oracle.SUM and len(oshape) > 0
+        c0 = rand(rng, oshape, dtype) if use_beta else None
+        print("case", case, shape, keep, flush=True)
+        got, ref = _reduce_check(tf, oracle, a, list(range(rank)), keep, op_tf, op_or, alpha=2.0 if use_beta else 1.0,
+                                 beta=-0.5 if use_beta else 0.0, c0=c0)
+        kernels.add(tf.last_kernel())
+        if op_or == oracle.SUM:
+            assert relerr(got, ref) < 10 * TOL[dtype], (case, shape, keep, tf.last_kernel())
+        else:
+            assert np.array_equal(got, ref), (case, shape, keep)
+    assert any("reduce_fast_kernel" in k for k in kernels), kernels
