@@ -105,6 +105,10 @@ int32_t launch_emul(int dtype, const void* a, const void* b, void* c, std::vecto
 // C[kept] = alpha*reduce(A[kept, red]) + beta*C ; kept: s[0]=A, s[1]=C ; red: s[0]=A
 int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, std::vector<Axis> red, int reduce_op,
                       Scalar alpha, Scalar beta, void* stream);
+// The general (any extents, any strides) reduction kernel; with b != nullptr the reduced quantity is the product A*B of
+// two operands read at the same coordinates (sum only).  Axis slots here: 0 = A, 1 = C, 2 = B.
+int32_t launch_reduce_general(int dtype, const void* a, const void* b, void* c, std::vector<Axis> kept, std::vector<Axis> red,
+                              int reduce_op, Scalar alpha, Scalar beta, void* stream);
 // C = alpha*A*B + beta*C over classified axes
 int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes axes, Scalar alpha,
                         Scalar beta, void* stream);

@@ -553,6 +553,22 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
             for (auto& x : *grp) kept.push_back(x);
         int32_t st_dot = TFH_OK;
         if (try_dot(dtype, a, b, c, kept, red, alpha, beta, stream, st_dot)) return st_dot;
+        // extents that kernel does not tile: the general reduction kernel with a second operand (axis slots A, C, B),
+        // the operand with more elements first.  Shapes beyond its axis limits go on to the tiled kernels.
+        auto elems = [&](int slot) {
+            double n = 1;
+            for (auto* grp : {&kept, &red})
+                for (auto& x : *grp)
+                    if (x.s[slot] != 0) n *= (double)x.n;
+            return n;
+        };
+        const int pa = elems(1) > elems(0) ? 1 : 0, pb = 1 - pa;
+        std::vector<Axis> kept2, red2;
+        for (auto& x : kept) kept2.push_back(Axis{x.n, {x.s[pa], x.s[2], x.s[pb]}, x.label});
+        for (auto& x : red) red2.push_back(Axis{x.n, {x.s[pa], 0, x.s[pb]}, x.label});
+        if (launch_reduce_general(dtype, pa == 0 ? a : b, pa == 0 ? b : a, c, kept2, red2, TFH_REDUCE_SUM, alpha, beta, stream) == TFH_OK)
+            return TFH_OK;
+        clear_error();
     }
     // lanes of the epilogue run along n: put C's fastest axis in the N group (swap operands if needed)
     if (min_stride(ax.M, 2) < min_stride(ax.N, 2)) {

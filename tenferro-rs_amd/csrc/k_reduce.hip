@@ -27,6 +27,7 @@ constexpr int THREADS = 256;
 
 struct ReduceArgs {
     const void* in;
+    const void* in_b;      // second operand of a product reduction (DOT), addressed through t_sb / g_sb / r_sb
     void* out;
     double* partial;       // [nchunks][kept_slots] accumulators (complex: 2 doubles each)
     int32_t nt, ng, nr;
@@ -37,12 +38,12 @@ struct ReduceArgs {
     int32_t use_beta;
     // thread tile, in A-memory order
     int32_t t_shift[MAXT], t_mask[MAXT], t_red[MAXT];
-    int64_t t_sa[MAXT], t_sc[MAXT], t_n[MAXT];
+    int64_t t_sa[MAXT], t_sc[MAXT], t_n[MAXT], t_sb[MAXT];
     // kept outer axes -> blockIdx.x
-    int64_t g_count[MAXG], g_sa[MAXG], g_sc[MAXG];
+    int64_t g_count[MAXG], g_sa[MAXG], g_sc[MAXG], g_sb[MAXG];
     int32_t g_tid[MAXG], g_text[MAXG];
     // serial reduced axes (innermost first)
-    int64_t r_count[MAXR], r_sa[MAXR], r_n[MAXR];
+    int64_t r_count[MAXR], r_sa[MAXR], r_n[MAXR], r_sb[MAXR];
     int32_t r_tid[MAXR], r_text[MAXR];
     int64_t r_total;       // product of r_count
     int64_t kept_slots;    // gridDim.x * kept lanes per block
@@ -58,6 +59,7 @@ __device__ __forceinline__ double identity(int op) {
 
 struct ThreadPos {
     int64_t in, out;      // element offsets of this thread (block origin + in-tile position)
+    int64_t in_b;         // ... in the second operand of a product reduction
     int64_t lim[MAXT];    // remaining extent of each tile axis at this block
     int32_t tc[MAXT];     // in-tile coordinate per tile axis
     bool ok;              // inside the tensor on every kept tile axis
@@ -68,7 +70,7 @@ struct ThreadPos {
 
 __device__ __forceinline__ ThreadPos thread_pos(const ReduceArgs& a, int tid) {
     ThreadPos p;
-    p.in = p.out = 0;
+    p.in = p.out = p.in_b = 0;
 #pragma unroll
     for (int t = 0; t < MAXT; ++t) p.lim[t] = t < a.nt ? a.t_n[t] : 1;
     uint64_t bid = blockIdx.x;
@@ -77,6 +79,7 @@ __device__ __forceinline__ ThreadPos thread_pos(const ReduceArgs& a, int tid) {
         int64_t c = (int64_t)(bid - q * (uint64_t)a.g_count[g]);
         bid = q;
         p.in += c * a.g_sa[g];
+        p.in_b += c * a.g_sb[g];
         p.out += c * a.g_sc[g];
         int t = a.g_tid[g];
 #pragma unroll
@@ -95,6 +98,7 @@ __device__ __forceinline__ ThreadPos thread_pos(const ReduceArgs& a, int tid) {
             int c = (tid >> a.t_shift[t]) & a.t_mask[t];
             p.tc[t] = c;
             p.in += (int64_t)c * a.t_sa[t];
+            p.in_b += (int64_t)c * a.t_sb[t];
             if (a.t_red[t]) {
                 p.writer &= c == 0;
                 p.red_ok &= c < a.t_n[t];
@@ -109,12 +113,14 @@ __device__ __forceinline__ ThreadPos thread_pos(const ReduceArgs& a, int tid) {
     return p;
 }
 
-template <class R, bool CX>
+// DOT: the reduced quantity is the product A * B of two operands read at the same coordinates (sum only).
+template <class R, bool CX, bool DOT = false>
 __global__ void __launch_bounds__(THREADS) reduce_kernel(ReduceArgs a) {
     constexpr int NC = CX ? 2 : 1;
     __shared__ double lds[THREADS * NC];
     const ThreadPos p = thread_pos(a, threadIdx.x);
     const R* A = reinterpret_cast<const R*>(a.in) + p.in * NC;
+    const R* B = DOT ? reinterpret_cast<const R*>(a.in_b) + p.in_b * NC : nullptr;
     const int op = a.op;
     double acc_re = identity(op), acc_im = 0.0;
     // this block's slice of the serial reduced range
@@ -123,7 +129,7 @@ __global__ void __launch_bounds__(THREADS) reduce_kernel(ReduceArgs a) {
     const int64_t it1 = it0 + per < a.r_total ? it0 + per : a.r_total;
     // odometer start
     int64_t c[MAXR];
-    int64_t off = 0;
+    int64_t off = 0, off_b = 0;
     {
         int64_t lin = it0;
 #pragma unroll
@@ -134,6 +140,7 @@ __global__ void __launch_bounds__(THREADS) reduce_kernel(ReduceArgs a) {
                 c[r] = lin - q * a.r_count[r];
                 lin = q;
                 off += c[r] * a.r_sa[r];
+                if (DOT) off_b += c[r] * a.r_sb[r];
             }
         }
     }
@@ -152,7 +159,7 @@ __global__ void __launch_bounds__(THREADS) reduce_kernel(ReduceArgs a) {
     const bool load_ok = p.ok && p.red_ok;
     constexpr int U = 8;  // independent loads in flight per thread
     for (int64_t it = it0; it < it1; it += U) {
-        int64_t offs[U];
+        int64_t offs[U], offs_b[U];
         bool oks[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -162,35 +169,48 @@ __global__ void __launch_bounds__(THREADS) reduce_kernel(ReduceArgs a) {
                 if (r < a.nr) ok &= c[r] * a.r_text[r] + tcr[r] < a.r_n[r];
             oks[u] = ok;
             offs[u] = off;
+            offs_b[u] = off_b;
             // advance the odometer
             off += a.r_sa[0];
+            if (DOT) off_b += a.r_sb[0];
             if (++c[0] == a.r_count[0]) {
                 off -= a.r_sa[0] * a.r_count[0];
+                if (DOT) off_b -= a.r_sb[0] * a.r_count[0];
                 c[0] = 0;
 #pragma unroll
                 for (int r = 1; r < MAXR; ++r) {
                     if (r < a.nr) {
                         off += a.r_sa[r];
+                        if (DOT) off_b += a.r_sb[r];
                         if (++c[r] < a.r_count[r]) break;
                         off -= a.r_sa[r] * a.r_count[r];
+                        if (DOT) off_b -= a.r_sb[r] * a.r_count[r];
                         c[r] = 0;
                     }
                 }
             }
         }
-        R vre[U], vim[U];
+        R vre[U], vim[U], wre[U], wim[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            vre[u] = vim[u] = R(0);
+            vre[u] = vim[u] = wre[u] = wim[u] = R(0);
             if (oks[u]) {
                 vre[u] = A[offs[u] * NC];
                 if (CX) vim[u] = A[offs[u] * NC + 1];
+                if (DOT) {
+                    wre[u] = B[offs_b[u] * NC];
+                    if (CX) wim[u] = B[offs_b[u] * NC + 1];
+                }
             }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (oks[u]) {
-                if (CX) {
+                if (DOT) {
+                    const double ar = (double)vre[u], ai = (double)vim[u], br = (double)wre[u], bi = (double)wim[u];
+                    acc_re += CX ? ar * br - ai * bi : ar * br;
+                    if (CX) acc_im += ar * bi + ai * br;
+                } else if (CX) {
                     acc_re += (double)vre[u];
                     acc_im += (double)vim[u];
                 } else {
@@ -760,13 +780,21 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
         int32_t st_fast = TFH_OK;
         if (try_fast_reduce(dtype, a, c, kept, red, reduce_op, alpha, beta, stream, st_fast)) return st_fast;
     }
-    // merge axes (kept and reduced separately; slot 0 = A, slot 1 = C)
-    std::stable_sort(kept.begin(), kept.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[1]) > std::llabs(y.s[1]); });
     for (auto& x : kept) x.s[2] = 0;
-    fuse_axes(kept, 2);
     for (auto& x : red) x.s[1] = x.s[2] = 0;
-    std::stable_sort(red.begin(), red.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[0]) > std::llabs(y.s[0]); });
-    fuse_axes(red, 1);
+    return launch_reduce_general(dtype, a, nullptr, c, kept, red, reduce_op, alpha, beta, stream);
+}
+
+// The general kernel for any extents and strides.  Axis slots: 0 = A, 1 = C, 2 = B (the second operand of a product
+// reduction, b != nullptr; zero strides otherwise).
+int32_t launch_reduce_general(int dtype, const void* a, const void* b, void* c, std::vector<Axis> kept, std::vector<Axis> red,
+                              int reduce_op, Scalar alpha, Scalar beta, void* stream) {
+    // merge axes (kept and reduced separately)
+    std::stable_sort(kept.begin(), kept.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[1]) > std::llabs(y.s[1]); });
+    fuse_axes(kept, 3);
+    auto key_red = [](const Axis& x) { return x.s[0] == 0 ? INT64_MAX : std::llabs(x.s[0]); };
+    std::stable_sort(red.begin(), red.end(), [&](const Axis& x, const Axis& y) { return key_red(x) > key_red(y); });
+    fuse_axes(red, 3);
     for (auto& x : kept)
         if (x.s[1] == 0) return set_error(TFH_ERR_STRIDED, "output view has stride 0 on an axis of extent %lld", (long long)x.n);
     struct Ax {
@@ -811,6 +839,7 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
         ra.t_red[t] = all[i].red;
         ra.t_sa[t] = all[i].a.s[0];
         ra.t_sc[t] = all[i].a.s[1];
+        ra.t_sb[t] = all[i].a.s[2];
         ra.t_n[t] = all[i].a.n;
         if (all[i].red) ra.red_bits |= ra.t_mask[t] << shift;
         shift += all[i].tl;
@@ -834,6 +863,7 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
             int r = ra.nr++;
             ra.r_count[r] = cnt;
             ra.r_sa[r] = all[i].a.s[0] * text;
+            ra.r_sb[r] = all[i].a.s[2] * text;
             ra.r_n[r] = all[i].a.n;
             ra.r_tid[r] = tid_of[i];
             ra.r_text[r] = (int32_t)text;
@@ -843,6 +873,7 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
             ra.g_count[g] = cnt;
             ra.g_sa[g] = all[i].a.s[0] * text;
             ra.g_sc[g] = all[i].a.s[1] * text;
+            ra.g_sb[g] = all[i].a.s[2] * text;
             ra.g_tid[g] = tid_of[i];
             ra.g_text[g] = (int32_t)text;
             blocks *= (uint64_t)cnt;
@@ -859,6 +890,7 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
     ra.nchunks = nchunks;
     ra.kept_slots = (int64_t)blocks * THREADS;
     ra.in = a;
+    ra.in_b = b;
     ra.out = c;
     ra.op = reduce_op;
     ra.alpha_re = alpha.re;
@@ -875,12 +907,21 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
     }
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((uint32_t)blocks, (uint32_t)nchunks, 1), block(THREADS);
-    const int prof = prof_begin(PROF_REDUCE, stream);
-    switch (dtype) {
-        case TFH_F32: TFH_LAUNCH_TIMED((reduce_kernel<float, false>), grid, block, 0, st, ra); break;
-        case TFH_F64: TFH_LAUNCH_TIMED((reduce_kernel<double, false>), grid, block, 0, st, ra); break;
-        case TFH_C64: TFH_LAUNCH_TIMED((reduce_kernel<float, true>), grid, block, 0, st, ra); break;
-        default: TFH_LAUNCH_TIMED((reduce_kernel<double, true>), grid, block, 0, st, ra); break;
+    const int prof = prof_begin(b ? PROF_CONTRACT : PROF_REDUCE, stream);
+    if (b) {
+        switch (dtype) {
+            case TFH_F32: TFH_LAUNCH_TIMED((reduce_kernel<float, false, true>), grid, block, 0, st, ra); break;
+            case TFH_F64: TFH_LAUNCH_TIMED((reduce_kernel<double, false, true>), grid, block, 0, st, ra); break;
+            case TFH_C64: TFH_LAUNCH_TIMED((reduce_kernel<float, true, true>), grid, block, 0, st, ra); break;
+            default: TFH_LAUNCH_TIMED((reduce_kernel<double, true, true>), grid, block, 0, st, ra); break;
+        }
+    } else {
+        switch (dtype) {
+            case TFH_F32: TFH_LAUNCH_TIMED((reduce_kernel<float, false>), grid, block, 0, st, ra); break;
+            case TFH_F64: TFH_LAUNCH_TIMED((reduce_kernel<double, false>), grid, block, 0, st, ra); break;
+            case TFH_C64: TFH_LAUNCH_TIMED((reduce_kernel<float, true>), grid, block, 0, st, ra); break;
+            default: TFH_LAUNCH_TIMED((reduce_kernel<double, true>), grid, block, 0, st, ra); break;
+        }
     }
     prof_end(prof, stream);
     if (int32_t e = hip_check(hipGetLastError(), "reduce kernel launch")) return e;
