@@ -483,6 +483,9 @@ void launch_generic64(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st) {
         default: launch_tile<double, true, 64, 64>(g, grid, st); break;
     }
 }
+}  // namespace
+void launch_gemm_wave(int dtype, const gemm::GemmArgs& g, int64_t nwork, hipStream_t st);   // k_gemm_wave.hip
+namespace {
 void launch_128(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st) {
     switch (dtype) {
         case TFH_F32: launch_gemm128_f32(g, grid, g.a_kfast, g.b_kfast, st); break;
@@ -747,12 +750,19 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         nsplit = std::max(1, std::min(nsplit, 512));   // a single tile with a very long k still fills the chip
     }
     if (skinny) nsplit = 1;
+    // many tiny products (both free extents at most 32): one wave per 32x32 tile, no LDS staging (k_gemm_wave.hip)
+    const bool wavek = !skinny && M <= 32 && N <= 32 && nb >= 64 && kstages <= 64;
+    if (wavek) nsplit = 1;
     int64_t kps = ((kstages + nsplit - 1) / nsplit) * bke;
     nsplit = (int)((K + kps - 1) / kps);
     g.nsplit = nsplit;
     g.k_per_split = kps;
     g.tiles_m = (int)((M + bm - 1) / bm);
     g.tiles_n = (int)((NR + bm - 1) / bm);
+    if (wavek) {
+        g.tiles_m = (int)((M + 31) / 32);
+        g.tiles_n = (int)((NR + 31) / 32);
+    }
     if ((double)g.tiles_m * (double)g.tiles_n * (double)nb * (double)nsplit > 2147483647.0) {
         release_packed();
         return set_error(TFH_ERR_INVALID_ARGUMENT, "contraction too large for one launch (tiles %lld, batch*split %lld)",
@@ -893,7 +903,8 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         sk.b_in = (int32_t)inner_b; sk.c_in = (int32_t)inner_c;
         sk.alpha_re = alpha.re; sk.alpha_im = alpha.im; sk.beta_re = beta.re; sk.beta_im = beta.im;
         launch_gemm_skinny(dtype, sk, st);
-    } else if (use128) launch_128(dtype, g, grid, st);
+    } else if (wavek) launch_gemm_wave(dtype, g, nb * g.tiles_m * g.tiles_n, st);
+    else if (use128) launch_128(dtype, g, grid, st);
     else launch_generic64(dtype, g, grid, st);
     prof_end(prof, stream);
     release_packed();   // stream-ordered: the next user of these blocks is enqueued after this kernel

@@ -1429,3 +1429,34 @@ def test_reduce_random_shapes_that_tile(tf, oracle, dtype):
         else:
             assert np.array_equal(got, ref), (case, shape, keep)
     assert any("reduce_fast_kernel" in k for k in kernels), kernels
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("m,k,n,nbatch", [(8, 8, 8, 500), (16, 16, 16, 300), (32, 32, 32, 100), (5, 7, 3, 1000), (1, 9, 17, 200),
+                                          (20, 50, 31, 128), (32, 1, 32, 64), (3, 200, 2, 400)])
+def test_batches_of_tiny_products_take_the_wave_kernel(tf, oracle, dtype, m, k, n, nbatch):
+    # many products with both free extents at most 32: one wave per 32x32 tile, operands loaded straight into the MFMA
+    # layout with bounds masks.  Odd extents, k that is not a multiple of the step, alpha/beta, operand orders.
+    rng = np.random.default_rng(103)
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    for ma, mb, mc in [("bmk", "bkn", "bmn"), ("kbm", "nbk", "bnm")]:
+        ext = dict(b=nbatch, m=m, k=k, n=n)
+        a, b = rand(rng, [ext[l] for l in ma], dtype), rand(rng, [ext[l] for l in mb], dtype)
+        cshape = [ext[l] for l in mc]
+        for alpha, beta in [(1.0, 0.0), ((0.7 - 1.1j, -0.3 + 0.2j) if cplx else (0.7, -0.3))]:
+            c0 = rand(rng, cshape, dtype)
+            ref = c0.copy()
+            oracle.contract(a, lab(ma), b, lab(mb), ref, lab(mc), alpha=alpha, beta=beta)
+            out = dev(tf, c0)
+            plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [a.shape, b.shape, cshape])
+            tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, out)
+            if m > 1 and n > 1:      # (an empty free group goes to the product-reduction kernels instead)
+                assert "gemm_wave_kernel" in tf.last_kernel(), tf.last_kernel()
+            assert relerr(out.to_numpy(), ref) < TOL[dtype], (ma, mb, mc, alpha, beta)
+    # BatchedGemm descriptor, exact on small integers
+    ai = rng.integers(-4, 5, (nbatch, m, k)).astype(dtype)
+    bi = rng.integers(-4, 5, (nbatch, k, n)).astype(dtype)
+    out = tf.Tensor.empty([nbatch, m, n], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.BatchedGemm([nbatch], m, n, k), [ai.shape, bi.shape, [nbatch, m, n]])
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, ai), dev(tf, bi)], 0.0, out)
+    assert np.array_equal(out.to_numpy(), np.matmul(ai, bi))
