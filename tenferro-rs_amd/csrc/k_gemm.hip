@@ -1003,6 +1003,10 @@ int32_t grouped_plan_init(tfh_plan& plan) {
         if (M < 96 || (cx ? 2 * N : N) < 96) ++small;
     }
     gs->bm = small * 2 > plan.n_groups ? 64 : 128;
+    // every problem tiny (M, N <= 32): 32x32 tiles, one wave each (k_gemm_wave.hip)
+    bool all_tiny = plan.n_groups >= 64;
+    for (int gi = 0; gi < plan.n_groups; ++gi) all_tiny = all_tiny && mnk[(size_t)gi][0] <= 32 && mnk[(size_t)gi][1] <= 32 && mnk[(size_t)gi][2] <= 1024;
+    if (all_tiny) gs->bm = 32;
     for (int gi = 0; gi < plan.n_groups; ++gi) {
         int64_t M = mnk[(size_t)gi][0], N = mnk[(size_t)gi][1], K = mnk[(size_t)gi][2];
         int64_t NR = cx ? 2 * N : N;
@@ -1135,7 +1139,8 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
     g.tile_map = gs->tile_map_dev;
     dim3 grid((uint32_t)gs->tile_map_host.size(), 1, 1);
     const int prof = prof_begin(PROF_CONTRACT, stream);
-    if (gs->bm == 128) launch_128(dtype, g, grid, st);
+    if (gs->bm == 32) launch_gemm_wave(dtype, g, (int64_t)gs->tile_map_host.size(), st);
+    else if (gs->bm == 128) launch_128(dtype, g, grid, st);
     else launch_generic64(dtype, g, grid, st);
     prof_end(prof, stream);
     return hip_check(hipGetLastError(), "grouped contraction launch");

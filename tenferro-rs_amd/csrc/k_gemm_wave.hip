@@ -27,25 +27,46 @@ __global__ void __launch_bounds__(THREADS) gemm_wave_kernel(GemmArgs g, int64_t 
     const int lane = threadIdx.x & 63, j = lane & 15, gq = lane >> 4;
     const int64_t work = (int64_t)blockIdx.x * (THREADS / 64) + (threadIdx.x >> 6);
     if (work >= nwork) return;   // whole waves leave; there is no block-level synchronisation below
-    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    const int64_t batch = work / tiles;
-    const int tile = (int)(work - batch * tiles), tile_m = tile % g.tiles_m, tile_n = tile / g.tiles_m;
-    const int64_t M = g.M, N = g.N, K = g.K;
+    int64_t M = g.M, N = g.N, K = g.K;
+    OffFn am = g.am, ak = g.ak, bk = g.bk, bn = g.bn, cm = g.cm, cn = g.cn;
+    const E* A;
+    const E* B;
+    R* Cb;
+    int tile_m, tile_n;
+    if (g.problems) {   // grouped launch: one record per problem, one map entry per tile
+        const int4 tm = g.tile_map[work];
+        const GroupProblem& p = g.problems[tm.x];
+        M = p.M; N = p.N; K = p.K;
+        A = reinterpret_cast<const E*>(p.A);
+        B = reinterpret_cast<const E*>(p.B);
+        Cb = reinterpret_cast<R*>(p.C);
+        am = OffFn{nullptr, p.sam}; ak = OffFn{nullptr, p.sak}; bk = OffFn{nullptr, p.sbk};
+        bn = OffFn{nullptr, p.sbn}; cm = OffFn{nullptr, p.scm}; cn = OffFn{nullptr, p.scn};
+        tile_m = tm.y;
+        tile_n = tm.z;
+    } else {
+        const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+        const int64_t batch = work / tiles;
+        const int tile = (int)(work - batch * tiles);
+        tile_m = tile % g.tiles_m;
+        tile_n = tile / g.tiles_m;
+        A = reinterpret_cast<const E*>(g.A) + off_of(g.ab, batch);
+        B = reinterpret_cast<const E*>(g.B) + off_of(g.bb, batch);
+        Cb = reinterpret_cast<R*>(g.C) + off_of(g.cb, batch) * EC;
+    }
     const int64_t NR = N * EC, KR = K * EC;
     const int64_t m0 = (int64_t)tile_m * 32, n0r = (int64_t)tile_n * 32;
 
-    const E* A = reinterpret_cast<const E*>(g.A) + off_of(g.ab, batch);
-    const E* B = reinterpret_cast<const E*>(g.B) + off_of(g.bb, batch);
     // this lane's two rows of A and two (real) columns of B; -1 marks the ones outside the matrices
     int64_t ra[2], cb[2];
     int pb[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int64_t row = m0 + j + 16 * i;
-        ra[i] = row < M ? off_of(g.am, row) : -1;
+        ra[i] = row < M ? off_of(am, row) : -1;
         const int64_t col = n0r + j + 16 * i;
         pb[i] = CX ? (int)(col & 1) : 0;
-        cb[i] = col < NR ? off_of(g.bn, CX ? col >> 1 : col) : -1;
+        cb[i] = col < NR ? off_of(bn, CX ? col >> 1 : col) : -1;
     }
     acc_t acc[2][2];
 #pragma unroll
@@ -62,7 +83,7 @@ __global__ void __launch_bounds__(THREADS) gemm_wave_kernel(GemmArgs g, int64_t 
             const bool kok = kk < KR;
             const int64_t ke = kok ? (CX ? kk >> 1 : kk) : 0;
             const int q = CX ? (int)(kk & 1) : 0;
-            const int64_t ka = off_of(g.ak, ke), kb = off_of(g.bk, ke);
+            const int64_t ka = off_of(ak, ke), kb = off_of(bk, ke);
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 av[u][i] = R(0);
@@ -93,7 +114,6 @@ __global__ void __launch_bounds__(THREADS) gemm_wave_kernel(GemmArgs g, int64_t 
     }
 
     // ---- epilogue: the same arithmetic as the tiled kernels; real column n0r + 16 jb + j
-    R* Cb = reinterpret_cast<R*>(g.C) + off_of(g.cb, batch) * EC;
     const R ar = (R)g.alpha_re, ai = (R)g.alpha_im, br = (R)g.beta_re, bi = (R)g.beta_im;
     int64_t coff[2];
     bool cok[2];
@@ -101,7 +121,7 @@ __global__ void __launch_bounds__(THREADS) gemm_wave_kernel(GemmArgs g, int64_t 
     for (int jb = 0; jb < 2; ++jb) {
         const int64_t col = n0r + 16 * jb + j;
         cok[jb] = col < NR;
-        coff[jb] = cok[jb] ? off_of(g.cn, CX ? col >> 1 : col) * EC + (CX ? (col & 1) : 0) : 0;
+        coff[jb] = cok[jb] ? off_of(cn, CX ? col >> 1 : col) * EC + (CX ? (col & 1) : 0) : 0;
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -109,7 +129,7 @@ __global__ void __launch_bounds__(THREADS) gemm_wave_kernel(GemmArgs g, int64_t 
         for (int r = 0; r < 4; ++r) {
             const int64_t row = m0 + 16 * i + Mfma<R>::row(lane, r);
             const bool rok = row < M;
-            const int64_t roff = rok ? off_of(g.cm, row) * EC : 0;
+            const int64_t roff = rok ? off_of(cm, row) * EC : 0;
 #pragma unroll
             for (int jb = 0; jb < 2; ++jb) {
                 R v = acc[i][jb][r];

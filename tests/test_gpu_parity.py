@@ -352,6 +352,16 @@ def test_grouped_odd_extents_on_128_tiles(tf, oracle, dtype):
     assert "gemm128_kernel" in tf.last_kernel(), tf.last_kernel()
 
 
+@pytest.mark.parametrize("dtype", ALL)
+def test_grouped_tiny_problems_take_the_wave_kernel(tf, oracle, dtype):
+    # 300 problems with every extent between 1 and 32 (a block-sparse tensor with small blocks): one grouped launch,
+    # one wave per 32x32 tile
+    rng = np.random.default_rng(79)
+    dims = [tuple(int(v) for v in rng.integers(1, 33, 3)) for _ in range(300)]
+    assert _grouped_case(tf, oracle, dims, dtype, 79) < TOL[dtype]
+    assert "gemm_wave_kernel" in tf.last_kernel(), tf.last_kernel()
+
+
 def test_config4_grouped_full_size(tf, oracle):
     # 128 blocks, i,j,k iid from {64,...,1024}: every block <= 1e-12 against the oracle, one launch
     from tenferro_rs_amd import inputs
