@@ -32,7 +32,7 @@ PEAK = {"hbm": 8000.0, "f32": 157.3, "f64": 78.6}   # GB/s, TFLOP/s (MI355X publ
 # WRITE_SIZE) summarised in profiles/bench_hbm_traffic_pmc.txt, each scaled by what the same counter read for plain
 # 1 GiB device copies in the same run (x2.0 and x1.0).  A profiler cannot run inside this script; these are that run's
 # figures for exactly these workloads.
-TRAFFIC = {"c1": 249.0e6, "c2_permute": 268.6e6, "c2_reduce": 134.9e6, "c3": 7087.4e6, "c4": 3067.6e6}
+TRAFFIC = {"c1": 249.0e6, "c2_permute": 268.6e6, "c2_reduce": 134.9e6, "c3": 7071.7e6, "c4": 3065.9e6}
 SPINUP_S = 0.3   # seconds of untimed device spin-up per configuration
 METRIC = "contraction TFLOP/s & % MFMA peak (f64/f32); permute/reduce GB/s & % HBM peak"
 
