@@ -1470,3 +1470,59 @@ def test_batches_of_tiny_products_take_the_wave_kernel(tf, oracle, dtype, m, k, 
     plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.BatchedGemm([nbatch], m, n, k), [ai.shape, bi.shape, [nbatch, m, n]])
     tf.HipBackend.execute(plan, 1.0, [dev(tf, ai), dev(tf, bi)], 0.0, out)
     assert np.array_equal(out.to_numpy(), np.matmul(ai, bi))
+
+
+def test_calls_from_several_host_threads_on_their_own_streams(tf, oracle):
+    # the library's state (per-stream workspaces, pools, table caches, error slots) is process-global behind a mutex and
+    # calls are documented as thread-safe: four host threads, each with its own stream, run a mix of contractions
+    # (tables, split-K, packing), einsum trees, permutes and reductions at once; every result is checked
+    import threading
+    import torch
+    rng = np.random.default_rng(104)
+    work = []
+    for t in range(4):
+        a, b = rand(rng, (24, 8, 20, 12 + t), np.float64), rand(rng, (12 + t, 30, 8), np.float64)      # "ajbk,kcj->abc"
+        ref = np.empty((24, 20, 30))
+        oracle.contract(a, lab("ajbk"), b, lab("kcj"), ref, lab("abc"))
+        p = rand(rng, (16, 8 + t, 16, 8), np.float64)
+        pref = np.ascontiguousarray(p.transpose(3, 1, 0, 2))
+        rref = p.sum(axis=(1, 3))
+        ops = [rand(rng, s_, np.complex128) for s_ in [(9, 3, 8 + t), (9, 2, 7), (3, 2, 2, 4), (8 + t, 2, 6)]]
+        eref = np.einsum("awc,asx,wstv,cty->xvy", *ops)
+        work.append((a, b, ref, p, pref, rref, ops, eref))
+    errors = []
+
+    def body(t):
+        try:
+            a, b, ref, p, pref, rref, ops, eref = work[t]
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                st = stream.cuda_stream
+                da, db, dp = dev(tf, a), dev(tf, b), dev(tf, p)
+                dops = [dev(tf, o) for o in ops]
+                stream.synchronize()
+                plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Contract(lab("ajbk"), lab("kcj"), lab("abc")), [a.shape, b.shape, ref.shape])
+                pplan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute([0, 1, 2, 3], [3, 1, 0, 2]), [p.shape, pref.shape])
+                rplan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Reduce([0, 1, 2, 3], [0, 2], tf.ReduceOp.Sum), [p.shape, rref.shape])
+                for it in range(25):
+                    out = tf.Tensor.empty(list(ref.shape), tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+                    pout = tf.Tensor.empty(list(pref.shape), tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+                    rout = tf.Tensor.empty(list(rref.shape), tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+                    tf.HipBackend.execute(plan, 1.0, [da, db], 0.0, out, st)
+                    tf.HipBackend.execute(pplan, 1.0, [dp], 0.0, pout, st)
+                    tf.HipBackend.execute(rplan, 1.0, [dp], 0.0, rout, st)
+                    e = tf.einsum("awc,asx,wstv,cty->xvy", dops, st)
+                    stream.synchronize()
+                    assert relerr(out.to_numpy(), ref) < 1e-12
+                    assert pout.to_numpy().tobytes() == pref.tobytes()
+                    assert relerr(rout.to_numpy(), rref) < 1e-12
+                    assert relerr(e.to_numpy(), eref) < 1e-12
+        except BaseException as ex:      # noqa: BLE001 -- reported by the main thread
+            errors.append((t, repr(ex)))
+
+    threads = [threading.Thread(target=body, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
