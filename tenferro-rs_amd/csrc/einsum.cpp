@@ -562,6 +562,8 @@ double tfh_tree_mac_count(const tfh_tree* t) { return t ? t->macs : 0; }
 double tfh_tree_peak_intermediate(const tfh_tree* t) { return t ? t->peak : 0; }
 
 // ---- executor ----------------------------------------------------------------------------------------------
+}  // extern "C"
+
 namespace {
 struct Operand {          // a node as the executor sees it: unique labels + strides
     std::vector<uint32_t> labels;
@@ -605,6 +607,8 @@ int32_t reduce_or_copy(int dtype, const Operand& src, const Operand& dst, Scalar
     return launch_reduce(dtype, src.ptr, dst.ptr, kept, red, TFH_REDUCE_SUM, alpha, beta, stream);
 }
 }  // namespace
+
+extern "C" {
 
 int32_t tfh_einsum_execute(int32_t dtype, const tfh_tree* tree, const tfh_view* operands, int32_t n_operands,
                            const void* alpha, const void* beta, tfh_view* output, uint64_t donate_mask, tfh_stream stream) {
