@@ -64,9 +64,10 @@ __device__ __forceinline__ void lds_store_pack(R* p, const R (&x)[N]) {
     *reinterpret_cast<Raw*>(p) = __builtin_bit_cast(Raw, t);
 }
 
-template <class R, bool CX>
+// BNV: real columns per tile, 128 or 64 (a thin right-hand side: 33..95 real columns)
+template <class R, bool CX, int BNV = 128>
 struct Cfg128 {
-    static constexpr int BM = 128, BN = 128;
+    static constexpr int BM = 128, BN = BNV;
     static constexpr int BKR = 128 / sizeof(R);           // real k per stage: 128 bytes per row
     static constexpr int EC = CX ? 2 : 1;                 // reals per element
     static constexpr int BKE = BKR / EC;                  // elements of k per stage
@@ -79,7 +80,7 @@ struct Cfg128 {
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 16, TN = WN / 16;
     static constexpr int MIN_WAVES = 2;   // waves per SIMD the register budget is sized for
     static constexpr size_t LDS_BYTES = (size_t)2 * (BM + BN) * PITCH * sizeof(R);
-    static_assert(TM == 4 && TN == 4, "the chunk swizzle assumes four 16-row blocks per wave tile");
+    static_assert(TM == 4 && (TN == 4 || TN == 2), "the chunk swizzle assumes four 16-row blocks per wave row");
     // LDS index of real k `rk` in real row `rr`
     __device__ static __forceinline__ int lds_idx(int rr, int rk) { return rr * PITCH + (((rk / CH) ^ ((rr >> 4) & 3)) * CH) + rk % CH; }
 };
@@ -87,9 +88,9 @@ struct Cfg128 {
 // Per-thread, loop-invariant description of one operand's share of a stage (ROWS element rows x BKE k).
 //   KFAST : load l covers row rq + l*RP, k elements kq .. kq+V-1
 //   else  : load l = p*V + j covers rows rq .. rq+V-1 at k element (p*KP + kq)*V + j
-template <class R, bool CX, int ROWS, bool KFAST, int V, int RM>
+template <class R, bool CX, int ROWS, bool KFAST, int V, int RM, int BNV = 128>
 struct OperandMap {
-    typedef Cfg128<R, CX> C_;
+    typedef Cfg128<R, CX, BNV> C_;
     static constexpr int EC = C_::EC, PN = V * EC;
     static constexpr int KV = C_::BKE / V;             // KFAST: loads per row
     static constexpr int RP = C_::NT / KV;             // KFAST: rows per pass
@@ -223,9 +224,9 @@ struct OperandMap {
     }
 };
 
-template <class R, bool CX, bool AKF, bool BKF, int VA, int VB>
-__global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES)) gemm128_kernel(GemmArgs g) {
-    typedef Cfg128<R, CX> C_;
+template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128>
+__global__ void __launch_bounds__((Cfg128<R, CX, BNV>::NT), (Cfg128<R, CX, BNV>::MIN_WAVES)) gemm128_kernel(GemmArgs g) {
+    typedef Cfg128<R, CX, BNV> C_;
     typedef typename ElemT<R, CX>::type E;
     typedef typename Mfma<R>::acc_t acc_t;
     constexpr int BM = C_::BM, BN = C_::BN, BKE = C_::BKE, PITCH = C_::PITCH, BNE = C_::BNE, CH = C_::CH;
@@ -270,8 +271,8 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
     const int rowsA = (int)(M - m0 < BM ? M - m0 : BM), rowsB = (int)(N - n0 < BNE ? N - n0 : BNE);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    typedef OperandMap<R, CX, BM, AKF, VA, 1> MapA;
-    typedef OperandMap<R, CX, BNE, BKF, VB, (CX ? 2 : 1)> MapB;
+    typedef OperandMap<R, CX, BM, AKF, VA, 1, BNV> MapA;
+    typedef OperandMap<R, CX, BNE, BKF, VB, (CX ? 2 : 1), BNV> MapB;
     MapA ma;
     MapB mb;
     ma.init(am, ak, m0, rowsA);
@@ -288,6 +289,9 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
 
     const int wm0 = (wave / C_::WAVES_N) * C_::WM, wn0 = (wave % C_::WAVES_N) * C_::WN;
     const int lrow = lane & 15, lgrp = lane >> 4;
+    // chunk swizzle of this wave's B rows: block j of the wave starts at row wn0 + 16 j, i.e. (row >> 4) & 3 = j for a
+    // 64-column wave tile and 2 (wave column) + j for a 32-column one
+    const int swb0 = TN == 4 ? 0 : (wn0 >> 4) & 3;
 
     acc_t acc[TM][TN];
 #pragma unroll
@@ -333,7 +337,7 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
 #pragma unroll
             for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const Chunk*>(as + i * 16 * PITCH + ((2 * lgrp + h) ^ i) * CH);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const Chunk*>(bs + j * 16 * PITCH + ((2 * lgrp + h) ^ j) * CH);
+            for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const Chunk*>(bs + j * 16 * PITCH + ((2 * lgrp + h) ^ ((swb0 + j) & 3)) * CH);
 #pragma unroll
             for (int c = 0; c < CH; ++c)
 #pragma unroll
@@ -368,7 +372,7 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
 #pragma unroll
             for (int i = 0; i < TM; ++i) a[h][i] = *reinterpret_cast<const Chunk*>(as + i * 16 * PITCH + ((2 * lgrp + h) ^ i) * CH);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) b[h][j] = *reinterpret_cast<const Chunk*>(bs + j * 16 * PITCH + ((2 * lgrp + h) ^ j) * CH);
+            for (int j = 0; j < TN; ++j) b[h][j] = *reinterpret_cast<const Chunk*>(bs + j * 16 * PITCH + ((2 * lgrp + h) ^ ((swb0 + j) & 3)) * CH);
         }
         if (!tab) {
             sa = uniform_ptr(sa);
@@ -520,28 +524,29 @@ __global__ void __launch_bounds__((Cfg128<R, CX>::NT), (Cfg128<R, CX>::MIN_WAVES
         }
 }
 
-template <class R, bool CX, bool AKF, bool BKF, int VA, int VB>
+template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128>
 inline void launch_gemm128_variant(const GemmArgs& g, dim3 grid, hipStream_t st) {
     static bool once = [] {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm128_kernel<R, CX, AKF, BKF, VA, VB>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg128<R, CX>::LDS_BYTES);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm128_kernel<R, CX, AKF, BKF, VA, VB, BNV>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg128<R, CX, BNV>::LDS_BYTES);
         return true;
     }();
     (void)once;
-    typedef Cfg128<R, CX> C_;
+    typedef Cfg128<R, CX, BNV> C_;
     const size_t lds = C_::LDS_BYTES;
     const dim3 block(C_::NT);
-    TFH_LAUNCH_TIMED((gemm128_kernel<R, CX, AKF, BKF, VA, VB>), grid, block, lds, st, g);
+    TFH_LAUNCH_TIMED((gemm128_kernel<R, CX, AKF, BKF, VA, VB, BNV>), grid, block, lds, st, g);
+    if (BNV == 64) note_kernel("(gemm128_kernel, 128x64 tiles)");
 }
 
-template <class R, bool CX, int V>
+template <class R, bool CX, int V, int BNV = 128>
 inline void launch_gemm128_layout(const GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
     if (akf) {
-        if (bkf) launch_gemm128_variant<R, CX, true, true, V, V>(g, grid, st);
-        else launch_gemm128_variant<R, CX, true, false, V, V>(g, grid, st);
+        if (bkf) launch_gemm128_variant<R, CX, true, true, V, V, BNV>(g, grid, st);
+        else launch_gemm128_variant<R, CX, true, false, V, V, BNV>(g, grid, st);
     } else {
-        if (bkf) launch_gemm128_variant<R, CX, false, true, V, V>(g, grid, st);
-        else launch_gemm128_variant<R, CX, false, false, V, V>(g, grid, st);
+        if (bkf) launch_gemm128_variant<R, CX, false, true, V, V, BNV>(g, grid, st);
+        else launch_gemm128_variant<R, CX, false, false, V, V, BNV>(g, grid, st);
     }
 }
 
@@ -558,6 +563,21 @@ inline void launch_gemm128_any(const GemmArgs& g, dim3 grid, bool akf, bool bkf,
     launch_gemm128_layout<R, CX, 1>(g, grid, akf, bkf, st);
 }
 
+// 128 x 64 tiles for a thin right-hand side.  The row-contiguous B loader of f32 / complex64 with 16-byte accesses has
+// more threads than 64 columns give work to, so those two combinations use element-wise accesses.
+template <class R, bool CX>
+inline void launch_gemm128x64_any(const GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
+    constexpr int VMAX = Cfg128<R, CX>::VMAX;
+    constexpr bool thin_ok = VMAX > 1 && (sizeof(R) == 8 || false);   // 16-byte accesses divide the 64-column tile
+    if constexpr (thin_ok) {
+        if (g.vec) {
+            launch_gemm128_layout<R, CX, VMAX, 64>(g, grid, akf, bkf, st);
+            return;
+        }
+    }
+    launch_gemm128_layout<R, CX, 1, 64>(g, grid, akf, bkf, st);
+}
+
 }  // namespace gemm
 
 // One translation unit per dtype instantiates its four layout variants.
@@ -565,5 +585,10 @@ void launch_gemm128_f32(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, 
 void launch_gemm128_f64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
 void launch_gemm128_c64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
 void launch_gemm128_c128(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+// ... and the same layouts with 128 x 64 tiles
+void launch_gemm128x64_f32(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+void launch_gemm128x64_f64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+void launch_gemm128x64_c64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+void launch_gemm128x64_c128(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
 
 }  // namespace tfh

@@ -486,7 +486,16 @@ void launch_generic64(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st) {
 }  // namespace
 void launch_gemm_wave(int dtype, const gemm::GemmArgs& g, int64_t nwork, hipStream_t st);   // k_gemm_wave.hip
 namespace {
-void launch_128(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st) {
+void launch_128(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st, int bn = 128) {
+    if (bn == 64) {
+        switch (dtype) {
+            case TFH_F32: launch_gemm128x64_f32(g, grid, g.a_kfast, g.b_kfast, st); break;
+            case TFH_F64: launch_gemm128x64_f64(g, grid, g.a_kfast, g.b_kfast, st); break;
+            case TFH_C64: launch_gemm128x64_c64(g, grid, g.a_kfast, g.b_kfast, st); break;
+            default: launch_gemm128x64_c128(g, grid, g.a_kfast, g.b_kfast, st); break;
+        }
+        return;
+    }
     switch (dtype) {
         case TFH_F32: launch_gemm128_f32(g, grid, g.a_kfast, g.b_kfast, st); break;
         case TFH_F64: launch_gemm128_f64(g, grid, g.a_kfast, g.b_kfast, st); break;
@@ -580,6 +589,20 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         std::swap(M, N);
         for (auto* grp : {&ax.batch, &ax.M, &ax.N, &ax.K})
             for (auto& x : *grp) std::swap(x.s[0], x.s[1]);
+    }
+    // 128x64 tiles take a thin free group (33..95 real columns) as N: if it is M that is thin, exchange the operands
+    // (C is then written along its slower axis, which is the small side of the problem)
+    {
+        const int ec = is_complex(dtype) ? 2 : 1;
+        // (a small operator against a long tensor keeps its orientation: the streaming kernel looks at it below)
+        const bool streamable = (dtype == TFH_F64 || dtype == TFH_C128) && M <= SKINNY_MAX_M && K * ec <= SKINNY_MAX_KR && N >= 4096;
+        if (M < 96 && M * ec >= 33 && N * ec >= 96 && !streamable) {
+            std::swap(a, b);
+            std::swap(ax.M, ax.N);
+            std::swap(M, N);
+            for (auto* grp : {&ax.batch, &ax.M, &ax.N, &ax.K})
+                for (auto& x : *grp) std::swap(x.s[0], x.s[1]);
+        }
     }
     // loaders run their lanes along k when the operand is contiguous in k, along the row index otherwise
     bool a_kfast = min_stride(ax.K, 0) <= min_stride(ax.M, 0);
@@ -713,13 +736,19 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     // tile shape, split-K
     const bool cx = is_complex(dtype);
     const int64_t NR = cx ? 2 * N : N;
-    int bm = (M >= 96 && NR >= 96) ? 128 : 64;
-    auto tiles_for = [&](int t) { return ((M + t - 1) / t) * ((NR + t - 1) / t) * nb; };
+    // 128x128 tiles, 128x64 for a thin right-hand side (33..95 real columns), else 64x64
+    int bm = 64, bn = 64;
+    if (M >= 96 && NR >= 96) bm = bn = 128;
+    else if (M >= 96 && NR >= 33) bm = 128;
+    auto tiles_for = [&](int tm_, int tn_) { return ((M + tm_ - 1) / tm_) * ((NR + tn_ - 1) / tn_) * nb; };
     const int bke = bke_of(dtype);
     const int64_t kstages = (K + bke - 1) / bke;
-    // too few 128x128 tiles to fill 256 CUs and too little k to split: fall back to 64x64 tiles
-    if (bm == 128 && tiles_for(128) < 192 && kstages < 32 && tiles_for(64) >= 2 * tiles_for(128)) bm = 64;
-    const int64_t tiles = tiles_for(bm);
+    // too few large tiles to fill 256 CUs and too little k to split: fall back to 64x64 tiles
+    if (bm == 128 && tiles_for(bm, bn) < 192 && kstages < 32 && tiles_for(64, 64) >= 2 * tiles_for(bm, bn)) bm = bn = 64;
+    // thin tiles that cannot reach one block per CU even with the deepest split: 64x64 tiles give twice the blocks
+    if (bm == 128 && bn == 64 && tiles_for(128, 64) * std::max<int64_t>(1, kstages / 8) < 256 && tiles_for(64, 64) >= 2 * tiles_for(128, 64))
+        bm = 64;
+    const int64_t tiles = tiles_for(bm, bn);
     int nsplit = 1;
     if (bm == 128 && tiles >= 32 && kstages >= 16) {
         // 128x128 tiles: 512 blocks are resident at a time (two per CU).  Estimated time of a split count s, in us, from
@@ -728,7 +757,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         // latency exposed (x1.25), and the fold moves the partials twice.  Picks the s with the least estimate: it
         // trades the idle tail of a partly filled last round against per-block overhead and partial traffic.
         auto estimate = [&](int s_) {
-            const double per_block = ((double)((kstages + s_ - 1) / s_) + 8.0) * 1.95;
+            const double per_block = ((double)((kstages + s_ - 1) / s_) + 8.0) * 1.95 * (double)bn / 128.0;
             const int64_t blocks = tiles * s_, full = blocks / 512, rem = blocks % 512;
             double t = (double)full * 2.0 * per_block;
             if (rem > 256) t += 2.0 * per_block;
@@ -758,7 +787,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     g.nsplit = nsplit;
     g.k_per_split = kps;
     g.tiles_m = (int)((M + bm - 1) / bm);
-    g.tiles_n = (int)((NR + bm - 1) / bm);
+    g.tiles_n = (int)((NR + bn - 1) / bn);
     if (wavek) {
         g.tiles_m = (int)((M + 31) / 32);
         g.tiles_n = (int)((NR + 31) / 32);
@@ -777,9 +806,9 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     reach(ax.N, 1, lo_b, hi_b); reach(ax.K, 1, lo_b, hi_b);
     if ((hi_a - lo_a + 1) * (int64_t)eb >= ((int64_t)1 << 32) || (hi_b - lo_b + 1) * (int64_t)eb >= ((int64_t)1 << 32)) use128 = false;
     if (!use128 && bm == 128) {
-        bm = 64;
+        bm = bn = 64;
         g.tiles_m = (int)((M + bm - 1) / bm);
-        g.tiles_n = (int)((NR + bm - 1) / bm);
+        g.tiles_n = (int)((NR + bn - 1) / bn);
     }
     const bool ktab32 = use128 && (ax.K.size() > 1);   // k tables for both operands or for none
     g.vec = use128 && vec_ok(dtype, a_kfast ? ax.K : ax.M, a_kfast ? ax.M : ax.K, a_kfast, 0) &&
@@ -904,7 +933,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         sk.alpha_re = alpha.re; sk.alpha_im = alpha.im; sk.beta_re = beta.re; sk.beta_im = beta.im;
         launch_gemm_skinny(dtype, sk, st);
     } else if (wavek) launch_gemm_wave(dtype, g, nb * g.tiles_m * g.tiles_n, st);
-    else if (use128) launch_128(dtype, g, grid, st);
+    else if (use128) launch_128(dtype, g, grid, st, bn);
     else launch_generic64(dtype, g, grid, st);
     prof_end(prof, stream);
     release_packed();   // stream-ordered: the next user of these blocks is enqueued after this kernel

@@ -751,6 +751,34 @@ def test_contract_odd_extents_take_the_straddling_vector_path(tf, oracle, dtype,
         assert relerr(out.to_numpy(), ref) < TOL[dtype], (m, k, n)
 
 
+THIN_SIZES = [(257, 1025, 33), (130, 523, 64), (300, 1040, 95), (47, 1031, 260), (64, 520, 1300), (1801, 66, 67), (513, 5, 80)]
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("layout", LAYOUTS, ids=["NN", "NT", "TN", "TT"])
+def test_contract_thin_side_takes_128x64_tiles(tf, oracle, dtype, layout):
+    # one free group of 33..95 real columns and a long other side: 128x64 tiles of the large-tile kernel, whichever
+    # operand is the thin one (the operands are exchanged so that it becomes the right-hand side)
+    ma, mb = layout
+    rng = np.random.default_rng(147)
+    ec = 2 if np.issubdtype(dtype, np.complexfloating) else 1
+    for m, k, n in THIN_SIZES:
+        ext = dict(m=m, k=k, n=n)
+        a = rand(rng, [ext[l] for l in ma], dtype)
+        b = rand(rng, [ext[l] for l in mb], dtype)
+        c0 = rand(rng, (m, n), dtype)
+        ref = c0.copy()
+        oracle.contract(a, lab(ma), b, lab(mb), ref, lab("mn"), alpha=0.5, beta=-1.5)
+        out = dev(tf, c0)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab("mn")), [a.shape, b.shape, [m, n]])
+        print("thin", dtype.__name__, ma, mb, m, k, n, flush=True)
+        tf.HipBackend.execute(plan, 0.5, [dev(tf, a), dev(tf, b)], -1.5, out)
+        thin = min(m, n)
+        if 33 <= thin * ec < 96:
+            assert "gemm128_kernel, 128x64" in tf.last_kernel(), (m, k, n, tf.last_kernel())
+        assert relerr(out.to_numpy(), ref) < TOL[dtype], (m, k, n, tf.last_kernel())
+
+
 def test_contract_operand_ending_at_the_end_of_its_allocation(tf, oracle):
     # the operands are the tail of exactly-sized device buffers: a read past the last element would leave the buffer
     rng = np.random.default_rng(48)
