@@ -529,6 +529,14 @@ public:
         check(tfh_tree_optimize(subscripts.get(), s.ptrs.data(), s.ranks.data(), (int32_t)shapes.size(), &t));
         return ContractionTree(t);
     }
+    // The tree `optimize` returns, shared through the library's cache of optimised networks (no counterpart in the
+    // reference: the einsum functions that take no plan use it so that a repeated call does not search again).
+    static ContractionTree optimize_cached(const Subscripts& subscripts, const std::vector<std::vector<size_t>>& shapes) {
+        detail::Shapes s(shapes);
+        tfh_tree* t = nullptr;
+        check(tfh_tree_optimize_cached(subscripts.get(), s.ptrs.data(), s.ranks.data(), (int32_t)shapes.size(), &t));
+        return ContractionTree(t);
+    }
     static ContractionTree from_pairs(const Subscripts& subscripts, const std::vector<std::vector<size_t>>& shapes,
                                       const std::vector<std::pair<size_t, size_t>>& pairs) {
         detail::Shapes s(shapes);
@@ -599,7 +607,7 @@ void einsum_with_plan_into(const ContractionTree& tree, const std::vector<const 
 template <class T>
 void einsum_with_subscripts_into(const Subscripts& subscripts, const std::vector<const Tensor<T>*>& operands, T alpha, T beta, Tensor<T>& output) {   // :545-582
     detail::common_space(operands);
-    einsum_with_plan_into(ContractionTree::optimize(subscripts, detail::shapes_of(operands)), operands, alpha, beta, output);
+    einsum_with_plan_into(ContractionTree::optimize_cached(subscripts, detail::shapes_of(operands)), operands, alpha, beta, output);
 }
 template <class T>
 void einsum_into(const std::string& notation, const std::vector<const Tensor<T>*>& operands, T alpha, T beta, Tensor<T>& output) {   // :500-543
@@ -616,7 +624,7 @@ Tensor<T> einsum_with_plan(const ContractionTree& tree, const std::vector<const 
 template <class T>
 Tensor<T> einsum_with_subscripts(const Subscripts& subscripts, const std::vector<const Tensor<T>*>& operands) {
     detail::common_space(operands);
-    return einsum_with_plan(ContractionTree::optimize(subscripts, detail::shapes_of(operands)), operands);
+    return einsum_with_plan(ContractionTree::optimize_cached(subscripts, detail::shapes_of(operands)), operands);
 }
 template <class T>
 Tensor<T> einsum(const std::string& notation, const std::vector<const Tensor<T>*>& operands) {
@@ -639,7 +647,7 @@ template <class T>
 Tensor<T> einsum_with_subscripts_owned(const Subscripts& subscripts, std::vector<Tensor<T>> operands) {
     auto ptrs = detail::pointers(operands);
     detail::common_space(ptrs);
-    auto tree = ContractionTree::optimize(subscripts, detail::shapes_of(ptrs));
+    auto tree = ContractionTree::optimize_cached(subscripts, detail::shapes_of(ptrs));
     return einsum_with_plan_owned(tree, std::move(operands));
 }
 template <class T>

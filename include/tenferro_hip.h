@@ -189,6 +189,15 @@ int32_t tfh_tree_optimize(const tfh_subscripts* s, const int64_t* const* shapes,
 int32_t tfh_tree_from_pairs(const tfh_subscripts* s, const int64_t* const* shapes, const int32_t* ranks,
                             int32_t n_inputs, const int32_t* pairs, int32_t n_pairs, tfh_tree** out);
 void tfh_tree_destroy(tfh_tree* t);
+/* The same tree as tfh_tree_optimize, from a process-wide cache keyed on the subscripts (labels, grouping) and the
+ * shapes: the string and allocating forms of einsum (tenferro-einsum/src/lib.rs:393-434, :541-582) optimise the same
+ * network on every call, which costs 5 us for two operands and milliseconds for eight.  The tree is shared and
+ * immutable; release it with tfh_tree_destroy like any other (trees are reference counted, so one that the cache has
+ * dropped stays valid for its holders).  At most 512 networks are kept, least recently used dropped first. */
+int32_t tfh_tree_optimize_cached(const tfh_subscripts* s, const int64_t* const* shapes, const int32_t* ranks,
+                                 int32_t n_inputs, tfh_tree** out);
+int32_t tfh_tree_cache_stats(int64_t* hits, int64_t* misses, int64_t* entries);   /* any pointer may be null */
+int32_t tfh_tree_cache_clear(void);
 int32_t tfh_tree_n_inputs(const tfh_tree* t);
 int32_t tfh_tree_n_steps(const tfh_tree* t);
 /* Step i contracts operands (lhs, rhs) into intermediate n_inputs + i. */

@@ -95,6 +95,8 @@ def lib():
             getattr(L, name).argtypes = [C.c_void_p]
         L.tfh_subscripts_input_rank.argtypes = [C.c_void_p, C.c_int32]
         L.tfh_tree_optimize.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
+        L.tfh_tree_optimize_cached.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
+        L.tfh_tree_cache_stats.argtypes = [C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
         L.tfh_tree_from_pairs.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p]
         L.tfh_plan_create.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
         L.tfh_plan_create_grouped.argtypes = [C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
@@ -490,6 +492,15 @@ class ContractionTree:
         return cls(out.value)
 
     @classmethod
+    def optimize_cached(cls, subscripts, shapes):
+        """The tree `optimize` returns, shared through the library's cache of optimised networks (no counterpart in the
+        reference: the einsum functions that take no plan use it so that a repeated call does not search again)."""
+        ptrs, ranks, keep = _shapes_c(shapes)
+        out = C.c_void_p()
+        _check(lib().tfh_tree_optimize_cached(subscripts._h, ptrs, ranks, len(shapes), C.byref(out)))
+        return cls(out.value)
+
+    @classmethod
     def from_pairs(cls, subscripts, shapes, pairs):
         ptrs, ranks, keep = _shapes_c(shapes)
         flat = [int(x) for p in pairs for x in p]
@@ -849,7 +860,7 @@ def einsum_with_plan(tree, operands, stream=None, _donate=0):
 def einsum_with_subscripts(subscripts, operands, stream=None):
     """:397-412"""
     _dispatch_check(operands)
-    tree = ContractionTree.optimize(subscripts, [t.dims() for t in operands])
+    tree = ContractionTree.optimize_cached(subscripts, [t.dims() for t in operands])
     return einsum_with_plan(tree, operands, stream)
 
 
@@ -860,7 +871,7 @@ def einsum(subscripts, operands, stream=None):
 
 def einsum_with_subscripts_into(subscripts, operands, alpha, beta, output, stream=None):
     """:578-582"""
-    tree = ContractionTree.optimize(subscripts, [t.dims() for t in operands])
+    tree = ContractionTree.optimize_cached(subscripts, [t.dims() for t in operands])
     einsum_with_plan_into(tree, operands, alpha, beta, output, stream)
 
 
@@ -880,7 +891,7 @@ def einsum_with_plan_owned(tree, operands, stream=None):
 
 def einsum_with_subscripts_owned(subscripts, operands, stream=None):
     """:474-480"""
-    tree = ContractionTree.optimize(subscripts, [t.dims() for t in operands])
+    tree = ContractionTree.optimize_cached(subscripts, [t.dims() for t in operands])
     return einsum_with_plan_owned(tree, operands, stream)
 
 
@@ -896,6 +907,13 @@ PROF_CONTRACT, PROF_COPY, PROF_REDUCE = 0, 1, 2
 def profile_enable(on=True):
     """Bracket the dominant kernel of every launch with HIP events on its stream (tfh_profile_enable)."""
     _check(lib().tfh_profile_enable(1 if on else 0))
+
+
+def tree_cache_stats():
+    """(hits, misses, entries) of the library's cache of optimised einsum networks."""
+    h, m, e = C.c_int64(), C.c_int64(), C.c_int64()
+    _check(lib().tfh_tree_cache_stats(C.byref(h), C.byref(m), C.byref(e)))
+    return h.value, m.value, e.value
 
 
 def last_kernel():

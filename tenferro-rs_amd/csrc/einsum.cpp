@@ -6,12 +6,16 @@
 // device memory taken from the stream's block cache and are laid out so that the step that consumes
 // them reads its contracted modes contiguously.  The host never waits.
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <functional>
+#include <list>
 #include <map>
+#include <mutex>
 #include <set>
 #include <string>
+#include <unordered_map>
 
 #include "internal.hpp"
 
@@ -48,6 +52,7 @@ struct tfh_tree {
     std::vector<TreeNode> nodes;    // inputs after diagonal/pre-reduction (unique labels), then intermediates
     std::vector<TreeStep> steps;
     double macs = 0, peak = 0;
+    std::atomic<int> refs{1};   // the creator's reference; the tree cache and each of its hits hold one more
 };
 
 namespace {
@@ -374,6 +379,22 @@ void finish_tree(tfh_tree& t) {
 
 }  // namespace
 
+// ---- tree cache: the allocating / string forms of einsum optimise the same network on every call
+namespace {
+constexpr size_t TREE_CACHE_ENTRIES = 512;
+struct TreeCache {
+    std::mutex mu;
+    std::list<std::string> order;   // most recently used first
+    std::unordered_map<std::string, std::pair<tfh_tree*, std::list<std::string>::iterator>> map;
+    int64_t hits = 0, misses = 0;
+};
+TreeCache& tree_cache() {
+    static TreeCache* c = new TreeCache();   // never destroyed: trees may be released during process exit
+    return *c;
+}
+void put_u64(std::string& k, uint64_t v) { k.append(reinterpret_cast<const char*>(&v), sizeof v); }
+}  // namespace
+
 extern "C" {
 
 int32_t tfh_subscripts_new(const uint32_t* labels, const int32_t* ranks, int32_t n_inputs, const uint32_t* output,
@@ -534,7 +555,92 @@ int32_t tfh_tree_from_pairs(const tfh_subscripts* s, const int64_t* const* shape
     return TFH_OK;
 }
 
-void tfh_tree_destroy(tfh_tree* t) { delete t; }
+void tfh_tree_destroy(tfh_tree* t) {
+    if (t && t->refs.fetch_sub(1, std::memory_order_acq_rel) == 1) delete t;
+}
+
+int32_t tfh_tree_optimize_cached(const tfh_subscripts* s, const int64_t* const* shapes, const int32_t* ranks, int32_t n_inputs,
+                                 tfh_tree** out) {
+    if (!out) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
+    *out = nullptr;
+    if (!s || n_inputs != (int32_t)s->inputs.size() || (n_inputs > 0 && (!shapes || !ranks)))
+        return tfh_tree_optimize(s, shapes, ranks, n_inputs, out);   // reports the error
+    // key: the labels of every operand and of the output, the grouping the parentheses spell, and the extents
+    std::string key;
+    put_u64(key, (uint64_t)n_inputs);
+    for (int i = 0; i < n_inputs; ++i) {
+        if (ranks[i] != (int32_t)s->inputs[i].size() || (ranks[i] > 0 && !shapes[i])) return tfh_tree_optimize(s, shapes, ranks, n_inputs, out);
+        put_u64(key, (uint64_t)ranks[i]);
+        for (int d = 0; d < ranks[i]; ++d) {
+            put_u64(key, s->inputs[i][d]);
+            put_u64(key, (uint64_t)shapes[i][d]);
+        }
+    }
+    put_u64(key, (uint64_t)s->output.size());
+    for (uint32_t l : s->output) put_u64(key, l);
+    if (s->has_parens) {
+        std::function<void(int)> emit = [&](int n) {
+            if (s->nest[n].leaf >= 0) {
+                put_u64(key, (uint64_t)s->nest[n].leaf);
+                return;
+            }
+            put_u64(key, ~(uint64_t)0);
+            for (int c : s->nest[n].children) emit(c);
+            put_u64(key, ~(uint64_t)1);
+        };
+        emit(s->root);
+    }
+    TreeCache& c = tree_cache();
+    {
+        std::lock_guard<std::mutex> lk(c.mu);
+        auto it = c.map.find(key);
+        if (it != c.map.end()) {
+            c.order.splice(c.order.begin(), c.order, it->second.second);
+            it->second.first->refs.fetch_add(1, std::memory_order_relaxed);
+            *out = it->second.first;
+            ++c.hits;
+            clear_error();
+            return TFH_OK;
+        }
+    }
+    tfh_tree* t = nullptr;
+    if (int32_t e = tfh_tree_optimize(s, shapes, ranks, n_inputs, &t)) return e;
+    {
+        std::lock_guard<std::mutex> lk(c.mu);
+        ++c.misses;
+        if (c.map.find(key) == c.map.end()) {   // (another thread may have inserted the same network meanwhile)
+            while (c.map.size() >= TREE_CACHE_ENTRIES) {
+                auto victim = c.map.find(c.order.back());
+                tfh_tree_destroy(victim->second.first);   // callers that still hold it keep it alive
+                c.map.erase(victim);
+                c.order.pop_back();
+            }
+            c.order.push_front(key);
+            t->refs.fetch_add(1, std::memory_order_relaxed);
+            c.map.emplace(key, std::make_pair(t, c.order.begin()));
+        }
+    }
+    *out = t;
+    return TFH_OK;
+}
+
+int32_t tfh_tree_cache_stats(int64_t* hits, int64_t* misses, int64_t* entries) {
+    TreeCache& c = tree_cache();
+    std::lock_guard<std::mutex> lk(c.mu);
+    if (hits) *hits = c.hits;
+    if (misses) *misses = c.misses;
+    if (entries) *entries = (int64_t)c.map.size();
+    return TFH_OK;
+}
+
+int32_t tfh_tree_cache_clear(void) {
+    TreeCache& c = tree_cache();
+    std::lock_guard<std::mutex> lk(c.mu);
+    for (auto& kv : c.map) tfh_tree_destroy(kv.second.first);
+    c.map.clear();
+    c.order.clear();
+    return TFH_OK;
+}
 int32_t tfh_tree_n_inputs(const tfh_tree* t) { return t ? t->n_inputs : 0; }
 int32_t tfh_tree_n_steps(const tfh_tree* t) { return t ? (int32_t)t->steps.size() : 0; }
 int32_t tfh_tree_step(const tfh_tree* t, int32_t i, int32_t* lhs, int32_t* rhs) {

@@ -142,6 +142,14 @@ static void gpu_checks() {
     CHECK(rel_frobenius(einsum_with_plan<double>(tree, {&A, &B}).to_vec(), ref) < 1e-12);
     CHECK(rel_frobenius(einsum_with_subscripts<double>(subs, {&A, &B}).to_vec(), ref) < 1e-12);
     CHECK(rel_frobenius(einsum_owned<double>("ij,jk->ik", {A, B}).to_vec(), ref) < 1e-12);
+    {   // the plan-less forms share one cached tree per network: a repeated call is a hit and gives the same result
+        int64_t h0 = 0, m0 = 0, h1 = 0, m1 = 0;
+        tfh_tree_cache_stats(&h0, &m0, nullptr);
+        CHECK(rel_frobenius(einsum<double>("ij,jk->ik", {&A, &B}).to_vec(), ref) < 1e-12);
+        CHECK(rel_frobenius(einsum<double>("ij,jk->ik", {&A, &B}).to_vec(), ref) < 1e-12);
+        tfh_tree_cache_stats(&h1, &m1, nullptr);
+        CHECK(h1 - h0 == 2 && m1 == m0);
+    }
     // the copies handed over above share A's and B's buffers, so nothing was donated and both are intact
     CHECK(A.to_vec() == ha && B.to_vec() == hb);
     {   // a chain whose operands are moved in: each is the sole owner of its buffer, which may then hold an intermediate

@@ -263,6 +263,82 @@ def test_tree_greedy_beyond_twelve_operands(tf):
     assert len(tree.steps) == n - 1 and tree.mac_count == (n - 1) * 64
 
 
+def test_tree_cache_shares_a_network_and_tells_networks_apart(tf):
+    # the plan-less einsum functions take their tree from a cache keyed on labels, grouping and extents: the same
+    # network is searched once, every differing ingredient is its own entry, errors are reported as by optimize
+    L = tf.lib()
+    L.tfh_tree_cache_clear()
+    h0, m0, e0 = tf.tree_cache_stats()
+    assert e0 == 0
+    net, shapes = "awc,asx,wstv,cty->xvy", [[8, 4, 8], [8, 2, 8], [4, 2, 2, 4], [8, 2, 8]]
+    t1 = tf.ContractionTree.optimize_cached(tf.Subscripts.parse(net), shapes)
+    t2 = tf.ContractionTree.optimize_cached(tf.Subscripts.parse(net), shapes)       # another Subscripts object, same key
+    fresh = tf.ContractionTree.optimize(tf.Subscripts.parse(net), shapes)
+    assert t1._h == t2._h != fresh._h
+    assert t1.steps == fresh.steps and t1.mac_count == fresh.mac_count and t1.output_dims == fresh.output_dims
+    h1, m1, e1 = tf.tree_cache_stats()
+    assert (h1 - h0, m1 - m0, e1) == (1, 1, 1)
+    others = [tf.ContractionTree.optimize_cached(tf.Subscripts.parse(n), sh) for n, sh in [
+        (net, [[8, 4, 8], [8, 2, 16], [4, 2, 2, 4], [8, 2, 16]]),              # other extents
+        ("awc,asx,wstv,cty->xyv", shapes),                                        # other output order
+        ("awc,asx,wstv,cyt->xvy", [[8, 4, 8], [8, 2, 8], [4, 2, 2, 4], [8, 8, 2]]),   # other operand labels
+        ("(awc,asx),(wstv,cty)->xvy", shapes),                                    # forced grouping
+        ("(awc,cty),(asx,wstv)->xvy", [shapes[0], shapes[3], shapes[1], shapes[2]])]]   # another grouping and operand order
+    handles = {t1._h} | {t._h for t in others}
+    assert len(handles) == 6 and tf.tree_cache_stats()[2] == 6
+    # integer-label subscripts with the same labels hit the entry of the parsed string
+    ints = tf.Subscripts.new([[ord(c) for c in term] for term in "awc,asx,wstv,cty".split(",")], [ord(c) for c in "xvy"])
+    assert tf.ContractionTree.optimize_cached(ints, shapes)._h == t1._h
+    with pytest.raises(tf.ShapeMismatch):
+        tf.ContractionTree.optimize_cached(tf.Subscripts.parse("ij,jk->ik"), [[3, 4], [5, 6]])
+    with pytest.raises(tf.RankMismatch):
+        tf.ContractionTree.optimize_cached(tf.Subscripts.parse("ij,jk->ik"), [[3, 4], [4, 6, 1]])
+    with pytest.raises(tf.InvalidArgument):
+        tf.ContractionTree.optimize_cached(tf.Subscripts.parse("ij,jk->ik"), [[3, 4]])
+    assert tf.tree_cache_stats()[2] == 6          # failures leave no entry
+
+
+def test_tree_cache_drops_the_least_recently_used_and_holders_keep_their_tree(tf):
+    L = tf.lib()
+    L.tfh_tree_cache_clear()
+    s = tf.Subscripts.parse("ij,jk,kl->il")
+    first = tf.ContractionTree.optimize_cached(s, [[2, 3], [3, 4], [4, 1000]])
+    steps, macs = first.steps, first.mac_count
+    for n in range(1, 700):                        # more networks than the cache keeps (512)
+        tf.ContractionTree.optimize_cached(s, [[2, 3], [3, 4], [4, n]])
+        if n % 100 == 0:                           # keep one entry in use: it must survive
+            tf.ContractionTree.optimize_cached(s, [[2, 3], [3, 4], [4, 1]])
+    hits, misses, entries = tf.tree_cache_stats()
+    assert entries == 512
+    assert first.steps == steps and first.mac_count == macs      # dropped by the cache, alive for its holder
+    again = tf.ContractionTree.optimize_cached(s, [[2, 3], [3, 4], [4, 1000]])
+    assert again._h != first._h and again.steps == steps         # searched again after the drop
+    h2 = tf.tree_cache_stats()[0]
+    tf.ContractionTree.optimize_cached(s, [[2, 3], [3, 4], [4, 1]])
+    assert tf.tree_cache_stats()[0] == h2 + 1                    # the entry kept in use is still cached
+    L.tfh_tree_cache_clear()
+    assert tf.tree_cache_stats()[2] == 0 and again.steps == steps
+
+
+def test_tree_cache_is_safe_from_several_threads(tf):
+    import threading
+    tf.lib().tfh_tree_cache_clear()
+    s = tf.Subscripts.parse("ab,bc,cd,de->ae")
+    ref = {n: tf.ContractionTree.optimize(s, [[n, 5], [5, 7], [7, 3], [3, n]]).steps for n in range(1, 40)}
+    bad = []
+    def work(seed):
+        rng = np.random.default_rng(seed)
+        for _ in range(400):
+            n = int(rng.integers(1, 40))
+            t = tf.ContractionTree.optimize_cached(s, [[n, 5], [5, 7], [7, 3], [3, n]])
+            if t.steps != ref[n]:
+                bad.append(n)
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(8)]
+    for t in threads: t.start()
+    for t in threads: t.join()
+    assert not bad and tf.tree_cache_stats()[2] == 39
+
+
 # ---------------------------------------------------------------------------------------------- Tensor metadata
 def test_tensor_metadata_reference_doc_examples(tf):
     T, col = tf.Tensor, tf.MemoryOrder.ColumnMajor
