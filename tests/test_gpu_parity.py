@@ -1554,3 +1554,77 @@ def test_calls_from_several_host_threads_on_their_own_streams(tf, oracle):
     for th in threads:
         th.join()
     assert not errors, errors
+
+
+def test_operand_above_4_gib(tf, oracle):
+    # An f32 matrix of 40000 x 30000 (4.8 GB): element byte offsets pass 2^32, so the large-tile kernel's 32-bit
+    # addressing does not apply and the kernels with 64-bit addressing take over.  The tensor is too large for the
+    # oracle as a whole: data movement is checked through the involution (bit for bit, on the device) and arithmetic
+    # against the oracle on sampled rows, some of them beyond the 4 GiB mark and on tile boundaries.
+    import torch
+    m, k = 40000, 30000
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    x = torch.randn(m, k, dtype=torch.float32, device="cuda", generator=gen)
+    X = tf.Tensor.from_torch(x)
+    rows = [0, 1, 63, 64, 127, 128, 20011, 35791, 35792, 39935, 39936, 39999]
+    xs = x[rows].cpu().numpy()
+    rng = np.random.default_rng(111)
+
+    t = tf.Tensor.empty([k, m], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
+    back = tf.Tensor.empty([m, k], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
+    tf.HipBackend.execute(tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Permute([0, 1], [1, 0]), [[m, k], [k, m]]), 1.0, [X], 0.0, t)
+    tf.HipBackend.execute(tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Permute([0, 1], [1, 0]), [[k, m], [m, k]]), 1.0, [t], 0.0, back)
+    assert torch.equal(back._buf.view(m, k), x)
+    assert np.array_equal(t._buf.view(k, m)[:, rows].cpu().numpy(), xs.T)
+    del back, t
+
+    def sampled(out, width):
+        return out._buf.view(m, width)[rows].cpu().numpy() if width else out._buf[rows].cpu().numpy()
+
+    v = rand(rng, (k,), np.float32)
+    out = tf.Tensor.empty([m], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
+    tf.HipBackend.execute(tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Contract(lab("mk"), lab("k"), lab("m")), [[m, k], [k], [m]]), 1.0, [X, dev(tf, v)], 0.0, out)
+    ref = np.empty(len(rows), np.float32)
+    oracle.contract(xs, lab("mk"), v, lab("k"), ref, lab("m"))
+    assert relerr(sampled(out, 0), ref) < 1e-5, tf.last_kernel()
+
+    tf.HipBackend.execute(tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Reduce([0, 1], [0], tf.ReduceOp.Sum), [[m, k], [m]]), 1.0, [X], 0.0, out)
+    oracle.reduce(xs, [0, 1], ref, [0])
+    assert relerr(sampled(out, 0), ref) < 1e-5, tf.last_kernel()
+
+    for n in (64, 256):      # a thin and a wide right-hand side
+        w = rand(rng, (k, n), np.float32)
+        out = tf.Tensor.empty([m, n], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
+        tf.HipBackend.execute(tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Contract(lab("mk"), lab("kn"), lab("mn")), [[m, k], [k, n], [m, n]]), 1.0, [X, dev(tf, w)], 0.0, out)
+        assert "gemm_kernel" in tf.last_kernel(), tf.last_kernel()     # 64-bit addressing
+        ref = np.empty((len(rows), n), np.float32)
+        oracle.contract(xs, lab("mk"), w, lab("kn"), ref, lab("mn"))
+        assert relerr(sampled(out, n), ref) < 1e-5, n
+
+
+def test_long_grids_and_high_rank(tf, oracle):
+    # extents past the 65535 limit of a grid's y and z dimensions, many small outputs, a rank-12 permutation
+    rng = np.random.default_rng(112)
+    x = rand(rng, (70000, 3, 5), np.float64)
+    out = dev(tf, np.zeros((5, 70000, 3)))
+    tf.HipBackend.execute(tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute([0, 1, 2], [2, 0, 1]), [x.shape, out.dims()]), 1.0, [dev(tf, x)], 0.0, out)
+    assert out.to_numpy().tobytes() == np.ascontiguousarray(x.transpose(2, 0, 1)).tobytes()
+    for shape, keep in [((300000, 7), 0), ((7, 300000), 1)]:
+        y = rand(rng, shape, np.float64)
+        ref = np.empty(300000)
+        oracle.reduce(y, [0, 1], ref, [keep])
+        out = dev(tf, np.zeros(300000))
+        tf.HipBackend.execute(tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Reduce([0, 1], [keep], tf.ReduceOp.Sum), [list(shape), [300000]]), 1.0, [dev(tf, y)], 0.0, out)
+        assert relerr(out.to_numpy(), ref) < 1e-12, shape
+    a, b = rand(rng, (70000, 3, 4), np.float64), rand(rng, (70000, 4, 5), np.float64)
+    ref = np.empty((70000, 3, 5))
+    oracle.contract(a, lab("bij"), b, lab("bjk"), ref, lab("bik"))
+    got = tf.einsum("bij,bjk->bik", [dev(tf, a), dev(tf, b)])
+    assert relerr(got.to_numpy(), ref) < 1e-12, tf.last_kernel()
+    shape = [2, 3] * 6
+    perm = [11, 0, 9, 2, 7, 4, 5, 6, 3, 8, 1, 10]
+    z = rand(rng, shape, np.float64)
+    oshape = [shape[q] for q in perm]
+    out = dev(tf, np.zeros(oshape))
+    tf.HipBackend.execute(tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute(list(range(12)), perm), [shape, oshape]), 1.0, [dev(tf, z)], 0.0, out)
+    assert out.to_numpy().tobytes() == np.ascontiguousarray(z.transpose(perm)).tobytes()
