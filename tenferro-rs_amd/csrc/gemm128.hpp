@@ -275,10 +275,17 @@ __global__ void __launch_bounds__((Cfg128<R, CX, BNV>::NT), (Cfg128<R, CX, BNV>:
     typedef OperandMap<R, CX, BNE, BKF, VB, (CX ? 2 : 1), BNV> MapB;
     MapA ma;
     MapB mb;
-    ma.init(am, ak, m0, rowsA);
+    // single-stride rows: the tile's first row goes into the 64-bit base and the offsets start at row 0, so that they
+    // span one tile whatever the operand's size.  A vector moved back at a matrix edge can start a few rows before
+    // the tile: the host's bias leaves room for that.  Grouped problems carry no bias (and are small): their offsets
+    // stay relative to the problem's first row.
+    const bool rebase_a = !am.tab && !g.problems, rebase_b = !bn.tab && !g.problems;
+    if (rebase_a) Ap += (int64_t)(int32_t)am.stride * m0;
+    if (rebase_b) Bp += (int64_t)(int32_t)bn.stride * n0;
+    ma.init(am, ak, rebase_a ? 0 : m0, rowsA);
 #pragma unroll
     for (int l = 0; l < MapA::NL; ++l) ma.voff[l] += g.problems ? 0u : g.bias_a32;
-    mb.init(bn, bk, n0, rowsB);
+    mb.init(bn, bk, rebase_b ? 0 : n0, rowsB);
 #pragma unroll
     for (int l = 0; l < MapB::NL; ++l) mb.voff[l] += g.problems ? 0u : g.bias_b32;
     // uniform bases; single-stride k advances them by one stage per iteration

@@ -798,12 +798,27 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
                          (long long)g.tiles_m * g.tiles_n, (long long)(nb * nsplit));
     }
 
-    // The 128x128 kernel addresses each operand as a uniform base + 32-bit byte offset: usable when the
-    // bytes reachable inside one batch entry span less than 4 GiB (larger operands take the generic kernel).
+    // The 128x128 kernel addresses each operand as a uniform 64-bit base + unsigned 32-bit byte offsets.  A group
+    // with a single stride is folded into the base (the tile's first row, the stage's first k), so its offsets only
+    // cover one tile or stage -- taken as 128 indices with 8 of slack either way, because a vector that is moved back
+    // at a matrix edge can start a few rows before its tile; a multi-axis group goes through a 32-bit table over its
+    // whole extent.  Usable when the offsets of
+    // an operand span less than 4 GiB: always for operands below 4 GiB, and for larger ones whose long groups have
+    // a single stride (anything else takes the generic kernel with 64-bit offsets).
     bool use128 = bm == 128 && !skinny;
     int64_t lo_a = 0, hi_a = 0, lo_b = 0, hi_b = 0;
-    reach(ax.M, 0, lo_a, hi_a); reach(ax.K, 0, lo_a, hi_a);
-    reach(ax.N, 1, lo_b, hi_b); reach(ax.K, 1, lo_b, hi_b);
+    auto tile_reach = [&](const std::vector<Axis>& grp, int slot, int64_t& lo, int64_t& hi) {
+        if (grp.size() == 1) {
+            const int64_t s_ = grp[0].s[slot], top = std::min<int64_t>(grp[0].n, 128) + 8;
+            if (std::llabs(s_) * (int64_t)eb >= ((int64_t)1 << 31)) use128 = false;   // the kernel steps the base by a signed 32-bit stride
+            lo += std::min(-8 * s_, top * s_);
+            hi += std::max(-8 * s_, top * s_);
+        } else {
+            reach(grp, slot, lo, hi);
+        }
+    };
+    tile_reach(ax.M, 0, lo_a, hi_a); tile_reach(ax.K, 0, lo_a, hi_a);
+    tile_reach(ax.N, 1, lo_b, hi_b); tile_reach(ax.K, 1, lo_b, hi_b);
     if ((hi_a - lo_a + 1) * (int64_t)eb >= ((int64_t)1 << 32) || (hi_b - lo_b + 1) * (int64_t)eb >= ((int64_t)1 << 32)) use128 = false;
     if (!use128 && bm == 128) {
         bm = bn = 64;

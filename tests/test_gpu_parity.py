@@ -751,7 +751,10 @@ def test_contract_odd_extents_take_the_straddling_vector_path(tf, oracle, dtype,
         assert relerr(out.to_numpy(), ref) < TOL[dtype], (m, k, n)
 
 
-THIN_SIZES = [(257, 1025, 33), (130, 523, 64), (300, 1040, 95), (47, 1031, 260), (64, 520, 1300), (1801, 66, 67), (513, 5, 80)]
+THIN_SIZES = [(257, 1025, 33), (130, 523, 64), (300, 1040, 95), (47, 1031, 260), (64, 520, 1300), (1801, 66, 67), (513, 5, 80),
+              # a last tile with fewer valid rows than a 16-byte vector and a short k: the vector moved back at the
+              # edge starts before its tile
+              (257, 40, 65), (385, 100, 65), (130, 24, 67), (65, 40, 257)]
 
 
 @pytest.mark.parametrize("dtype", ALL)
@@ -1593,13 +1596,33 @@ def test_operand_above_4_gib(tf, oracle):
     assert relerr(sampled(out, 0), ref) < 1e-5, tf.last_kernel()
 
     for n in (64, 256):      # a thin and a wide right-hand side
+        # rows and k of the big operand have one stride each: the large-tile kernel folds the tile's first row and the
+        # stage's first k into its 64-bit base, so its 32-bit offsets only span a tile
         w = rand(rng, (k, n), np.float32)
         out = tf.Tensor.empty([m, n], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
         tf.HipBackend.execute(tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Contract(lab("mk"), lab("kn"), lab("mn")), [[m, k], [k, n], [m, n]]), 1.0, [X, dev(tf, w)], 0.0, out)
-        assert "gemm_kernel" in tf.last_kernel(), tf.last_kernel()     # 64-bit addressing
+        assert "gemm128_kernel" in tf.last_kernel(), tf.last_kernel()
         ref = np.empty((len(rows), n), np.float32)
         oracle.contract(xs, lab("mk"), w, lab("kn"), ref, lab("mn"))
         assert relerr(sampled(out, n), ref) < 1e-5, n
+        # the big operand on the right (k-contiguous rows of B), the output transposed
+        out = tf.Tensor.empty([n, m], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
+        tf.HipBackend.execute(tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Contract(lab("kn"), lab("mk"), lab("nm")), [[k, n], [m, k], [n, m]]), 1.0, [dev(tf, w), X], 0.0, out)
+        assert "gemm128_kernel" in tf.last_kernel(), tf.last_kernel()
+        assert relerr(out._buf.view(n, m)[:, rows].cpu().numpy(), ref.T) < 1e-5, n
+    # the same matrix as a [200, 199, k] view of [200, 200, k]: the row group has two strides that do not fuse, its
+    # 32-bit table would have to span the whole operand -- the kernel with 64-bit offsets takes it
+    n = 256
+    X3 = tf.Tensor(x.view(-1), [200, 199, k], [200 * k, k, 1], 0, tf.GpuMemory(0), tf.dtype_code(np.dtype(np.float32)))
+    out = tf.Tensor.empty([200, 199, n], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
+    tf.HipBackend.execute(tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Contract(lab("abk"), lab("kn"), lab("abn")), [[200, 199, k], [k, n], [200, 199, n]]), 1.0, [X3, dev(tf, w)], 0.0, out)
+    assert "(gemm_kernel" in tf.last_kernel(), tf.last_kernel()
+    pick = [(0, 0), (0, 198), (1, 0), (99, 57), (178, 190), (179, 0), (199, 198)]
+    xs3 = np.stack([x[a_ * 200 + b_].cpu().numpy() for a_, b_ in pick])
+    ref = np.empty((len(pick), n), np.float32)
+    oracle.contract(xs3, lab("mk"), w, lab("kn"), ref, lab("mn"))
+    got = np.stack([out._buf.view(200, 199, n)[a_, b_].cpu().numpy() for a_, b_ in pick])
+    assert relerr(got, ref) < 1e-5
 
 
 def test_long_grids_and_high_rank(tf, oracle):
