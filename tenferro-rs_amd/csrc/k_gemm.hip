@@ -754,14 +754,15 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         // 128x128 tiles: 512 blocks are resident at a time (two per CU).  Estimated time of a split count s, in us, from
         // what the kernel measures on this device: a block-stage takes 1.95 us of a CU's matrix cores, a block costs
         // about eight more stages of prologue and epilogue, two blocks sharing a CU overlap fully, one alone leaves
-        // latency exposed (x1.25), and the fold moves the partials twice.  Picks the s with the least estimate: it
+        // latency exposed (x1.7 when the whole launch is one block per CU, x1.25 for the tail of a longer launch), and
+        // the fold moves the partials twice.  Picks the s with the least estimate: it
         // trades the idle tail of a partly filled last round against per-block overhead and partial traffic.
         auto estimate = [&](int s_) {
             const double per_block = ((double)((kstages + s_ - 1) / s_) + 8.0) * 1.95 * (double)bn / 128.0;
             const int64_t blocks = tiles * s_, full = blocks / 512, rem = blocks % 512;
             double t = (double)full * 2.0 * per_block;
             if (rem > 256) t += 2.0 * per_block;
-            else if (rem > 0) t += 1.25 * per_block;
+            else if (rem > 0) t += (full == 0 ? 1.7 : 1.25) * per_block;
             if (s_ > 1) t += 3.0 + (double)s_ * (double)(nb * M * NR * rb) * 2.0 / 10e6;
             return t;
         };
