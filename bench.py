@@ -32,7 +32,7 @@ PEAK = {"hbm": 8000.0, "f32": 157.3, "f64": 78.6}   # GB/s, TFLOP/s (MI355X publ
 # WRITE_SIZE) summarised in profiles/bench_hbm_traffic_pmc.txt, each scaled by what the same counter read for plain
 # 1 GiB device copies in the same run (x2.0 and x1.0).  A profiler cannot run inside this script; these are that run's
 # figures for exactly these workloads.
-TRAFFIC = {"c1": 249.0e6, "c2_permute": 268.6e6, "c2_reduce": 134.9e6, "c3": 7071.7e6, "c4": 3065.9e6}
+TRAFFIC = {"c1": 249.0e6, "c2_permute": 268.6e6, "c2_reduce": 134.9e6, "c3": 7079.5e6, "c4": 3066.4e6}
 SPINUP_S = 0.3   # seconds of untimed device spin-up per configuration
 METRIC = "contraction TFLOP/s & % MFMA peak (f64/f32); permute/reduce GB/s & % HBM peak"
 
@@ -147,7 +147,7 @@ def run_c1(h):
         "roofline": {"bound": "mfma", "achieved": flops / (kms * 1e-3) / 1e12, "peak": PEAK["f32"], "unit": "TFLOP/s",
                      "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f32"], "traffic": TRAFFIC["c1"],
                      "traffic_unit": "HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, calibrated)",
-                     "kernel": "gemm128_kernel<float, false, true, true, 4, 4> (split-K 8)", "kernel_ms": kms, "launches_per_step": per_step},
+                     "kernel": "gemm128_kernel<float, false, true, true, 4, 4, 128> (split-K 8)", "kernel_ms": kms, "launches_per_step": per_step},
     }
     if h.cpu:
         ref = np.empty((a, b, c), np.float32)
@@ -230,7 +230,7 @@ def run_c3(h):
         "peak_intermediate_bytes": tree.peak_intermediate * 16,
         "roofline": {"bound": "mfma", "achieved": flops / (total_kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
                      "frac": flops / (total_kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": TRAFFIC["c3"],
-                     "kernel": "gemm128_kernel<double, true, ..., 1, 1> x2 + gemm_skinny_kernel<true> x1 (the three pairwise contractions of the tree)",
+                     "kernel": "gemm128_kernel<double, true, ..., 1, 1, 128> x2 + gemm_skinny_kernel<true> x1 (the three pairwise contractions of the tree)",
                      "kernel_ms": total_kms, "launches_per_step": per_step},
     }
     if h.cpu:
@@ -263,7 +263,7 @@ def run_c4(h):
         "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
         "roofline": {"bound": "mfma", "achieved": flops / (kms * 1e-3) / 1e12, "peak": PEAK["f64"], "unit": "TFLOP/s",
                      "frac": flops / (kms * 1e-3) / 1e12 / PEAK["f64"], "traffic": TRAFFIC["c4"],
-                     "kernel": "gemm128_kernel<double, false, true, false, 2, 2> (grouped)", "kernel_ms": kms, "launches_per_step": per_step},
+                     "kernel": "gemm128_kernel<double, false, true, false, 2, 2, 128> (grouped)", "kernel_ms": kms, "launches_per_step": per_step},
     }
     if h.cpu:
         refs = [np.empty((i, k)) for i, j, k in dims]
