@@ -262,8 +262,11 @@ private:
     std::shared_ptr<void> e_;
 };
 
+template <class T> class TensorView;
+
 template <class T>
 class Tensor {   // tenferro-tensor/src/lib.rs:167-181
+    friend class TensorView<T>;
 public:
     // ---- constructors (:336-369)
     static Tensor zeros(const std::vector<size_t>& dims, LogicalMemorySpace space, MemoryOrder order) { return filled(dims, space, order, T(0)); }
@@ -300,6 +303,7 @@ public:
         return StridedView<T>{(T*)buf_->dev, dims_, strides_, offset_};
     }
     StridedViewMut<T> view_mut() { return view(); }
+    TensorView<T> tensor_view() const;   // :455-470: waits, then a borrowed view without a pending event
 
     // ---- zero-copy metadata operations (:502-548)
     Tensor permute(const std::vector<size_t>& perm) const {
@@ -487,6 +491,34 @@ private:
         return t;
     }
 };
+
+// Borrowed counterpart of Tensor (tenferro-tensor/src/lib.rs:183-300): shares the source's buffer (a reference count
+// stands in for the borrow), carries no pending event, offers the zero-copy view operations and the copying
+// to_tensor / contiguous / conj.
+template <class T>
+class TensorView {
+public:
+    const std::vector<size_t>& dims() const { return t_.dims(); }
+    const std::vector<ptrdiff_t>& strides() const { return t_.strides(); }
+    size_t ndim() const { return t_.ndim(); }
+    LogicalMemorySpace logical_memory_space() const { return t_.logical_memory_space(); }
+    std::optional<ComputeDevice> preferred_compute_device() const { return t_.preferred_compute_device(); }
+    TensorView permute(const std::vector<size_t>& perm) const { return TensorView(t_.permute(perm)); }                              // :250
+    TensorView broadcast(const std::vector<size_t>& target) const { return TensorView(t_.broadcast(target)); }                      // :262
+    TensorView diagonal(const std::vector<std::pair<size_t, size_t>>& axes) const { return TensorView(t_.diagonal(axes)); }         // :272
+    Tensor<T> to_tensor(MemoryOrder order) const { return t_.contiguous(order); }    // :281: always a fresh buffer
+    Tensor<T> contiguous(MemoryOrder order) const { return t_.contiguous(order); }   // :286
+    Tensor<T> conj() const { return t_.conj(); }                                     // :293
+private:
+    friend class Tensor<T>;
+    explicit TensorView(Tensor<T> t) : t_(std::move(t)) { t_.event_.reset(); }
+    Tensor<T> t_;
+};
+template <class T>
+TensorView<T> Tensor<T>::tensor_view() const {
+    wait();
+    return TensorView<T>(*this);
+}
 
 // ---------------------------------------------------------------------------------------------- tenferro-einsum
 class Subscripts {   // tenferro-einsum/src/lib.rs:239-283

@@ -785,6 +785,31 @@ class Tensor:
         self.event = CompletionEvent(st)
         return self
 
+    def view(self):
+        """:445-449: the element view for host-side inspection.  Waits for pending work.  A main-memory tensor gives a
+        numpy view with this tensor's dims and element strides over its buffer; device memory cannot back a host slice
+        (use to_numpy, or to_memory_space_async, for a copy)."""
+        self.wait()
+        if self.logical_memory_space_.kind != 0:
+            raise InvalidArgument("invalid argument: view() of a tensor in GPU memory; copy it with to_memory_space_async first")
+        return self._host_view(False)
+
+    def _host_view(self, writeable):
+        flat = np.asarray(self._buf).reshape(-1)
+        isz = flat.dtype.itemsize
+        return np.lib.stride_tricks.as_strided(flat[self._offset:], shape=self._dims, strides=[st * isz for st in self._strides],
+                                               writeable=writeable and flat.flags.writeable)
+
+    def view_mut(self):
+        """:452-454"""
+        self.view()
+        return self._host_view(True)
+
+    def tensor_view(self):
+        """:455-470: waits, then a borrowed view (event None) sharing this tensor's buffer."""
+        self.wait()
+        return TensorView(self._like(self._dims, self._strides))
+
     def to_memory_space_async(self, target):
         """:660-671: same space -> self; Main->Gpu / Gpu->Main copy the underlying buffer."""
         if target == self.logical_memory_space_:
@@ -831,6 +856,64 @@ def _dispatch_check(operands, op_kind=OpKind.Contract):
     if not devices or devices[0].kind != ComputeDevice.HIP or space.kind != 1 or devices[0].device_id != space.space_id:
         raise NoCompatibleComputeDevice(f"no compatible compute device for Contract on {space!r}", space, op_kind)
     return space
+
+
+class TensorView:
+    """tenferro-tensor/src/lib.rs:183-300: the borrowed counterpart of Tensor.  It shares the source tensor's buffer,
+    carries no pending event (tensor_view() has waited) and offers the zero-copy view operations plus the copying
+    to_tensor / contiguous / conj."""
+
+    def __init__(self, tensor):
+        self._t = tensor
+        self._t.event = None
+
+    def dims(self):
+        return self._t.dims()
+
+    def strides(self):
+        return self._t.strides()
+
+    def ndim(self):
+        return self._t.ndim()
+
+    def logical_memory_space(self):
+        return self._t.logical_memory_space()
+
+    def preferred_compute_device(self):
+        return self._t.preferred_compute_device()
+
+    def permute(self, perm):
+        """:250-252"""
+        return TensorView(self._t.permute(perm))
+
+    def broadcast(self, target_dims):
+        """:262-264"""
+        return TensorView(self._t.broadcast(target_dims))
+
+    def diagonal(self, axes):
+        """:272-274"""
+        return TensorView(self._t.diagonal(axes))
+
+    def to_tensor(self, order):
+        """:281-283: always a fresh buffer, laid out in `order`."""
+        t = self._t
+        if t.logical_memory_space_.kind == 0:
+            return Tensor.from_slice(t.to_numpy().ravel(order="F" if order == MemoryOrder.ColumnMajor else "C"), t._dims, order)
+        out = Tensor.empty(t._dims, t.logical_memory_space_, order, t.dtype)
+        modes = list(range(t.ndim()))
+        st = current_stream()
+        HipBackend.execute(HipBackend.plan(t.dtype, PrimDescriptor.Permute(modes, modes), [t._dims, t._dims]), 1.0, [t], 0.0, out, st)
+        out.event = CompletionEvent(st)
+        return out
+
+    def contiguous(self, order):
+        """:286-288: "a contiguous copy of this view's data"."""
+        return self.to_tensor(order)
+
+    def conj(self):
+        """:293-299"""
+        return self._t.conj()
+
 
 
 def einsum_with_plan_into(tree, operands, alpha, beta, output, stream=None, _donate=0):

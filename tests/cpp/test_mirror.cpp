@@ -103,6 +103,17 @@ static void host_checks() {
     auto row = Tensor<double>::from_slice({1, 2, 3}, {3}, MemoryOrder::RowMajor).broadcast({2, 3});
     CHECK(row.strides() == (std::vector<ptrdiff_t>{0, 1}) && row.to_vec() == (std::vector<double>{1, 2, 3, 1, 2, 3}));
     CHECK(raises(Error::Kind::ShapeMismatch, [] { Tensor<double>::from_slice({1, 2, 3}, {2, 2}, MemoryOrder::RowMajor); }));
+    // TensorView (:183-300): borrowed metadata view, zero-copy permute / broadcast / diagonal
+    {
+        auto v = a.tensor_view();
+        CHECK(v.dims() == a.dims() && v.strides() == a.strides() && v.ndim() == 3 && v.logical_memory_space() == a.logical_memory_space());
+        auto vp = v.permute({2, 0, 1});
+        CHECK(vp.dims() == ap.dims() && vp.strides() == ap.strides());
+        CHECK(sq.tensor_view().diagonal({{0, 1}}).strides() == (std::vector<ptrdiff_t>{4}));
+        CHECK(Tensor<double>::from_slice({1, 2, 3}, {3}, MemoryOrder::RowMajor).tensor_view().broadcast({2, 3}).strides() == (std::vector<ptrdiff_t>{0, 1}));
+        CHECK(raises(Error::Kind::InvalidArgument, [&] { v.permute({0, 0, 1}); }));
+        CHECK(raises(Error::Kind::NoCompatibleComputeDevice, [&] { v.to_tensor(MemoryOrder::RowMajor); }));
+    }
     // no CPU compute in this library: an operation on main-memory operands names the missing device
     CHECK(raises(Error::Kind::NoCompatibleComputeDevice, [&] { einsum<double>("ij,jk->ik", {&sq, &sq}); }));
     CHECK(raises(Error::Kind::NoCompatibleComputeDevice, [&] { sq.conj(); }));
@@ -142,6 +153,17 @@ static void gpu_checks() {
     CHECK(rel_frobenius(einsum_with_plan<double>(tree, {&A, &B}).to_vec(), ref) < 1e-12);
     CHECK(rel_frobenius(einsum_with_subscripts<double>(subs, {&A, &B}).to_vec(), ref) < 1e-12);
     CHECK(rel_frobenius(einsum_owned<double>("ij,jk->ik", {A, B}).to_vec(), ref) < 1e-12);
+    {   // TensorView on the device: a permuted view materialised in either order, and its conjugate-free copy
+        auto v = A.tensor_view().permute({1, 0});
+        auto tr = v.to_tensor(MemoryOrder::RowMajor);
+        CHECK(tr.is_contiguous() && tr.dims() == (std::vector<size_t>{n, n}) && tr.strides() == (std::vector<ptrdiff_t>{(ptrdiff_t)n, 1}));
+        auto got = tr.to_vec();
+        bool same = true;
+        for (size_t i = 0; i < n && same; ++i)
+            for (size_t j = 0; j < n; ++j) same = same && got[i * n + j] == ha[j * n + i];
+        CHECK(same);
+        CHECK(v.contiguous(MemoryOrder::ColumnMajor).strides() == (std::vector<ptrdiff_t>{1, (ptrdiff_t)n}));
+    }
     {   // the plan-less forms share one cached tree per network: a repeated call is a hit and gives the same result
         int64_t h0 = 0, m0 = 0, h1 = 0, m1 = 0;
         tfh_tree_cache_stats(&h0, &m0, nullptr);

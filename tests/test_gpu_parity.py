@@ -1651,3 +1651,25 @@ def test_long_grids_and_high_rank(tf, oracle):
     out = dev(tf, np.zeros(oshape))
     tf.HipBackend.execute(tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute(list(range(12)), perm), [shape, oshape]), 1.0, [dev(tf, z)], 0.0, out)
     assert out.to_numpy().tobytes() == np.ascontiguousarray(z.transpose(perm)).tobytes()
+
+
+def test_tensor_view_materialises_on_the_device(tf, oracle):
+    # TensorView (tenferro-tensor/src/lib.rs:183-300) over device memory: zero-copy permute / diagonal / broadcast, then
+    # to_tensor / contiguous / conj run the copy kernels; bit-exact against the oracle's permute
+    rng = np.random.default_rng(120)
+    x = rand(rng, (6, 5, 6, 4), np.complex128)
+    v = dev(tf, x).tensor_view()
+    assert v.logical_memory_space() == tf.GpuMemory(0) and v.dims() == [6, 5, 6, 4]
+    p = v.permute([3, 0, 2, 1])
+    ref = np.empty((4, 6, 6, 5), np.complex128)
+    oracle.permute(x, [0, 1, 2, 3], ref, [3, 0, 2, 1])
+    for order in (tf.MemoryOrder.RowMajor, tf.MemoryOrder.ColumnMajor):
+        t = p.to_tensor(order)
+        assert t.is_contiguous() and t.to_numpy().tobytes() == ref.tobytes()
+        assert p.contiguous(order).to_numpy().tobytes() == ref.tobytes()
+    d = v.diagonal([(0, 2)])                   # axes 0 and 2 merged: dims [6, 5, 4]
+    assert d.dims() == [6, 5, 4]
+    assert d.to_tensor(tf.MemoryOrder.RowMajor).to_numpy().tobytes() == np.ascontiguousarray(np.einsum("ijik->ijk", x)).tobytes()
+    b = dev(tf, x[:, :1]).tensor_view().broadcast([6, 5, 6, 4])
+    assert b.to_tensor(tf.MemoryOrder.RowMajor).to_numpy().tobytes() == np.ascontiguousarray(np.broadcast_to(x[:, :1], x.shape)).tobytes()
+    assert p.conj().to_numpy().tobytes() == np.conj(ref).tobytes()

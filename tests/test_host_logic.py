@@ -382,3 +382,36 @@ def test_seeded_inputs_are_pure_functions_of_the_index():
     assert abs(c.real.std() * 32 - 1) < 0.02 and abs(c.imag.std() * 32 - 1) < 0.02 and abs(np.corrcoef(c.real, c.imag)[0, 1]) < 0.02
     dims = inputs.draw_block_dims(1004, 128)
     assert len(dims) == 128 and all(v % 64 == 0 and 64 <= v <= 1024 for d in dims for v in d)
+
+
+def test_tensor_view_and_host_views(tf):
+    # TensorView (tenferro-tensor/src/lib.rs:183-300) and view()/view_mut() (:445-454) on main-memory tensors
+    T, row, col = tf.Tensor, tf.MemoryOrder.RowMajor, tf.MemoryOrder.ColumnMajor
+    data = np.arange(24.0)
+    a = T.from_slice(data, [2, 3, 4], row)
+    v = a.tensor_view()
+    assert v.dims() == [2, 3, 4] and v.strides() == [12, 4, 1] and v.ndim() == 3
+    assert v.logical_memory_space() == tf.MainMemory and v.preferred_compute_device() is None
+    vp = v.permute([2, 0, 1])
+    assert vp.dims() == [4, 2, 3] and vp.strides() == [1, 12, 4]
+    t = vp.to_tensor(row)                                   # a copy, contiguous in the requested order
+    assert t.strides() == [6, 3, 1] and np.array_equal(t.to_numpy(), data.reshape(2, 3, 4).transpose(2, 0, 1))
+    assert vp.contiguous(col).strides() == [1, 4, 8]
+    assert np.array_equal(vp.contiguous(col).to_numpy(), data.reshape(2, 3, 4).transpose(2, 0, 1))
+    same = v.to_tensor(row)                                 # already contiguous: still a fresh buffer
+    assert same._buf is not a._buf and np.array_equal(same.to_numpy(), a.to_numpy())
+    sq = T.from_slice(np.arange(9.0), [3, 3], row)
+    d = sq.tensor_view().diagonal([(0, 1)])
+    assert d.dims() == [3] and d.strides() == [4] and list(d.to_tensor(row).to_numpy()) == [0.0, 4.0, 8.0]
+    b = T.from_slice(np.array([1.0, 2.0, 3.0]), [3, 1], row).tensor_view().broadcast([3, 4])
+    assert b.strides() == [1, 0] and b.to_tensor(row).to_numpy().tolist() == [[1.0] * 4, [2.0] * 4, [3.0] * 4]
+    z = T.from_slice(np.array([1 + 2j, 3 - 4j]), [2], row).tensor_view().conj()
+    assert z.to_numpy().tolist() == [1 - 2j, 3 + 4j]       # :617-620
+    with pytest.raises(tf.InvalidArgument):
+        v.permute([0, 0, 1])
+    # view(): the strided element view of a main-memory tensor
+    w = a.permute([1, 2, 0]).view()
+    assert w.shape == (3, 4, 2) and np.array_equal(w, data.reshape(2, 3, 4).transpose(1, 2, 0)) and not w.flags.writeable
+    m = a.view_mut()
+    m[1, 2, 3] = -1.0
+    assert a.to_numpy()[1, 2, 3] == -1.0
