@@ -570,15 +570,25 @@ inline void launch_gemm128_any(const GemmArgs& g, dim3 grid, bool akf, bool bkf,
     launch_gemm128_layout<R, CX, 1>(g, grid, akf, bkf, st);
 }
 
-// 128 x 64 tiles for a thin right-hand side.  The row-contiguous B loader of f32 / complex64 with 16-byte accesses has
-// more threads than 64 columns give work to, so those two combinations use element-wise accesses.
+// 128 x 64 tiles for a thin right-hand side.  A row-contiguous B of f32 / complex64 has more threads than 16-byte
+// accesses over 64 columns give work to: that loader uses 8-byte accesses (two f32, one complex64).
 template <class R, bool CX>
 inline void launch_gemm128x64_any(const GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
     constexpr int VMAX = Cfg128<R, CX>::VMAX;
-    constexpr bool thin_ok = VMAX > 1 && (sizeof(R) == 8 || false);   // 16-byte accesses divide the 64-column tile
-    if constexpr (thin_ok) {
+    if constexpr (VMAX > 1) {
         if (g.vec) {
-            launch_gemm128_layout<R, CX, VMAX, 64>(g, grid, akf, bkf, st);
+            if constexpr (sizeof(R) == 8) {
+                launch_gemm128_layout<R, CX, VMAX, 64>(g, grid, akf, bkf, st);
+            } else {
+                constexpr int VBR = VMAX / 2;
+                if (bkf) {
+                    if (akf) launch_gemm128_variant<R, CX, true, true, VMAX, VMAX, 64>(g, grid, st);
+                    else launch_gemm128_variant<R, CX, false, true, VMAX, VMAX, 64>(g, grid, st);
+                } else {
+                    if (akf) launch_gemm128_variant<R, CX, true, false, VMAX, VBR, 64>(g, grid, st);
+                    else launch_gemm128_variant<R, CX, false, false, VMAX, VBR, 64>(g, grid, st);
+                }
+            }
             return;
         }
     }
