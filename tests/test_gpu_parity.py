@@ -389,6 +389,37 @@ def test_elementwise_mul_conj_fill(tf, oracle, dtype):
     assert ones.strides() == [1, 7]
 
 
+@pytest.mark.parametrize("dtype", ALL)
+def test_elementwise_mul_second_operand_in_another_axis_order(tf, oracle, dtype):
+    # the second operand's contiguous axis is neither A's nor the output's: it is brought into the output's axis order
+    # first (a pool block, released in stream order); strided / reversed / broadcast operands and an output that is
+    # a view are covered, and the operands must come out unchanged
+    rng = np.random.default_rng(130)
+    shape = (70, 50, 60)
+    a = rand(rng, shape, dtype)
+    cases = {
+        "reversed modes": rand(rng, shape[::-1], dtype).transpose(2, 1, 0),
+        "middle axis contiguous": rand(rng, (70, 60, 50), dtype).transpose(0, 2, 1),
+        "reversed and stepped": rand(rng, (60, 100, 70), dtype)[::-1, ::2, :].transpose(2, 1, 0),
+        "broadcast": np.broadcast_to(rand(rng, (1, 50, 1), dtype), shape),
+    }
+    for name, b in cases.items():
+        for alpha, beta in [(1.0, 0.0), (0.5, -1.5)]:
+            big = rand(rng, (70, 50, 120), dtype)
+            c0 = big[:, :, ::2]                                   # the output is a stepped view
+            ref = c0.copy()
+            oracle.elementwise_mul(a, np.ascontiguousarray(b), ref, alpha=alpha, beta=beta)
+            da, db, dc = dev(tf, a), dev(tf, b), dev(tf, c0)
+            plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.ElementwiseMul(), [a.shape, b.shape, c0.shape])
+            tf.HipBackend.execute(plan, alpha, [da, db], beta, dc)
+            assert relerr(dc.to_numpy(), ref) < TOL[dtype], (name, alpha, beta)
+            assert np.array_equal(db.to_numpy(), b) and np.array_equal(da.to_numpy(), a), name
+    # through einsum: a Hadamard product whose operands list their modes in different orders
+    x, y = rand(rng, (64, 48, 40), dtype), rand(rng, (40, 48, 64), dtype)
+    got = tf.einsum("ijk,kji->ijk", [dev(tf, x), dev(tf, y)])
+    assert relerr(got.to_numpy(), x * y.transpose(2, 1, 0)) < TOL[dtype]
+
+
 def test_conj_reference_doc_example(tf):
     # tenferro-tensor/src/lib.rs:612-620
     a = dev(tf, np.array([1 + 2j, 3 - 4j]))
