@@ -415,7 +415,17 @@ int32_t plan_tiles(std::vector<Axis> axes, int elem_bytes, int max_tile_elems, b
     std::stable_sort(in_order.begin(), in_order.end(), [&](int x, int y) { return key_in(x) < key_in(y); });
 
     std::vector<int> tl(na, 0);  // log2 tile extent per axis
-    auto full = [&](int i) { return ceil_log2(axes[i].n); };
+    // An extent that is not a power of two makes its last tile partial, and one partial tile takes the whole launch
+    // off the kernel's fast path.  When the extent has a power-of-two divisor of at least 128 bytes (96 = 3 x 32), the
+    // tile is first tried no longer than that divisor; the plan is kept if every tile then comes out full.
+    bool capped = false;
+    auto full = [&](int i) {
+        const int64_t n = axes[i].n;
+        const int whole = ceil_log2(n);
+        if (!capped || (n & (n - 1)) == 0) return whole;
+        const int d = __builtin_ctzll((unsigned long long)n);
+        return ((int64_t)elem_bytes << d) >= 128 ? d : whole;
+    };
     auto tile_axes = [&]() { int c = 0; for (int i = 0; i < na; ++i) c += tl[i] > 0; return c; };
     auto prod_log2 = [&]() { int p = 0; for (int i = 0; i < na; ++i) p += tl[i]; return p; };
     const int budget = ceil_log2(max_tile_elems);
@@ -430,26 +440,43 @@ int32_t plan_tiles(std::vector<Axis> axes, int elem_bytes, int max_tile_elems, b
             want = std::min(want, tl[i] + budget - prod_log2());
             tl[i] = want;
             run += want;
-            if (want < full(i)) break;
+            if (want < ceil_log2(axes[i].n)) break;   // the run ends at an axis the tile covers only partly
         }
     };
-    take_run(out_order);
-    if (two_sided) take_run(in_order);
-    // spend the rest of the budget: alternately lengthen the output-side and the input-side run
-    for (int side = 0; prod_log2() < budget; side ^= 1) {
-        bool grew = false;
-        for (int pass = 0; pass < 2 && !grew; ++pass) {
-            const std::vector<int>& order = ((side ^ pass) == 0 || !two_sided) ? out_order : in_order;
-            for (int i : order) {
-                if (tl[i] < full(i) && (tl[i] > 0 || tile_axes() < MAXT)) {
-                    ++tl[i];
-                    grew = true;
-                    break;
+    auto choose = [&]() {
+        std::fill(tl.begin(), tl.end(), 0);
+        take_run(out_order);
+        if (two_sided) take_run(in_order);
+        // spend the rest of the budget: alternately lengthen the output-side and the input-side run
+        for (int side = 0; prod_log2() < budget; side ^= 1) {
+            bool grew = false;
+            for (int pass = 0; pass < 2 && !grew; ++pass) {
+                const std::vector<int>& order = ((side ^ pass) == 0 || !two_sided) ? out_order : in_order;
+                for (int i : order) {
+                    if (tl[i] < full(i) && (tl[i] > 0 || tile_axes() < MAXT)) {
+                        ++tl[i];
+                        grew = true;
+                        break;
+                    }
+                    if (tl[i] < ceil_log2(axes[i].n)) break;  // cannot extend this run past a partial axis
                 }
-                if (tl[i] < full(i)) break;  // cannot extend this run past a partial axis
             }
+            if (!grew) break;
         }
-        if (!grew) break;
+    };
+    for (int i = 0; i < na; ++i) capped = capped || (axes[i].n & (axes[i].n - 1)) != 0;
+    if (capped) {
+        choose();
+        bool all_full = true;
+        for (int i = 0; i < na; ++i) all_full = all_full && (tl[i] == 0 || axes[i].n % ((int64_t)1 << tl[i]) == 0);
+        const std::vector<int> tl_capped = tl;
+        const int elems_capped = prod_log2();
+        capped = false;
+        choose();
+        // (a capped plan whose tile came out tiny would trade the fast path for too little work per block)
+        if (all_full && (elems_capped >= 10 || elems_capped + 1 >= prod_log2())) tl = tl_capped;
+    } else {
+        choose();
     }
     // tile axis ids
     std::vector<int> ids;

@@ -848,6 +848,16 @@ def test_permute_extents_with_divisor_tiles(tf, oracle, dtype):
     big = rand(rng, (64, 131), dtype)
     got, ref = _permute_check(tf, oracle, big[:, 1:129], (1, 0))
     assert got.tobytes() == ref.tobytes()
+    # extents with a power-of-two divisor of at least 128 bytes (96 = 3 x 32, 160 = 5 x 32, 48 = 3 x 16): the tiles are
+    # cut to that divisor, every tile is full and the launch stays on the kernel's fast path
+    # (the last shape's divisor tiles would hold 256 elements only: it keeps the general path)
+    for shape, perm, fast in [((96, 96, 96), (2, 1, 0), True), ((96, 256, 128), (1, 2, 0), True), ((160, 3, 160), (2, 1, 0), True),
+                              ((192, 5, 320), (2, 0, 1), True), ((48, 48, 48, 16), (3, 1, 0, 2), False)]:
+        a = rand(rng, shape, dtype)
+        got, ref = _permute_check(tf, oracle, a, perm)
+        assert got.tobytes() == ref.tobytes(), (shape, perm)
+        if np.dtype(dtype).itemsize >= 8:
+            assert tf.last_kernel().endswith("true>)") == fast, (shape, perm, tf.last_kernel())
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex128])
