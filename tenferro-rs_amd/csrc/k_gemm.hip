@@ -745,6 +745,10 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     const int64_t kstages = (K + bke - 1) / bke;
     // too few large tiles to fill 256 CUs and too little k to split: fall back to 64x64 tiles
     if (bm == 128 && tiles_for(bm, bn) < 192 && kstages < 32 && tiles_for(64, 64) >= 2 * tiles_for(bm, bn)) bm = bn = 64;
+    // large tiles that stay at half a block per CU or less even with the deepest split (512^3 f64: 16 tiles x 4): the
+    // 64x64 kernel fills the chip better (18 us against 29 us; from 768^3 on the large tiles win)
+    if (bm == 128 && bn == 128 && tiles_for(128, 128) * std::max<int64_t>(1, kstages / 8) <= 128 && tiles_for(64, 64) >= 2 * tiles_for(128, 128))
+        bm = bn = 64;
     // thin tiles that cannot reach one block per CU even with the deepest split: 64x64 tiles give twice the blocks
     if (bm == 128 && bn == 64 && tiles_for(128, 64) * std::max<int64_t>(1, kstages / 8) < 256 && tiles_for(64, 64) >= 2 * tiles_for(128, 64))
         bm = 64;

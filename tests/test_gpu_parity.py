@@ -691,12 +691,12 @@ def test_reduce_misaligned_base_and_split_reductions(tf, oracle):
 
 
 BIG_CASES = [
-    # k long enough (>= 32 stages) that the few 128x128 tiles are preferred to 64x64 ones and split over k
-    ("ajbk,kcj->abc", dict(a=16, j=24, b=16, k=48, c=160)),     # two-mode k through offset tables, packed B
-    ("mk,kn->mn", dict(m=300, k=1103, n=260)),                   # ragged edges and a k tail
-    ("km,nk->mn", dict(m=256, k=1040, n=384)),
-    ("mk,nk->nm", dict(m=200, k=1030, n=130)),                   # operands swap
-    ("bmk,kbn->bmn", dict(b=3, m=130, k=1050, n=140)),           # batch
+    # enough 128x128 tiles and k stages (tiles x stages / 8 > 128) that they are preferred to 64x64 tiles and split over k
+    ("ajbk,kcj->abc", dict(a=48, j=24, b=16, k=48, c=672)),     # two-mode k through offset tables, packed B
+    ("mk,kn->mn", dict(m=812, k=1103, n=772)),                   # ragged edges and a k tail
+    ("km,nk->mn", dict(m=768, k=1040, n=896)),
+    ("mk,nk->nm", dict(m=712, k=1030, n=642)),                   # operands swap
+    ("bmk,kbn->bmn", dict(b=3, m=386, k=1050, n=396)),           # batch
 ]
 
 
@@ -757,8 +757,8 @@ def test_config3_full_size_complex128(tf, oracle):
 # sizes that the launcher gives to the 128x128 kernel: a long k (>= 32 stages) over few tiles, or many tiles over a k
 # shorter than one vector
 # (the last three leave fewer k than one vector in the final stage: its window then starts inside the previous stage)
-ODD_SIZES = [(129, 1031, 133), (255, 1077, 257), (1801, 5, 1795), (1810, 3, 1811), (1793, 4, 1800), (193, 1058, 97),
-             (257, 1025, 129), (130, 1027, 131), (1801, 66, 1795)]
+ODD_SIZES = [(641, 1031, 645), (767, 1077, 769), (1801, 5, 1795), (1810, 3, 1811), (1793, 4, 1800), (4673, 1058, 97),
+             (769, 1025, 641), (642, 1027, 643), (1801, 66, 1795)]
 LAYOUTS = [("mk", "kn"), ("mk", "nk"), ("km", "kn"), ("km", "nk")]
 
 
@@ -813,10 +813,28 @@ def test_contract_thin_side_takes_128x64_tiles(tf, oracle, dtype, layout):
         assert relerr(out.to_numpy(), ref) < TOL[dtype], (m, k, n, tf.last_kernel())
 
 
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("layout", LAYOUTS, ids=["NN", "NT", "TN", "TT"])
+def test_contract_odd_extents_few_tiles(tf, oracle, dtype, layout):
+    # the same kind of extents with so few tiles that the 64x64 kernel (or, for complex128, the large-tile one) is chosen
+    ma, mb = layout
+    rng = np.random.default_rng(148)
+    for m, k, n in [(129, 1031, 133), (255, 1077, 257), (193, 1058, 97), (257, 1025, 129), (130, 1027, 131), (131, 37, 129), (300, 5, 310)]:
+        ext = dict(m=m, k=k, n=n)
+        a = rand(rng, [ext[l] for l in ma], dtype)
+        b = rand(rng, [ext[l] for l in mb], dtype)
+        ref = np.empty((m, n), dtype)
+        oracle.contract(a, lab(ma), b, lab(mb), ref, lab("mn"))
+        out = dev(tf, np.full((m, n), np.nan, dtype))
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab("mn")), [a.shape, b.shape, [m, n]])
+        tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
+        assert relerr(out.to_numpy(), ref) < TOL[dtype], (m, k, n, tf.last_kernel())
+
+
 def test_contract_operand_ending_at_the_end_of_its_allocation(tf, oracle):
     # the operands are the tail of exactly-sized device buffers: a read past the last element would leave the buffer
     rng = np.random.default_rng(48)
-    for dtype, m, k, n in [(np.float32, 131, 1033, 129), (np.float64, 129, 523, 131)]:
+    for dtype, m, k, n in [(np.float32, 643, 1033, 641), (np.float64, 641, 523, 643)]:
         for ma, mb in LAYOUTS:
             ext = dict(m=m, k=k, n=n)
             a = rand(rng, [ext[l] for l in ma], dtype)
@@ -948,7 +966,7 @@ def test_contract_random_label_patterns_and_views(tf, oracle, dtype, big):
 
 @pytest.mark.parametrize("dtype", ALL)
 def test_contract_random_layouts_on_the_128_tile_kernel(tf, oracle, dtype):
-    # random shapes sized for the 128x128 kernel (both free products >= 97, k of a thousand or more, so >= 32 stages):
+    # random shapes sized for the 128x128 kernel (both free products >= 700, k of a thousand or more: enough tiles and stages):
     # one or two modes per group, random axis orders, random strided / reversed / offset views, odd extents.  Most
     # cases are contiguous along some operand direction (16-byte loads with their tail handling), the stepped views are not.
     rng = np.random.default_rng(58)
@@ -959,7 +977,7 @@ def test_contract_random_layouts_on_the_128_tile_kernel(tf, oracle, dtype):
         nb, nm, nn, nk = int(rng.integers(0, 2)), int(rng.integers(1, 3)), int(rng.integers(1, 3)), int(rng.integers(1, 3))
         batch, fm, fn, kk = labels[:nb], labels[nb:nb + nm], labels[nb + nm:nb + nm + nn], labels[nb + nm + nn:nb + nm + nn + nk]
         ext = {}
-        for grp, lo, hi in ((fm, 97, 300), (fn, 97, 300), (kk, 1000, 1100)):
+        for grp, lo, hi in ((fm, 700, 860), (fn, 700, 860), (kk, 1000, 1100)):
             ext[grp[0]] = int(rng.integers(lo, hi + 1))
             for l in grp[1:]:
                 ext[l] = int(rng.integers(1, 4))
