@@ -8,6 +8,12 @@
  * boundary as a run-time tag (tfh_dtype) because generics cannot; a Rust binding
  * monomorphises back (`impl TensorPrims<Standard> for HipBackend`).
  *
+ * Threads: every entry point may be called from any thread, and calls that enqueue on
+ * DIFFERENT streams may run concurrently.  Each stream owns scratch memory (offset tables,
+ * split-K partials, einsum intermediates) that the kernels of successive calls reuse in
+ * stream order, so calls that enqueue on the SAME stream must not overlap in time: the
+ * caller serialises them, as it would the launches themselves.
+ *
  * Reference interfaces replaced (paths relative to the tenferro-rs workspace):
  *   tenferro-prims/src/lib.rs:278-340   trait TensorPrims<A> { plan, execute, has_extension_for }
  *   tenferro-prims/src/lib.rs:152-245   enum PrimDescriptor

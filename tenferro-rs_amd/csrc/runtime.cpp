@@ -117,7 +117,25 @@ int32_t pool_alloc(void* stream, size_t bytes, void** out) {
         return TFH_OK;
     }
     void* p = nullptr;
-    if (int32_t e = hip_check(hipMalloc(&p, bytes), "hipMalloc(intermediate)")) return e;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        // out of device memory: the blocks cached for reuse (on every stream of this device) are given back once the
+        // work that may still read them has finished, and the allocation is tried once more
+        (void)hipGetLastError();
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return set_error(TFH_ERR_DEVICE, "hipMalloc(intermediate): out of memory for %zu bytes while the stream is being captured", bytes);
+        }
+        if (int32_t e = hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize")) return e;
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        for (auto& kv : g_scratch) {
+            if (kv.first.first != dev) continue;
+            for (auto& b : kv.second.free_blocks) (void)hipFree(b.second);
+            kv.second.free_blocks.clear();
+        }
+        if (int32_t e = hip_check(hipMalloc(&p, bytes), "hipMalloc(intermediate)")) return e;
+    }
     s->live[p] = bytes;
     *out = p;
     return TFH_OK;

@@ -1732,3 +1732,39 @@ def test_tensor_view_materialises_on_the_device(tf, oracle):
     b = dev(tf, x[:, :1]).tensor_view().broadcast([6, 5, 6, 4])
     assert b.to_tensor(tf.MemoryOrder.RowMajor).to_numpy().tobytes() == np.ascontiguousarray(np.broadcast_to(x[:, :1], x.shape)).tobytes()
     assert p.conj().to_numpy().tobytes() == np.conj(ref).tobytes()
+
+
+def test_intermediates_cached_for_reuse_are_given_back_when_the_device_runs_out_of_memory(tf):
+    # The intermediates of a contraction tree come from a per-stream cache of device blocks that keeps them after the
+    # call.  With the device nearly full, a tree whose intermediate fits no cached block and no free memory must still
+    # run: the cached blocks are released and the allocation is tried again.  The free memory is bounded with one large
+    # untouched allocation; the three intermediates (2.0, 2.6, 3.4 GiB) each exceed what the earlier ones can hold.
+    import torch
+    assert tf.lib().tfh_release_workspaces() == 0
+    torch.cuda.empty_cache()
+    gib = 1 << 30
+    free, _ = torch.cuda.mem_get_info()
+    if free < 16 * gib:
+        pytest.skip("needs 16 GiB of free device memory")
+    try:
+        ballast = torch.empty(free - 6 * gib, dtype=torch.uint8, device="cuda")
+    except RuntimeError:
+        pytest.skip("one allocation of all but 6 GiB of the free device memory is not available")
+    try:
+        rng = np.random.default_rng(130)
+        subs = tf.Subscripts.parse("ij,jk,kl->il")
+        for step, n in enumerate((16384, 18688, 21376)):
+            a, b, c = rand(rng, (n, 2), np.float64), rand(rng, (2, n), np.float64), rand(rng, (n, 3), np.float64)
+            tree = tf.ContractionTree.from_pairs(subs, [a.shape, b.shape, c.shape], [(0, 1), (3, 2)])   # (A B) first: n x n
+            assert tree.peak_intermediate == n * n
+            if step == 2:
+                torch.cuda.synchronize()
+                assert torch.cuda.mem_get_info()[0] < n * n * 8   # the cached blocks hold what this step would need
+            out = tf.einsum_with_plan(tree, [dev(tf, a), dev(tf, b), dev(tf, c)])
+            assert relerr(out.to_numpy(), a @ (b @ c)) < 1e-12
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] < 6 * gib - 21376 * 21376 * 8 + gib   # the last intermediate stays cached
+    finally:
+        del ballast
+        assert tf.lib().tfh_release_workspaces() == 0
+        torch.cuda.empty_cache()
