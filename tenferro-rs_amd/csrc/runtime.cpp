@@ -39,6 +39,28 @@ StreamScratch* scratch_for(void* stream, int32_t* err) {
     if (*err) return nullptr;
     return &g_scratch[{dev, stream}];
 }
+
+// hipMalloc that, when the device is out of memory, gives back the blocks cached for reuse on every stream of the
+// current device (after the work that may still read them has finished) and tries once more.  `stream`: the stream
+// the caller enqueues on, checked for an ongoing graph capture (which forbids the synchronisation); g_mu is held.
+int32_t malloc_or_release(void** p, size_t bytes, void* stream, const char* what) {
+    if (hipMalloc(p, bytes) == hipSuccess) return TFH_OK;
+    (void)hipGetLastError();
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return set_error(TFH_ERR_DEVICE, "%s: out of memory for %zu bytes while the stream is being captured", what, bytes);
+    }
+    if (int32_t e = hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize")) return e;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    for (auto& kv : g_scratch) {
+        if (kv.first.first != dev) continue;
+        for (auto& b : kv.second.free_blocks) (void)hipFree(b.second);
+        kv.second.free_blocks.clear();
+    }
+    return hip_check(hipMalloc(p, bytes), what);
+}
 }  // namespace
 
 int32_t workspace(void* stream, size_t bytes, void** out) {
@@ -55,7 +77,7 @@ int32_t workspace(void* stream, size_t bytes, void** out) {
             s->ws_bytes = 0;
         }
         size_t want = std::max<size_t>(bytes + bytes / 4, (size_t)1 << 20);
-        if (int32_t e = hip_check(hipMalloc(&s->ws, want), "hipMalloc(workspace)")) return e;
+        if (int32_t e = malloc_or_release(&s->ws, want, stream, "hipMalloc(workspace)")) return e;
         s->ws_bytes = want;
     }
     *out = s->ws;
@@ -117,25 +139,7 @@ int32_t pool_alloc(void* stream, size_t bytes, void** out) {
         return TFH_OK;
     }
     void* p = nullptr;
-    if (hipMalloc(&p, bytes) != hipSuccess) {
-        // out of device memory: the blocks cached for reuse (on every stream of this device) are given back once the
-        // work that may still read them has finished, and the allocation is tried once more
-        (void)hipGetLastError();
-        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
-            (void)hipGetLastError();
-            return set_error(TFH_ERR_DEVICE, "hipMalloc(intermediate): out of memory for %zu bytes while the stream is being captured", bytes);
-        }
-        if (int32_t e = hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize")) return e;
-        int dev = 0;
-        (void)hipGetDevice(&dev);
-        for (auto& kv : g_scratch) {
-            if (kv.first.first != dev) continue;
-            for (auto& b : kv.second.free_blocks) (void)hipFree(b.second);
-            kv.second.free_blocks.clear();
-        }
-        if (int32_t e = hip_check(hipMalloc(&p, bytes), "hipMalloc(intermediate)")) return e;
-    }
+    if (int32_t e = malloc_or_release(&p, bytes, stream, "hipMalloc(intermediate)")) return e;
     s->live[p] = bytes;
     *out = p;
     return TFH_OK;
@@ -315,7 +319,10 @@ int32_t tfh_preferred_compute_devices(int32_t space_kind, int64_t space_id, int3
 int32_t tfh_malloc(size_t bytes, void** out) {
     if (!out) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
     *out = nullptr;
-    return hip_check(hipMalloc(out, bytes ? bytes : 1), "hipMalloc");
+    if (hipMalloc(out, bytes ? bytes : 1) == hipSuccess) return TFH_OK;
+    (void)hipGetLastError();
+    std::lock_guard<std::mutex> lk(tfh::g_mu);
+    return tfh::malloc_or_release(out, bytes ? bytes : 1, nullptr, "hipMalloc");
 }
 int32_t tfh_free(void* ptr) { return hip_check(hipFree(ptr), "hipFree"); }
 int32_t tfh_memcpy_h2d(void* dst, const void* src, size_t bytes, tfh_stream stream) {

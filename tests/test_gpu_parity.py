@@ -1764,6 +1764,10 @@ def test_intermediates_cached_for_reuse_are_given_back_when_the_device_runs_out_
             assert relerr(out.to_numpy(), a @ (b @ c)) < 1e-12
         torch.cuda.synchronize()
         assert torch.cuda.mem_get_info()[0] < 6 * gib - 21376 * 21376 * 8 + gib   # the last intermediate stays cached
+        import ctypes
+        p = ctypes.c_void_p()
+        assert tf.lib().tfh_malloc(4 * gib, ctypes.byref(p)) == 0 and p.value     # tfh_malloc gives the cache back too
+        assert tf.lib().tfh_free(p) == 0
     finally:
         del ballast
         assert tf.lib().tfh_release_workspaces() == 0
