@@ -338,7 +338,10 @@ struct FastReduceArgs {
     int64_t t_sa[MAXT], t_sc[MAXT];
     int64_t g_count[MAXG], g_sa[MAXG], g_sc[MAXG];
     int64_t r_count[MAXR], r_sa[MAXR];
-    int32_t r_total, pad_;
+    int32_t r_total;
+    // >= 0: the blocks of group (blockIdx.x >> rot_shift) start their serial range at index group % r_total and wrap
+    // round (mode 0 only); < 0: every block starts at index 0
+    int32_t rot_shift;
     int64_t ks_sa, ks_sc;     // strides of the block-serial kept axis
     int32_t bf_bit[3];        // BF: the three lowest reduced thread-id bits inside a wave
     // few outputs, long serial range: blockIdx.y takes `rps` serial indices and writes raw partial results (mode 1),
@@ -373,8 +376,9 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
     const int tid = threadIdx.x;
     const int r_begin = a.mode == 1 ? (int)blockIdx.y * a.rps : 0;
     const int r_count = a.mode == 2 ? 0 : (a.mode == 1 ? (a.r_total - r_begin < a.rps ? a.r_total - r_begin : a.rps) : a.r_total);
+    const int rot = a.rot_shift >= 0 && a.mode == 0 ? (int)((blockIdx.x >> a.rot_shift) % (uint32_t)r_count) : 0;
     for (int i = tid; i < r_count; i += THREADS) {
-        int64_t lin = r_begin + i, off = 0;
+        int64_t lin = r_begin + (i + rot >= r_count ? i + rot - r_count : i + rot), off = 0;
 #pragma unroll
         for (int r = 0; r < MAXR; ++r)
             if (r < a.nr) {
@@ -715,6 +719,20 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
     }
 
     fa.r_total = (int32_t)r_total;
+    // A serial axis with a kept axis outside it (sum over a middle axis): the blocks of the launch run in step, so at
+    // any moment they would all read the same serial index -- addresses that differ by the outer axis's stride, a large
+    // power of two in the usual case, which fall into the same DRAM banks.  Groups of 32 consecutive blocks start at
+    // different serial indices instead (the order of a block's additions stays fixed, so results are reproducible).
+    // 16^6 f64 summed over axes 1 and 4: 25.2 -> 24.1 us; [16,64,16,1024] over axis 1: 30.2 -> 26.1 us; 32^5 f32 over
+    // axis 1: 33.8 -> 29.9 us.  A serial axis that is outermost keeps the plain order: there the blocks sweep one
+    // contiguous slab after another, and rotating them measured 2-6 % slower.
+    fa.rot_shift = -1;
+    if (nchunks == 1 && r_total >= 4 && blocks >= 512 && fa.nr >= 1 && fa.ng >= 1) {
+        int64_t serial_min = INT64_MAX, grid_max = 0;
+        for (int r = 0; r < fa.nr; ++r) serial_min = std::min<int64_t>(serial_min, std::llabs(fa.r_sa[r]));
+        for (int g = 0; g < fa.ng; ++g) grid_max = std::max<int64_t>(grid_max, std::llabs(fa.g_sa[g]));
+        if (grid_max > serial_min) fa.rot_shift = 5;
+    }
     fa.in = a;
     fa.out = c;
     fa.op = reduce_op;
