@@ -1734,6 +1734,42 @@ def test_tensor_view_materialises_on_the_device(tf, oracle):
     assert p.conj().to_numpy().tobytes() == np.conj(ref).tobytes()
 
 
+def test_rotated_serial_starts_sum_every_index_exactly_once(tf):
+    # The fast reduction and product-reduction kernels start the serial range of a block group (or of a chunk of a
+    # split range) at a rotated index and wrap round.  Small-integer inputs make every sum exact in f64 and f32, so a
+    # serial index that is skipped or taken twice -- counts that are not powers of two, a last chunk shorter than the
+    # others -- shows as an inequality.  Shapes: a middle axis of 12 and of 7 with serial steps of 128 KB under >= 512
+    # blocks (rotation by block group), 1000 and 777 rows summed into few outputs (rotation by chunk).
+    rng = np.random.default_rng(131)
+    lab = lambda t: [ord(ch) for ch in t]
+
+    def ints(shape, dtype):
+        return rng.integers(-3, 4, size=shape).astype(dtype)
+
+    for dtype in (np.float64, np.float32):
+        for shape, red in (((24, 12, 16, 1024), (1,)), ((40, 7, 32, 512), (1,)), ((1000, 96, 128), (0,)), ((777, 2048), (0,)),
+                           ((6, 5, 9, 16, 2048), (1, 2))):
+            a = ints(shape, dtype)
+            modes = list(range(len(shape)))
+            kept = [m for m in modes if m not in red]
+            out = dev(tf, np.full([shape[m] for m in kept], np.nan, dtype))
+            plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Reduce(modes, kept, tf.ReduceOp.Sum), [list(shape), [shape[m] for m in kept]])
+            tf.HipBackend.execute(plan, 1.0, [dev(tf, a)], 0.0, out)
+            assert "reduce_fast_kernel" in tf.last_kernel(), (shape, tf.last_kernel())
+            assert np.array_equal(out.to_numpy(), a.sum(axis=red, dtype=np.float64).astype(dtype)), (shape, red, dtype)
+        # the same through the product reduction: a vector contracted with a middle axis, vector x matrix
+        for sub, sa, sb in (("ajbi,j->abi", (24, 12, 16, 1024), (12,)), ("ajbi,j->abi", (40, 7, 32, 512), (7,)),
+                            ("i,ij->j", (1000,), (1000, 4096)), ("i,ij->j", (777,), (777, 2048))):
+            ia, ib, ic = sub.replace("->", ",").split(",")
+            x, y = ints(sa, dtype), ints(sb, dtype)
+            ref = np.einsum(sub, x.astype(np.float64), y.astype(np.float64))
+            out = dev(tf, np.full(ref.shape, np.nan, dtype))
+            plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ia), lab(ib), lab(ic)), [list(sa), list(sb), list(ref.shape)])
+            tf.HipBackend.execute(plan, 1.0, [dev(tf, x), dev(tf, y)], 0.0, out)
+            assert "dot_fast_kernel" in tf.last_kernel(), (sub, sa, tf.last_kernel())
+            assert np.array_equal(out.to_numpy(), ref.astype(dtype)), (sub, sa, dtype)
+
+
 def test_intermediates_cached_for_reuse_are_given_back_when_the_device_runs_out_of_memory(tf):
     # The intermediates of a contraction tree come from a per-stream cache of device blocks that keeps them after the
     # call.  With the device nearly full, a tree whose intermediate fits no cached block and no free memory must still
