@@ -1734,6 +1734,48 @@ def test_tensor_view_materialises_on_the_device(tf, oracle):
     assert p.conj().to_numpy().tobytes() == np.conj(ref).tobytes()
 
 
+def test_reduce_over_short_contiguous_rows(tf, oracle):
+    # A reduced contiguous axis of 2..32 elements inside a long kept axis, extents that do not tile (17, 31, 3; an even 6
+    # under an odd row count): 256 rows per block go through LDS and every thread adds up its own row.  Sum (exact on
+    # small integers, and against the oracle on random data), max/min, alpha/beta on a permuted output, a sliced operand
+    # whose outer axes do not merge, both real dtypes; complex and rows longer than 32 stay on the general kernel.
+    rng = np.random.default_rng(132)
+    for dtype in (np.float64, np.float32):
+        for shape, red in (((100, 100, 100, 17), (3,)), ((15, 17, 33, 65, 31), (4,)), ((4097, 333, 3), (2,)), ((1001, 1025, 6), (2,)),
+                           ((3000, 32), (1,)), ((70000, 2), (1,))):
+            a = rng.integers(-3, 4, size=shape).astype(dtype)
+            modes = list(range(len(shape)))
+            kept = [m for m in modes if m not in red]
+            oshape = [shape[m] for m in kept]
+            out = dev(tf, np.full(oshape, np.nan, dtype))
+            tf.HipBackend.execute(tf.HipBackend.plan(dtype, tf.PrimDescriptor.Reduce(modes, kept, tf.ReduceOp.Sum), [list(shape), oshape]), 1.0, [dev(tf, a)], 0.0, out)
+            assert "reduce_shortrow_kernel" in tf.last_kernel(), (shape, tf.last_kernel())
+            assert np.array_equal(out.to_numpy(), a.sum(axis=red, dtype=np.float64).astype(dtype)), (shape, dtype)
+        x = rand(rng, (37, 1500, 17), dtype)
+        got, ref = _reduce_check(tf, oracle, x, [0, 1, 2], [0, 1], tf.ReduceOp.Sum, oracle.SUM)
+        assert "reduce_shortrow_kernel" in tf.last_kernel() and relerr(got, ref) < TOL[dtype]
+        for op_tf, op_or in [(tf.ReduceOp.Max, oracle.MAX), (tf.ReduceOp.Min, oracle.MIN)]:
+            got, ref = _reduce_check(tf, oracle, x, [0, 1, 2], [0, 1], op_tf, op_or)
+            assert "reduce_shortrow_kernel" in tf.last_kernel() and np.array_equal(got, ref)
+        # output axes exchanged (C strides 1 and 37), alpha and beta
+        c0 = rand(rng, (1500, 37), dtype)
+        got, ref = _reduce_check(tf, oracle, x, [0, 1, 2], [1, 0], tf.ReduceOp.Sum, oracle.SUM, alpha=-1.5, beta=0.25, c0=c0)
+        assert "reduce_shortrow_kernel" in tf.last_kernel() and relerr(got, ref) < TOL[dtype]
+        # a slice: the outer axis does not merge with the rows' axis
+        big = rand(rng, (9, 1400, 13), dtype)
+        got, ref = _reduce_check(tf, oracle, big[:, 100:1300, :], [0, 1, 2], [0, 1], tf.ReduceOp.Sum, oracle.SUM)
+        assert "reduce_shortrow_kernel" in tf.last_kernel() and relerr(got, ref) < TOL[dtype]
+        # rows that are not dense (every second one): the general kernel
+        got, ref = _reduce_check(tf, oracle, big[:, ::2, :], [0, 1, 2], [0, 1], tf.ReduceOp.Sum, oracle.SUM)
+        assert "reduce_shortrow_kernel" not in tf.last_kernel() and relerr(got, ref) < TOL[dtype]
+    z = rand(rng, (2000, 17), np.complex128)
+    got, ref = _reduce_check(tf, oracle, z, [0, 1], [0], tf.ReduceOp.Sum, oracle.SUM)
+    assert "reduce_shortrow_kernel" not in tf.last_kernel() and relerr(got, ref) < 1e-12
+    w = rand(rng, (2000, 33), np.float64)
+    got, ref = _reduce_check(tf, oracle, w, [0, 1], [0], tf.ReduceOp.Sum, oracle.SUM)
+    assert "reduce_shortrow_kernel" not in tf.last_kernel() and relerr(got, ref) < 1e-12
+
+
 def test_rotated_serial_starts_sum_every_index_exactly_once(tf):
     # The fast reduction and product-reduction kernels start the serial range of a block group (or of a chunk of a
     # split range) at a rotated index and wrap round.  Small-integer inputs make every sum exact in f64 and f32, so a
