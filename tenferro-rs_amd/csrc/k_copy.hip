@@ -12,6 +12,8 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <string>
+#include <vector>
 
 #include "internal.hpp"
 #include "launch.hpp"
@@ -314,6 +316,121 @@ __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
         __syncthreads();
         tile = next;
         o = o2;
+    }
+}
+
+// ---- tiles of many short axes ---------------------------------------------------------------------------------------
+// A tensor of many small extents (3^14, 2^16, [3,4]x6: spins and qubits) has no long axis to tile: four power-of-two tile
+// axes give runs of a few elements and, for extents that are no powers of two, mostly idle lanes (3^14 reversed:
+// 161 GB/s).  Here a tile is the product of WHOLE axes -- as many as it takes to reach 512-byte runs on both sides --
+// and the position-to-offset maps of a tile, which no longer are shifts and masks, come from three tables built once
+// per layout (input offset in read order; output offset and LDS position in write order) and kept in registers for
+// all the tiles a block moves.  Every tile is full by construction.
+constexpr int TAB_MAX_AXES = 16;
+struct TabCopyArgs {
+    const void* in;
+    void* out;
+    const uint32_t* tab;   // [3][E]: input element offset of read position r; output offset and LDS position of write position w
+    int32_t E, ng;
+    int64_t ntiles;
+    int64_t g_count[MAXG], g_si[MAXG], g_so[MAXG];
+};
+struct TabBuildArgs {
+    uint32_t* tab;
+    int32_t E, nt;
+    int32_t r_ext[TAB_MAX_AXES], w_ext[TAB_MAX_AXES], w_rpos[TAB_MAX_AXES];
+    int64_t r_si[TAB_MAX_AXES], w_so[TAB_MAX_AXES];
+};
+__global__ void __launch_bounds__(THREADS) tabcopy_build_kernel(TabBuildArgs b) {
+    const int i = blockIdx.x * THREADS + threadIdx.x;
+    if (i >= b.E) return;
+    int lin = i;
+    int64_t off = 0;
+    for (int t = 0; t < b.nt; ++t) {
+        const int q = lin / b.r_ext[t];
+        off += (int64_t)(lin - q * b.r_ext[t]) * b.r_si[t];
+        lin = q;
+    }
+    b.tab[i] = (uint32_t)off;
+    lin = i;
+    off = 0;
+    int pos = 0;
+    for (int t = 0; t < b.nt; ++t) {
+        const int q = lin / b.w_ext[t], c = lin - q * b.w_ext[t];
+        off += (int64_t)c * b.w_so[t];
+        pos += c * b.w_rpos[t];
+        lin = q;
+    }
+    b.tab[b.E + i] = (uint32_t)off;
+    b.tab[2 * b.E + i] = (uint32_t)pos;
+}
+
+template <class V, int EPT>
+__global__ void __launch_bounds__(THREADS) tabcopy_kernel(TabCopyArgs a) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    V* lds = reinterpret_cast<V*>(smem_raw);
+    const int tid = threadIdx.x, E = a.E;
+    uint32_t roff[EPT], woff[EPT], lpos[EPT];
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+        const int r = tid + THREADS * j;
+        roff[j] = woff[j] = lpos[j] = 0;
+        if (r < E) {
+            roff[j] = a.tab[r];
+            woff[j] = a.tab[E + r];
+            lpos[j] = swz((int)a.tab[2 * E + r]);
+        }
+    }
+    auto origin = [&](uint64_t tile, int64_t& oi, int64_t& oo) {
+        oi = oo = 0;
+        for (int g = 0; g < a.ng; ++g) {
+            const uint64_t q = tile / (uint64_t)a.g_count[g];
+            const int64_t c = (int64_t)(tile - q * (uint64_t)a.g_count[g]);
+            tile = q;
+            oi += c * a.g_si[g];
+            oo += c * a.g_so[g];
+        }
+        oi = uniform64(oi);
+        oo = uniform64(oo);
+    };
+    V regs[EPT];
+    auto load = [&](int64_t oi) {
+        const V* in = reinterpret_cast<const V*>(a.in) + oi;
+#pragma unroll
+        for (int j = 0; j < EPT; ++j)
+            if (tid + THREADS * j < E) regs[j] = load_stream<Pack<V, 1>>(in + roff[j]).v[0];
+    };
+    uint64_t tile = blockIdx.x;
+    if (tile >= (uint64_t)a.ntiles) return;
+    int64_t oi, oo;
+    origin(tile, oi, oo);
+    load(oi);
+    for (;;) {
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) {
+            const int r = tid + THREADS * j;
+            if (r < E) lds[swz(r)] = regs[j];
+        }
+        __syncthreads();
+        const uint64_t next = tile + gridDim.x;
+        const bool more = next < (uint64_t)a.ntiles;
+        int64_t oi2 = 0, oo2 = 0;
+        if (more) {   // the next tile's loads are in flight while this one is written out
+            origin(next, oi2, oo2);
+            load(oi2);
+        }
+        V* out = reinterpret_cast<V*>(a.out) + oo;
+#pragma unroll
+        for (int j = 0; j < EPT; ++j)
+            if (tid + THREADS * j < E) {
+                Pack<V, 1> x;
+                x.v[0] = lds[lpos[j]];
+                store_stream<Pack<V, 1>>(out + woff[j], x);
+            }
+        if (!more) break;
+        __syncthreads();
+        tile = next;
+        oo = oo2;
     }
 }
 
@@ -635,6 +752,173 @@ bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
 }  // namespace
 
+namespace {
+// Contiguous run (elements) a tile of the shift-and-mask plan reads (slot 0) or writes (slot 1), and the share of its
+// positions that hold an element (tile extents are powers of two, the axes need not be).
+void masked_plan_quality(const CopyArgs& a, int64_t& run_in, int64_t& run_out, double& filled) {
+    run_in = run_out = 1;
+    filled = 1.0;
+    bool go = true;
+    for (int t = 0; t < a.nt && go; ++t) {
+        const int64_t ext = a.r_mask[t] + 1, n = a.t_n[a.r_id[t]], use = std::min(ext, n);
+        if (std::llabs(a.r_si[t]) != run_in) break;
+        run_in *= use;
+        go = use == n;
+    }
+    go = true;
+    for (int t = 0; t < a.nt && go; ++t) {
+        const int64_t ext = a.w_mask[t] + 1, n = a.t_n[a.w_id[t]], use = std::min(ext, n);
+        if (std::llabs(a.w_so[t]) != run_out) break;
+        run_out *= use;
+        go = use == n;
+    }
+    for (int t = 0; t < a.nt; ++t) {
+        const int64_t ext = a.r_mask[t] + 1, n = a.t_n[a.r_id[t]];
+        filled *= (double)std::min(ext, n) / (double)ext;   // (a last partial tile along a long axis is ignored)
+    }
+}
+
+template <class V>
+void launch_tabcopy(const TabCopyArgs& ta, int ept, dim3 grid, size_t lds, hipStream_t st) {
+    if (ept <= 8) TFH_LAUNCH_TIMED((tabcopy_kernel<V, 8>), grid, dim3(THREADS), lds, st, ta);
+    else if (ept <= 16) TFH_LAUNCH_TIMED((tabcopy_kernel<V, 16>), grid, dim3(THREADS), lds, st, ta);
+    else TFH_LAUNCH_TIMED((tabcopy_kernel<V, 32>), grid, dim3(THREADS), lds, st, ta);
+}
+
+// A bit-exact move whose shift-and-mask tiles come out with short runs or mostly empty: tiles of whole axes, driven by
+// tables.  Returns true when it launched (status holds the outcome).
+bool try_table_copy(int eb, const void* in, void* out, std::vector<Axis> axes, const TilePlan& tp, void* stream, int32_t& status) {
+    status = TFH_OK;
+    int64_t total = 1;
+    for (auto& x : axes) total *= x.n;
+    if (total < 65536) return false;
+    int64_t run_in_old, run_out_old;
+    double filled;
+    masked_plan_quality(tp.args, run_in_old, run_out_old, filled);
+    const double old_q = (double)std::min<int64_t>(std::min(run_in_old, run_out_old) * eb, 512) * (tp.all_full ? 1.0 : filled);
+    if (old_q >= 256.0) return false;
+    std::stable_sort(axes.begin(), axes.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[1]) > std::llabs(y.s[1]); });
+    fuse_axes(axes, 2);
+    const int na = (int)axes.size();
+    if (na < 2 || na > MAXG) return false;
+    for (auto& x : axes)
+        if (x.s[0] <= 0 || x.s[1] <= 0) return false;   // broadcast or reversed axes stay with the general path
+    std::vector<int> in_order(na), out_order(na);
+    for (int i = 0; i < na; ++i) in_order[i] = out_order[i] = i;
+    std::stable_sort(in_order.begin(), in_order.end(), [&](int x, int y) { return axes[x].s[0] < axes[y].s[0]; });
+    std::stable_sort(out_order.begin(), out_order.end(), [&](int x, int y) { return axes[x].s[1] < axes[y].s[1]; });
+    // whole axes, alternately from the input's and the output's fastest end, while the tile fits and a side is short
+    const int64_t emax = std::min<int64_t>(61440 / eb, (int64_t)THREADS * 32);
+    const int64_t want = std::max<int64_t>(1, 512 / eb);
+    std::vector<char> in_tile(na, 0);
+    int64_t E = 1, run[2] = {1, 1};
+    size_t pos[2] = {0, 0};
+    bool open_[2] = {true, true};
+    const std::vector<int>* order[2] = {&in_order, &out_order};
+    auto advance = [&](int side) {   // run of a side = product of the leading axes of its order that are in the tile
+        while (pos[side] < (size_t)na && in_tile[(*order[side])[pos[side]]]) {
+            const Axis& x = axes[(*order[side])[pos[side]]];
+            if (x.s[side] != run[side]) { open_[side] = false; break; }   // not contiguous with the run so far
+            run[side] *= x.n;
+            ++pos[side];
+        }
+        if (pos[side] == (size_t)na) open_[side] = false;
+    };
+    for (;;) {
+        advance(0);
+        advance(1);
+        int side = -1;
+        if (open_[0] && run[0] < want && (!(open_[1] && run[1] < want) || run[0] <= run[1])) side = 0;
+        else if (open_[1] && run[1] < want) side = 1;
+        if (side < 0) break;
+        const int i = (*order[side])[pos[side]];
+        if (axes[i].s[side] != run[side] || E * axes[i].n > emax) { open_[side] = false; continue; }
+        in_tile[i] = 1;
+        E *= axes[i].n;
+    }
+    // runs reached with a small tile (a few short axes serve both sides): more whole axes, the input's innermost free
+    // axis and the output's in turn, until a block has 2048 elements to move per tile
+    for (int side = 0, idle = 0; E < 2048 && idle < 2; side ^= 1) {
+        int pick = -1;
+        for (int i : *order[side])
+            if (!in_tile[i]) { pick = i; break; }
+        if (pick < 0 || E * axes[pick].n > emax) { ++idle; continue; }
+        idle = 0;
+        in_tile[pick] = 1;
+        E *= axes[pick].n;
+    }
+    if (E < 512) return false;
+    const double new_q = (double)std::min<int64_t>(std::min(run[0], run[1]) * eb, 512);
+    if (new_q < 2.0 * old_q) return false;
+    // tile axes in read order (with their LDS strides) and in write order
+    TabBuildArgs tb;
+    std::memset(&tb, 0, sizeof tb);
+    std::vector<int> rpos(na, 0);
+    int64_t lo = 1, span_in = 0, span_out = 0;
+    std::string key = "copytab|" + std::to_string(eb);
+    for (int i : in_order)
+        if (in_tile[i]) {
+            if (tb.nt == TAB_MAX_AXES) return false;
+            tb.r_ext[tb.nt] = (int32_t)axes[i].n;
+            tb.r_si[tb.nt] = axes[i].s[0];
+            rpos[i] = (int)lo;
+            lo *= axes[i].n;
+            ++tb.nt;
+            span_in += (axes[i].n - 1) * axes[i].s[0];
+            span_out += (axes[i].n - 1) * axes[i].s[1];
+            key += "|" + std::to_string(axes[i].n) + "," + std::to_string(axes[i].s[0]) + "," + std::to_string(axes[i].s[1]);
+        }
+    if (span_in >= ((int64_t)1 << 32) || span_out >= ((int64_t)1 << 32)) return false;   // 32-bit element offsets
+    int w = 0;
+    for (int i : out_order)
+        if (in_tile[i]) {
+            tb.w_ext[w] = (int32_t)axes[i].n;
+            tb.w_so[w] = axes[i].s[1];
+            tb.w_rpos[w] = rpos[i];
+            ++w;
+        }
+    tb.E = (int32_t)E;
+    TabCopyArgs ta;
+    std::memset(&ta, 0, sizeof ta);
+    ta.in = in;
+    ta.out = out;
+    ta.E = (int32_t)E;
+    int64_t ntiles = 1;
+    for (int i = na - 1; i >= 0; --i)   // fastest tile index: the innermost axis outside the tile (neighbouring tiles abut)
+        if (!in_tile[i]) {
+            ta.g_count[ta.ng] = axes[i].n;
+            ta.g_si[ta.ng] = axes[i].s[0];
+            ta.g_so[ta.ng] = axes[i].s[1];
+            ++ta.ng;
+            ntiles *= axes[i].n;
+        }
+    ta.ntiles = ntiles;
+    if (ntiles < 8) return false;
+    void* tab = nullptr;
+    bool fresh = false;
+    if ((status = table_cache_get(stream, key, (size_t)3 * E * sizeof(uint32_t), &tab, &fresh)) != TFH_OK) return true;
+    if (!tab) return false;   // no cached block to be had (cache full, stream being captured): the masked tiles do it
+    hipStream_t st = (hipStream_t)stream;
+    if (fresh) {
+        tb.tab = (uint32_t*)tab;
+        hipLaunchKernelGGL(tabcopy_build_kernel, dim3((uint32_t)((E + THREADS - 1) / THREADS)), dim3(THREADS), 0, st, tb);
+        table_cache_commit(stream, key);
+    }
+    ta.tab = (const uint32_t*)tab;
+    const int ept = (int)((E + THREADS - 1) / THREADS);
+    const size_t lds = (size_t)(E + E / 32 + 4) * eb;
+    const size_t per_cu = std::max<size_t>(1, std::min<size_t>(4, (size_t)(160 * 1024) / (lds + 512)));
+    const dim3 grid((uint32_t)std::min<int64_t>(ntiles, (int64_t)(256 * per_cu)));
+    const int prof = prof_begin(PROF_COPY, stream);
+    if (eb == 4) launch_tabcopy<uint32_t>(ta, ept, grid, lds, st);
+    else if (eb == 8) launch_tabcopy<uint64_t>(ta, ept, grid, lds, st);
+    else launch_tabcopy<double2>(ta, ept, grid, lds, st);
+    prof_end(prof, stream);
+    status = hip_check(hipGetLastError(), "copy kernel launch");
+    return true;
+}
+}  // namespace
+
 int32_t launch_copy(int dtype, const void* in, void* out, std::vector<Axis> axes, Scalar alpha, Scalar beta, bool conj,
                     void* stream) {
     const int eb = (int)dtype_size(dtype);
@@ -652,6 +936,8 @@ int32_t launch_copy(int dtype, const void* in, void* out, std::vector<Axis> axes
     const bool cx = is_complex(dtype);
     const bool raw = alpha.is_one() && beta.is_zero() && !(conj && cx);
     if (raw) {
+        int32_t st_tab = TFH_OK;
+        if (try_table_copy(eb, in, out, axes, tp, stream, st_tab)) return st_tab;
         switch (eb) {
             case 4: return run_copy<uint32_t, RawOp<uint32_t>, true>(tp, RawOp<uint32_t>(), false, vin, vout, st);
             case 8: return run_copy<uint64_t, RawOp<uint64_t>, true>(tp, RawOp<uint64_t>(), false, vin, vout, st);

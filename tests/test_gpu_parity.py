@@ -1734,6 +1734,46 @@ def test_tensor_view_materialises_on_the_device(tf, oracle):
     assert p.conj().to_numpy().tobytes() == np.conj(ref).tobytes()
 
 
+def test_permute_tensors_of_many_short_axes(tf):
+    # Tensors of many small extents (spins, qubits): the tile is a product of whole axes and its position-to-offset maps
+    # come from cached tables.  Bit-exact against numpy for reversals, a cyclic shift and neighbour exchanges, extents that
+    # are and are not powers of two, 4-, 8- and 16-byte elements, a sliced operand (strides that are not the dense ones),
+    # the second call on a layout (tables from the cache) and a call after the caches were released.
+    rng = np.random.default_rng(133)
+    cases = [((3,) * 14, tuple(reversed(range(14))), np.float64), ((3,) * 12, tuple(reversed(range(12))), np.complex128),
+             ((3,) * 13, (0, 2, 1, 3, 5, 4, 6, 8, 7, 9, 11, 10, 12), np.float32), ((5,) * 8, tuple(reversed(range(8))), np.float64),
+             ((3, 4) * 5, tuple(reversed(range(10))), np.float64), ((2, 3) * 7, tuple(reversed(range(14))), np.float64),
+             ((4,) * 10, tuple(reversed(range(10))), np.float32), ((2,) * 16, tuple(reversed(range(16))), np.complex64),
+             ((6,) * 7, (3, 4, 5, 6, 0, 1, 2), np.float64), ((100, 50, 20, 17), (0, 1, 3, 2), np.float64)]
+    used = 0
+    for shape, perm, dtype in cases:
+        x = rand(rng, shape, dtype)
+        oshape = [shape[q] for q in perm]
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Permute(list(range(len(shape))), list(perm)), [list(shape), oshape])
+        for rep in range(2):
+            out = dev(tf, np.zeros(oshape, dtype))
+            tf.HipBackend.execute(plan, 1.0, [dev(tf, x)], 0.0, out)
+            used += "tabcopy_kernel" in tf.last_kernel()
+            assert out.to_numpy().tobytes() == np.ascontiguousarray(x.transpose(perm)).tobytes(), (shape, perm, dtype, tf.last_kernel())
+    assert used >= 14, used            # most of these shapes take the table-driven tiles, on both calls
+    # a slice of a larger tensor: strides of the operand are not those of a dense tensor
+    big = rand(rng, (4,) + (3,) * 12, np.float64)
+    x = big[1]
+    perm = tuple(reversed(range(12)))
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute(list(range(12)), list(perm)), [[3] * 12, [3] * 12])
+    out = dev(tf, np.zeros((3,) * 12))
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, x)], 0.0, out)
+    assert out.to_numpy().tobytes() == np.ascontiguousarray(x.transpose(perm)).tobytes()
+    assert tf.lib().tfh_release_workspaces() == 0
+    tf.HipBackend.execute(plan, 1.0, [dev(tf, x)], 0.0, out)
+    assert "tabcopy_kernel" in tf.last_kernel() and out.to_numpy().tobytes() == np.ascontiguousarray(x.transpose(perm)).tobytes()
+    # alpha/beta and conj keep the masked tiles (the table path moves raw bits only)
+    z = rand(rng, (3,) * 12, np.complex128)
+    got = dev(tf, np.zeros((3,) * 12, np.complex128))
+    tf.HipBackend.execute(tf.HipBackend.plan(np.complex128, tf.PrimDescriptor.Permute(list(range(12)), list(perm)), [[3] * 12, [3] * 12]), 2.0, [dev(tf, z)], 0.0, got)
+    assert "tabcopy_kernel" not in tf.last_kernel() and np.array_equal(got.to_numpy(), 2.0 * z.transpose(perm))
+
+
 def test_reduce_over_short_contiguous_rows(tf, oracle):
     # A reduced contiguous axis of 2..32 elements inside a long kept axis, extents that do not tile (17, 31, 3; an even 6
     # under an odd row count): 256 rows per block go through LDS and every thread adds up its own row.  Sum (exact on
