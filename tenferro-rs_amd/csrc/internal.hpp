@@ -112,6 +112,10 @@ int32_t launch_reduce_general(int dtype, const void* a, const void* b, void* c, 
 // C = alpha*A*B + beta*C over classified axes
 int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes axes, Scalar alpha,
                         Scalar beta, void* stream);
+// A tiny operator (<= 8 free and <= 8 contracted indices) applied to a long tensor: the streaming kernel of
+// k_gemm_tiny.hip.  Returns false when the shape is not one it takes; true when it launched (status holds the outcome).
+bool try_tiny_operator(int dtype, const void* a, const void* b, void* c, const ContractAxes& ax, Scalar alpha, Scalar beta,
+                       void* stream, int32_t& status);
 // Matrix-vector-like contractions (one free group empty): the streaming product-reduction kernel of k_dot.hip.  Returns
 // false when the shape is not one it tiles; true when it launched (status holds the outcome).  Axis strides: A, B, C.
 bool try_dot(int dtype, const void* a, const void* b, void* c, std::vector<Axis> kept, std::vector<Axis> red, Scalar alpha,

@@ -559,6 +559,11 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     }
     // One free group empty (matrix-vector, vector-matrix, dot and batched dot products): there is nothing for a tile
     // of MFMAs to reuse -- a reduction of the elementwise product, bound by HBM (k_dot.hip)
+    // a tiny operator applied to a long tensor (a gate on a leg of a state): a stream over the long operand
+    if (M > 1 && N > 1) {
+        int32_t st_tiny = TFH_OK;
+        if (try_tiny_operator(dtype, a, b, c, ax, alpha, beta, stream, st_tiny)) return st_tiny;
+    }
     if (M == 1 || N == 1) {
         std::vector<Axis> kept, red = ax.K;
         for (auto* grp : {&ax.batch, &ax.M, &ax.N})

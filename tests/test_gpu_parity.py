@@ -1734,6 +1734,58 @@ def test_tensor_view_materialises_on_the_device(tf, oracle):
     assert p.conj().to_numpy().tobytes() == np.conj(ref).tobytes()
 
 
+def test_contract_tiny_operator_applied_to_a_long_tensor(tf):
+    # One operand with at most 8 free and 8 contracted indices, the other long (a gate on one or two legs of a state):
+    # the streaming kernel, against numpy's einsum in double precision.  Legs at the front, in the middle and at the end,
+    # extents 2, 3 and 8, either operand order, two-leg gates, alpha/beta, a sliced long operand, an output whose
+    # contiguous axis is not the long operand's (scalar accesses), all four dtypes; exact on small integers.
+    rng = np.random.default_rng(134)
+    lab = lambda t: [ord(ch) for ch in t]
+
+    def run(sub, sa, sb, dtype, alpha=1.0, beta=0.0, views=None, out_order="C", exact=False):
+        ia, ib, ic = sub.replace("->", ",").split(",")
+        if exact:
+            x, y = rng.integers(-3, 4, size=sa).astype(dtype), rng.integers(-3, 4, size=sb).astype(dtype)
+        else:
+            x, y = rand(rng, sa, dtype), rand(rng, sb, dtype)
+        if views:
+            x, y = views(x, y)
+        ref = np.einsum(sub, x.astype(np.complex128), y.astype(np.complex128))
+        c0 = rand(rng, ref.shape, dtype)
+        c0 = np.asfortranarray(c0) if out_order == "F" else c0
+        out = dev(tf, c0 if beta != 0.0 else np.full_like(c0, np.nan))
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ia), lab(ib), lab(ic)), [list(x.shape), list(y.shape), list(ref.shape)])
+        tf.HipBackend.execute(plan, alpha, [dev(tf, x), dev(tf, y)], beta, out)
+        assert "tiny_operator_kernel" in tf.last_kernel(), (sub, sa, sb, tf.last_kernel())
+        want = alpha * ref + (beta * c0 if beta != 0.0 else 0.0)
+        if exact:
+            assert np.array_equal(out.to_numpy(), want.real.astype(dtype)), (sub, sa, sb, dtype)
+        else:
+            assert relerr(out.to_numpy(), want) < TOL[dtype], (sub, sa, sb, dtype)
+
+    for dtype in ALL:
+        run("ab,xby->xay", (2, 2), (64, 2, 1024), dtype)
+        run("ab,xby->xay", (2, 2), (1, 2, 131072), dtype)
+        run("ab,xby->xay", (2, 2), (131072, 2, 1), dtype)
+        run("ab,xby->xay", (3, 3), (243, 3, 729), dtype)
+        run("xby,ba->xay", (64, 2, 1024), (2, 2), dtype)                       # the operator second
+        run("abcd,xcydz->xaybz", (2, 2, 2, 2), (32, 2, 32, 2, 64), dtype)       # two legs
+        run("ab,xby->xay", (8, 8), (64, 8, 1024), dtype, alpha=-0.5, beta=2.0)
+        run("ab,xby->xay", (5, 3), (100, 3, 700), dtype)                       # rectangular, nothing a power of two
+        run("ab,xby->xay", (2, 2), (65, 2, 1023), dtype)                       # odd inner extent: scalar accesses
+        run("ab,xby->xay", (2, 2), (64, 2, 1024), dtype, out_order="F")         # the output contiguous along x
+        run("ab,xby->xay", (4, 4), (70, 4, 1100), dtype, views=lambda x, y: (x.T, y[3:67, :, 50:1074]))   # transposed operator, sliced tensor
+        run("ab,xby->yax", (2, 2), (64, 2, 1024), dtype)                       # the long axes exchanged in the output
+    run("ab,xby->xay", (2, 2), (64, 2, 1024), np.float64, exact=True)
+    run("abcd,xcydz->xaybz", (2, 2, 2, 2), (32, 2, 32, 2, 64), np.float32, exact=True)
+    if True:
+        z = (rng.integers(-2, 3, size=(2, 2)) + 1j * rng.integers(-2, 3, size=(2, 2))).astype(np.complex128)
+        t = (rng.integers(-2, 3, size=(32, 2, 2048)) + 1j * rng.integers(-2, 3, size=(32, 2, 2048))).astype(np.complex128)
+        out = dev(tf, np.zeros((32, 2, 2048), np.complex128))
+        tf.HipBackend.execute(tf.HipBackend.plan(np.complex128, tf.PrimDescriptor.Contract(lab("ab"), lab("xby"), lab("xay")), [[2, 2], [32, 2, 2048], [32, 2, 2048]]), 1.0, [dev(tf, z), dev(tf, t)], 0.0, out)
+        assert "tiny_operator_kernel" in tf.last_kernel() and np.array_equal(out.to_numpy(), np.einsum("ab,xby->xay", z, t))
+
+
 def test_permute_tensors_of_many_short_axes(tf):
     # Tensors of many small extents (spins, qubits): the tile is a product of whole axes and its position-to-offset maps
     # come from cached tables.  Bit-exact against numpy for reversals, a cyclic shift and neighbour exchanges, extents that
