@@ -1037,10 +1037,10 @@ int32_t launch_emul(int dtype, const void* a, const void* b, void* c, std::vecto
     set_scalars(tp.args, alpha, beta, false);
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
-        case TFH_F32: hipLaunchKernelGGL((emul_kernel<float, false>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
-        case TFH_F64: hipLaunchKernelGGL((emul_kernel<double, false>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
-        case TFH_C64: hipLaunchKernelGGL((emul_kernel<float, true>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
-        default: hipLaunchKernelGGL((emul_kernel<double, true>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
+        case TFH_F32: TFH_LAUNCH_TIMED((emul_kernel<float, false>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
+        case TFH_F64: TFH_LAUNCH_TIMED((emul_kernel<double, false>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
+        case TFH_C64: TFH_LAUNCH_TIMED((emul_kernel<float, true>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
+        default: TFH_LAUNCH_TIMED((emul_kernel<double, true>), tp.grid, dim3(THREADS), 0, st, tp.args, tp.ept); break;
     }
     pool_free(stream, packed);   // stream-ordered: the block is reused only by later work on this stream
     return hip_check(hipGetLastError(), "elementwise kernel launch");

@@ -1786,6 +1786,27 @@ def test_contract_tiny_operator_applied_to_a_long_tensor(tf):
         assert "tiny_operator_kernel" in tf.last_kernel() and np.array_equal(out.to_numpy(), np.einsum("ab,xby->xay", z, t))
 
 
+def test_contract_without_a_summed_index_scales_through_the_elementwise_kernel(tf):
+    # "asx,x->asx", "ij,i->ij": a tensor scaled along some of its axes.  One free group is empty and nothing is summed, so
+    # the elementwise kernel does it with the missing axes as broadcast axes; extents that tile and extents that do not,
+    # alpha/beta, all dtypes (4-byte elements keep the product-reduction kernel where the extents tile).
+    rng = np.random.default_rng(135)
+    lab = lambda t: [ord(ch) for ch in t]
+    for dtype in ALL:
+        for sub, sa, sb in (("asx,x->asx", (100, 3, 1000), (1000,)), ("asx,a->asx", (128, 2, 1024), (128,)), ("ij,j->ij", (1021, 1031), (1031,)),
+                            ("ij,i->ji", (512, 300), (512,)), ("abcd,ca->abcd", (16, 9, 32, 40), (32, 16))):
+            ia, ib, ic = sub.replace("->", ",").split(",")
+            x, y = rand(rng, sa, dtype), rand(rng, sb, dtype)
+            ref = np.einsum(sub, x.astype(np.complex128), y.astype(np.complex128))
+            c0 = rand(rng, ref.shape, dtype)
+            out = dev(tf, c0)
+            plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ia), lab(ib), lab(ic)), [list(sa), list(sb), list(ref.shape)])
+            tf.HipBackend.execute(plan, 2.0, [dev(tf, x), dev(tf, y)], -1.0, out)
+            if np.dtype(dtype).itemsize >= 8 or sa in ((100, 3, 1000), (1021, 1031), (512, 300), (16, 9, 32, 40)):
+                assert "emul_kernel" in tf.last_kernel(), (sub, sa, dtype, tf.last_kernel())
+            assert relerr(out.to_numpy(), 2.0 * ref - c0) < TOL[dtype], (sub, sa, dtype)
+
+
 def test_permute_tensors_of_many_short_axes(tf):
     # Tensors of many small extents (spins, qubits): the tile is a product of whole axes and its position-to-offset maps
     # come from cached tables.  Bit-exact against numpy for reversals, a cyclic shift and neighbour exchanges, extents that
