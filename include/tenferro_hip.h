@@ -159,6 +159,21 @@ int32_t tfh_execute_grouped(const tfh_plan* plan, const void* alpha,
                             const tfh_view* inputs, int32_t n_inputs,
                             const void* beta, tfh_view* outputs, tfh_stream stream);
 
+/* tfh_execute for callers that cannot allocate device memory.  No counterpart in the reference: it is for code
+ * under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same arguments, same kernels
+ * and same results as tfh_execute, but the device scratch of the call (offset tables, split-K partials, partial sums
+ * of a split reduction, a packed copy of an operand) comes from one fixed array of TFH_STATIC_SCRATCH_BYTES that is
+ * part of the library's code object on every device it runs on; the call allocates and frees nothing on the device.
+ * A call that needs more scratch than that fails with TFH_ERR_INVALID_ARGUMENT and a message that gives the
+ * amounts (kernels that precede the oversized request may already have been enqueued; the output is then
+ * unspecified).  All calls on one device share the array: calls that overlap in time on one device, on any
+ * streams or threads, race on it -- order them on one stream or with events.  Grouped plans are not taken. */
+#define TFH_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+size_t tfh_static_scratch_bytes(void);
+int32_t tfh_execute_static(const tfh_plan* plan, const void* alpha,
+                           const tfh_view* inputs, int32_t n_inputs,
+                           const void* beta, tfh_view* output, tfh_stream stream);
+
 /* Tensor::conj / into_conj (tenferro-tensor/src/lib.rs:622-658): out = conj(in) elementwise,
  * same dims; a plain copy for real dtypes.  in and out may be the same view (into_conj). */
 int32_t tfh_conj(int32_t dtype, const tfh_view* in, tfh_view* out, tfh_stream stream);

@@ -78,6 +78,9 @@ def lib():
             getattr(L, name).argtypes = [C.c_void_p]
         L.tfh_execute.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
         L.tfh_execute_grouped.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.tfh_execute_static.argtypes = L.tfh_execute.argtypes
+        L.tfh_static_scratch_bytes.restype = C.c_size_t
+        L.tfh_static_scratch_bytes.argtypes = []
         L.tfh_einsum_execute.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p,
                                          C.c_uint64, C.c_void_p]
         L.tfh_conj.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
@@ -406,6 +409,16 @@ class HipBackend:
         st = current_stream() if stream is None else stream
         _check(lib().tfh_execute(plan._h, _scalar_c(plan.dtype, alpha), views, len(inputs), _scalar_c(plan.dtype, beta),
                                  C.byref(vo), st))
+
+    @staticmethod
+    def execute_static(plan, alpha, inputs, beta, output, stream=None):
+        """execute() without device allocations: the scratch of the call comes from the library's fixed array
+        (tfh_execute_static; no counterpart in the reference).  Calls that overlap on one device race on that array."""
+        views = (tfh_view * max(len(inputs), 1))(*[view_of(t) for t in inputs])
+        vo = view_of(output)
+        st = current_stream() if stream is None else stream
+        _check(lib().tfh_execute_static(plan._h, _scalar_c(plan.dtype, alpha), views, len(inputs), _scalar_c(plan.dtype, beta),
+                                        C.byref(vo), st))
 
     @staticmethod
     def has_extension_for(dtype, ext):

@@ -139,6 +139,11 @@ void table_cache_commit(void* stream, const std::string& key);
 // stream's cache; reuse on the same stream needs no synchronisation).
 int32_t pool_alloc(void* stream, size_t bytes, void** out);
 void pool_free(void* stream, void* ptr);
+// Between arena_begin() and arena_end() on one host thread, workspace() and pool_alloc() hand out consecutive pieces of
+// the given device region instead of allocating (an error once it is used up), pool_free() does nothing and the table
+// cache is bypassed.
+void arena_begin(void* base, size_t bytes);
+void arena_end();
 int32_t hip_check(int err, const char* what);
 // Event bracket around a dominant kernel while profiling is enabled (runtime.cpp); -1 when disabled.
 enum { PROF_CONTRACT = 0, PROF_COPY = 1, PROF_REDUCE = 2 };

@@ -33,6 +33,25 @@ constexpr size_t TABLE_CACHE_ENTRIES = 256;
 std::mutex g_mu;
 std::map<std::pair<int, void*>, StreamScratch> g_scratch;   // (device, stream)
 
+// While a call made through tfh_execute_static is running on this thread, every piece of device scratch it asks for
+// (workspace, packed operands, offset tables) is carved out of a fixed region handed in by arena_begin(); nothing is
+// allocated, cached or freed.
+struct Arena {
+    char* base = nullptr;
+    size_t cap = 0, used = 0;
+    bool active = false;
+};
+thread_local Arena t_arena;
+int32_t arena_alloc(size_t bytes, void** out, const char* what) {
+    const size_t at = (t_arena.used + 255) & ~(size_t)255;
+    if (bytes > t_arena.cap || at > t_arena.cap - bytes)
+        return set_error(TFH_ERR_INVALID_ARGUMENT, "%s: the call needs %zu bytes of scratch memory beyond the %zu already taken; the static scratch holds %zu",
+                         what, bytes, at, t_arena.cap);
+    *out = t_arena.base + at;
+    t_arena.used = at + bytes;
+    return TFH_OK;
+}
+
 StreamScratch* scratch_for(void* stream, int32_t* err) {
     int dev = 0;
     *err = hip_check(hipGetDevice(&dev), "hipGetDevice");
@@ -63,7 +82,11 @@ int32_t malloc_or_release(void** p, size_t bytes, void* stream, const char* what
 }
 }  // namespace
 
+void arena_begin(void* base, size_t bytes) { t_arena = Arena{(char*)base, bytes, 0, true}; }
+void arena_end() { t_arena = Arena{}; }
+
 int32_t workspace(void* stream, size_t bytes, void** out) {
+    if (t_arena.active) return arena_alloc(bytes, out, "workspace");
     std::lock_guard<std::mutex> lk(g_mu);
     int32_t err;
     StreamScratch* s = scratch_for(stream, &err);
@@ -87,6 +110,7 @@ int32_t workspace(void* stream, size_t bytes, void** out) {
 int32_t table_cache_get(void* stream, const std::string& key, size_t bytes, void** tables, bool* fresh) {
     *tables = nullptr;
     *fresh = false;
+    if (t_arena.active) return TFH_OK;   // no cache in a call that must not allocate: the tables go to its workspace
     std::lock_guard<std::mutex> lk(g_mu);
     int32_t err;
     StreamScratch* s = scratch_for(stream, &err);
@@ -126,6 +150,7 @@ void table_cache_commit(void* stream, const std::string& key) {
 }
 
 int32_t pool_alloc(void* stream, size_t bytes, void** out) {
+    if (t_arena.active) return arena_alloc(bytes, out, "packed operand");
     std::lock_guard<std::mutex> lk(g_mu);
     int32_t err;
     StreamScratch* s = scratch_for(stream, &err);
@@ -146,7 +171,7 @@ int32_t pool_alloc(void* stream, size_t bytes, void** out) {
 }
 
 void pool_free(void* stream, void* ptr) {
-    if (!ptr) return;
+    if (!ptr || t_arena.active) return;   // arena blocks live until the call ends
     std::lock_guard<std::mutex> lk(g_mu);
     int32_t err;
     StreamScratch* s = scratch_for(stream, &err);
