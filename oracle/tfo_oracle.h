@@ -6,8 +6,11 @@
  *
  * The reference's own CPU backend is unimplemented (tenferro-prims/src/lib.rs:419-439 are
  * `todo!()`), so every function here follows the *documented formula* of the item it cites and
- * is pinned by the checks in tests/test_oracle_*.py (numpy cross-checks, closed forms, brute
- * force, the reference's doc examples).  Numerical parity with a reference implementation is
+ * is pinned by the checks in tests/test_oracle.py and tests/test_golden.py (numpy cross-checks at
+ * single-block and multi-block sizes, closed forms, brute force, the reference's doc examples,
+ * exactly representable operands for the alpha/beta epilogue).  f32 products are accumulated in
+ * f32 inside a cache block and in f64 across blocks: on outputs whose terms cancel the result
+ * carries the rounding error of an f32 inner product (tests/golden/cancelling_f32.npz).  Numerical parity with a reference implementation is
  * therefore "parity unpinned": there is no reference implementation to compare with.
  */
 #ifndef TFO_ORACLE_H

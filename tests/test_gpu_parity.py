@@ -34,6 +34,23 @@ def relerr(x, ref):
     return d / n if n > 0 else d
 
 
+def contraction_within_tolerance(x, ref, dtype, scale, k):
+    """The parity rule for a contraction result.  The stated tolerance (TOL) is a relative Frobenius error against the
+    norm of the reference, and a well-conditioned output meets it.  An output whose terms cancel cannot: two backends
+    that each round every one of k products and partial sums (the CPU restatement accumulates f32 in f32 inside a cache
+    block, the matrix cores accumulate f32 in f32) may differ by the textbook bound on a rounded inner product,
+    2 * gamma with gamma = (k + 2) * u (u = 2^-24 or 2^-53; 4 real operations per complex one) times `scale`, the
+    same contraction over absolute values |alpha| * |A| . |B| + |beta| * |C0|.  A wrong or dropped term is of the
+    order scale / k, far above that."""
+    d = np.linalg.norm((np.asarray(x, np.complex128) - ref).ravel())
+    n = np.linalg.norm(np.asarray(ref).ravel())
+    if d <= TOL[dtype] * n:
+        return True
+    u = 2.0 ** -24 if dtype in (np.float32, np.complex64) else 2.0 ** -53
+    ops = 4 if np.issubdtype(dtype, np.complexfloating) else 1
+    return d <= 2 * ops * (k + 2) * u * np.linalg.norm(np.asarray(scale).ravel())
+
+
 def dev(tf, arr):
     """Device Tensor with the same dims, element strides and offset as the numpy view `arr`."""
     import torch
@@ -960,8 +977,54 @@ def test_contract_random_label_patterns_and_views(tf, oracle, dtype, big):
         out = dev(tf, c0) if cshape else tf.Tensor.empty([], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
         plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [a.shape, b.shape, cshape])
         tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, out)
-        err = relerr(out.to_numpy(), ref)
-        assert err < TOL[dtype], (case, ma, mb, mc, ext, err)
+        # the same contraction over absolute values, in f64: the scale of the rounding-error bound
+        scale = np.abs(c0).astype(np.float64) if use_beta else np.zeros(cshape)
+        oracle.contract(np.abs(a).astype(np.float64), lab(ma), np.abs(b).astype(np.float64), lab(mb), scale, lab(mc),
+                        alpha=abs(alpha), beta=abs(beta) if use_beta else 0.0)
+        k = int(np.prod([ext[l] for l in set(ma) & set(mb) - set(mc)], dtype=np.int64))
+        assert contraction_within_tolerance(out.to_numpy(), ref, dtype, scale, k), (case, ma, mb, mc, ext, relerr(out.to_numpy(), ref))
+
+
+def _cancelling():
+    import os
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "cancelling_f32.npz"))
+
+
+def test_f32_cancelling_dot_product_regression(tf, oracle):
+    # "dc,dc->" (d = 6, c = 5), alpha = 0.7, thirty f32 terms whose sum is 1/1428 of the sum of their magnitudes.  A
+    # randomized run once reported 2.18e-5 between the device and the CPU restatement on it: the restatement adds f32
+    # products in f32 inside a cache block and carries all of that error; a product with an empty free group runs as a
+    # reduction that accumulates in f64 on the device, which returns the exact result rounded once.
+    fx = _cancelling()
+    a, b, alpha = fx["dot_a"], fx["dot_b"], float(fx["alpha"])
+    exact, scale = float(fx["dot_exact"]), float(fx["dot_abs"])
+    out = tf.Tensor.empty([], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
+    plan = tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Contract(lab("dc"), lab("dc"), []), [a.shape, b.shape, []])
+    tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], 0.0, out)
+    got = float(out.to_numpy())
+    assert "dot" in tf.last_kernel() or "reduce" in tf.last_kernel(), tf.last_kernel()
+    assert abs(got - exact) <= 2.0 ** -23 * abs(exact)          # one rounding of the result and one of alpha
+    ref = np.empty([], np.float32)
+    oracle.contract(a, lab("dc"), b, lab("dc"), ref, [], alpha=alpha)
+    assert abs(float(ref) - exact) > 1e-5 * abs(exact)          # the restatement is the side that misses 1e-5 here ...
+    assert contraction_within_tolerance(got, ref, np.float32, scale, 30)   # ... and is inside the rounding bound
+
+
+def test_f32_cancelling_sums_on_the_matrix_cores(tf, oracle):
+    # the same thirty terms under two free axes ("fdc,dce->fe"): the f32 matrix-core kernel accumulates in f32, so on
+    # these outputs it is held to the rounding bound, not to 1e-5 of the (cancelled) result
+    fx = _cancelling()
+    a, b, alpha = fx["mat_a"], fx["mat_b"], float(fx["alpha"])
+    exact, scale = fx["mat_exact"], fx["mat_abs"]
+    out = tf.Tensor.empty([2, 3], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
+    plan = tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Contract(lab("fdc"), lab("dce"), lab("fe")), [a.shape, b.shape, [2, 3]])
+    tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], 0.0, out)
+    assert "gemm" in tf.last_kernel(), tf.last_kernel()
+    got = out.to_numpy().astype(np.float64)
+    assert np.linalg.norm(got - exact) <= (30 + 2) * 2.0 ** -24 * np.linalg.norm(scale)
+    ref = np.empty([2, 3], np.float32)
+    oracle.contract(a, lab("fdc"), b, lab("dce"), ref, lab("fe"), alpha=alpha)
+    assert contraction_within_tolerance(out.to_numpy(), ref, np.float32, scale, 30)
 
 
 @pytest.mark.parametrize("dtype", ALL)

@@ -400,3 +400,101 @@ def test_beta_zero_never_reads_the_output(oracle):
     p = np.full((7, 6), np.nan)
     oracle.permute(a, [0, 1], p, [1, 0], alpha=2.0)
     assert np.isfinite(p).all()
+
+
+# ------------------------------------------------------------------------------------------------ f32 under cancellation
+def lab(s):
+    return [ord(c) for c in s]
+
+
+def _cancelling():
+    import os
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "cancelling_f32.npz"))
+
+
+def test_f32_cancelling_sums_blocked_path_within_the_rounding_bound_and_brute_force_exact(oracle):
+    # tests/golden/cancelling_f32.npz: thirty f32 terms whose sum is 1/1428 of the sum of their magnitudes, with the
+    # exact result from numpy in f64.  The blocked path adds f32 products in f32 inside a cache block: its error is
+    # bounded by (k + 2) * 2^-24 * sum|a||b| -- and on the first case it is 2.2e-5 of the result, i.e. this path cannot
+    # meet a 1e-5 tolerance that is measured against a cancelled result.  The brute-force path (long double) is exact.
+    fx = _cancelling()
+    alpha = float(fx["alpha"])
+    for a, ma, b, mb, mc, exact, scale in [(fx["dot_a"], "dc", fx["dot_b"], "dc", "", fx["dot_exact"], fx["dot_abs"]),
+                                           (fx["mat_a"], "fdc", fx["mat_b"], "dce", "fe", fx["mat_exact"], fx["mat_abs"])]:
+        shape = [dict(zip(ma + mb, a.shape + b.shape))[l] for l in mc]
+        got = np.empty(shape, np.float32)
+        oracle.contract(a, lab(ma), b, lab(mb), got, lab(mc), alpha=alpha)
+        assert np.linalg.norm(got - exact) <= 32 * 2.0 ** -24 * np.linalg.norm(scale)
+        gold = np.empty(shape, np.float32)
+        oracle.contract(a, lab(ma), b, lab(mb), gold, lab(mc), alpha=alpha, naive=True)
+        assert np.all(np.abs(gold - exact) <= 2.0 ** -23 * np.abs(exact))
+    got = np.empty([], np.float32)
+    oracle.contract(fx["dot_a"], lab("dc"), fx["dot_b"], lab("dc"), got, [], alpha=alpha)
+    assert 1e-5 < abs(float(got) - float(fx["dot_exact"])) / abs(float(fx["dot_exact"])) < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.complex64])
+def test_f32_alpha_beta_epilogue_is_exact_on_dyadic_cancelling_sums(oracle, dtype):
+    # quarter-integers in [-2, 2]: every product, partial sum and the alpha/beta combination below is exactly
+    # representable in f32, so whatever the order of additions the blocked path must return numpy's f64 result bit for
+    # bit -- a wrong sign, a dropped beta term or alpha applied twice cannot hide behind rounding.  Columns of B are
+    # arranged in +/- pairs so that most sums cancel to small values.
+    rng = np.random.default_rng(77)
+    m, n, k = 37, 29, 96
+    def draw(shape):
+        x = rng.integers(-8, 9, shape).astype(np.float64) / 4.0
+        if np.issubdtype(dtype, np.complexfloating):
+            x = x + 1j * rng.integers(-8, 9, shape).astype(np.float64) / 4.0
+        return x
+    a = draw((m, k))
+    a[:, k // 2:] = a[:, :k // 2]                 # a row is its first half twice ...
+    b = draw((k, n))
+    b[k // 2:, : n // 2] = -b[:k // 2, : n // 2]  # ... and the left columns of B change sign half way: those sums are exactly 0
+    c0 = draw((m, n))
+    alpha, beta = (0.5 - 0.25j, -0.25 + 2j) if np.issubdtype(dtype, np.complexfloating) else (0.5, -0.25)
+    want = (alpha * (a @ b) + beta * c0).astype(dtype)
+    assert np.all((a @ b)[:, : n // 2] == 0)
+    got = c0.astype(dtype)
+    oracle.contract(a.astype(dtype), lab("mk"), b.astype(dtype), lab("kn"), got, lab("mn"), alpha=alpha, beta=beta)
+    assert got.tobytes() == want.tobytes()
+
+
+# ------------------------------------------------------------------------------------------------ several cache blocks, all threads
+@pytest.mark.parametrize("dtype", [np.float64, np.complex128, np.float32])
+def test_contract_blocked_path_across_cache_blocks_against_numpy(oracle, dtype):
+    # 700 x 1100 x 900: several blocks along every loop of the blocked kernel (with edge blocks that are not full),
+    # all threads at work -- the code path that produces the full-size references of the benchmark.  numpy's matmul (BLAS)
+    # is the independent check; f32 is compared with the f64 product rounded once.
+    rng = np.random.default_rng(91)
+    m, k, n = 700, 1100, 900
+    a = rng.standard_normal((m, k))
+    b = rng.standard_normal((k, n))
+    if np.issubdtype(dtype, np.complexfloating):
+        a = a + 1j * rng.standard_normal((m, k))
+        b = b + 1j * rng.standard_normal((k, n))
+    a, b = a.astype(dtype), b.astype(dtype)
+    c0 = rng.standard_normal((m, n)).astype(dtype)
+    wide = np.complex128 if np.issubdtype(dtype, np.complexfloating) else np.float64
+    want = 0.5 * (a.astype(wide) @ b.astype(wide)) - 1.5 * c0.astype(wide)
+    got = c0.copy()
+    oracle.contract(a, lab("mk"), b, lab("kn"), got, lab("mn"), alpha=0.5, beta=-1.5)
+    err = np.linalg.norm(got - want) / np.linalg.norm(want)
+    assert err < (2e-6 if dtype == np.float32 else 1e-14), err
+    # transposed storage of both operands and of the output (the packing routines' other branches)
+    got_t = np.asfortranarray(c0.copy())
+    oracle.contract(np.asfortranarray(a), lab("mk"), np.asfortranarray(b), lab("kn"), got_t, lab("mn"), alpha=0.5, beta=-1.5)
+    assert np.linalg.norm(got_t - want) / np.linalg.norm(want) < (2e-6 if dtype == np.float32 else 1e-14)
+
+
+def test_contract_benchmark_pattern_with_fused_groups_against_numpy(oracle):
+    # "ajbk,kcj->abc" with a = 16 (the f32 benchmark configuration at a quarter of its rows): fused row and k groups
+    # with different orders in the two operands, K = 12288 over many cache blocks; against numpy's einsum in f64
+    rng = np.random.default_rng(92)
+    a_, j, b_, k, c = 16, 128, 64, 96, 256
+    A = rng.standard_normal((a_, j, b_, k)).astype(np.float32)
+    B = rng.standard_normal((k, c, j)).astype(np.float32)
+    want = np.einsum("ajbk,kcj->abc", A.astype(np.float64), B.astype(np.float64), optimize=True)
+    got = np.empty((a_, b_, c), np.float32)
+    oracle.contract(A, lab("ajbk"), B, lab("kcj"), got, lab("abc"))
+    err = np.linalg.norm(got - want) / np.linalg.norm(want)
+    assert err < 2e-6, err   # f32 accumulation inside a cache block, f64 across blocks
