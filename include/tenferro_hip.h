@@ -293,9 +293,14 @@ int32_t tfh_stream_wait_event(tfh_stream s, tfh_event e);  /* chaining without a
  * launch count of one kind since the last enable, then forgets those records. */
 int32_t tfh_profile_enable(int32_t on);
 int32_t tfh_profile_collect(int32_t kind, double* total_ms, int32_t* launches);
+/* The same records by kernel, before tfh_profile_collect forgets them: the index-th distinct kernel (in order of its
+ * first launch) among the records of one kind, its label as tfh_last_kernel spells it, the summed duration and
+ * the number of its launches.  *launches == 0 and an empty name: index is past the last kernel. */
+int32_t tfh_profile_kernel(int32_t kind, int32_t index, char* name, size_t cap, double* total_ms, int32_t* launches);
 
-/* Diagnostic, no counterpart in the reference: the source-level name (template arguments as written in the
- * library) of the dominant kernel most recently launched by the calling thread, "" before the first one.
+/* Diagnostic, no counterpart in the reference: the name, in parentheses and with its template arguments as
+ * instantiated ("(gemm128_kernel<double, true, false, true, 1, 1, 128>)", what a kernel trace shows without namespaces
+ * and parameter list), of the dominant kernel most recently launched by the calling thread, "" before the first one.
  * Tests use it to check which kernel a call was routed to. */
 const char* tfh_last_kernel(void);
 

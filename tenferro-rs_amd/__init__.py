@@ -113,6 +113,7 @@ def lib():
         L.tfh_has_extension.argtypes = [C.c_int32, C.c_int32]
         L.tfh_profile_enable.argtypes = [C.c_int32]
         L.tfh_profile_collect.argtypes = [C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_int32)]
+        L.tfh_profile_kernel.argtypes = [C.c_int32, C.c_int32, C.c_char_p, C.c_size_t, C.POINTER(C.c_double), C.POINTER(C.c_int32)]
         L.tfh_last_kernel.restype = C.c_char_p
         L.tfh_last_kernel.argtypes = []
         L.tfh_subscripts_labels.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]
@@ -1022,3 +1023,16 @@ def profile_collect(kind):
     ms, n = C.c_double(), C.c_int32()
     _check(lib().tfh_profile_collect(kind, C.byref(ms), C.byref(n)))
     return ms.value, n.value
+
+
+def profile_kernels(kind):
+    """[(kernel label, total milliseconds, launches)] of one kind since profile_enable, by kernel, in order of first
+    launch (tfh_profile_kernel).  Call before profile_collect, which forgets the records."""
+    out = []
+    buf = C.create_string_buffer(512)
+    while True:
+        ms, n = C.c_double(), C.c_int32()
+        _check(lib().tfh_profile_kernel(kind, len(out), buf, 512, C.byref(ms), C.byref(n)))
+        if n.value == 0:
+            return out
+        out.append((buf.value.decode(), ms.value, n.value))

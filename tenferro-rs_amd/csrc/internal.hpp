@@ -158,7 +158,8 @@ struct ProfEvents {
     void* start = nullptr;
     void* stop = nullptr;
 };
-ProfEvents prof_take();
+// `name`: the label of the kernel that takes them, kept with the record (tfh_profile_kernel).
+ProfEvents prof_take(const char* name = nullptr);
 
 // Byte pointer of a view's element 0.
 inline char* view_ptr(const tfh_view& v, int dtype) { return (char*)v.base + v.offset * (int64_t)dtype_size(dtype); }

@@ -187,6 +187,7 @@ namespace {
 struct ProfRec {
     int kind;
     hipEvent_t a, b;
+    const char* name = "";   // label of the kernel that took the events (static storage)
 };
 std::mutex g_prof_mu;
 bool g_prof_on = false;
@@ -221,9 +222,17 @@ int prof_begin(int kind, void* stream) {
     g_prof.push_back(r);
     return (int)g_prof.size() - 1;
 }
-ProfEvents prof_take() {
+ProfEvents prof_take(const char* name) {
     ProfEvents e = t_pending;
     t_pending = ProfEvents{};
+    if (e.start && name) {
+        std::lock_guard<std::mutex> lk(g_prof_mu);
+        for (auto it = g_prof.rbegin(); it != g_prof.rend(); ++it)
+            if (it->a == (hipEvent_t)e.start) {
+                it->name = name;
+                break;
+            }
+    }
     return e;
 }
 void prof_end(int token, void* stream) {
@@ -277,6 +286,32 @@ int32_t tfh_profile_collect(int32_t kind, double* total_ms, int32_t* launches) {
     tfh::g_prof.swap(keep);
     *total_ms = total;
     *launches = n;
+    return TFH_OK;
+}
+
+int32_t tfh_profile_kernel(int32_t kind, int32_t index, char* name, size_t cap, double* total_ms, int32_t* launches) {
+    if (!name || !cap || !total_ms || !launches || index < 0) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer or negative index");
+    std::lock_guard<std::mutex> lk(tfh::g_prof_mu);
+    std::vector<const char*> names;   // distinct labels of this kind in order of first launch (labels are unique pointers per kernel)
+    for (auto& r : tfh::g_prof) {
+        if (r.kind != kind) continue;
+        bool seen = false;
+        for (const char* n : names) seen = seen || std::string(n) == r.name;
+        if (!seen) names.push_back(r.name);
+    }
+    name[0] = 0;
+    *total_ms = 0;
+    *launches = 0;
+    if ((size_t)index >= names.size()) return TFH_OK;
+    snprintf(name, cap, "%s", names[(size_t)index]);
+    for (auto& r : tfh::g_prof) {
+        if (r.kind != kind || std::string(r.name) != names[(size_t)index]) continue;
+        if (int32_t e = hip_check(hipEventSynchronize(r.b), "hipEventSynchronize")) return e;
+        float ms = 0;
+        if (int32_t e = hip_check(hipEventElapsedTime(&ms, r.a, r.b), "hipEventElapsedTime")) return e;
+        *total_ms += ms;
+        ++*launches;
+    }
     return TFH_OK;
 }
 
