@@ -24,6 +24,7 @@ namespace {
 constexpr int MAXT = 4;    // tile axes
 constexpr int MAXG = 16;   // grid axes
 constexpr int THREADS = 256;
+constexpr int MAXU = 16;   // accesses per thread and side in the large-tile variant
 
 struct CopyArgs {
     const void* in;
@@ -49,6 +50,17 @@ struct CopyArgs {
     int32_t g_text[MAXG];  // tile extent of that axis (1 if untiled)
     double alpha_re, alpha_im, beta_re, beta_im;
     int32_t conj, use_beta;
+    // large-tile variant: access u of a thread is at tile position (u * threads + tid) * vector length; the part of its
+    // offsets that depends on u alone (byte offsets on either side, LDS position of the written element) comes from the
+    // host, so a thread works out its own part once instead of sixteen times
+    uint32_t u_roff[MAXU], u_woff[MAXU];
+    int32_t u_wl[MAXU];
+    uint32_t walk_inc[4];   // mixed-radix digits of the block count (the distance between a block's successive tiles)
+    uint32_t walk_magic[4]; // floor(2^32 / g_count[g]): the first tile's digits by multiply-high instead of division
+    // byte strides of the tile axes in read and in write order and the rebase distances, all modulo 2^32 (in-tile
+    // offsets span less than 4 GiB, so wrapped 32-bit sums are exact): a thread's own part of its offsets in a dozen
+    // 32-bit multiply-adds
+    uint32_t r_sb[MAXT], w_sb[MAXT], in_rebase_b, out_rebase_b;
 };
 
 __device__ __forceinline__ int swz(int r) { return r + (r >> 5); }
@@ -91,6 +103,48 @@ __device__ __forceinline__ BlockOrigin block_origin(const CopyArgs& a, uint64_t 
     for (int t = 0; t < MAXT; ++t) o.lim[t] = uniform64(o.lim[t]);
     return o;
 }
+
+// The tiles a persistent block moves are gridDim.x apart.  Instead of decomposing every tile index by division (64-bit
+// divisions run on the vector unit, hundreds of cycles per grid axis between a barrier and the next tile's loads), the
+// block keeps the mixed-radix digits of its tile index and adds the digits of gridDim.x with carry: scalar adds and
+// compares only.  Digits fit 32 bits (the host takes the fast path only then).
+constexpr int WALKG = 4;   // grid axes the walk handles (the host checks)
+struct TileWalk {   // (grid axes past a.ng have count 1 and stride 0 on the host side: no conditions in here)
+    uint32_t c[WALKG], inc[WALKG];
+    __device__ __forceinline__ void start(const CopyArgs& a, uint32_t first) {
+#pragma unroll
+        for (int g = 0; g < WALKG; ++g) {
+            // n >= 1: mulhi(first, floor(2^32 / n)) is the quotient or one less
+            const uint32_t n = (uint32_t)a.g_count[g];
+            uint32_t q = __umulhi(first, a.walk_magic[g]), rem = first - q * n;
+            if (rem >= n) {
+                ++q;
+                rem -= n;
+            }
+            c[g] = rem;
+            first = q;
+            inc[g] = a.walk_inc[g];
+        }
+    }
+    __device__ __forceinline__ void advance(const CopyArgs& a) {
+        uint32_t carry = 0;
+#pragma unroll
+        for (int g = 0; g < WALKG; ++g) {
+            const uint32_t n = (uint32_t)a.g_count[g];
+            const uint32_t v = c[g] + inc[g] + carry;   // < 2 n
+            carry = v >= n ? 1u : 0u;
+            c[g] = v >= n ? v - n : v;
+        }
+    }
+    __device__ __forceinline__ void offsets(const CopyArgs& a, int64_t& in, int64_t& out) const {
+        in = out = 0;
+#pragma unroll
+        for (int g = 0; g < WALKG; ++g) {
+            in += (int64_t)c[g] * a.g_si[g];
+            out += (int64_t)c[g] * a.g_so[g];
+        }
+    }
+};
 
 // ---- element operations -----------------------------------------------------------------------------
 template <class V>
@@ -178,8 +232,12 @@ __device__ __forceinline__ void store_stream(void* p, const P& x) {
 // Interior tiles take a fast path: the in-tile byte offsets and LDS positions of each thread's accesses are
 // computed once (32-bit) and reused for every tile against a uniform per-tile base; edge tiles and tensors
 // whose tiles span 4 GiB recompute coordinates with bounds checks.
-template <class V, class Op, int EPT, int VR, int VW, bool READ_OLD, bool FAST>
-__global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
+// FULL (with FAST): the tile has exactly EPT * NTH elements, so no access is masked and the tile loop is straight-line
+// code.  With per-access masks every load sits in its own conditional block; the compiler then cannot tell that the
+// previous tile's loads have completed and makes each load of the next tile wait for the one before it.
+template <class V, class Op, int EPT, int VR, int VW, bool READ_OLD, bool FAST, int NTH = THREADS, bool FULL = false>
+__global__ void __launch_bounds__(NTH) copy_kernel(CopyArgs a, Op op) {
+    prefetch_kernel_arguments<sizeof(CopyArgs)>();
     extern __shared__ __align__(16) unsigned char smem_raw[];
     V* lds = reinterpret_cast<V*>(smem_raw);
     constexpr int NR = EPT / VR, NW = EPT / VW;
@@ -188,37 +246,70 @@ __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
     uint32_t roff[FAST ? NR : 1], woff[FAST ? NW : 1];
     int wl[FAST ? NW : 1];
     uint32_t rmask = 0, wmask = 0;
+    if constexpr (FULL) {
+        static_assert(NR <= MAXU && NW <= MAXU, "the host provides MAXU per-access offsets");
+        // tile coordinates are bit fields of the tile position, and the position splits into disjoint bits from the
+        // thread and from u: offsets are sums of a per-thread part (here) and a per-u part (from the host)
+        const int r0 = tid * VR;
+        uint32_t mine = 0u - a.in_rebase_b;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t) mine += (uint32_t)((r0 >> a.r_shift[t]) & a.r_mask[t]) * a.r_sb[t];
+#pragma clang loop unroll(full)
+        for (int u = 0; u < NR; ++u) roff[u] = mine + a.u_roff[u];
+    } else {
 #pragma clang loop unroll(full)
     for (int u = 0; u < (FAST ? NR : 0); ++u) {
-        const int r = (u * THREADS + tid) * VR;
+        const int r = (u * NTH + tid) * VR;
         int64_t off = 0;
 #pragma unroll
         for (int t = 0; t < MAXT; ++t) off += (int64_t)((r >> a.r_shift[t]) & a.r_mask[t]) * a.r_si[t];
         roff[u] = (uint32_t)((off - a.in_rebase) * (int64_t)sizeof(V));
         rmask |= (r < a.tile_elems ? 1u : 0u) << u;
     }
-#pragma clang loop unroll(full)
-    for (int u = 0; u < (FAST ? NW : 0); ++u) {
-        const int w = (u * THREADS + tid) * VW;
-        int64_t off = 0;
+    }
+    if constexpr (FULL) {
+        const int w0 = tid * VW;
+        uint32_t mine = 0u - a.out_rebase_b;
         int r = 0;
 #pragma unroll
         for (int t = 0; t < MAXT; ++t) {
-            const int c = (w >> a.w_shift[t]) & a.w_mask[t];
-            off += (int64_t)c * a.w_so[t];
+            const int c = (w0 >> a.w_shift[t]) & a.w_mask[t];
+            mine += (uint32_t)c * a.w_sb[t];
             r += c * a.w_rpos[t];
         }
-        woff[u] = (uint32_t)((off - a.out_rebase) * (int64_t)sizeof(V));
-        wl[u] = r;
-        wmask |= (w < a.tile_elems ? 1u : 0u) << u;
+#pragma clang loop unroll(full)
+        for (int u = 0; u < NW; ++u) {
+            woff[u] = mine + a.u_woff[u];
+            wl[u] = r + a.u_wl[u];
+        }
+    } else {
+#pragma clang loop unroll(full)
+        for (int u = 0; u < (FAST ? NW : 0); ++u) {
+            const int w = (u * NTH + tid) * VW;
+            int64_t off = 0;
+            int r = 0;
+#pragma unroll
+            for (int t = 0; t < MAXT; ++t) {
+                const int c = (w >> a.w_shift[t]) & a.w_mask[t];
+                off += (int64_t)c * a.w_so[t];
+                r += c * a.w_rpos[t];
+            }
+            woff[u] = (uint32_t)((off - a.out_rebase) * (int64_t)sizeof(V));
+            wl[u] = r;
+            wmask |= (w < a.tile_elems ? 1u : 0u) << u;
+        }
     }
 
     auto load = [&](const BlockOrigin& o) {
         if constexpr (FAST) {
-            const gcptr base = (gcptr)(uintptr_t)(reinterpret_cast<const V*>(a.in) + o.in + a.in_rebase);
+            // the complete tile base goes through readfirstlane: an opaque scalar that the optimiser cannot split up again
+            // (it otherwise hoists "input pointer + thread offset" out of the tile loop as 64-bit vector addresses, adds the
+            // tile origin to each on the vector unit, and lets those address registers share the loads' destinations, so
+            // that every load of the next tile waits for the previous one)
+            const gcptr base = (gcptr)(uintptr_t)uniform64((int64_t)(uintptr_t)(reinterpret_cast<const V*>(a.in) + o.in + a.in_rebase));
 #pragma clang loop unroll(full)
             for (int u = 0; u < NR; ++u) {
-                if ((rmask >> u) & 1u) {
+                if (FULL || ((rmask >> u) & 1u)) {
                     const Pack<V, VR> p = gload_pack<Pack<V, VR>>(base, roff[u]);
 #pragma unroll
                     for (int j = 0; j < VR; ++j) regs[u * VR + j] = p.v[j];
@@ -231,7 +322,7 @@ __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
         const V* in = reinterpret_cast<const V*>(a.in) + o.in;
 #pragma clang loop unroll(full)
         for (int u = 0; u < NR; ++u) {
-            const int r = (u * THREADS + tid) * VR;
+            const int r = (u * NTH + tid) * VR;
             bool ok = r < a.tile_elems;
             int64_t off = 0;
 #pragma unroll
@@ -250,13 +341,25 @@ __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
     };
     uint64_t tile = blockIdx.x;
     if (tile >= (uint64_t)a.ntiles) return;
-    BlockOrigin o = block_origin(a, tile);
+    BlockOrigin o;
+    o.in = o.in2 = o.out = 0;
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) o.lim[t] = 0;   // (the straight-line variant never looks at lim)
+    TileWalk walk;
+    if constexpr (FULL) {
+        walk.start(a, (uint32_t)tile);
+        walk.offsets(a, o.in, o.out);
+    } else {
+        o = block_origin(a, tile);
+    }
     load(o);
+    // (nothing that the tile loop needs later -- LDS positions, write offsets -- is to be computed ahead of these loads)
+    if constexpr (FULL) __builtin_amdgcn_sched_barrier(0);
     for (;;) {
 #pragma clang loop unroll(full)
         for (int u = 0; u < NR; ++u) {
-            const int r = (u * THREADS + tid) * VR;
-            if (FAST ? (bool)((rmask >> u) & 1u) : r < a.tile_elems) {
+            const int r = (u * NTH + tid) * VR;
+            if (FULL || (FAST ? (bool)((rmask >> u) & 1u) : r < a.tile_elems)) {
 #pragma unroll
                 for (int j = 0; j < VR; ++j) lds[swz(r) + j] = regs[u * VR + j];
             }
@@ -266,14 +369,19 @@ __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
         const bool more = next < (uint64_t)a.ntiles;
         BlockOrigin o2 = o;
         if (more) {
-            o2 = block_origin(a, next);
+            if constexpr (FULL) {
+                walk.advance(a);
+                walk.offsets(a, o2.in, o2.out);
+            } else {
+                o2 = block_origin(a, next);
+            }
             load(o2);
         }
         if constexpr (FAST) {
-            const gmptr base = (gmptr)(uintptr_t)(reinterpret_cast<V*>(a.out) + o.out + a.out_rebase);
+            const gmptr base = (gmptr)(uintptr_t)uniform64((int64_t)(uintptr_t)(reinterpret_cast<V*>(a.out) + o.out + a.out_rebase));
 #pragma clang loop unroll(full)
             for (int u = 0; u < NW; ++u) {
-                if ((wmask >> u) & 1u) {
+                if (FULL || ((wmask >> u) & 1u)) {
                     Pack<V, VW> x, old;
 #pragma unroll
                     for (int j = 0; j < VW; ++j) x.v[j] = lds[swz(wl[u] + j * a.w_rpos[0])];
@@ -289,7 +397,7 @@ __global__ void __launch_bounds__(THREADS) copy_kernel(CopyArgs a, Op op) {
             asm volatile("" : "+v"(tid));
 #pragma clang loop unroll(full)
             for (int u = 0; u < NW; ++u) {
-                const int w = (u * THREADS + tid) * VW;
+                const int w = (u * NTH + tid) * VW;
                 bool ok = w < a.tile_elems;
                 int64_t off = 0;
                 int r = 0;
@@ -454,6 +562,7 @@ __global__ void __launch_bounds__(THREADS) fill_kernel(CopyArgs a, V value, int 
 
 template <class R, bool CX>
 __global__ void __launch_bounds__(THREADS) emul_kernel(CopyArgs a, int ept) {
+    prefetch_kernel_arguments<sizeof(CopyArgs)>();
     constexpr int NC = CX ? 2 : 1;
     const BlockOrigin o = block_origin(a, (uint64_t)blockIdx.x + (uint64_t)blockIdx.y * gridDim.x);
     const R* A = reinterpret_cast<const R*>(a.in) + o.in * NC;
@@ -509,7 +618,10 @@ struct TilePlan {
 
 // axes: s[0] = input stride, s[1] = output stride, s[2] = second input stride (emul only).
 // order_slot: which slot defines the read order (0) -- the write order is always slot 1.
-int32_t plan_tiles(std::vector<Axis> axes, int elem_bytes, int max_tile_elems, bool two_sided, TilePlan& tp) {
+// grow_side / grow_log2: after the tile is chosen within max_tile_elems, the run of one side (0 = input, 1 = output) is
+// lengthened by up to grow_log2 more doublings (the large-tile variant of the copy kernel).
+int32_t plan_tiles(std::vector<Axis> axes, int elem_bytes, int max_tile_elems, bool two_sided, TilePlan& tp, int grow_side = -1,
+                   int grow_log2 = 0) {
     CopyArgs& a = tp.args;
     std::memset(&a, 0, sizeof a);
     for (auto& x : axes)
@@ -579,6 +691,21 @@ int32_t plan_tiles(std::vector<Axis> axes, int elem_bytes, int max_tile_elems, b
                 }
             }
             if (!grew) break;
+        }
+        if (grow_side >= 0) {
+            const std::vector<int>& order = grow_side == 1 ? out_order : in_order;
+            for (int more = 0; more < grow_log2; ++more) {
+                bool grew = false;
+                for (int i : order) {
+                    if (tl[i] < full(i) && (tl[i] > 0 || tile_axes() < MAXT)) {
+                        ++tl[i];
+                        grew = true;
+                        break;
+                    }
+                    if (tl[i] < ceil_log2(axes[i].n)) break;
+                }
+                if (!grew) break;
+            }
         }
     };
     for (int i = 0; i < na; ++i) capped = capped || (axes[i].n & (axes[i].n - 1)) != 0;
@@ -667,6 +794,7 @@ int32_t plan_tiles(std::vector<Axis> axes, int elem_bytes, int max_tile_elems, b
             a.g_text[g] = (int32_t)text;
             blocks *= (uint64_t)cnt;
         }
+    for (int g = a.ng; g < MAXG; ++g) a.g_count[g] = 1;   // neutral: the kernels' unconditional tile walk relies on it
     a.ntiles = (int64_t)blocks;
     // 4 resident blocks per CU on 256 CUs; block counts from 512 to 4096 measure within 2% of each other
     tp.persistent = (uint32_t)std::min<uint64_t>(blocks, 1024);
@@ -704,6 +832,49 @@ void set_scalars(CopyArgs& a, Scalar alpha, Scalar beta, bool conj) {
     a.beta_im = beta.im;
     a.conj = conj;
     a.use_beta = !beta.is_zero();
+}
+
+// Large tiles (raw moves only): 512 threads move a tile of 32 elements per thread (128 KB of 8-byte elements), one block
+// per CU.  Every tile is full and both sides take 16-byte accesses.
+template <class V, int EPT>
+void launch_copy_large(TilePlan& tp, size_t lds, hipStream_t st) {
+    constexpr int VEC = 16 / sizeof(V);
+    {   // the per-u parts of the offsets (see CopyArgs)
+        CopyArgs& a = tp.args;
+        uint32_t step = tp.persistent;
+        for (int g = 0; g < WALKG; ++g) {
+            a.walk_inc[g] = step % (uint32_t)a.g_count[g];
+            step /= (uint32_t)a.g_count[g];
+            a.walk_magic[g] = a.g_count[g] <= 1 ? 0xffffffffu : (uint32_t)(((uint64_t)1 << 32) / (uint64_t)a.g_count[g]);
+        }
+        for (int t = 0; t < MAXT; ++t) {
+            a.r_sb[t] = (uint32_t)(a.r_si[t] * (int64_t)sizeof(V));
+            a.w_sb[t] = (uint32_t)(a.w_so[t] * (int64_t)sizeof(V));
+        }
+        a.in_rebase_b = (uint32_t)(a.in_rebase * (int64_t)sizeof(V));
+        a.out_rebase_b = (uint32_t)(a.out_rebase * (int64_t)sizeof(V));
+        for (int u = 0; u < EPT / VEC; ++u) {
+            const int pos = u * 512 * VEC;
+            int64_t offr = 0, offw = 0;
+            int rp = 0;
+            for (int t = 0; t < MAXT; ++t) {
+                offr += (int64_t)((pos >> a.r_shift[t]) & a.r_mask[t]) * a.r_si[t];
+                const int c = (pos >> a.w_shift[t]) & a.w_mask[t];
+                offw += (int64_t)c * a.w_so[t];
+                rp += c * a.w_rpos[t];
+            }
+            a.u_roff[u] = (uint32_t)(offr * (int64_t)sizeof(V));
+            a.u_woff[u] = (uint32_t)(offw * (int64_t)sizeof(V));
+            a.u_wl[u] = rp;
+        }
+    }
+    static bool once = [] {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&copy_kernel<V, RawOp<V>, EPT, VEC, VEC, false, true, 512, true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        return true;
+    }();
+    (void)once;
+    TFH_LAUNCH_TIMED((copy_kernel<V, RawOp<V>, EPT, VEC, VEC, false, true, 512, true>), dim3(tp.persistent), dim3(512), lds, st, tp.args, RawOp<V>());
 }
 
 template <class V, class Op, int EPT, int VR, int VW>
@@ -938,6 +1109,36 @@ int32_t launch_copy(int dtype, const void* in, void* out, std::vector<Axis> axes
     if (raw) {
         int32_t st_tab = TFH_OK;
         if (try_table_copy(eb, in, out, axes, tp, stream, st_tab)) return st_tab;
+        // Large tiles.  When the rows a tile touches on one side lie far apart (an axis that is contiguous on one side
+        // and the slowest on the other: strides of megabytes inside every tile), 512-byte runs on that side cost 10-17 %
+        // of the rate; four times the tile, spent on that side's run alone (2 KB), gets most of it back.
+        if (tp.all_full && ((vin && vout) || eb == 16) && tp.args.tile_elems == max_tile) {
+            int64_t far_[2] = {0, 0};
+            for (int t = 0; t < tp.args.nt; ++t) {
+                far_[0] = std::max<int64_t>(far_[0], std::llabs(tp.args.r_si[t]) * eb);
+                far_[1] = std::max<int64_t>(far_[1], std::llabs(tp.args.w_so[t]) * eb);
+            }
+            const int side = far_[1] >= far_[0] ? 1 : 0;
+            const bool want = far_[side] >= ((int64_t)1 << 20);
+            TilePlan big;
+            if (want && plan_tiles(axes, eb, max_tile, true, big, side, 2) == TFH_OK && big.all_full && ((big.vec_in && big.vec_out) || eb == 16) &&
+                big.args.tile_elems == 4 * max_tile && big.args.ntiles >= 256 && big.args.ntiles < ((int64_t)1 << 30) && big.args.ng <= WALKG) {
+                big.args.in = in;
+                big.args.out = out;
+                set_scalars(big.args, alpha, beta, conj);
+                big.persistent = (uint32_t)std::min<int64_t>(big.args.ntiles, 256);
+                const size_t lds = (size_t)(big.args.tile_elems + big.args.tile_elems / 32 + 4) * eb;
+                const int prof = prof_begin(PROF_COPY, st);
+                switch (eb) {
+                    case 4: launch_copy_large<uint32_t, 32>(big, lds, st); break;
+                    case 8: launch_copy_large<uint64_t, 32>(big, lds, st); break;
+                    default: launch_copy_large<double2, 16>(big, lds, st); break;
+                }
+                prof_end(prof, st);
+                return hip_check(hipGetLastError(), "copy kernel launch");
+            }
+            clear_error();
+        }
         switch (eb) {
             case 4: return run_copy<uint32_t, RawOp<uint32_t>, true>(tp, RawOp<uint32_t>(), false, vin, vout, st);
             case 8: return run_copy<uint64_t, RawOp<uint64_t>, true>(tp, RawOp<uint64_t>(), false, vin, vout, st);

@@ -61,6 +61,7 @@ __device__ __forceinline__ RVec<R, N> load_stream(const R* p) {
 // KV: A's contiguous axis is kept (VEC outputs per lane).  BB: B has stride 0 along that axis.  CX: complex product.
 template <class R, int VEC, bool KV, bool BB, bool CX>
 __global__ void __launch_bounds__(THREADS) dot_fast_kernel(DotArgs a) {
+    prefetch_kernel_arguments<sizeof(DotArgs)>();
     constexpr int NV = CX ? 2 : (KV ? VEC : 1);   // accumulators per lane (complex: re, im)
     constexpr int LV = CX ? 2 : VEC;              // components per load of A
     constexpr int LB = CX ? 2 : (BB ? 1 : VEC);   // components per load of B

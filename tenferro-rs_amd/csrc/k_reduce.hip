@@ -116,12 +116,13 @@ __device__ __forceinline__ ThreadPos thread_pos(const ReduceArgs& a, int tid) {
 // DOT: the reduced quantity is the product A * B of two operands read at the same coordinates (sum only).
 template <class R, bool CX, bool DOT = false>
 __global__ void __launch_bounds__(THREADS) reduce_kernel(ReduceArgs a) {
+    prefetch_kernel_arguments<sizeof(ReduceArgs)>();
     constexpr int NC = CX ? 2 : 1;
     __shared__ double lds[THREADS * NC];
     const ThreadPos p = thread_pos(a, threadIdx.x);
     const R* A = reinterpret_cast<const R*>(a.in) + p.in * NC;
     const R* B = DOT ? reinterpret_cast<const R*>(a.in_b) + p.in_b * NC : nullptr;
-    const int op = a.op;
+    const int op = DOT ? (int)TFH_REDUCE_SUM : a.op;   // (a product reduction is always a sum: the selects fold away)
     double acc_re = identity(op), acc_im = 0.0;
     // this block's slice of the serial reduced range
     const int64_t per = (a.r_total + a.nchunks - 1) / a.nchunks;
@@ -351,7 +352,21 @@ struct FastReduceArgs {
     double* partial;          // [nchunks][nblocks][THREADS][NV]
     int64_t vc_stride;        // C stride between the VEC outputs of one lane (KV)
     double alpha, beta;
+    // floor(2^32 / n) for every grid count and for r_total: division by a launch constant as a multiply-high and one
+    // correction step on the scalar unit (a 32-bit division costs ~25 vector instructions in every wave, and with eight
+    // blocks per CU all starting at once every instruction before the first load is time the memory system idles)
+    uint32_t g_magic[MAXG], rot_magic;
 };
+// n >= 1, x < 2^32: the quotient estimate mulhi(x, floor(2^32 / n)) is the quotient or one less
+__device__ __forceinline__ uint32_t div_magic(uint32_t x, uint32_t n, uint32_t magic, uint32_t& rem) {
+    uint32_t q = __umulhi(x, magic);
+    rem = x - q * n;
+    if (rem >= n) {
+        ++q;
+        rem -= n;
+    }
+    return q;
+}
 
 template <class R, int N>
 struct alignas(sizeof(R) * N) RVec {
@@ -367,8 +382,11 @@ __device__ __forceinline__ RVec<R, N> load_stream(const R* p) {
     return __builtin_bit_cast(RVec<R, N>, __builtin_nontemporal_load(reinterpret_cast<const Raw*>(p)));
 }
 
-template <class R, int VEC, bool KV, int KS, bool BF>
+// SUM: the operation is known to be a sum (otherwise it is a.op at run time, and every element pays for an add, a
+// max, a min and the selects between them: ten f64 instructions per 16 bytes loaded instead of two)
+template <class R, int VEC, bool KV, int KS, bool BF, bool SUM = false>
 __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) {
+    prefetch_kernel_arguments<sizeof(FastReduceArgs)>();
     constexpr int NV = KV ? VEC : 1;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     int64_t* rtab = reinterpret_cast<int64_t*>(smem_raw);                               // [r_total]
@@ -377,16 +395,27 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
     const int r_begin = a.mode == 1 ? (int)blockIdx.y * a.rps : 0;
     const int r_count = a.mode == 2 ? 0 : (a.mode == 1 ? (a.r_total - r_begin < a.rps ? a.r_total - r_begin : a.rps) : a.r_total);
     // (a split reduction rotates every chunk by its own number: the chunks run in step as well, a power of two apart)
-    int rot = a.rot_shift >= 0 && a.mode == 0 ? (int)((blockIdx.x >> a.rot_shift) % (uint32_t)r_count) : 0;
+    int rot = 0;
+    if (a.rot_shift >= 0 && a.mode == 0) {
+        uint32_t rem;
+        (void)div_magic(blockIdx.x >> a.rot_shift, (uint32_t)r_count, a.rot_magic, rem);
+        rot = (int)rem;
+    }
     if (a.mode == 1 && r_count > 0) rot = (int)(blockIdx.y % (uint32_t)r_count);
     for (int i = tid; i < r_count; i += THREADS) {
-        int64_t lin = r_begin + (i + rot >= r_count ? i + rot - r_count : i + rot), off = 0;
+        // (the serial range is at most FAST_MAX_RTAB long: 32-bit arithmetic, and the outermost axis takes what is left)
+        uint32_t lin = (uint32_t)(r_begin + (i + rot >= r_count ? i + rot - r_count : i + rot));
+        int64_t off = 0;
 #pragma unroll
         for (int r = 0; r < MAXR; ++r)
             if (r < a.nr) {
-                int64_t q = lin / a.r_count[r];
-                off += (lin - q * a.r_count[r]) * a.r_sa[r];
-                lin = q;
+                if (r + 1 < a.nr) {
+                    const uint32_t n = (uint32_t)a.r_count[r], q = lin / n;
+                    off += (int64_t)(lin - q * n) * a.r_sa[r];
+                    lin = q;
+                } else {
+                    off += (int64_t)lin * a.r_sa[r];
+                }
             }
         rtab[i] = off;
     }
@@ -395,11 +424,10 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
     {
         uint32_t bid = blockIdx.x;   // the grid (and so every count) is below 2^31
         for (int g = 0; g < a.ng; ++g) {
-            const uint32_t n = (uint32_t)a.g_count[g], q = bid / n;
-            const int64_t c = (int64_t)(bid - q * n);
-            bid = q;
-            org_in += c * a.g_sa[g];
-            org_out += c * a.g_sc[g];
+            uint32_t c;
+            bid = div_magic(bid, (uint32_t)a.g_count[g], a.g_magic[g], c);
+            org_in += (int64_t)c * a.g_sa[g];
+            org_out += (int64_t)c * a.g_sc[g];
         }
     }
     int64_t toff_in = 0, toff_out = 0;
@@ -411,7 +439,7 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
         if (a.t_red[t]) writer &= c == 0;
         else toff_out += (int64_t)c * a.t_sc[t];
     }
-    const int op = a.op;
+    const int op = SUM ? (int)TFH_REDUCE_SUM : a.op;
     __syncthreads();
     const R* A = reinterpret_cast<const R*>(a.in) + org_in + toff_in;
     double acc[KS][NV];
@@ -577,19 +605,24 @@ __global__ void __launch_bounds__(THREADS) reduce_fast_kernel(FastReduceArgs a) 
     }
 }
 
-template <class R, int VEC, bool KV>
-void launch_fast_ks(const FastReduceArgs& fa, dim3 grid, int ks, bool bf, hipStream_t st) {
+template <class R, int VEC, bool KV, bool SUM>
+void launch_fast_op(const FastReduceArgs& fa, dim3 grid, int ks, bool bf, hipStream_t st) {
     const int nv = KV ? VEC : 1;
     if (ks == 8 && bf) {
         size_t lds = FAST_MAX_RTAB * sizeof(int64_t) + (size_t)nv * THREADS * sizeof(double);
-        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 8, true>), grid, dim3(THREADS), lds, st, fa);
+        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 8, true, SUM>), grid, dim3(THREADS), lds, st, fa);
     } else if (ks == 8) {
         size_t lds = FAST_MAX_RTAB * sizeof(int64_t) + (size_t)8 * nv * THREADS * sizeof(double);
-        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 8, false>), grid, dim3(THREADS), lds, st, fa);
+        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 8, false, SUM>), grid, dim3(THREADS), lds, st, fa);
     } else {
         size_t lds = FAST_MAX_RTAB * sizeof(int64_t) + (size_t)nv * THREADS * sizeof(double);
-        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 1, false>), grid, dim3(THREADS), lds, st, fa);
+        TFH_LAUNCH_TIMED((reduce_fast_kernel<R, VEC, KV, 1, false, SUM>), grid, dim3(THREADS), lds, st, fa);
     }
+}
+template <class R, int VEC, bool KV>
+void launch_fast_ks(const FastReduceArgs& fa, dim3 grid, int ks, bool bf, hipStream_t st) {
+    if (fa.op == TFH_REDUCE_SUM) launch_fast_op<R, VEC, KV, true>(fa, grid, ks, bf, st);
+    else launch_fast_op<R, VEC, KV, false>(fa, grid, ks, bf, st);
 }
 template <class R>
 void launch_fast(const FastReduceArgs& fa, dim3 grid, int vec, bool kv, int ks, bool bf, hipStream_t st) {
@@ -719,7 +752,6 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
         fa.g_sc[0] *= 8;
         blocks /= 8;
     }
-
     fa.r_total = (int32_t)r_total;
     // A serial axis with a kept axis outside it (sum over a middle axis): the blocks of the launch run in step, so at
     // any moment they would all read the same serial index -- addresses that differ by the outer axis's stride, a large
@@ -738,6 +770,9 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
         // (serial steps of at least 32 KB: shorter ones measured within 2 % either way)
         if (grid_max > serial_min && serial_min * rbytes >= 32768) fa.rot_shift = 5;
     }
+    auto magic_of = [](int64_t n) { return n <= 1 ? 0xffffffffu : (uint32_t)(((uint64_t)1 << 32) / (uint64_t)n); };
+    for (int g = 0; g < fa.ng; ++g) fa.g_magic[g] = magic_of(fa.g_count[g]);
+    fa.rot_magic = magic_of(r_total);
     fa.in = a;
     fa.out = c;
     fa.op = reduce_op;

@@ -51,6 +51,25 @@ def contraction_within_tolerance(x, ref, dtype, scale, k):
     return d <= 2 * ops * (k + 2) * u * np.linalg.norm(np.asarray(scale).ravel())
 
 
+def copy_kernel_is_fast(label):
+    """Whether a copy_kernel label names the variant without bounds checks: the seventh template argument of
+    copy_kernel<V, Op, EPT, VR, VW, READ_OLD, FAST, threads, FULL>."""
+    assert label.startswith("(copy_kernel<"), label
+    args, depth, cur = [], 0, ""
+    for ch in label[len("(copy_kernel<"):-2]:
+        if ch == "<":
+            depth += 1
+        elif ch == ">":
+            depth -= 1
+        if ch == "," and depth == 0:
+            args.append(cur.strip())
+            cur = ""
+        else:
+            cur += ch
+    args.append(cur.strip())
+    return args[6] == "true"
+
+
 def dev(tf, arr):
     """Device Tensor with the same dims, element strides and offset as the numpy view `arr`."""
     import torch
@@ -619,6 +638,30 @@ def _permute_check(tf, oracle, a, perm, alpha=1.0, beta=0.0, b0=None):
     return out.to_numpy(), ref
 
 
+@pytest.mark.parametrize("dtype,shape", [(np.float32, (16,) * 6), (np.float64, (16, 16, 16, 16, 16, 8)), (np.complex128, (16, 16, 16, 8, 16, 8)),
+                                         (np.float64, (4, 16, 16, 16, 16, 16))])
+def test_permute_large_tiles_for_far_apart_rows_bit_exact(tf, oracle, dtype, shape):
+    # an axis that is contiguous on one side and the slowest on the other: every tile touches rows megabytes apart,
+    # and the copy takes the large-tile variant (512 threads, four times the tile, the longer run on the scattered
+    # side).  Bit-exact against numpy's transpose; the identity and a near-identity stay on the ordinary tiles.
+    rng = np.random.default_rng(44)
+    a = rand(rng, shape, dtype)
+    da = dev(tf, a)
+    large = 0
+    for perm in [(5, 2, 0, 4, 1, 3), (1, 2, 3, 4, 5, 0), (2, 4, 1, 5, 3, 0), (5, 0, 1, 2, 3, 4), (0, 1, 2, 3, 4, 5), (0, 1, 2, 5, 3, 4)]:
+        oshape = [shape[p] for p in perm]
+        out = tf.Tensor.empty(oshape, tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Permute(list(range(6)), list(perm)), [shape, oshape])
+        tf.HipBackend.execute(plan, 1.0, [da], 0.0, out)
+        label = tf.last_kernel()
+        is_large = label.endswith("512, true>)")
+        large += is_large
+        assert out.to_numpy().tobytes() == np.ascontiguousarray(a.transpose(perm)).tobytes(), (perm, label)
+        if perm in [(0, 1, 2, 3, 4, 5), (0, 1, 2, 5, 3, 4)]:
+            assert not is_large, (perm, label)
+    assert large >= 2, large
+
+
 @pytest.mark.parametrize("dtype", ALL)
 def test_permute_power_of_two_shapes_take_the_vector_path(tf, oracle, dtype):
     # every tile full, contiguous fastest axes on both sides: 16-byte accesses, no bounds checks
@@ -626,7 +669,7 @@ def test_permute_power_of_two_shapes_take_the_vector_path(tf, oracle, dtype):
     a = rand(rng, (32, 8, 64, 16), dtype)
     for perm in [(3, 1, 0, 2), (0, 1, 2, 3), (2, 3, 0, 1), (1, 0, 3, 2)]:
         got, ref = _permute_check(tf, oracle, a, perm)
-        assert tf.last_kernel().startswith("(copy_kernel") and tf.last_kernel().endswith("true>)"), tf.last_kernel()   # FAST
+        assert copy_kernel_is_fast(tf.last_kernel()), tf.last_kernel()
         assert got.tobytes() == ref.tobytes(), perm
     b0 = rand(rng, (16, 8, 32, 64), dtype)
     alpha, beta = (0.5 - 2j, 1.5 + 1j) if np.issubdtype(dtype, np.complexfloating) else (0.5, -1.5)
@@ -643,7 +686,7 @@ def test_permute_misaligned_base_and_odd_inner_extent(tf, oracle):
     assert got.tobytes() == ref.tobytes()
     b = rng.standard_normal((64, 30, 17))            # partial tiles on every axis
     got, ref = _permute_check(tf, oracle, b, (2, 1, 0))
-    assert tf.last_kernel().startswith("(copy_kernel") and tf.last_kernel().endswith("false>)"), tf.last_kernel()      # bounds-checked
+    assert not copy_kernel_is_fast(tf.last_kernel()), tf.last_kernel()      # bounds-checked
     assert got.tobytes() == ref.tobytes()
 
 
@@ -892,7 +935,7 @@ def test_permute_extents_with_divisor_tiles(tf, oracle, dtype):
         got, ref = _permute_check(tf, oracle, a, perm)
         assert got.tobytes() == ref.tobytes(), (shape, perm)
         if np.dtype(dtype).itemsize >= 8:
-            assert tf.last_kernel().endswith("true>)") == fast, (shape, perm, tf.last_kernel())
+            assert copy_kernel_is_fast(tf.last_kernel()) == fast, (shape, perm, tf.last_kernel())
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex128])
@@ -1362,7 +1405,7 @@ def test_reduce_rows_and_inner_axes_take_the_butterfly_fold(tf, oracle, dtype):
         a = ints(shape)
         got, ref = _reduce_check(tf, oracle, a, ma, mc, tf.ReduceOp.Sum, oracle.SUM)
         if dtype == np.float64:      # (the other element sizes tile these shapes differently; they are checked for their results)
-            assert "8, true>" in tf.last_kernel(), (shape, tf.last_kernel())
+            assert ", 8, true, " in tf.last_kernel(), (shape, tf.last_kernel())
         assert np.array_equal(got, ref), shape
     a = rand(rng, (32768, 256), dtype)
     c0 = rand(rng, (32768,), dtype)
@@ -1371,7 +1414,7 @@ def test_reduce_rows_and_inner_axes_take_the_butterfly_fold(tf, oracle, dtype):
     if not cplx:
         for op_tf, op_or in [(tf.ReduceOp.Max, oracle.MAX), (tf.ReduceOp.Min, oracle.MIN)]:
             got, ref = _reduce_check(tf, oracle, a, [0, 1], [0], op_tf, op_or)
-            assert dtype != np.float64 or "8, true>" in tf.last_kernel()
+            assert dtype != np.float64 or ", 8, true, " in tf.last_kernel()
             assert np.array_equal(got, ref)
 
 
