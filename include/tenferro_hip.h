@@ -271,9 +271,19 @@ int32_t tfh_set_device(int32_t device_id);
 /* DataBuffer::Hip storage (tenferro-tensor/src/lib.rs:133-137). */
 int32_t tfh_malloc(size_t bytes, void** out);
 int32_t tfh_free(void* ptr);
-int32_t tfh_memcpy_h2d(void* dst, const void* src, size_t bytes, tfh_stream stream);   /* to_memory_space_async, :660-671 */
+/* Tensor::to_memory_space_async (tenferro-tensor/src/lib.rs:660-671).  Host memory from tfh_host_malloc (page-locked)
+ * is copied by the copy engine directly and the call returns at once; the transfer is complete when work enqueued on
+ * `stream` after it runs (record an event).  Ordinary (pageable) host memory goes through two 16 MiB pinned staging
+ * buffers of the stream, in chunks, the host filling or emptying one while the engine works on the other: the call
+ * returns when the host side is done -- host-to-device: the source may be reused, the last chunk is on its way in
+ * stream order; device-to-host: the data is in `dst`.  Either way the transfer runs beside kernels of other streams. */
+int32_t tfh_memcpy_h2d(void* dst, const void* src, size_t bytes, tfh_stream stream);
 int32_t tfh_memcpy_d2h(void* dst, const void* src, size_t bytes, tfh_stream stream);
 int32_t tfh_memcpy_d2d(void* dst, const void* src, size_t bytes, tfh_stream stream);
+/* Page-locked host memory for transfers that return immediately (no counterpart in the reference, whose host tensors
+ * are ordinary Vec<T>; a MainMemory tensor that is meant to move may be allocated here). */
+int32_t tfh_host_malloc(size_t bytes, void** out);
+int32_t tfh_host_free(void* ptr);
 
 int32_t tfh_stream_create(tfh_stream* out);
 int32_t tfh_stream_destroy(tfh_stream s);
@@ -304,7 +314,9 @@ int32_t tfh_profile_kernel(int32_t kind, int32_t index, char* name, size_t cap, 
  * Tests use it to check which kernel a call was routed to. */
 const char* tfh_last_kernel(void);
 
-/* Releases the cached workspace, intermediate buffers and offset tables of every stream (after a synchronize). */
+/* Releases the cached workspace, intermediate buffers and offset tables of every stream (after a synchronize).
+ * Buffers that were handed out while their stream was being captured into a HIP graph are part of that graph and are
+ * passed over, here and whenever the library frees or regrows a cache: they stay until the process ends. */
 int32_t tfh_release_workspaces(void);
 
 #ifdef __cplusplus

@@ -86,6 +86,8 @@ def lib():
         L.tfh_conj.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
         L.tfh_fill.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
         L.tfh_memcpy_h2d.argtypes = L.tfh_memcpy_d2h.argtypes = L.tfh_memcpy_d2d.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.tfh_host_malloc.argtypes = [C.c_size_t, C.POINTER(C.c_void_p)]
+        L.tfh_host_free.argtypes = [C.c_void_p]
         L.tfh_malloc.argtypes = [C.c_size_t, C.POINTER(C.c_void_p)]
         L.tfh_event_record.argtypes = [C.c_void_p, C.c_void_p]
         L.tfh_stream_wait_event.argtypes = [C.c_void_p, C.c_void_p]
@@ -373,6 +375,33 @@ def view_of(t):
     return v
 
 
+_in_flight = []     # (event, buffers): device buffers that kernels on a stream other than torch's current one may still use
+
+
+def _enqueue_on(tensors, st):
+    """Stream-side prologue of a call that enqueues on stream `st`: pending completion events of the tensors become
+    stream dependencies (tenferro-einsum/src/lib.rs:146-177), never host waits."""
+    for t in tensors:
+        if isinstance(t, Tensor) and t.event is not None:
+            _check(lib().tfh_stream_wait_event(st, t.event._h))
+
+
+def _completed_on(outputs, st, used=()):
+    """The outputs of a call enqueued on `st` carry an event recorded behind it (tenferro-tensor/src/lib.rs:301-309).
+    When `st` is not the stream torch's allocator ordered the buffers on, the buffers of every tensor the call used are
+    held until that event has completed: dropping a tensor right after the call must not hand its memory to other work
+    while the kernels enqueued here still run.  (Holding references rather than telling the allocator about the stream:
+    the allocator would touch the stream again when the buffer is freed, and the caller may have destroyed it by then.)"""
+    import torch
+    ev = CompletionEvent(st)
+    for t in outputs:
+        if isinstance(t, Tensor):
+            t.event = ev
+    if st and st != torch.cuda.current_stream().cuda_stream:
+        _in_flight[:] = [(e, bufs) for e, bufs in _in_flight if not e.ready()]
+        _in_flight.append((ev, [t._buf for t in list(used) + list(outputs) if isinstance(t, Tensor)]))
+
+
 class HipPlan:
     """Plan<T> of the Hip backend (tenferro-prims/src/lib.rs:279-280)."""
 
@@ -408,8 +437,10 @@ class HipBackend:
         views = (tfh_view * max(len(inputs), 1))(*[view_of(t) for t in inputs])
         vo = view_of(output)
         st = current_stream() if stream is None else stream
+        _enqueue_on(list(inputs) + [output], st)
         _check(lib().tfh_execute(plan._h, _scalar_c(plan.dtype, alpha), views, len(inputs), _scalar_c(plan.dtype, beta),
                                  C.byref(vo), st))
+        _completed_on([output], st, inputs)
 
     @staticmethod
     def execute_static(plan, alpha, inputs, beta, output, stream=None):
@@ -418,8 +449,10 @@ class HipBackend:
         views = (tfh_view * max(len(inputs), 1))(*[view_of(t) for t in inputs])
         vo = view_of(output)
         st = current_stream() if stream is None else stream
+        _enqueue_on(list(inputs) + [output], st)
         _check(lib().tfh_execute_static(plan._h, _scalar_c(plan.dtype, alpha), views, len(inputs), _scalar_c(plan.dtype, beta),
                                         C.byref(vo), st))
+        _completed_on([output], st, inputs)
 
     @staticmethod
     def has_extension_for(dtype, ext):
@@ -447,7 +480,9 @@ class HipBackend:
         views = (tfh_view * len(flat))(*flat)
         outs = (tfh_view * len(outputs))(*[view_of(t) for t in outputs])
         st = current_stream() if stream is None else stream
+        _enqueue_on([t for pair in inputs for t in pair] + list(outputs), st)
         _check(lib().tfh_execute_grouped(plan._h, _scalar_c(plan.dtype, alpha), views, 2, _scalar_c(plan.dtype, beta), outs, st))
+        _completed_on(outputs, st, [t for pair in inputs for t in pair])
 
 
 # ---------------------------------------------------------------------------------------------- einsum front end
@@ -938,12 +973,10 @@ def einsum_with_plan_into(tree, operands, alpha, beta, output, stream=None, _don
     vo = output._view()
     st = current_stream() if stream is None else stream
     # pending events of the operands are stream dependencies, never host waits (:146-177)
-    for t in list(operands) + [output]:
-        if t.event is not None:
-            _check(lib().tfh_stream_wait_event(st, t.event._h))
+    _enqueue_on(list(operands) + [output], st)
     _check(lib().tfh_einsum_execute(dt, tree._h, views, len(operands), _scalar_c(dt, alpha), _scalar_c(dt, beta), C.byref(vo),
                                     C.c_uint64(_donate), st))
-    output.event = CompletionEvent(st)
+    _completed_on([output], st, operands)
 
 
 def einsum_with_plan(tree, operands, stream=None, _donate=0):

@@ -224,47 +224,36 @@ struct OperandMap {
     }
 };
 
+// What one block works on: the problem (extents, operand bases, strides), its tile, batch entry and k split.
+struct TileCtx {
+    int64_t M, N, K;
+    gptr Ap, Bp;
+    void* Cp;
+    Off32 am, ak, bk, bn;
+    OffFn cm, cn;
+    int tile_m, tile_n;
+    int64_t batch;
+    int split;
+    bool grouped;   // a problem of a grouped launch: plain strided matrices, offsets relative to the problem's first element
+};
+
 template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128>
-__global__ void __launch_bounds__((Cfg128<R, CX, BNV>::NT), (Cfg128<R, CX, BNV>::MIN_WAVES)) gemm128_kernel(GemmArgs g) {
+__device__ __forceinline__ void gemm128_body(const GemmArgs& g, const TileCtx& t, unsigned char* smem_raw) {
     typedef Cfg128<R, CX, BNV> C_;
-    typedef typename ElemT<R, CX>::type E;
     typedef typename Mfma<R>::acc_t acc_t;
     constexpr int BM = C_::BM, BN = C_::BN, BKE = C_::BKE, PITCH = C_::PITCH, BNE = C_::BNE, CH = C_::CH;
     constexpr int TM = C_::TM, TN = C_::TN;
-    extern __shared__ __align__(16) unsigned char smem_raw[];
     R* As = reinterpret_cast<R*>(smem_raw);   // [2][BM][PITCH]
     R* Bs = As + 2 * BM * PITCH;              // [2][BN][PITCH]
 
-    int64_t M = g.M, N = g.N, K = g.K;
-    gptr Ap = as_global(g.A32);
-    gptr Bp = as_global(g.B32);
-    void* Cp = g.C;
-    Off32 am = g.am32, ak = g.ak32, bk = g.bk32, bn = g.bn32;
-    OffFn cm = g.cm, cn = g.cn;
-    int tile_m, tile_n;
-    int64_t batch = 0;
-    int split = 0;
-    if (g.problems) {
-        const int4 tm = g.tile_map[blockIdx.x];
-        const GroupProblem& p = g.problems[tm.x];
-        M = p.M; N = p.N; K = p.K;
-        Ap = as_global(p.A); Bp = as_global(p.B); Cp = p.C;
-        am.stride = (uint32_t)(p.sam * (int64_t)sizeof(E)); ak.stride = (uint32_t)(p.sak * (int64_t)sizeof(E));
-        bk.stride = (uint32_t)(p.sbk * (int64_t)sizeof(E)); bn.stride = (uint32_t)(p.sbn * (int64_t)sizeof(E));
-        cm.stride = p.scm; cn.stride = p.scn;
-        tile_m = tm.y;
-        tile_n = tm.z;
-    } else {
-        // one-dimensional grid: tiles of one (batch, split) pair are adjacent logical positions
-        const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n;
-        const uint64_t lb = logical_block(blockIdx.x, gridDim.x);
-        const uint32_t lz = (uint32_t)(lb / tiles);
-        tile_of((uint32_t)(lb % tiles), g.tiles_m, g.tiles_n, tile_m, tile_n);
-        split = (int)(lz % (uint32_t)g.nsplit);
-        batch = lz / (uint32_t)g.nsplit;
-        Ap += off_of(g.ab, batch) * (int64_t)sizeof(E);
-        Bp += off_of(g.bb, batch) * (int64_t)sizeof(E);
-    }
+    const int64_t M = t.M, N = t.N, K = t.K;
+    gptr Ap = t.Ap, Bp = t.Bp;
+    void* Cp = t.Cp;
+    const Off32 am = t.am, ak = t.ak, bk = t.bk, bn = t.bn;
+    const OffFn cm = t.cm, cn = t.cn;
+    const int tile_m = t.tile_m, tile_n = t.tile_n;
+    const int64_t batch = t.batch;
+    const int split = t.split;
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BNE;
     const int64_t kbeg = (int64_t)split * g.k_per_split;
     const int64_t kend = (g.nsplit > 1 && kbeg + g.k_per_split < K) ? kbeg + g.k_per_split : K;
@@ -279,15 +268,15 @@ __global__ void __launch_bounds__((Cfg128<R, CX, BNV>::NT), (Cfg128<R, CX, BNV>:
     // span one tile whatever the operand's size.  A vector moved back at a matrix edge can start a few rows before
     // the tile: the host's bias leaves room for that.  Grouped problems carry no bias (and are small): their offsets
     // stay relative to the problem's first row.
-    const bool rebase_a = !am.tab && !g.problems, rebase_b = !bn.tab && !g.problems;
+    const bool rebase_a = !am.tab && !t.grouped, rebase_b = !bn.tab && !t.grouped;
     if (rebase_a) Ap += (int64_t)(int32_t)am.stride * m0;
     if (rebase_b) Bp += (int64_t)(int32_t)bn.stride * n0;
     ma.init(am, ak, rebase_a ? 0 : m0, rowsA);
 #pragma unroll
-    for (int l = 0; l < MapA::NL; ++l) ma.voff[l] += g.problems ? 0u : g.bias_a32;
+    for (int l = 0; l < MapA::NL; ++l) ma.voff[l] += t.grouped ? 0u : g.bias_a32;
     mb.init(bn, bk, rebase_b ? 0 : n0, rowsB);
 #pragma unroll
-    for (int l = 0; l < MapB::NL; ++l) mb.voff[l] += g.problems ? 0u : g.bias_b32;
+    for (int l = 0; l < MapB::NL; ++l) mb.voff[l] += t.grouped ? 0u : g.bias_b32;
     // uniform bases; single-stride k advances them by one stage per iteration
     gptr sa = Ap + (ak.tab ? 0 : (int64_t)(int32_t)ak.stride * kbeg);
     gptr sb = Bp + (bk.tab ? 0 : (int64_t)(int32_t)bk.stride * kbeg);
@@ -486,7 +475,7 @@ __global__ void __launch_bounds__((Cfg128<R, CX, BNV>::NT), (Cfg128<R, CX, BNV>:
             }
         return;
     }
-    R* Cb = reinterpret_cast<R*>(Cp) + (g.problems ? 0 : off_of(g.cb, batch)) * (CX ? 2 : 1);
+    R* Cb = reinterpret_cast<R*>(Cp) + (t.grouped ? 0 : off_of(g.cb, batch)) * (CX ? 2 : 1);
     const R ar = (R)g.alpha_re, ai = (R)g.alpha_im, br = (R)g.beta_re, bi = (R)g.beta_im;
     int64_t coff[TN];
     bool cok[TN];
@@ -531,6 +520,90 @@ __global__ void __launch_bounds__((Cfg128<R, CX, BNV>::NT), (Cfg128<R, CX, BNV>:
         }
 }
 
+// One tile of a uniform launch (single problem, batched, split-K) or of a grouped launch whose tiles all have this shape.
+template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128>
+__global__ void __launch_bounds__((Cfg128<R, CX, BNV>::NT), (Cfg128<R, CX, BNV>::MIN_WAVES)) gemm128_kernel(GemmArgs g) {
+    typedef typename ElemT<R, CX>::type E;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    TileCtx t;
+    t.M = g.M; t.N = g.N; t.K = g.K;
+    t.Ap = as_global(g.A32);
+    t.Bp = as_global(g.B32);
+    t.Cp = g.C;
+    t.am = g.am32; t.ak = g.ak32; t.bk = g.bk32; t.bn = g.bn32;
+    t.cm = g.cm; t.cn = g.cn;
+    t.batch = 0;
+    t.split = 0;
+    t.grouped = g.problems != nullptr;
+    if (g.problems) {
+        const int4 tm = g.tile_map[blockIdx.x];
+        const GroupProblem& p = g.problems[tm.x];
+        t.M = p.M; t.N = p.N; t.K = p.K;
+        t.Ap = as_global(p.A); t.Bp = as_global(p.B); t.Cp = p.C;
+        t.am.stride = (uint32_t)(p.sam * (int64_t)sizeof(E)); t.ak.stride = (uint32_t)(p.sak * (int64_t)sizeof(E));
+        t.bk.stride = (uint32_t)(p.sbk * (int64_t)sizeof(E)); t.bn.stride = (uint32_t)(p.sbn * (int64_t)sizeof(E));
+        t.cm.stride = p.scm; t.cn.stride = p.scn;
+        t.tile_m = tm.y;
+        t.tile_n = tm.z;
+    } else {
+        // one-dimensional grid: tiles of one (batch, split) pair are adjacent logical positions
+        const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n;
+        const uint64_t lb = logical_block(blockIdx.x, gridDim.x);
+        const uint32_t lz = (uint32_t)(lb / tiles);
+        tile_of((uint32_t)(lb % tiles), g.tiles_m, g.tiles_n, t.tile_m, t.tile_n);
+        t.split = (int)(lz % (uint32_t)g.nsplit);
+        t.batch = lz / (uint32_t)g.nsplit;
+        t.Ap += off_of(g.ab, t.batch) * (int64_t)sizeof(E);
+        t.Bp += off_of(g.bb, t.batch) * (int64_t)sizeof(E);
+    }
+    gemm128_body<R, CX, AKF, BKF, VA, VB, BNV>(g, t, smem_raw);
+}
+
+// Grouped launch with a tile shape per map entry (tile_map[].w): 0 = 128 x 128; 1 = 128 rows x 64 real columns (a last
+// column strip of at most 64); 2 = 64 rows x 128 real columns (a last row strip of at most 64), computed as the transposed
+// product with the operands exchanged, so that the strip is again the thin right-hand side; -1 = no tile (padding that
+// keeps the per-XCD lists of the map equally long).  The branch is uniform over the block; the three bodies never run
+// in the same block, so registers and LDS are those of the largest.
+template <class R, bool CX, bool AKF, bool BKF, int V>
+__global__ void __launch_bounds__((Cfg128<R, CX, 128>::NT), (Cfg128<R, CX, 128>::MIN_WAVES)) gemm128_grouped_kernel(GemmArgs g) {
+    typedef typename ElemT<R, CX>::type E;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int4 tm = g.tile_map[blockIdx.x];
+    if (tm.x < 0) return;
+    const GroupProblem& p = g.problems[tm.x];
+    const int kind = __builtin_amdgcn_readfirstlane(tm.w);
+    TileCtx t;
+    t.batch = 0;
+    t.split = 0;
+    t.grouped = true;
+    t.tile_m = tm.y;
+    t.tile_n = tm.z;
+    t.K = p.K;
+    t.Cp = p.C;
+    t.am.tab = t.ak.tab = t.bk.tab = t.bn.tab = nullptr;
+    t.cm.tab = t.cn.tab = nullptr;
+    constexpr int64_t EB = (int64_t)sizeof(E);
+    // a row-contiguous B of 4-byte reals has more threads than 16-byte accesses over 64 columns: 8-byte accesses there
+    constexpr int VTHIN = (V > 1 && sizeof(R) == 4) ? V / 2 : V;
+    if (kind != 2) {
+        t.M = p.M; t.N = p.N;
+        t.Ap = as_global(p.A); t.Bp = as_global(p.B);
+        t.am.stride = (uint32_t)(p.sam * EB); t.ak.stride = (uint32_t)(p.sak * EB);
+        t.bk.stride = (uint32_t)(p.sbk * EB); t.bn.stride = (uint32_t)(p.sbn * EB);
+        t.cm.stride = p.scm; t.cn.stride = p.scn;
+        if (kind == 0) gemm128_body<R, CX, AKF, BKF, V, V, 128>(g, t, smem_raw);
+        else gemm128_body<R, CX, AKF, BKF, V, (BKF ? V : VTHIN), 64>(g, t, smem_raw);
+    } else {
+        // C^T = B^T A^T: the body's A is B seen with rows n, its B is A seen with columns m
+        t.M = p.N; t.N = p.M;
+        t.Ap = as_global(p.B); t.Bp = as_global(p.A);
+        t.am.stride = (uint32_t)(p.sbn * EB); t.ak.stride = (uint32_t)(p.sbk * EB);
+        t.bk.stride = (uint32_t)(p.sak * EB); t.bn.stride = (uint32_t)(p.sam * EB);
+        t.cm.stride = p.scn; t.cn.stride = p.scm;
+        gemm128_body<R, CX, BKF, AKF, V, (AKF ? V : VTHIN), 64>(g, t, smem_raw);
+    }
+}
+
 template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128>
 inline void launch_gemm128_variant(const GemmArgs& g, dim3 grid, hipStream_t st) {
     static bool once = [] {
@@ -570,6 +643,32 @@ inline void launch_gemm128_any(const GemmArgs& g, dim3 grid, bool akf, bool bkf,
     launch_gemm128_layout<R, CX, 1>(g, grid, akf, bkf, st);
 }
 
+// Grouped launch with per-tile shapes (16-byte accesses only: g.vec; the scalar-access fallback keeps uniform tiles).
+template <class R, bool CX, bool AKF, bool BKF>
+inline void launch_gemm128_grouped_variant(const GemmArgs& g, dim3 grid, hipStream_t st) {
+    constexpr int V = Cfg128<R, CX>::VMAX;
+    static bool once = [] {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm128_grouped_kernel<R, CX, AKF, BKF, V>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg128<R, CX, 128>::LDS_BYTES);
+        return true;
+    }();
+    (void)once;
+    typedef Cfg128<R, CX, 128> C_;
+    const size_t lds = C_::LDS_BYTES;
+    const dim3 block(C_::NT);
+    TFH_LAUNCH_TIMED((gemm128_grouped_kernel<R, CX, AKF, BKF, V>), grid, block, lds, st, g);
+}
+template <class R, bool CX>
+inline void launch_gemm128_grouped_any(const GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
+    if (akf) {
+        if (bkf) launch_gemm128_grouped_variant<R, CX, true, true>(g, grid, st);
+        else launch_gemm128_grouped_variant<R, CX, true, false>(g, grid, st);
+    } else {
+        if (bkf) launch_gemm128_grouped_variant<R, CX, false, true>(g, grid, st);
+        else launch_gemm128_grouped_variant<R, CX, false, false>(g, grid, st);
+    }
+}
+
 // 128 x 64 tiles for a thin right-hand side.  A row-contiguous B of f32 / complex64 has more threads than 16-byte
 // accesses over 64 columns give work to: that loader uses 8-byte accesses (two f32, one complex64).
 template <class R, bool CX>
@@ -607,5 +706,10 @@ void launch_gemm128x64_f32(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bk
 void launch_gemm128x64_f64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
 void launch_gemm128x64_c64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
 void launch_gemm128x64_c128(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+// ... and the grouped kernel with a tile shape per map entry
+void launch_gemm128_grouped_f32(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+void launch_gemm128_grouped_f64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+void launch_gemm128_grouped_c64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+void launch_gemm128_grouped_c128(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
 
 }  // namespace tfh

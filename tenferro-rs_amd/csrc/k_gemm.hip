@@ -22,6 +22,7 @@
 #include <array>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
 
 #include "gemm128.hpp"
@@ -1020,27 +1021,30 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
 
 // ---- grouped launch ------------------------------------------------------------------------------------------
 struct GroupedState {
-    std::vector<int4> tile_map_host;
+    std::vector<int4> tile_map_host;   // (problem, tile_m, tile_n, shape); shape: see gemm128_grouped_kernel; problem -1 = padding
+    std::vector<int4> tile_map_uniform;   // every tile 128 x 128 (the scalar-access fallback of the 128 kernel)
     int bm = 128;
+    bool shaped = false;               // tile_map_host carries per-tile shapes (128-tile plans)
     std::mutex mu;
-    int4* tile_map_dev = nullptr;       // uploaded on first execute
-    GroupProblem* problems_dev = nullptr;
-    int device = -1;
+    struct DeviceMaps { int4* shaped = nullptr; int4* uniform = nullptr; };
+    std::map<int, DeviceMaps> maps;    // per device: the tile maps never change after the plan is made, so they are uploaded once
 };
 
 void grouped_state_destroy(GroupedState* s) {
     if (!s) return;
-    if (s->tile_map_dev) (void)hipFree(s->tile_map_dev);
-    if (s->problems_dev) (void)hipFree(s->problems_dev);
+    for (auto& kv : s->maps) {
+        if (kv.second.shaped) (void)hipFree(kv.second.shaped);
+        if (kv.second.uniform) (void)hipFree(kv.second.uniform);
+    }
     delete s;
 }
 
 int32_t grouped_plan_init(tfh_plan& plan) {
-    // Tile list over all problems, heaviest tiles (largest K) first so the tail of the launch is short.
     auto* gs = new (std::nothrow) GroupedState();
     if (!gs) return set_error(TFH_ERR_DEVICE, "out of host memory");
     const bool cx = is_complex(plan.dtype);
-    struct T { int p, tm, tn; int64_t k; };
+    const int ec = cx ? 2 : 1;
+    struct T { int p, tm, tn, kind; int64_t k; };
     std::vector<T> tiles;
     int64_t small = 0;
     std::vector<std::array<int64_t, 3>> mnk((size_t)plan.n_groups);
@@ -1075,17 +1079,110 @@ int32_t grouped_plan_init(tfh_plan& plan) {
     bool all_tiny = plan.n_groups >= 64;
     for (int gi = 0; gi < plan.n_groups; ++gi) all_tiny = all_tiny && mnk[(size_t)gi][0] <= 32 && mnk[(size_t)gi][1] <= 32 && mnk[(size_t)gi][2] <= 1024;
     if (all_tiny) gs->bm = 32;
-    for (int gi = 0; gi < plan.n_groups; ++gi) {
-        int64_t M = mnk[(size_t)gi][0], N = mnk[(size_t)gi][1], K = mnk[(size_t)gi][2];
-        int64_t NR = cx ? 2 * N : N;
-        for (int64_t tm = 0; tm * gs->bm < M; ++tm)
-            for (int64_t tn = 0; tn * gs->bm < NR; ++tn) tiles.push_back({gi, (int)tm, (int)tn, K});
+    if (gs->bm != 128) {
+        for (int gi = 0; gi < plan.n_groups; ++gi) {
+            int64_t M = mnk[(size_t)gi][0], N = mnk[(size_t)gi][1], K = mnk[(size_t)gi][2];
+            int64_t NR = cx ? 2 * N : N;
+            for (int64_t tm = 0; tm * gs->bm < M; ++tm)
+                for (int64_t tn = 0; tn * gs->bm < NR; ++tn) tiles.push_back({gi, (int)tm, (int)tn, 0, K});
+        }
+        // heaviest tiles (largest K) first, so that the tail of the launch is short
+        std::stable_sort(tiles.begin(), tiles.end(), [](const T& x, const T& y) { return x.k > y.k; });
+        for (auto& t : tiles) gs->tile_map_host.push_back(make_int4(t.p, t.tm, t.tn, 0));
+        plan.grouped = gs;
+        return TFH_OK;
     }
-    // Heaviest tiles (largest K) first so that the tail of the launch is short.  The XCDs take the list round-robin,
-    // so each gets an equal share of every problem; giving whole problems to one XCD for L2 locality measured 10%
-    // slower (the balance is worth more than the operand re-use).
+    // 128-row tiles.  A last strip of at most 64 rows or 64 real columns gets tiles of that shape instead of a padded
+    // 128 x 128 one (extents that are odd multiples of 64 -- half of all extents drawn from {64, 128, ...} -- would
+    // otherwise compute 10 % more than the products need): shape 1 = 128 x 64, shape 2 = 64 x 128 (run transposed).
+    // Two row panels of a problem (256 rows of A, every column tile, walked column by column) form a unit: its tiles read
+    // the same rows of A and, side by side, the same columns of B.  Units are dealt to the eight XCDs -- block i of a
+    // launch runs on XCD i % 8, each with an L2 of its own -- longest first onto the XCD with the least work so far, and
+    // every XCD runs its units in the order of their k (a lone tile with a long k that started late would run on after
+    // everything else has finished).  Measured on the benchmark's 128 blocks: dealing the tiles out one by one in the
+    // order of their k, each problem spread over all eight L2s, fetches 2.82 GB for 0.68 GB of operands; units of one
+    // row panel 2.09 GB, of two 1.59 GB, of four 1.30 GB, at the same speed within 1 % (832 / 825 / 831 us) -- while units
+    // kept in the order of their total work instead of their k lost 10 %.
+    struct Unit { std::vector<T> tiles; double cost; };
+    std::vector<Unit> units;
+    // a 128 x 64 tile does half the multiply-adds of a full tile in about 0.63 of its time (measured on thin products)
+    const double thin_cost = 0.63;
+    for (int gi = 0; gi < plan.n_groups; ++gi) {
+        const int64_t M = mnk[(size_t)gi][0], N = mnk[(size_t)gi][1], K = mnk[(size_t)gi][2];
+        const int64_t NR = N * ec;
+        if (M == 0 || N == 0) continue;
+        const int64_t full_m = M / 128, rem_m = M % 128, full_n = NR / 128, rem_n = NR % 128;
+        // (a transposed strip is 64 real columns of the transposed product, i.e. 64 / ec rows of this one)
+        const bool thin_m = rem_m > 0 && rem_m * ec <= 64, thin_n = rem_n > 0 && rem_n <= 64;
+        const int64_t rows128 = full_m + ((rem_m > 0 && !thin_m) ? 1 : 0);   // row panels of 128 (the last one padded)
+        const int64_t cols128 = full_n + ((rem_n > 0 && !thin_n) ? 1 : 0);
+        const double kcost = (double)((K + 15) / 16 + 8);   // stages plus about eight stages' worth of prologue and epilogue
+        const int64_t upanels = 2;   // row panels per unit
+        for (int64_t tm0 = 0; tm0 < rows128; tm0 += upanels) {
+            Unit u;
+            u.cost = 0;
+            const int64_t tm1 = std::min(rows128, tm0 + upanels);
+            // column by column, so that the unit's row panels read a column of B at the same time
+            for (int64_t tn = 0; tn < cols128; ++tn)
+                for (int64_t tm = tm0; tm < tm1; ++tm) {
+                    u.tiles.push_back({gi, (int)tm, (int)tn, 0, K});
+                    u.cost += kcost;
+                }
+            if (thin_n)   // column strip: tile_n counts 64-column tiles
+                for (int64_t tm = tm0; tm < tm1; ++tm) {
+                    u.tiles.push_back({gi, (int)tm, (int)(2 * cols128), 1, K});
+                    u.cost += thin_cost * kcost;
+                }
+            units.push_back(std::move(u));
+        }
+        if (thin_m) {   // row strip, transposed: the body's rows are the columns (128 per tile), its 64-wide tile_n counts rows
+            Unit u;
+            u.cost = 0;
+            const int64_t cols = (N + 127) / 128;
+            for (int64_t tn = 0; tn < cols; ++tn) {
+                u.tiles.push_back({gi, (int)tn, (int)(2 * rows128 * ec), 2, K});
+                u.cost += thin_cost * kcost;
+            }
+            units.push_back(std::move(u));
+        }
+    }
+    std::stable_sort(units.begin(), units.end(), [](const Unit& x, const Unit& y) { return x.cost > y.cost; });
+    std::array<std::vector<T>, XCDS> per_xcd;
+    std::array<double, XCDS> load{};
+    std::array<std::vector<const Unit*>, XCDS> units_of;
+    for (auto& u : units) {
+        int best = 0;
+        for (int x = 1; x < XCDS; ++x)
+            if (load[(size_t)x] < load[(size_t)best]) best = x;
+        load[(size_t)best] += u.cost;
+        units_of[(size_t)best].push_back(&u);
+    }
+    for (int x = 0; x < XCDS; ++x) {
+        // an XCD starts its longest tiles first (largest k), whatever the size of the unit they belong to: a lone tile
+        // with a long k that started late would run on after everything else has finished
+        std::stable_sort(units_of[(size_t)x].begin(), units_of[(size_t)x].end(),
+                             [](const Unit* a, const Unit* b) { return a->tiles[0].k > b->tiles[0].k; });
+        for (const Unit* u : units_of[(size_t)x])
+            for (auto& t : u->tiles) per_xcd[(size_t)x].push_back(t);
+    }
+    size_t longest = 0;
+    for (auto& v : per_xcd) longest = std::max(longest, v.size());
+    for (size_t i = 0; i < longest; ++i)
+        for (int x = 0; x < XCDS; ++x) {
+            const auto& v = per_xcd[(size_t)x];
+            if (i < v.size()) gs->tile_map_host.push_back(make_int4(v[i].p, v[i].tm, v[i].tn, v[i].kind));
+            else gs->tile_map_host.push_back(make_int4(-1, 0, 0, -1));
+        }
+    while (!gs->tile_map_host.empty() && gs->tile_map_host.back().x < 0) gs->tile_map_host.pop_back();
+    gs->shaped = true;
+    // uniform 128 x 128 tiles for operands that do not allow 16-byte accesses
+    for (int gi = 0; gi < plan.n_groups; ++gi) {
+        const int64_t M = mnk[(size_t)gi][0], NR = mnk[(size_t)gi][1] * ec, K = mnk[(size_t)gi][2];
+        for (int64_t tm = 0; tm * 128 < M; ++tm)
+            for (int64_t tn = 0; tn * 128 < NR; ++tn) tiles.push_back({gi, (int)tm, (int)tn, 0, K});
+    }
     std::stable_sort(tiles.begin(), tiles.end(), [](const T& x, const T& y) { return x.k > y.k; });
-    for (auto& t : tiles) gs->tile_map_host.push_back(make_int4(t.p, t.tm, t.tn, 0));
+    for (auto& t : tiles) gs->tile_map_uniform.push_back(make_int4(t.p, t.tm, t.tn, 0));
     plan.grouped = gs;
     return TFH_OK;
 }
@@ -1152,38 +1249,12 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
     }
     if (gs->bm == 128 && !ok128)
         return set_error(TFH_ERR_INVALID_ARGUMENT, "grouped contraction: an operand has a negative stride or spans 4 GiB or more");
-    {
-        std::lock_guard<std::mutex> lk(gs->mu);
-        int dev = 0;
-        if (int32_t e = hip_check(hipGetDevice(&dev), "hipGetDevice")) return e;
-        if (!gs->tile_map_dev || gs->device != dev) {
-            if (gs->tile_map_dev) (void)hipFree(gs->tile_map_dev);
-            if (gs->problems_dev) (void)hipFree(gs->problems_dev);
-            gs->tile_map_dev = nullptr;
-            gs->problems_dev = nullptr;
-            size_t nb = gs->tile_map_host.size() * sizeof(int4);
-            if (int32_t e = hip_check(hipMalloc((void**)&gs->tile_map_dev, std::max<size_t>(nb, 16)), "hipMalloc(tile map)")) return e;
-            if (int32_t e = hip_check(hipMalloc((void**)&gs->problems_dev, sizeof(GroupProblem) * (size_t)plan.n_groups), "hipMalloc(problem table)")) return e;
-            if (nb)
-                if (int32_t e = hip_check(hipMemcpy(gs->tile_map_dev, gs->tile_map_host.data(), nb, hipMemcpyHostToDevice), "upload tile map")) return e;
-            gs->device = dev;
-        }
-    }
     if (gs->tile_map_host.empty()) return TFH_OK;
-    for (int first = 0; first < plan.n_groups; first += PROBS_PER_SET) {
-        ProblemSet s;
-        s.first = first;
-        s.count = std::min(PROBS_PER_SET, plan.n_groups - first);
-        std::memcpy(s.p, probs.data() + first, sizeof(GroupProblem) * (size_t)s.count);
-        hipLaunchKernelGGL(set_problems_kernel, dim3(1), dim3(64), 0, st, gs->problems_dev, s);
-    }
     GemmArgs g;
     std::memset(&g, 0, sizeof g);
     g.nbatch = 1;
     g.nsplit = 1;
-    g.a_kfast = 1;   // per-problem choice is not available in one launch: assume row-major operands,
-    g.b_kfast = 0;   // i.e. A contiguous in k, B contiguous in n (the block-sparse "ij,jk->ik" case)
-    // pick the mapping from the first problem's strides
+    // one loader layout per launch, from the first problem's strides (row-major operands: A contiguous in k, B in n)
     g.a_kfast = std::llabs(probs[0].sak) <= std::llabs(probs[0].sam) || probs[0].M == 1;
     g.b_kfast = std::llabs(probs[0].sbk) <= std::llabs(probs[0].sbn) || probs[0].N == 1;
     // 16-byte accesses: every problem is contiguous along the direction the mapping names, with an extent there that
@@ -1200,15 +1271,61 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
         else if (!(g.a_kfast ? vec_side(true, p.sak, p.K, p.sam, p.M) : vec_side(false, p.sam, p.M, p.sak, p.K))) vec = false;
         else if (!(g.b_kfast ? vec_side(true, p.sbk, p.K, p.sbn, p.N) : vec_side(false, p.sbn, p.N, p.sbk, p.K))) vec = false;
     }
+    // Tiles of their own shape for the last strips need 16-byte accesses on both operands (or 16-byte elements); in a
+    // transposed strip tile the operands change places, so both must also satisfy the other's rule.
+    bool shaped = gs->shaped && gs->bm == 128 && (vec || V == 1);
+    if (shaped && V > 1)
+        for (auto& p : probs) {
+            // transposed: the body's A is B (lanes along n when B is row-contiguous), its B is A
+            if (!(g.b_kfast ? vec_side(true, p.sbk, p.K, p.sbn, p.N) : vec_side(false, p.sbn, p.N, p.sbk, p.K))) shaped = false;
+            if (!(g.a_kfast ? vec_side(true, p.sak, p.K, p.sam, p.M) : vec_side(false, p.sam, p.M, p.sak, p.K))) shaped = false;
+        }
+    const std::vector<int4>& map_host = shaped ? gs->tile_map_host : (gs->bm == 128 ? gs->tile_map_uniform : gs->tile_map_host);
+    // The tile maps never change: one upload per device, the first time the plan runs there (this allocates and waits,
+    // so a grouped plan is run once eagerly before it is captured into a graph, like every other first call).
+    int4* map_dev = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(gs->mu);
+        int dev = 0;
+        if (int32_t e = hip_check(hipGetDevice(&dev), "hipGetDevice")) return e;
+        GroupedState::DeviceMaps& dm = gs->maps[dev];
+        int4*& slot = (shaped || gs->bm != 128) ? dm.shaped : dm.uniform;
+        if (!slot) {
+            const size_t nb = map_host.size() * sizeof(int4);
+            if (int32_t e = hip_check(hipMalloc((void**)&slot, std::max<size_t>(nb, 16)), "hipMalloc(tile map)")) return e;
+            if (int32_t e = hip_check(hipMemcpy(slot, map_host.data(), nb, hipMemcpyHostToDevice), "upload tile map")) return e;
+        }
+        map_dev = slot;
+    }
+    // The problem records belong to the call: they go into this stream's workspace (stream order keeps them intact until
+    // the contraction that reads them has run), written from kernel arguments -- no host staging, capturable.  Two
+    // executes of one plan on two streams therefore never share records.
+    void* ws = nullptr;
+    if (int32_t e = workspace(stream, sizeof(GroupProblem) * (size_t)plan.n_groups, &ws)) return e;
+    GroupProblem* problems_dev = (GroupProblem*)ws;
+    for (int first = 0; first < plan.n_groups; first += PROBS_PER_SET) {
+        ProblemSet s;
+        s.first = first;
+        s.count = std::min(PROBS_PER_SET, plan.n_groups - first);
+        std::memcpy(s.p, probs.data() + first, sizeof(GroupProblem) * (size_t)s.count);
+        hipLaunchKernelGGL(set_problems_kernel, dim3(1), dim3(64), 0, st, problems_dev, s);
+    }
     g.vec = gs->bm == 128 && vec;
     g.alpha_re = alpha.re; g.alpha_im = alpha.im; g.beta_re = beta.re; g.beta_im = beta.im;
     g.use_beta = !beta.is_zero();
-    g.problems = gs->problems_dev;
-    g.tile_map = gs->tile_map_dev;
-    dim3 grid((uint32_t)gs->tile_map_host.size(), 1, 1);
+    g.problems = problems_dev;
+    g.tile_map = map_dev;
+    dim3 grid((uint32_t)map_host.size(), 1, 1);
     const int prof = prof_begin(PROF_CONTRACT, stream);
-    if (gs->bm == 32) launch_gemm_wave(dtype, g, (int64_t)gs->tile_map_host.size(), st);
-    else if (gs->bm == 128) launch_128(dtype, g, grid, st);
+    if (gs->bm == 32) launch_gemm_wave(dtype, g, (int64_t)map_host.size(), st);
+    else if (shaped) {
+        switch (dtype) {
+            case TFH_F32: launch_gemm128_grouped_f32(g, grid, g.a_kfast, g.b_kfast, st); break;
+            case TFH_F64: launch_gemm128_grouped_f64(g, grid, g.a_kfast, g.b_kfast, st); break;
+            case TFH_C64: launch_gemm128_grouped_c64(g, grid, g.a_kfast, g.b_kfast, st); break;
+            default: launch_gemm128_grouped_c128(g, grid, g.a_kfast, g.b_kfast, st); break;
+        }
+    } else if (gs->bm == 128) launch_128(dtype, g, grid, st);
     else launch_generic64(dtype, g, grid, st);
     prof_end(prof, stream);
     return hip_check(hipGetLastError(), "grouped contraction launch");

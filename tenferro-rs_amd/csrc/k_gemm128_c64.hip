@@ -8,4 +8,7 @@ void launch_gemm128_c64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, 
 void launch_gemm128x64_c64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
     gemm::launch_gemm128x64_any<float, true>(g, grid, akf, bkf, st);
 }
+void launch_gemm128_grouped_c64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
+    gemm::launch_gemm128_grouped_any<float, true>(g, grid, akf, bkf, st);
+}
 }  // namespace tfh

@@ -8,4 +8,7 @@ void launch_gemm128_f64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, 
 void launch_gemm128x64_f64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
     gemm::launch_gemm128x64_any<double, false>(g, grid, akf, bkf, st);
 }
+void launch_gemm128_grouped_f64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
+    gemm::launch_gemm128_grouped_any<double, false>(g, grid, akf, bkf, st);
+}
 }  // namespace tfh

@@ -3,8 +3,11 @@
 // the GPU-async vocabulary of tenferro-tensor/src/lib.rs:301-309, 660-713.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <cstring>
 #include <map>
 #include <mutex>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -18,16 +21,37 @@ int32_t hip_check(int err, const char* what) {
 }
 
 namespace {
+// A buffer that was handed out while its stream was being captured into a graph is part of that graph: replays read
+// and write it long after the call that took it has returned.  Such buffers are "pinned": nothing here frees them
+// before the process ends (a workspace that has to grow is retired instead of freed, tfh_release_workspaces and the
+// out-of-memory path pass them over).  Pinned blocks still serve later calls on their stream, which stream order keeps
+// apart from a replay launched into the same stream.
 struct StreamScratch {
     void* ws = nullptr;
     size_t ws_bytes = 0;
+    bool ws_pinned = false;
+    std::vector<void*> retired;                 // pinned workspaces that were outgrown
     std::multimap<size_t, void*> free_blocks;   // cached intermediates by size
     std::map<void*, size_t> live;
+    std::set<void*> pinned_blocks;              // intermediates handed out during a capture
     // offset tables of contractions already run on this stream, by the dims and strides they were built from
-    struct Tables { void* dev; size_t bytes; bool filled; };
+    struct Tables { void* dev; size_t bytes; bool filled; bool pinned; };
     std::map<std::string, Tables> tables;
     size_t table_bytes = 0;
+    // two pinned host buffers for transfers from and to pageable host memory (allocated on first use)
+    void* bounce[2] = {nullptr, nullptr};
+    hipEvent_t bounce_ev[2] = {nullptr, nullptr};
+    bool bounce_busy[2] = {false, false};   // a copy recorded in bounce_ev may still be using the buffer
 };
+constexpr size_t BOUNCE_BYTES = (size_t)16 << 20;
+bool capturing(void* stream) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return cs != hipStreamCaptureStatusNone;
+}
 constexpr size_t TABLE_CACHE_BYTES = (size_t)64 << 20;   // per stream; beyond it tables go to the workspace again
 constexpr size_t TABLE_CACHE_ENTRIES = 256;
 std::mutex g_mu;
@@ -75,8 +99,15 @@ int32_t malloc_or_release(void** p, size_t bytes, void* stream, const char* what
     (void)hipGetDevice(&dev);
     for (auto& kv : g_scratch) {
         if (kv.first.first != dev) continue;
-        for (auto& b : kv.second.free_blocks) (void)hipFree(b.second);
-        kv.second.free_blocks.clear();
+        auto& fb = kv.second.free_blocks;
+        for (auto it = fb.begin(); it != fb.end();) {
+            if (kv.second.pinned_blocks.count(it->second)) {
+                ++it;
+                continue;
+            }
+            (void)hipFree(it->second);
+            it = fb.erase(it);
+        }
     }
     return hip_check(hipMalloc(p, bytes), what);
 }
@@ -91,18 +122,26 @@ int32_t workspace(void* stream, size_t bytes, void** out) {
     int32_t err;
     StreamScratch* s = scratch_for(stream, &err);
     if (!s) return err;
+    const bool cap = capturing(stream);
     if (bytes > s->ws_bytes) {
         if (s->ws) {
-            // kernels already enqueued may still read the old buffer
-            if (int32_t e = hip_check(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize")) return e;
-            (void)hipFree(s->ws);
+            if (s->ws_pinned || cap) {
+                // a captured graph holds the old buffer (or is being recorded right now, when nothing may wait): keep it
+                s->retired.push_back(s->ws);
+            } else {
+                // kernels already enqueued may still read the old buffer
+                if (int32_t e = hip_check(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize")) return e;
+                (void)hipFree(s->ws);
+            }
             s->ws = nullptr;
             s->ws_bytes = 0;
+            s->ws_pinned = false;
         }
         size_t want = std::max<size_t>(bytes + bytes / 4, (size_t)1 << 20);
         if (int32_t e = malloc_or_release(&s->ws, want, stream, "hipMalloc(workspace)")) return e;
         s->ws_bytes = want;
     }
+    if (cap) s->ws_pinned = true;
     *out = s->ws;
     return TFH_OK;
 }
@@ -117,23 +156,21 @@ int32_t table_cache_get(void* stream, const std::string& key, size_t bytes, void
     if (!s) return err;
     auto it = s->tables.find(key);
     if (it != s->tables.end()) {
-        if (it->second.filled && it->second.bytes == bytes) *tables = it->second.dev;
+        if (it->second.filled && it->second.bytes == bytes) {
+            *tables = it->second.dev;
+            if (capturing(stream)) it->second.pinned = true;
+        }
         return TFH_OK;
     }
     if (s->tables.size() >= TABLE_CACHE_ENTRIES || s->table_bytes + bytes > TABLE_CACHE_BYTES) return TFH_OK;
-    // no allocation while the stream is being captured into a graph: the call then builds its tables in the workspace
-    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess) {
-        (void)hipGetLastError();
-        return TFH_OK;
-    }
-    if (cs != hipStreamCaptureStatusNone) return TFH_OK;
+    // no new cache entry while the stream is being captured into a graph: the call then builds its tables in the workspace
+    if (capturing(stream)) return TFH_OK;
     void* p = nullptr;
     if (hipMalloc(&p, bytes) != hipSuccess) {
         (void)hipGetLastError();   // out of memory for the cache is not an error of the call
         return TFH_OK;
     }
-    s->tables[key] = StreamScratch::Tables{p, bytes, false};
+    s->tables[key] = StreamScratch::Tables{p, bytes, false, false};
     s->table_bytes += bytes;
     *tables = p;
     *fresh = true;
@@ -156,16 +193,19 @@ int32_t pool_alloc(void* stream, size_t bytes, void** out) {
     StreamScratch* s = scratch_for(stream, &err);
     if (!s) return err;
     bytes = std::max<size_t>((bytes + 255) & ~(size_t)255, 256);
+    const bool cap = capturing(stream);
     auto it = s->free_blocks.lower_bound(bytes);
     if (it != s->free_blocks.end() && it->first <= bytes + bytes / 4) {
         *out = it->second;
         s->live[*out] = it->first;
         s->free_blocks.erase(it);
+        if (cap) s->pinned_blocks.insert(*out);
         return TFH_OK;
     }
     void* p = nullptr;
     if (int32_t e = malloc_or_release(&p, bytes, stream, "hipMalloc(intermediate)")) return e;
     s->live[p] = bytes;
+    if (cap) s->pinned_blocks.insert(p);
     *out = p;
     return TFH_OK;
 }
@@ -182,6 +222,83 @@ void pool_free(void* stream, void* ptr) {
     s->free_blocks.emplace(it->second, ptr);
     s->live.erase(it);
 }
+
+namespace {
+// Is this host pointer page-locked memory the device can read and write directly?
+bool is_pinned_host(const void* p) {
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();   // ordinary (pageable) memory is unknown to the runtime
+        return false;
+    }
+    return attr.type == hipMemoryTypeHost;
+}
+
+int32_t bounce_buffers(void* stream, StreamScratch** out) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    int32_t err;
+    StreamScratch* s = scratch_for(stream, &err);
+    if (!s) return err;
+    for (int i = 0; i < 2; ++i) {
+        if (!s->bounce[i]) {
+            if (int32_t e = hip_check(hipHostMalloc(&s->bounce[i], BOUNCE_BYTES, hipHostMallocDefault), "hipHostMalloc(staging buffer)")) return e;
+            if (int32_t e = hip_check(hipEventCreateWithFlags(&s->bounce_ev[i], hipEventDisableTiming), "hipEventCreate")) return e;
+        }
+    }
+    *out = s;   // (entries of the map stay where they are: the buffers can be used without the lock)
+    return TFH_OK;
+}
+
+// Pageable host memory cannot be the source or target of an asynchronous copy: the transfer goes through two pinned
+// staging buffers in chunks, the host filling (or emptying) one while the copy engine works on the other, so that the
+// transfer proceeds at the engine's rate and runs beside kernels of other streams.  The call returns when the host side
+// is done: for host-to-device, when the last chunk has been handed to the stream; for device-to-host, when the data is in
+// `dst`.  Pinned memory (tfh_host_malloc) is copied directly and fully asynchronously.
+int32_t wait_bounce(StreamScratch* s, int b) {
+    if (!s->bounce_busy[b]) return TFH_OK;
+    s->bounce_busy[b] = false;
+    return hip_check(hipEventSynchronize(s->bounce_ev[b]), "hipEventSynchronize");
+}
+int32_t staged_h2d(void* dst, const void* src, size_t bytes, void* stream) {
+    StreamScratch* s = nullptr;
+    if (int32_t e = bounce_buffers(stream, &s)) return e;
+    size_t done = 0;
+    for (int i = 0; done < bytes; ++i) {
+        const int b = i & 1;
+        const size_t n = std::min(BOUNCE_BYTES, bytes - done);
+        if (int32_t e = wait_bounce(s, b)) return e;   // the copy that last used this buffer (of this or an earlier call) has finished
+        std::memcpy(s->bounce[b], (const char*)src + done, n);
+        if (int32_t e = hip_check(hipMemcpyAsync((char*)dst + done, s->bounce[b], n, hipMemcpyHostToDevice, (hipStream_t)stream), "hipMemcpyAsync(h2d)")) return e;
+        if (int32_t e = hip_check(hipEventRecord(s->bounce_ev[b], (hipStream_t)stream), "hipEventRecord")) return e;
+        s->bounce_busy[b] = true;
+        done += n;
+    }
+    return TFH_OK;
+}
+int32_t staged_d2h(void* dst, const void* src, size_t bytes, void* stream) {
+    StreamScratch* s = nullptr;
+    if (int32_t e = bounce_buffers(stream, &s)) return e;
+    const size_t nchunks = (bytes + BOUNCE_BYTES - 1) / BOUNCE_BYTES;
+    auto issue = [&](size_t c) {
+        const int b = (int)(c & 1);
+        const size_t at = c * BOUNCE_BYTES, n = std::min(BOUNCE_BYTES, bytes - at);
+        if (int32_t e = wait_bounce(s, b)) return e;   // an earlier host-to-device copy may still be reading it
+        if (int32_t e = hip_check(hipMemcpyAsync(s->bounce[b], (const char*)src + at, n, hipMemcpyDeviceToHost, (hipStream_t)stream), "hipMemcpyAsync(d2h)")) return e;
+        return hip_check(hipEventRecord(s->bounce_ev[b], (hipStream_t)stream), "hipEventRecord");
+    };
+    if (nchunks > 0)
+        if (int32_t e = issue(0)) return e;
+    for (size_t c = 0; c < nchunks; ++c) {
+        if (c + 1 < nchunks)
+            if (int32_t e = issue(c + 1)) return e;   // the engine fills the other buffer while the host empties this one
+        const int b = (int)(c & 1);
+        if (int32_t e = hip_check(hipEventSynchronize(s->bounce_ev[b]), "hipEventSynchronize")) return e;
+        const size_t at = c * BOUNCE_BYTES, n = std::min(BOUNCE_BYTES, bytes - at);
+        std::memcpy((char*)dst + at, s->bounce[b], n);
+    }
+    return TFH_OK;
+}
+}  // namespace
 
 namespace {
 struct ProfRec {
@@ -321,14 +438,29 @@ int32_t tfh_release_workspaces(void) {
     std::lock_guard<std::mutex> lk(tfh::g_mu);
     if (int32_t e = hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize")) return e;
     for (auto& kv : tfh::g_scratch) {
-        if (kv.second.ws) (void)hipFree(kv.second.ws);
-        kv.second.ws = nullptr;
-        kv.second.ws_bytes = 0;
-        for (auto& b : kv.second.free_blocks) (void)hipFree(b.second);
-        kv.second.free_blocks.clear();
-        for (auto& t : kv.second.tables) (void)hipFree(t.second.dev);
-        kv.second.tables.clear();
-        kv.second.table_bytes = 0;
+        auto& sc = kv.second;
+        if (sc.ws && !sc.ws_pinned) {
+            (void)hipFree(sc.ws);
+            sc.ws = nullptr;
+            sc.ws_bytes = 0;
+        }
+        for (auto it = sc.free_blocks.begin(); it != sc.free_blocks.end();) {
+            if (sc.pinned_blocks.count(it->second)) {
+                ++it;
+                continue;
+            }
+            (void)hipFree(it->second);
+            it = sc.free_blocks.erase(it);
+        }
+        for (auto it = sc.tables.begin(); it != sc.tables.end();) {
+            if (it->second.pinned) {
+                ++it;
+                continue;
+            }
+            (void)hipFree(it->second.dev);
+            sc.table_bytes -= it->second.bytes;
+            it = sc.tables.erase(it);
+        }
     }
     return TFH_OK;
 }
@@ -386,11 +518,25 @@ int32_t tfh_malloc(size_t bytes, void** out) {
 }
 int32_t tfh_free(void* ptr) { return hip_check(hipFree(ptr), "hipFree"); }
 int32_t tfh_memcpy_h2d(void* dst, const void* src, size_t bytes, tfh_stream stream) {
-    return hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream), "hipMemcpyAsync(h2d)");
+    if (bytes == 0) return TFH_OK;
+    if (!dst || !src) return set_error(TFH_ERR_INVALID_ARGUMENT, "null pointer");
+    if (tfh::is_pinned_host(src) || tfh::capturing(stream))
+        return hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream), "hipMemcpyAsync(h2d)");
+    return tfh::staged_h2d(dst, src, bytes, stream);
 }
 int32_t tfh_memcpy_d2h(void* dst, const void* src, size_t bytes, tfh_stream stream) {
-    return hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream), "hipMemcpyAsync(d2h)");
+    if (bytes == 0) return TFH_OK;
+    if (!dst || !src) return set_error(TFH_ERR_INVALID_ARGUMENT, "null pointer");
+    if (tfh::is_pinned_host(dst) || tfh::capturing(stream))
+        return hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream), "hipMemcpyAsync(d2h)");
+    return tfh::staged_d2h(dst, src, bytes, stream);
 }
+int32_t tfh_host_malloc(size_t bytes, void** out) {
+    if (!out) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
+    *out = nullptr;
+    return hip_check(hipHostMalloc(out, bytes ? bytes : 1, hipHostMallocDefault), "hipHostMalloc");
+}
+int32_t tfh_host_free(void* ptr) { return hip_check(hipHostFree(ptr), "hipHostFree"); }
 int32_t tfh_memcpy_d2d(void* dst, const void* src, size_t bytes, tfh_stream stream) {
     return hip_check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream), "hipMemcpyAsync(d2d)");
 }

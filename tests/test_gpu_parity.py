@@ -385,7 +385,89 @@ def test_grouped_odd_extents_on_128_tiles(tf, oracle, dtype):
     # (k tails of 1, 2, 5, 6 and 7 elements; edges of 1 and 3 rows), all large enough for 128x128 tiles
     dims = [(129, 1031, 133), (255, 66, 257), (193, 1058, 97), (300, 5, 310), (131, 130, 129), (257, 1025, 129), (300, 6, 310)]
     assert _grouped_case(tf, oracle, dims, dtype, 78) < TOL[dtype]
-    assert "gemm128_kernel" in tf.last_kernel(), tf.last_kernel()
+    assert "gemm128_kernel" in tf.last_kernel() or "gemm128_grouped_kernel" in tf.last_kernel(), tf.last_kernel()
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_grouped_tile_shapes_for_last_strips(tf, oracle, dtype):
+    # extents that leave a last strip of at most 64 rows or 64 real columns (odd multiples of 64, a strip of 1, of 63, of
+    # exactly 64; for complex a strip of 32 elements is 64 real columns) get tiles of that shape -- the row strip runs as
+    # the transposed product -- next to extents whose strip is wider than 64 and stays a padded 128 x 128 tile, extents
+    # below one tile on one side, and a corner where both strips meet; alpha and beta applied
+    dims = [(192, 80, 320), (320, 96, 192), (448, 40, 448), (129, 64, 191), (256, 33, 256), (191, 50, 129), (160, 72, 97),
+            (224, 24, 100), (100, 56, 224), (128, 16, 64), (64, 16, 128), (576, 8, 1088)]
+    from tenferro_rs_amd import inputs
+    As = [inputs.uniform(81, 3 * g, (i, j), dtype) for g, (i, j, k) in enumerate(dims)]
+    Bs = [inputs.uniform(81, 3 * g + 1, (j, k), dtype) for g, (i, j, k) in enumerate(dims)]
+    C0 = [inputs.uniform(81, 3 * g + 2, (i, k), dtype) for g, (i, j, k) in enumerate(dims)]
+    outs = [dev(tf, c) for c in C0]
+    desc = tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik"))
+    plan = tf.HipBackend.plan_grouped(dtype, desc, [[[i, j], [j, k], [i, k]] for (i, j, k) in dims])
+    alpha, beta = (0.7 - 1.1j, -0.3 + 0.2j) if np.issubdtype(dtype, np.complexfloating) else (0.7, -0.3)
+    tf.HipBackend.execute_grouped(plan, alpha, [(dev(tf, a), dev(tf, b)) for a, b in zip(As, Bs)], beta, outs)
+    assert "gemm128_grouped_kernel" in tf.last_kernel(), tf.last_kernel()
+    for a, b, c0, o, d in zip(As, Bs, C0, outs, dims):
+        ref = c0.copy()
+        oracle.contract(a, lab("ij"), b, lab("jk"), ref, lab("ik"), alpha=alpha, beta=beta)
+        assert relerr(o.to_numpy(), ref) < TOL[dtype], d
+
+
+def test_grouped_column_major_operands_and_views(tf, oracle):
+    # column-major blocks (A contiguous along its rows, B along k) and blocks cut out of larger buffers: the other
+    # loader layouts of the grouped kernel, with last strips in both directions
+    rng = np.random.default_rng(82)
+    dims = [(192, 70, 320), (320, 130, 192), (256, 64, 200), (200, 90, 256)]
+    As = [np.asfortranarray(rng.standard_normal((i, j))) for (i, j, k) in dims]
+    Bs = [np.asfortranarray(rng.standard_normal((j, k))) for (i, j, k) in dims]
+    outs = [tf.Tensor.empty([i, k], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64) for (i, j, k) in dims]
+    desc = tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik"))
+    plan = tf.HipBackend.plan_grouped(np.float64, desc, [[[i, j], [j, k], [i, k]] for (i, j, k) in dims])
+    ins = [(dev(tf, a.T).permute([1, 0]), dev(tf, b.T).permute([1, 0])) for a, b in zip(As, Bs)]
+    tf.HipBackend.execute_grouped(plan, 1.0, ins, 0.0, outs)
+    for a, b, o in zip(As, Bs, outs):
+        assert relerr(o.to_numpy(), a @ b) < 1e-12
+    big = [rng.standard_normal((i + 3, j + 8)) for (i, j, k) in dims]
+    bigb = [rng.standard_normal((j + 2, k + 6)) for (i, j, k) in dims]
+    As = [x[1:1 + i, 4:4 + j] for x, (i, j, k) in zip(big, dims)]
+    Bs = [x[2:2 + j, 2:2 + k] for x, (i, j, k) in zip(bigb, dims)]
+    tf.HipBackend.execute_grouped(plan, 1.0, [(dev(tf, a), dev(tf, b)) for a, b in zip(As, Bs)], 0.0, outs)
+    for a, b, o in zip(As, Bs, outs):
+        assert relerr(o.to_numpy(), a @ b) < 1e-12
+
+
+def test_grouped_plan_on_two_streams_with_different_operands(tf, oracle):
+    # one plan, two streams, two operand sets in flight at the same time: the problem records of a call live in the
+    # workspace of its own stream, so neither call sees the other's pointers
+    import ctypes
+    import torch
+    dims = [(192, 256, 320), (320, 192, 192), (256, 128, 256), (128, 320, 448)] * 6
+    rng = np.random.default_rng(83)
+    sets = []
+    for s in range(2):
+        As = [rng.standard_normal((i, j)) for (i, j, k) in dims]
+        Bs = [rng.standard_normal((j, k)) for (i, j, k) in dims]
+        outs = [tf.Tensor.empty([i, k], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64) for (i, j, k) in dims]
+        sets.append((As, Bs, [(dev(tf, a), dev(tf, b)) for a, b in zip(As, Bs)], outs))
+    desc = tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik"))
+    plan = tf.HipBackend.plan_grouped(np.float64, desc, [[[i, j], [j, k], [i, k]] for (i, j, k) in dims])
+    streams = []
+    for _ in range(2):
+        st = ctypes.c_void_p()
+        assert tf.lib().tfh_stream_create(ctypes.byref(st)) == 0
+        streams.append(st)
+    torch.cuda.synchronize()
+    try:
+        for rep in range(4):   # alternate the streams so that launches of both are queued together
+            for (As, Bs, ins, outs), st in zip(sets, streams):
+                tf.HipBackend.execute_grouped(plan, 1.0, ins, 0.0, outs, stream=st.value)
+        for st in streams:
+            assert tf.lib().tfh_stream_synchronize(st) == 0
+        for As, Bs, ins, outs in sets:
+            for a, b, o in zip(As, Bs, outs):
+                assert relerr(o.to_numpy(), a @ b) < 1e-12
+    finally:
+        for st in streams:
+            tf.lib().tfh_stream_destroy(st)
 
 
 @pytest.mark.parametrize("dtype", ALL)
@@ -600,6 +682,146 @@ def test_einsum_async_chaining(tf):
     d.wait()
     assert d.is_ready() and d.event is None
     assert relerr(d.to_numpy(), a @ b @ b) < 1e-12
+
+
+def _new_streams(tf, n):
+    import ctypes
+    out = []
+    for _ in range(n):
+        st = ctypes.c_void_p()
+        assert tf.lib().tfh_stream_create(ctypes.byref(st)) == 0
+        out.append(st)
+    return out
+
+
+def test_chaining_across_two_streams_through_the_completion_event(tf):
+    # tenferro-einsum/src/lib.rs:146-177: the producer runs on one stream, the consumer on another, and the only thing
+    # that orders them is the producer's completion event, which the consumer's stream is made to wait for.  The producer
+    # is long (2 x 2048^3 f64 per call, four calls queued) and the consumer is enqueued at once: without the wait it
+    # would read a half-written operand.  Both the einsum path and TensorPrims::execute.
+    import torch
+    rng = np.random.default_rng(35)
+    n = 2048
+    a = rng.standard_normal((n, n)) / 32
+    b = rng.standard_normal((n, n)) / 32
+    da, db = dev(tf, a), dev(tf, b)
+    sa, sb = _new_streams(tf, 2)
+    torch.cuda.synchronize()
+    try:
+        c = da
+        for _ in range(4):
+            c = tf.einsum("ij,jk->ik", [c, db], stream=sa.value)
+        assert c.event is not None
+        d = tf.einsum("ij,jk->ki", [c, db], stream=sb.value)       # consumer on the other stream
+        d.wait()
+        ref = a @ b @ b @ b @ b
+        assert relerr(d.to_numpy(), (ref @ b).T) < 1e-12
+        # the same through execute(): output.event is set by the producer and waited for by the consumer
+        plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik")), [[n, n], [n, n], [n, n]])
+        x = tf.Tensor.empty([n, n], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+        y = tf.Tensor.empty([n, n], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+        z = tf.Tensor.empty([n, n], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+        torch.cuda.synchronize()
+        tf.HipBackend.execute(plan, 1.0, [da, db], 0.0, x, stream=sa.value)
+        tf.HipBackend.execute(plan, 1.0, [x, db], 0.0, y, stream=sa.value)
+        assert y.event is not None
+        tf.HipBackend.execute(plan, 1.0, [y, db], 0.0, z, stream=sb.value)
+        z.wait()
+        assert relerr(z.to_numpy(), a @ b @ b @ b) < 1e-12
+    finally:
+        torch.cuda.synchronize()
+        for st in (sa, sb):
+            tf.lib().tfh_stream_destroy(st)
+
+
+def test_host_transfers_pageable_and_pinned_round_trip(tf):
+    # tfh_memcpy_h2d / tfh_memcpy_d2h (Tensor::to_memory_space_async): pageable memory goes through the stream's pinned
+    # staging buffers in 16 MiB chunks (sizes below, at and above one and two chunks, odd byte counts), pinned memory
+    # from tfh_host_malloc directly; data comes back bit for bit
+    import ctypes
+    import torch
+    L = tf.lib()
+    (st,) = _new_streams(tf, 1)
+    rng = np.random.default_rng(36)
+    try:
+        for nbytes in [1, 4097, (16 << 20) - 3, 16 << 20, (16 << 20) + 5, (40 << 20) + 1]:
+            src = rng.integers(0, 256, nbytes, dtype=np.uint8)
+            dbuf = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+            back = np.zeros(nbytes, np.uint8)
+            assert L.tfh_memcpy_h2d(dbuf.data_ptr(), src.ctypes.data, nbytes, st) == 0
+            assert L.tfh_memcpy_d2h(back.ctypes.data, dbuf.data_ptr(), nbytes, st) == 0   # returns with the data in place
+            assert np.array_equal(back, src), nbytes
+            assert np.array_equal(dbuf.cpu().numpy(), src), nbytes
+        # pinned: the calls return at once; the stream orders the copies
+        nbytes = (24 << 20) + 7
+        hp, hq = ctypes.c_void_p(), ctypes.c_void_p()
+        assert L.tfh_host_malloc(nbytes, ctypes.byref(hp)) == 0 and L.tfh_host_malloc(nbytes, ctypes.byref(hq)) == 0
+        src = rng.integers(0, 256, nbytes, dtype=np.uint8)
+        ctypes.memmove(hp.value, src.ctypes.data, nbytes)
+        dbuf = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        assert L.tfh_memcpy_h2d(dbuf.data_ptr(), hp, nbytes, st) == 0
+        assert L.tfh_memcpy_d2h(hq, dbuf.data_ptr(), nbytes, st) == 0
+        assert L.tfh_stream_synchronize(st) == 0
+        back = np.ctypeslib.as_array(ctypes.cast(hq.value, ctypes.POINTER(ctypes.c_uint8)), shape=(nbytes,))
+        assert np.array_equal(back, src)
+        assert L.tfh_host_free(hp) == 0 and L.tfh_host_free(hq) == 0
+    finally:
+        L.tfh_stream_destroy(st)
+
+
+def test_host_to_device_copy_runs_beside_a_contraction_on_another_stream(tf):
+    # a staged transfer from pageable memory on stream A and contractions on stream B, each alone and then together
+    # (the transfer from a second host thread, because its host side is busy copying into the staging buffers): together
+    # they must take clearly less than one after the other
+    import threading
+    import time
+    import torch
+    L = tf.lib()
+    sa, sb = _new_streams(tf, 2)
+    n = 3072
+    da = tf.Tensor.from_torch(torch.randn(n, n, dtype=torch.float64, device="cuda"))
+    db = tf.Tensor.from_torch(torch.randn(n, n, dtype=torch.float64, device="cuda"))
+    dc = tf.Tensor.empty([n, n], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik")), [[n, n], [n, n], [n, n]])
+    nbytes = 192 << 20
+    src = np.ones(nbytes, np.uint8)
+    dbuf = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+
+    def copy():
+        assert L.tfh_memcpy_h2d(dbuf.data_ptr(), src.ctypes.data, nbytes, sa) == 0
+        assert L.tfh_stream_synchronize(sa) == 0
+
+    def timed(fn):
+        t0 = time.perf_counter()
+        fn()
+        return time.perf_counter() - t0
+
+    try:
+        copy()                                                        # staging buffers allocated, pages touched
+        t_copy = min(timed(copy) for _ in range(3))
+        reps = 1
+        def compute():
+            for _ in range(reps):
+                tf.HipBackend.execute(plan, 1.0, [da, db], 0.0, dc, stream=sb.value)
+            assert L.tfh_stream_synchronize(sb) == 0
+        compute()
+        t_one = min(timed(compute) for _ in range(3))
+        reps = max(1, int(round(t_copy / t_one)))                     # about as much compute as the copy takes
+        t_comp = min(timed(compute) for _ in range(3))
+
+        def both():
+            th = threading.Thread(target=copy)
+            th.start()
+            compute()
+            th.join()
+        t_both = min(timed(both) for _ in range(3))
+        print("copy %.2f ms, compute %.2f ms, together %.2f ms" % (t_copy * 1e3, t_comp * 1e3, t_both * 1e3))
+        assert t_both < t_copy + t_comp - 0.4 * min(t_copy, t_comp), (t_copy, t_comp, t_both)
+    finally:
+        torch.cuda.synchronize()
+        for st in (sa, sb):
+            L.tfh_stream_destroy(st)
 
 
 def test_execute_errors(tf):
@@ -1200,6 +1422,65 @@ def test_calls_are_capturable_in_a_hip_graph_and_replay_correctly(tf, oracle):
         assert oP.to_numpy().tobytes() == p.tobytes(), replay
         assert relerr(oR.to_numpy(), r) < 1e-12, replay
         assert relerr(oE.to_numpy(), e) < 1e-12, replay
+
+
+def test_graph_replays_after_the_workspace_grew_and_the_caches_were_released(tf, oracle):
+    # A captured graph holds the addresses of the workspace, the offset tables and the intermediates its calls were
+    # given.  Later eager work on the same stream that needs a larger workspace, and tfh_release_workspaces, must leave
+    # those buffers alone (they are retired or passed over, never freed): the graph is replayed afterwards on new
+    # contents and must still give the eager result.
+    import torch
+    rng = np.random.default_rng(55)
+    A = rand(rng, (8, 32, 16, 48), np.float64)        # "ajbk,kcj->abc": packing, offset tables, split-K partials
+    B = rand(rng, (48, 64, 32), np.float64)
+    E1, E2, E3 = rand(rng, (40, 50), np.float64), rand(rng, (50, 30), np.float64), rand(rng, (30, 20), np.float64)
+    tA, tB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    tE = [torch.from_numpy(x).cuda() for x in (E1, E2, E3)]
+    dA, dB = tf.Tensor.from_torch(tA), tf.Tensor.from_torch(tB)
+    dE = [tf.Tensor.from_torch(t) for t in tE]
+    gpu0 = tf.GpuMemory(0)
+    oC = tf.Tensor.empty([8, 16, 64], gpu0, tf.MemoryOrder.RowMajor, np.float64)
+    oE = tf.Tensor.empty([40, 20], gpu0, tf.MemoryOrder.RowMajor, np.float64)
+    pc = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Contract(lab("ajbk"), lab("kcj"), lab("abc")), [A.shape, B.shape, [8, 16, 64]])
+    tree = tf.ContractionTree.optimize(tf.Subscripts.parse("ij,jk,kl->il"), [E1.shape, E2.shape, E3.shape])
+
+    def work():
+        tf.HipBackend.execute(pc, 1.0, [dA, dB], 0.0, oC)
+        tf.einsum_with_plan_into(tree, dE, 1.0, 0.0, oE)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()
+    side.synchronize()
+    oC.event = oE.event = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        work()
+    # eager work on the capture stream that needs a much larger workspace (a long k over few tiles: split-K partials)
+    big_a = tf.Tensor.from_torch(torch.randn(256, 1 << 15, dtype=torch.float64, device="cuda"))
+    big_b = tf.Tensor.from_torch(torch.randn(1 << 15, 256, dtype=torch.float64, device="cuda"))
+    big_c = tf.Tensor.empty([256, 256], gpu0, tf.MemoryOrder.RowMajor, np.float64)
+    pbig = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Contract(lab("mk"), lab("kn"), lab("mn")), [[256, 1 << 15], [1 << 15, 256], [256, 256]])
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        tf.HipBackend.execute(pbig, 1.0, [big_a, big_b], 0.0, big_c)
+    side.synchronize()
+    assert tf.lib().tfh_release_workspaces() == 0
+    # fresh allocations that would land in freed memory if anything of the graph's had been freed
+    filler = [torch.full((1 << 20,), float("nan"), dtype=torch.float64, device="cuda") for _ in range(8)]
+    for replay in range(2):
+        for t in [tA, tB] + tE:
+            t.mul_(-0.5).add_(0.25 * (replay + 1))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        c = np.empty((8, 16, 64))
+        oracle.contract(tA.cpu().numpy(), lab("ajbk"), tB.cpu().numpy(), lab("kcj"), c, lab("abc"))
+        e = tE[0].cpu().numpy() @ tE[1].cpu().numpy() @ tE[2].cpu().numpy()
+        assert relerr(oC.to_numpy(), c) < 1e-12, replay
+        assert relerr(oE.to_numpy(), e) < 1e-12, replay
+    del filler
 
 
 def test_owned_variant_keeps_intermediates_in_donated_operand_buffers(tf, oracle):
