@@ -152,6 +152,8 @@ struct StridedView {
     std::vector<size_t> dims;
     std::vector<ptrdiff_t> strides;
     ptrdiff_t offset = 0;
+    bool conj = false;   // read as the complex conjugate (TFH_VIEW_CONJ): Contract / Permute inputs and einsum operands only
+    StridedView conjugated() const { StridedView v = *this; v.conj = !conj; return v; }
     tfh_view raw() const {
         if (dims.size() > TFH_MAX_RANK) throw Error::InvalidArgument("rank above 16");
         tfh_view v;
@@ -159,6 +161,7 @@ struct StridedView {
         v.base = (void*)data;
         v.rank = (int32_t)dims.size();
         v.offset = offset;
+        v.flags = conj ? TFH_VIEW_CONJ : 0;
         for (size_t i = 0; i < dims.size(); ++i) { v.dims[i] = (int64_t)dims[i]; v.strides[i] = (int64_t)strides[i]; }
         return v;
     }

@@ -81,11 +81,18 @@ size_t tfh_dtype_size(int32_t dtype);
 typedef struct tfh_view {
     void* base;
     int32_t rank;
-    int32_t reserved;
+    int32_t flags;        /* TFH_VIEW_* bits; 0 for a plain view */
     int64_t offset;
     int64_t dims[TFH_MAX_RANK];
     int64_t strides[TFH_MAX_RANK];
 } tfh_view;
+
+/* TFH_VIEW_CONJ on an INPUT view of a complex dtype: the operation reads conj(element) instead of the element, without
+ * a conjugated copy -- the lazy form of Tensor::conj (tenferro-tensor/src/lib.rs:622-658), an addition to the
+ * reference's views.  Honoured by Contract, BatchedGemm, Permute and by the operands of tfh_einsum_execute: the
+ * contraction kernels flip the sign of the imaginary part while they stage the operand.  Ignored for real dtypes; any
+ * other operation, an output view and a grouped plan reject it with TFH_ERR_INVALID_ARGUMENT. */
+#define TFH_VIEW_CONJ 1
 
 /* ---- operation descriptor: PrimDescriptor (tenferro-prims/src/lib.rs:152-245) */
 typedef enum tfh_op {

@@ -28,7 +28,7 @@ _DT_NP = {v: k for k, v in _NP_DTYPES.items()}
 
 # ---------------------------------------------------------------------------------------------- C structs
 class tfh_view(C.Structure):
-    _fields_ = [("base", C.c_void_p), ("rank", C.c_int32), ("reserved", C.c_int32), ("offset", C.c_int64),
+    _fields_ = [("base", C.c_void_p), ("rank", C.c_int32), ("flags", C.c_int32), ("offset", C.c_int64),
                 ("dims", C.c_int64 * MAX_RANK), ("strides", C.c_int64 * MAX_RANK)]
 
 
@@ -647,6 +647,7 @@ class Tensor:
         self.logical_memory_space_, self.dtype, self.event = space, dtype, event
         self.preferred_compute_device_ = preferred
         self._lib_alloc = False     # the buffer was allocated by this module (not wrapped from the caller's tensor)
+        self._conj = False          # conj_on_load(): operations read conj(element) (TFH_VIEW_CONJ)
 
     def _sole_owner(self):
         """No other Tensor (a permute/broadcast/diagonal view) and no caller-held object shares the buffer."""
@@ -739,6 +740,18 @@ class Tensor:
         t = Tensor(self._buf, dims, strides, self._offset if offset is None else offset, self.logical_memory_space_,
                    self.dtype, self.event, self.preferred_compute_device_)
         t._lib_alloc = self._lib_alloc
+        t._conj = self._conj
+        return t
+
+    def conj_on_load(self):
+        """The lazy form of conj() (no counterpart in the reference, whose conj materialises): a view of the same buffer
+        that contractions, permutes and einsum read as conj(element) -- the kernels flip the sign of the imaginary part
+        while they stage the operand, so nothing is copied.  Real tensors come back unchanged.  The view and the views
+        made of it (permute, broadcast, diagonal) keep the flag; conj() of such a view is a plain copy, into_conj() just
+        drops the flag; it cannot be the output of an operation, and host access goes through conj() or to_numpy()."""
+        t = self._like(self._dims, self._strides)
+        if dtype_code(self.dtype) in (C64, C128):
+            t._conj = not self._conj
         return t
 
     def permute(self, perm):
@@ -792,6 +805,7 @@ class Tensor:
         v = tfh_view()
         v.base = self._buf.data_ptr()
         v.rank = len(self._dims)
+        v.flags = 1 if self._conj else 0      # TFH_VIEW_CONJ
         v.offset = self._offset
         for d in range(len(self._dims)):
             v.dims[d], v.strides[d] = self._dims[d], self._strides[d]
@@ -828,6 +842,9 @@ class Tensor:
         """:653-658: in place when the tensor lives on the device."""
         if self.logical_memory_space_.kind == 0:
             return self.conj()
+        if self._conj:                       # conj of a lazily conjugated view: the stored elements themselves
+            self._conj = False
+            return self
         vi = self._view()
         st = current_stream()
         _check(lib().tfh_conj(self.dtype, C.byref(vi), C.byref(vi), st))
@@ -841,6 +858,8 @@ class Tensor:
         self.wait()
         if self.logical_memory_space_.kind != 0:
             raise InvalidArgument("invalid argument: view() of a tensor in GPU memory; copy it with to_memory_space_async first")
+        if self._conj:
+            raise InvalidArgument("invalid argument: view() of a lazily conjugated tensor; materialise it with conj() first")
         return self._host_view(False)
 
     def _host_view(self, writeable):
@@ -863,6 +882,8 @@ class Tensor:
         """:660-671: same space -> self; Main->Gpu / Gpu->Main copy the underlying buffer."""
         if target == self.logical_memory_space_:
             return self
+        if self._conj:
+            raise InvalidArgument("invalid argument: a lazily conjugated tensor does not change memory space; materialise it with conj() first")
         import torch
         if target.kind == 1:
             buf = torch.from_numpy(np.ascontiguousarray(self._buf)).to(f"cuda:{target.space_id}", non_blocking=True)
@@ -887,7 +908,8 @@ class Tensor:
         self.wait()
         flat = self._buf if self.logical_memory_space_.kind == 0 else self._buf.cpu().numpy().ravel()
         isz = flat.dtype.itemsize
-        return np.lib.stride_tricks.as_strided(flat[self._offset:], self._dims, [s * isz for s in self._strides]).copy()
+        out = np.lib.stride_tricks.as_strided(flat[self._offset:], self._dims, [s * isz for s in self._strides]).copy()
+        return np.conj(out) if self._conj else out
 
 
 # ---------------------------------------------------------------------------------------------- einsum entry points

@@ -676,6 +676,7 @@ struct Operand {          // a node as the executor sees it: unique labels + str
     std::vector<int64_t> dims, strides;
     char* ptr = nullptr;
     void* owned = nullptr;   // pool block to release once consumed
+    bool conj = false;       // read as conj(element): an input view flagged TFH_VIEW_CONJ (complex dtypes)
 };
 
 // Diagonal view over repeated labels (zero-copy, tenferro-tensor/src/lib.rs:518-529).
@@ -700,7 +701,7 @@ int64_t count(const std::vector<int64_t>& dims) {
     return n;
 }
 
-// dst[dst_labels] = alpha * sum over missing labels of src + beta*dst
+// dst[dst_labels] = alpha * sum over missing labels of op(src) + beta*dst, op = conj when src.conj
 int32_t reduce_or_copy(int dtype, const Operand& src, const Operand& dst, Scalar alpha, Scalar beta, void* stream) {
     std::vector<Axis> kept, red;
     for (size_t d = 0; d < dst.labels.size(); ++d) {
@@ -709,8 +710,31 @@ int32_t reduce_or_copy(int dtype, const Operand& src, const Operand& dst, Scalar
     }
     for (size_t j = 0; j < src.labels.size(); ++j)
         if (find(dst.labels, src.labels[j]) < 0) red.push_back(Axis{src.dims[j], {src.strides[j], 0, 0}, src.labels[j]});
-    if (red.empty()) return launch_copy(dtype, src.ptr, dst.ptr, kept, alpha, beta, false, stream);
-    return launch_reduce(dtype, src.ptr, dst.ptr, kept, red, TFH_REDUCE_SUM, alpha, beta, stream);
+    if (red.empty()) return launch_copy(dtype, src.ptr, dst.ptr, kept, alpha, beta, src.conj, stream);
+    if (!src.conj) return launch_reduce(dtype, src.ptr, dst.ptr, kept, red, TFH_REDUCE_SUM, alpha, beta, stream);
+    // a flagged operand that is summed: a conjugated dense copy first (the reduction kernels do not conjugate)
+    std::vector<Axis> all;
+    int64_t n = 1;
+    for (size_t j = src.labels.size(); j-- > 0;) {
+        all.push_back(Axis{src.dims[j], {src.strides[j], n, 0}, src.labels[j]});
+        n *= src.dims[j];
+    }
+    void* tmp = nullptr;
+    if (int32_t e = pool_alloc(stream, (size_t)std::max<int64_t>(n, 1) * dtype_size(dtype), &tmp)) return e;
+    int32_t e = launch_copy(dtype, src.ptr, tmp, all, Scalar{1, 0}, Scalar{0, 0}, true, stream);
+    if (!e) {
+        Operand dense = src;
+        dense.ptr = (char*)tmp;
+        dense.conj = false;
+        int64_t st = 1;
+        for (size_t j = src.labels.size(); j-- > 0;) {
+            dense.strides[j] = st;
+            st *= src.dims[j];
+        }
+        e = reduce_or_copy(dtype, dense, dst, alpha, beta, stream);
+    }
+    pool_free(stream, tmp);
+    return e;
 }
 }  // namespace
 
@@ -728,6 +752,7 @@ int32_t tfh_einsum_execute(int32_t dtype, const tfh_tree* tree, const tfh_view* 
     }
     if (int32_t e = check_view_against(t.output_dims, *output, "output")) return e;
     if (!output->base) return set_error(TFH_ERR_INVALID_ARGUMENT, "output has a null base pointer");
+    if (output->flags & TFH_VIEW_CONJ) return set_error(TFH_ERR_INVALID_ARGUMENT, "TFH_VIEW_CONJ on an output view");
     const Scalar al = load_scalar(dtype, alpha), be = load_scalar(dtype, beta);
     const size_t eb = dtype_size(dtype);
     const Scalar one{1, 0}, zero{0, 0};
@@ -754,6 +779,7 @@ int32_t tfh_einsum_execute(int32_t dtype, const tfh_tree* tree, const tfh_view* 
     // leaves: diagonal views; labels private to one operand are summed into a temporary first
     for (int i = 0; i < n_operands; ++i) {
         Operand v = unique_view(t.input_labels[i], operands[i].dims, operands[i].strides, view_ptr(operands[i], dtype));
+        v.conj = (operands[i].flags & TFH_VIEW_CONJ) && is_complex(dtype);
         const TreeNode& leaf = t.nodes[i];
         if (n_operands == 1 || v.labels.size() == leaf.labels.size()) {
             nodes[i] = v;
@@ -878,7 +904,7 @@ int32_t tfh_einsum_execute(int32_t dtype, const tfh_tree* tree, const tfh_view* 
         ContractAxes ax;
         int32_t e = classify_contract(A.labels, A.dims.data(), A.strides.data(), B.labels, B.dims.data(), B.strides.data(), C.labels,
                                       C.dims.data(), C.strides.data(), ax);
-        if (!e) e = launch_contract(dtype, A.ptr, B.ptr, C.ptr, ax, last ? al : one, last ? be_final : zero, stream);
+        if (!e) e = launch_contract(dtype, A.ptr, B.ptr, C.ptr, ax, last ? al : one, last ? be_final : zero, stream, (A.conj ? 1 : 0) | (B.conj ? 2 : 0));
         // operands of this step are dead once its kernels are enqueued (stream order protects them)
         for (int side = 0; side < 2; ++side) {
             Operand& o = nodes[side ? t.steps[s].rhs : t.steps[s].lhs];

@@ -110,8 +110,9 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
 int32_t launch_reduce_general(int dtype, const void* a, const void* b, void* c, std::vector<Axis> kept, std::vector<Axis> red,
                               int reduce_op, Scalar alpha, Scalar beta, void* stream);
 // C = alpha*A*B + beta*C over classified axes
+// conj: bit 0 = conj(A), bit 1 = conj(B) (see k_gemm.hip)
 int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes axes, Scalar alpha,
-                        Scalar beta, void* stream);
+                        Scalar beta, void* stream, int conj = 0);
 // A tiny operator (<= 8 free and <= 8 contracted indices) applied to a long tensor: the streaming kernel of
 // k_gemm_tiny.hip.  Returns false when the shape is not one it takes; true when it launched (status holds the outcome).
 bool try_tiny_operator(int dtype, const void* a, const void* b, void* c, const ContractAxes& ax, Scalar alpha, Scalar beta,

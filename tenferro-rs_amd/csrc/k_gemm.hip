@@ -538,8 +538,64 @@ int bke_of(int dtype) {
 
 }  // namespace
 
+namespace {
+int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, ContractAxes ax, Scalar alpha, Scalar beta,
+                             void* stream, bool conj_a, bool conj_b);
+}
+
+// conj: bit 0 = use conj(A), bit 1 = use conj(B) (complex dtypes; ignored for real ones).  The tiled and the streaming
+// MFMA kernels conjugate an operand while they stage it (a sign flip on the way into LDS or into the registers), so a
+// flagged operand costs nothing.  Shapes that go to the kernels without that flip -- a free group of at most eight
+// indices: the tiny-operator, product-reduction and elementwise kernels -- get a conjugated copy of the flagged operand
+// first (one pass of the copy kernel over it).
 int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes ax, Scalar alpha, Scalar beta,
-                        void* stream) {
+                        void* stream, int conj) {
+    bool ca = (conj & 1) != 0 && is_complex(dtype), cb = (conj & 2) != 0 && is_complex(dtype);
+    if (!ca && !cb) return launch_contract_impl(dtype, a, b, c, ax, alpha, beta, stream, false, false);
+    const int64_t M = prod(ax.M), N = prod(ax.N);
+    if (M > 8 && N > 8) return launch_contract_impl(dtype, a, b, c, ax, alpha, beta, stream, ca, cb);
+    const size_t eb = dtype_size(dtype);
+    void* copies[2] = {nullptr, nullptr};
+    auto release = [&]() {
+        for (void* p : copies) pool_free(stream, p);
+    };
+    for (int slot = 0; slot < 2; ++slot) {
+        if (!(slot == 0 ? ca : cb)) continue;
+        // the operand's axes (those it has a stride on), densely re-strided in the order of their present strides
+        std::vector<Axis*> mine;
+        for (auto* grp : {&ax.batch, &ax.M, &ax.N, &ax.K})
+            for (auto& x : *grp)
+                if (x.s[slot] != 0 && x.n > 1) mine.push_back(&x);
+        std::stable_sort(mine.begin(), mine.end(), [slot](const Axis* x, const Axis* y) { return std::llabs(x->s[slot]) > std::llabs(y->s[slot]); });
+        int64_t elems = 1;
+        for (auto* x : mine) elems *= x->n;
+        if (int32_t e = pool_alloc(stream, (size_t)std::max<int64_t>(elems, 1) * eb, &copies[slot])) {
+            release();
+            return e;
+        }
+        std::vector<Axis> cp;
+        int64_t stride = 1;
+        for (size_t q = mine.size(); q-- > 0;) {
+            cp.push_back(Axis{mine[q]->n, {mine[q]->s[slot], stride, 0}, mine[q]->label});
+            mine[q]->s[slot] = stride;
+            stride *= mine[q]->n;
+        }
+        Scalar one, zero;
+        one.re = 1;
+        if (int32_t e = launch_copy(dtype, slot == 0 ? a : b, copies[slot], cp, one, zero, true, stream)) {
+            release();
+            return e;
+        }
+        (slot == 0 ? a : b) = copies[slot];
+    }
+    const int32_t e = launch_contract_impl(dtype, a, b, c, ax, alpha, beta, stream, false, false);
+    release();   // stream-ordered: the next user of these blocks is enqueued after the contraction
+    return e;
+}
+
+namespace {
+int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, ContractAxes ax, Scalar alpha, Scalar beta,
+                             void* stream, bool conj_a, bool conj_b) {
     const int rb = is_double(dtype) ? 8 : 4;
     const size_t eb = dtype_size(dtype);
     if (((uintptr_t)a % eb) || ((uintptr_t)b % eb) || ((uintptr_t)c % rb))
@@ -561,11 +617,11 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     // One free group empty (matrix-vector, vector-matrix, dot and batched dot products): there is nothing for a tile
     // of MFMAs to reuse -- a reduction of the elementwise product, bound by HBM (k_dot.hip)
     // a tiny operator applied to a long tensor (a gate on a leg of a state): a stream over the long operand
-    if (M > 1 && N > 1) {
+    if (M > 1 && N > 1 && !conj_a && !conj_b) {
         int32_t st_tiny = TFH_OK;
         if (try_tiny_operator(dtype, a, b, c, ax, alpha, beta, stream, st_tiny)) return st_tiny;
     }
-    if (M == 1 || N == 1) {
+    if ((M == 1 || N == 1) && !conj_a && !conj_b) {
         std::vector<Axis> kept, red = ax.K;
         for (auto* grp : {&ax.batch, &ax.M, &ax.N})
             for (auto& x : *grp) kept.push_back(x);
@@ -605,6 +661,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     // lanes of the epilogue run along n: put C's fastest axis in the N group (swap operands if needed)
     if (min_stride(ax.M, 2) < min_stride(ax.N, 2)) {
         std::swap(a, b);
+        std::swap(conj_a, conj_b);
         std::swap(ax.M, ax.N);
         std::swap(M, N);
         for (auto* grp : {&ax.batch, &ax.M, &ax.N, &ax.K})
@@ -618,6 +675,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         const bool streamable = (dtype == TFH_F64 || dtype == TFH_C128) && M <= SKINNY_MAX_M && K * ec <= SKINNY_MAX_KR && N >= 4096;
         if (M < 96 && M * ec >= 33 && N * ec >= 96 && !streamable) {
             std::swap(a, b);
+            std::swap(conj_a, conj_b);
             std::swap(ax.M, ax.N);
             std::swap(M, N);
             for (auto* grp : {&ax.batch, &ax.M, &ax.N, &ax.K})
@@ -671,12 +729,13 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
                 x.s[slot] = stride;
                 stride *= x.n;
             }
-        if (int32_t e = launch_copy(dtype, slot == 0 ? a : b, buf, cp, Scalar{1, 0}, Scalar{0, 0}, false, stream)) {
+        // (a flagged operand is conjugated by this copy, which it needs anyway)
+        if (int32_t e = launch_copy(dtype, slot == 0 ? a : b, buf, cp, Scalar{1, 0}, Scalar{0, 0}, slot == 0 ? conj_a : conj_b, stream)) {
             release_packed();
             return e;
         }
-        if (slot == 0) { a = buf; a_kfast = true; }
-        else { b = buf; b_kfast = true; }
+        if (slot == 0) { a = buf; a_kfast = true; conj_a = false; }
+        else { b = buf; b_kfast = true; conj_b = false; }
     }
     fuse_axes(ax.M, 3);
     fuse_axes(ax.N, 3);
@@ -706,6 +765,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
              std::llabs(in.s[2]) * SKINNY_UNIT * (int64_t)eb < ((int64_t)1 << 31);
         if (ok) {
             std::swap(a, b);
+            std::swap(conj_a, conj_b);
             std::swap(ax.M, ax.N);
             std::swap(M, N);
             std::swap(a_kfast, b_kfast);
@@ -750,6 +810,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     g.A = a; g.B = b; g.C = c;
     g.M = M; g.N = N; g.K = K; g.nbatch = nb;
     g.a_kfast = a_kfast; g.b_kfast = b_kfast;
+    g.conj_a = conj_a; g.conj_b = conj_b;
     g.alpha_re = alpha.re; g.alpha_im = alpha.im; g.beta_re = beta.re; g.beta_im = beta.im;
     g.use_beta = !beta.is_zero();
 
@@ -965,6 +1026,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         sk.M = (int32_t)M; sk.K = (int32_t)K;
         sk.kc = (int32_t)(cxd ? K : K / 2);
         sk.use_beta = g.use_beta;
+        sk.conj_a = conj_a; sk.conj_b = conj_b;
         sk.out_rows = out_rows;
         sk.plain = alpha.re == 1.0 && alpha.im == 0.0 && beta.is_zero();
         sk.units = Ntab;
@@ -1018,6 +1080,7 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
     }
     return TFH_OK;
 }
+}  // namespace
 
 // ---- grouped launch ------------------------------------------------------------------------------------------
 struct GroupedState {

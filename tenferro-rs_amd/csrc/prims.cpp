@@ -42,7 +42,8 @@ int32_t exec_permute(const tfh_plan& p, Scalar alpha, const tfh_view& a, Scalar 
         int j = find(p.modes_a, p.modes_c[d]);
         ax.push_back(Axis{b.dims[d], {a.strides[j], b.strides[d], 0}, p.modes_c[d]});
     }
-    return launch_copy(p.dtype, view_ptr(a, p.dtype), view_ptr(b, p.dtype), ax, alpha, beta, false, stream);
+    const bool conj = (a.flags & TFH_VIEW_CONJ) && is_complex(p.dtype);
+    return launch_copy(p.dtype, view_ptr(a, p.dtype), view_ptr(b, p.dtype), ax, alpha, beta, conj, stream);
 }
 
 int32_t reduce_moded(int dtype, const char* a_ptr, const ModedView& a, char* c_ptr, const tfh_view& c,
@@ -103,6 +104,13 @@ int32_t tfh_execute(const tfh_plan* plan, const void* alpha, const tfh_view* inp
     const int dt = plan->dtype;
     const Scalar al = load_scalar(dt, alpha), be = load_scalar(dt, beta);
     int32_t e = TFH_OK;
+    // TFH_VIEW_CONJ: inputs of Contract, BatchedGemm and Permute only
+    if (output->flags & TFH_VIEW_CONJ) return set_error(TFH_ERR_INVALID_ARGUMENT, "TFH_VIEW_CONJ on an output view");
+    int conj = 0;
+    for (int t = 0; t < n_inputs; ++t)
+        if ((inputs[t].flags & TFH_VIEW_CONJ) && is_complex(dt)) conj |= 1 << t;
+    if (conj && plan->op != TFH_OP_CONTRACT && plan->op != TFH_OP_BATCHED_GEMM && plan->op != TFH_OP_PERMUTE)
+        return set_error(TFH_ERR_INVALID_ARGUMENT, "TFH_VIEW_CONJ is honoured by Contract, BatchedGemm and Permute only (operation %d)", plan->op);
     switch (plan->op) {
         case TFH_OP_PERMUTE: e = exec_permute(*plan, al, inputs[0], be, *output, stream); break;
         case TFH_OP_REDUCE: {
@@ -130,7 +138,7 @@ int32_t tfh_execute(const tfh_plan* plan, const void* alpha, const tfh_view* inp
             ContractAxes ax;
             e = classify_contract(plan->modes_a, inputs[0].dims, inputs[0].strides, plan->modes_b, inputs[1].dims, inputs[1].strides,
                                   plan->modes_c, output->dims, output->strides, ax);
-            if (!e) e = launch_contract(dt, view_ptr(inputs[0], dt), view_ptr(inputs[1], dt), view_ptr(*output, dt), ax, al, be, stream);
+            if (!e) e = launch_contract(dt, view_ptr(inputs[0], dt), view_ptr(inputs[1], dt), view_ptr(*output, dt), ax, al, be, stream, conj);
             break;
         }
         default: e = set_error(TFH_ERR_INVALID_ARGUMENT, "unknown operation %d", plan->op);
@@ -144,6 +152,9 @@ int32_t tfh_execute_grouped(const tfh_plan* plan, const void* alpha, const tfh_v
     if (!plan || !alpha || !beta || !outputs || !inputs) return set_error(TFH_ERR_INVALID_ARGUMENT, "null argument");
     if (!plan->n_groups) return set_error(TFH_ERR_INVALID_ARGUMENT, "not a grouped plan");
     if (n_inputs != 2) return set_error(TFH_ERR_INVALID_ARGUMENT, "grouped contraction takes 2 inputs per group, got %d", n_inputs);
+    for (int i = 0; i < plan->n_groups; ++i)
+        if ((inputs[2 * i].flags | inputs[2 * i + 1].flags | outputs[i].flags) & TFH_VIEW_CONJ)
+            return set_error(TFH_ERR_INVALID_ARGUMENT, "TFH_VIEW_CONJ is not taken by a grouped plan (group %d)", i);
     int32_t e = launch_grouped(*plan, load_scalar(plan->dtype, alpha), inputs, load_scalar(plan->dtype, beta), outputs, stream);
     if (!e) clear_error();
     return e;
@@ -175,7 +186,10 @@ int32_t tfh_conj(int32_t dtype, const tfh_view* in, tfh_view* out, tfh_stream st
     std::vector<Axis> ax;
     if (int32_t e = view_axes(in, ax, 0)) return e;
     if (int32_t e = view_axes(out, ax, 1)) return e;
-    int32_t e = launch_copy(dtype, view_ptr(*in, dtype), view_ptr(*out, dtype), ax, Scalar{1, 0}, Scalar{0, 0}, true, stream);
+    if (out->flags & TFH_VIEW_CONJ) return set_error(TFH_ERR_INVALID_ARGUMENT, "TFH_VIEW_CONJ on an output view");
+    // (the conjugate of a view that is already read conjugated is a plain copy)
+    const bool conj = !((in->flags & TFH_VIEW_CONJ) && is_complex(dtype));
+    int32_t e = launch_copy(dtype, view_ptr(*in, dtype), view_ptr(*out, dtype), ax, Scalar{1, 0}, Scalar{0, 0}, conj, stream);
     if (!e) clear_error();
     return e;
 }

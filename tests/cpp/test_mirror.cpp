@@ -216,6 +216,19 @@ static void gpu_checks() {
         CHECK(rel_frobenius(out.to_vec(), expect) < 1e-12);
         auto Yback = std::move(Yc).into_conj();
         CHECK(Yback.to_vec() == hy);   // conj twice is the identity, bit for bit
+        // the same conjugate without a copy: a view flagged conjugate-on-load as an input of Contract
+        auto XY = Tensor<c128>::zeros({p, r}, gpu, MemoryOrder::RowMajor);
+        auto cplan = HipBackend::plan<c128>(PrimDescriptor::Contract({0, 1}, {1, 2}, {0, 2}), {{p, q}, {q, r}, {p, r}});
+        auto xv = X.view();
+        auto yv = Yback.view().conjugated();
+        auto xyv = XY.view_mut();
+        HipBackend::execute<c128>(cplan, c128(1), {&xv, &yv}, c128(0), xyv);
+        XY.mark(nullptr);
+        std::vector<c128> exy(p * r, c128(0));
+        for (size_t i = 0; i < p; ++i)
+            for (size_t k = 0; k < r; ++k)
+                for (size_t j = 0; j < q; ++j) exy[i * r + k] += hx[i * q + j] * std::conj(hy[j * r + k]);
+        CHECK(rel_frobenius(XY.to_vec(), exy) < 1e-12);
     }
 
     // TensorPrims::plan / execute on views: Permute is bit-exact, Reduce and ElementwiseMul follow alpha/beta

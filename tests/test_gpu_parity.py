@@ -684,6 +684,94 @@ def test_einsum_async_chaining(tf):
     assert relerr(d.to_numpy(), a @ b @ b) < 1e-12
 
 
+# ------------------------------------------------------------------------------------------------ conj on load
+def _contract_np(a, ma, b, mb, mc):
+    return np.einsum(f"{ma},{mb}->{mc}", a, b, optimize=True)
+
+
+@pytest.mark.parametrize("dtype", [np.complex64, np.complex128])
+def test_conj_on_load_in_every_contraction_kernel(tf, dtype):
+    # TFH_VIEW_CONJ (Tensor.conj_on_load): the operand is read as its conjugate, with no conjugated copy, by the four MFMA
+    # contraction kernels; shapes that go to the other kernels get a conjugated copy first.  Each shape with the flag on
+    # A, on B and on both, alpha and beta complex, against numpy on explicitly conjugated operands; the routing is
+    # checked so that every kernel's sign flip is exercised, including the paths that exchange the operands.
+    rng = np.random.default_rng(61)
+    tol = TOL[dtype]
+    cases = [   # (modes a, modes b, modes c, extents, substring of the kernel label expected)
+        ("mk", "kn", "mn", dict(m=1500, k=150, n=1000), ", 128>)"),
+        ("mk", "kn", "nm", dict(m=1500, k=150, n=1000), ", 128>)"),             # C's fastest axis is m: operands exchanged
+        ("km", "nk", "mn", dict(m=1500, k=150, n=1000), ", 128>)"),             # A column-contiguous, B k-contiguous
+        ("mk", "kn", "mn", dict(m=32768, k=64, n=40), "128x64 tiles"),                # thin right-hand side: 128x64 tiles
+        ("mk", "kn", "mn", dict(m=40, k=64, n=32768), "128x64 tiles"),                # thin left-hand side: exchanged
+        ("mk", "kn", "mn", dict(m=40, k=30, n=50), "(gemm_kernel"),
+        ("bmk", "bkn", "bmn", dict(b=70, m=20, k=24, n=18), "gemm_wave_kernel"),
+        ("xk", "mk", "xm", dict(x=4096, k=16, m=12), None),                     # small operator on a long tensor
+        ("mk", "k", "m", dict(m=500, k=300), None),                              # matrix . vector: conjugated copy, then the reduction kernel
+        ("ab", "xby", "xay", dict(a=2, b=2, x=300, y=300), None),               # tiny operator: conjugated copy
+        ("asx", "x", "asx", dict(a=30, s=2, x=40), None),                        # nothing summed: conjugated copy
+    ]
+    if dtype == np.complex128:
+        cases.append(("mk", "xk", "xm", dict(m=16, k=32, x=8192), "gemm_skinny_kernel"))
+        cases.append(("xk", "km", "xm", dict(m=16, k=32, x=8192), "gemm_skinny_kernel"))
+    seen = set()
+    for ma, mb, mc, ext, want in cases:
+        a = rand(rng, [ext[l] for l in ma], dtype)
+        b = rand(rng, [ext[l] for l in mb], dtype)
+        c0 = rand(rng, [ext[l] for l in mc], dtype)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [a.shape, b.shape, c0.shape])
+        alpha, beta = 0.7 - 1.1j, -0.3 + 0.2j
+        da, db = dev(tf, a), dev(tf, b)
+        for ca, cb in [(True, False), (False, True), (True, True)]:
+            out = dev(tf, c0)
+            tf.HipBackend.execute(plan, alpha, [da.conj_on_load() if ca else da, db.conj_on_load() if cb else db], beta, out)
+            label = tf.last_kernel()
+            if want is not None:
+                assert want in label, (ma, mb, mc, want, label)
+                seen.add(want)
+            ref = alpha * _contract_np(np.conj(a) if ca else a, ma, np.conj(b) if cb else b, mb, mc) + beta * c0
+            assert relerr(out.to_numpy(), ref) < tol, (ma, mb, mc, ca, cb, label)
+    assert {", 128>)", "128x64 tiles", "(gemm_kernel", "gemm_wave_kernel"} <= seen
+
+
+def test_conj_on_load_views_einsum_permute_and_rejections(tf, oracle):
+    rng = np.random.default_rng(62)
+    a = rand(rng, (12, 2, 14), np.complex128)
+    L = rand(rng, (12, 5, 12), np.complex128)
+    W = rand(rng, (5, 2, 2, 5), np.complex128)
+    dA, dL, dW = dev(tf, a), dev(tf, L), dev(tf, W)
+    # the benchmark's network with its fourth operand as a flagged view of the second: equal to the explicit conj(A)
+    lazy = tf.einsum("awc,asx,wstv,cty->xvy", [dL, dA, dW, dA.conj_on_load()])
+    eager = tf.einsum("awc,asx,wstv,cty->xvy", [dL, dA, dW, dA.conj()])
+    ref = np.einsum("awc,asx,wstv,cty->xvy", L, a, W, np.conj(a))
+    assert relerr(lazy.to_numpy(), ref) < 1e-12 and relerr(eager.to_numpy(), ref) < 1e-12
+    # views of a flagged tensor keep the flag; to_numpy shows the logical values; conj() of it is a plain copy
+    v = dA.conj_on_load().permute([2, 0, 1])
+    assert np.array_equal(v.to_numpy(), np.conj(a).transpose(2, 0, 1))
+    assert np.array_equal(dA.conj_on_load().conj().to_numpy(), a)
+    w = dA.conj_on_load()
+    assert w.into_conj() is w and np.array_equal(w.to_numpy(), a)
+    # Permute honours the flag (bit-exact sign flip), with alpha and beta too
+    out = tf.Tensor.empty([14, 12, 2], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.complex128)
+    plan = tf.HipBackend.plan(np.complex128, tf.PrimDescriptor.Permute([0, 1, 2], [2, 0, 1]), [a.shape, [14, 12, 2]])
+    tf.HipBackend.execute(plan, 1.0, [dA.conj_on_load()], 0.0, out)
+    assert out.to_numpy().tobytes() == np.ascontiguousarray(np.conj(a).transpose(2, 0, 1)).tobytes()
+    # a labelled sum of a flagged operand inside einsum (conj of the sum)
+    s = tf.einsum("asx->ax", [dA.conj_on_load()])
+    assert relerr(s.to_numpy(), np.conj(a).sum(axis=1)) < 1e-12
+    p = tf.einsum("asx,x->as", [dA.conj_on_load(), dev(tf, a[0, 0, :].copy())])
+    assert relerr(p.to_numpy(), np.einsum("asx,x->as", np.conj(a), a[0, 0, :])) < 1e-12
+    # real tensors: the flag is not set at all
+    r = dev(tf, rng.standard_normal((4, 4)))
+    assert r.conj_on_load()._conj is False
+    # not taken: other operations, outputs
+    red = tf.HipBackend.plan(np.complex128, tf.PrimDescriptor.Reduce([0, 1, 2], [0, 2], tf.ReduceOp.Sum), [a.shape, [12, 14]])
+    o2 = tf.Tensor.empty([12, 14], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.complex128)
+    with pytest.raises(tf.InvalidArgument):
+        tf.HipBackend.execute(red, 1.0, [dA.conj_on_load()], 0.0, o2)
+    with pytest.raises(tf.InvalidArgument):
+        tf.HipBackend.execute(plan, 1.0, [dA], 0.0, out.conj_on_load())
+
+
 def _new_streams(tf, n):
     import ctypes
     out = []
