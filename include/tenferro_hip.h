@@ -48,10 +48,18 @@ typedef enum tfh_status {
     TFH_ERR_STRIDED = 7                /* Error::Strided(StridedError)                     :156-158 */
 } tfh_status;
 
-/* Payload of the last failure on the calling thread. */
+/* Payload of the last failure on the calling thread: what a binding needs to rebuild the Error variant.
+ *   ShapeMismatch              expected[0..n_expected), got[0..n_got): the two shapes
+ *   RankMismatch               expected[0], got[0]: the two ranks (n_expected = n_got = 1)
+ *   NoCompatibleComputeDevice  expected[0..2) = the memory space as (tfh_space_kind, space id), got[0] = the tfh_op_kind
+ *   CrossMemorySpaceOperation  expected[0..2) = the left space, got[0..2) = the right space, each (tfh_space_kind, id);
+ *                              never returned by this library, whose views are bare device pointers: the binding,
+ *                              which knows where its tensors live, raises it before calling (the layout is fixed
+ *                              here so that every binding decodes status 5 the same way)
+ *   DeviceError, InvalidArgument, Strided   message only */
 typedef struct tfh_error_info {
     int32_t status;                    /* tfh_status of the failing call */
-    int32_t n_expected;                /* ShapeMismatch: rank of `expected`; RankMismatch: 1 */
+    int32_t n_expected;
     int32_t n_got;
     int32_t reserved;
     int64_t expected[TFH_MAX_RANK];

@@ -150,7 +150,10 @@ class DeviceError(Error):
 
 
 class NoCompatibleComputeDevice(Error):
+    """Fields `space` (LogicalMemorySpace) and `op` (an OpKind value), as in tenferro-device/src/lib.rs:134-140."""
     status = 4
+    space = None
+    op = None
 
 
 class CrossMemorySpaceOperation(Error):
@@ -179,7 +182,10 @@ def _check(status):
     got = list(info.got[:info.n_got]) if info.n_got else None
     if cls is RankMismatch and expected:
         expected, got = expected[0], got[0]
-    raise cls(info.message.decode(errors="replace"), expected, got)
+    err = cls(info.message.decode(errors="replace"), expected, got)
+    if cls is NoCompatibleComputeDevice and expected and len(expected) == 2 and got:
+        err.space, err.op = LogicalMemorySpace(int(expected[0]), int(expected[1])), int(got[0])
+    raise err
 
 
 # ---------------------------------------------------------------------------------------------- device model

@@ -58,6 +58,24 @@ int32_t set_rank_mismatch(int64_t expected, int64_t got) {
     snprintf(g_err.message, sizeof g_err.message, "rank mismatch: expected %lld, got %lld", (long long)expected, (long long)got);
     return TFH_ERR_RANK_MISMATCH;
 }
+
+int32_t set_no_compatible_device(int32_t space_kind, int64_t space_id, int32_t op_kind) {
+    static const char* kinds[] = {"Contract", "BatchedGemm", "Reduce", "Trace", "Permute", "ElementwiseMul"};
+    clear_error();
+    g_err.status = TFH_ERR_NO_COMPATIBLE_DEVICE;
+    g_err.n_expected = 2;   // the memory space: (tfh_space_kind, space id)
+    g_err.expected[0] = space_kind;
+    g_err.expected[1] = space_kind == TFH_SPACE_GPU_MEMORY ? space_id : 0;
+    g_err.n_got = 1;        // the operation: tfh_op_kind
+    g_err.got[0] = op_kind;
+    const char* op = op_kind >= 0 && op_kind <= TFH_KIND_ELEMENTWISE_MUL ? kinds[op_kind] : "?";
+    // "no compatible compute device for {op:?} on {space:?}" (tenferro-device/src/lib.rs:134)
+    if (space_kind == TFH_SPACE_GPU_MEMORY)
+        snprintf(g_err.message, sizeof g_err.message, "no compatible compute device for %s on GpuMemory { space_id: %lld }", op, (long long)space_id);
+    else
+        snprintf(g_err.message, sizeof g_err.message, "no compatible compute device for %s on MainMemory", op);
+    return TFH_ERR_NO_COMPATIBLE_DEVICE;
+}
 }  // namespace tfh
 
 extern "C" {

@@ -17,6 +17,7 @@ namespace tfh {
 int32_t set_error(int32_t status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int32_t set_shape_mismatch(const int64_t* expected, int n_expected, const int64_t* got, int n_got);
 int32_t set_rank_mismatch(int64_t expected, int64_t got);
+int32_t set_no_compatible_device(int32_t space_kind, int64_t space_id, int32_t op_kind);
 void clear_error();
 
 inline bool is_complex(int dt) { return dt == TFH_C64 || dt == TFH_C128; }

@@ -488,7 +488,6 @@ int32_t tfh_preferred_compute_devices(int32_t space_kind, int64_t space_id, int3
     if (!n) return set_error(TFH_ERR_INVALID_ARGUMENT, "null output pointer");
     *n = 0;
     if (op_kind < TFH_KIND_CONTRACT || op_kind > TFH_KIND_ELEMENTWISE_MUL) return set_error(TFH_ERR_INVALID_ARGUMENT, "unknown OpKind %d", op_kind);
-    static const char* kinds[] = {"Contract", "BatchedGemm", "Reduce", "Trace", "Permute", "ElementwiseMul"};
     if (space_kind == TFH_SPACE_GPU_MEMORY) {
         int32_t count = 0;
         if (int32_t e = tfh_device_count(&count)) return e;
@@ -500,11 +499,9 @@ int32_t tfh_preferred_compute_devices(int32_t space_kind, int64_t space_id, int3
             *n = 1;
             return TFH_OK;
         }
-        return set_error(TFH_ERR_NO_COMPATIBLE_DEVICE, "no compatible compute device for %s on GpuMemory { space_id: %lld }",
-                         kinds[op_kind], (long long)space_id);
+        return tfh::set_no_compatible_device(space_kind, space_id, op_kind);
     }
-    if (space_kind == TFH_SPACE_MAIN_MEMORY)
-        return set_error(TFH_ERR_NO_COMPATIBLE_DEVICE, "no compatible compute device for %s on MainMemory", kinds[op_kind]);
+    if (space_kind == TFH_SPACE_MAIN_MEMORY) return tfh::set_no_compatible_device(space_kind, 0, op_kind);
     return set_error(TFH_ERR_INVALID_ARGUMENT, "unknown memory space kind %d", space_kind);
 }
 

@@ -57,8 +57,10 @@ def test_dtype_sizes_extensions_and_device_display(tf):
 def test_preferred_compute_devices_main_memory_has_none(tf):
     # this library computes on HIP devices only
     with pytest.raises(tf.NoCompatibleComputeDevice) as e:
-        tf.preferred_compute_devices(tf.MainMemory, tf.OpKind.Contract)
-    assert "MainMemory" in str(e.value)
+        tf.preferred_compute_devices(tf.MainMemory, tf.OpKind.Reduce)
+    assert str(e.value) == "no compatible compute device for Reduce on MainMemory"
+    # the variant's two fields come back as data, not only as text (tenferro-device/src/lib.rs:134-140)
+    assert e.value.space == tf.MainMemory and e.value.op == tf.OpKind.Reduce
 
 
 # ---------------------------------------------------------------------------------------------- plan validation
