@@ -1209,24 +1209,22 @@ int32_t grouped_plan_init(tfh_plan& plan) {
             units.push_back(std::move(u));
         }
     }
-    std::stable_sort(units.begin(), units.end(), [](const Unit& x, const Unit& y) { return x.cost > y.cost; });
+    // Workgroups are dispatched in launch order, position i to XCD i % 8, and position i does not start before position
+    // i - 1 has: an XCD whose list holds longer tiles than the others' at the same depth holds all of them back.  So the
+    // units are taken in the order of their k (longest first; a lone tile with a long k that started late would also run
+    // on after everything else has finished) and each goes to the XCD with the least work so far: the eight lists then
+    // have the same k at the same depth and the same total.
+    std::stable_sort(units.begin(), units.end(), [](const Unit& x, const Unit& y) {
+        return x.tiles[0].k != y.tiles[0].k ? x.tiles[0].k > y.tiles[0].k : x.cost > y.cost;
+    });
     std::array<std::vector<T>, XCDS> per_xcd;
     std::array<double, XCDS> load{};
-    std::array<std::vector<const Unit*>, XCDS> units_of;
     for (auto& u : units) {
         int best = 0;
         for (int x = 1; x < XCDS; ++x)
             if (load[(size_t)x] < load[(size_t)best]) best = x;
         load[(size_t)best] += u.cost;
-        units_of[(size_t)best].push_back(&u);
-    }
-    for (int x = 0; x < XCDS; ++x) {
-        // an XCD starts its longest tiles first (largest k), whatever the size of the unit they belong to: a lone tile
-        // with a long k that started late would run on after everything else has finished
-        std::stable_sort(units_of[(size_t)x].begin(), units_of[(size_t)x].end(),
-                             [](const Unit* a, const Unit* b) { return a->tiles[0].k > b->tiles[0].k; });
-        for (const Unit* u : units_of[(size_t)x])
-            for (auto& t : u->tiles) per_xcd[(size_t)x].push_back(t);
+        for (auto& t : u.tiles) per_xcd[(size_t)best].push_back(t);
     }
     size_t longest = 0;
     for (auto& v : per_xcd) longest = std::max(longest, v.size());
