@@ -1158,15 +1158,13 @@ int32_t grouped_plan_init(tfh_plan& plan) {
     // 128-row tiles.  A last strip of at most 64 rows or 64 real columns gets tiles of that shape instead of a padded
     // 128 x 128 one (extents that are odd multiples of 64 -- half of all extents drawn from {64, 128, ...} -- would
     // otherwise compute 10 % more than the products need): shape 1 = 128 x 64, shape 2 = 64 x 128 (run transposed).
-    // Two row panels of a problem (256 rows of A, every column tile, walked column by column) form a unit: its tiles read
-    // the same rows of A and, side by side, the same columns of B.  Units are dealt to the eight XCDs -- block i of a
-    // launch runs on XCD i % 8, each with an L2 of its own -- longest first onto the XCD with the least work so far, and
-    // every XCD runs its units in the order of their k (a lone tile with a long k that started late would run on after
-    // everything else has finished).  Measured on the benchmark's 128 blocks: dealing the tiles out one by one in the
-    // order of their k, each problem spread over all eight L2s, fetches 2.82 GB for 0.68 GB of operands; units of one
-    // row panel 2.09 GB, of two 1.59 GB, of four 1.30 GB, at the same speed within 1 % (832 / 825 / 831 us) -- while units
-    // kept in the order of their total work instead of their k lost 10 %.
-    struct Unit { std::vector<T> tiles; double cost; };
+    // Two row panels of a problem (256 rows of A, every full column tile, walked column by column) form a unit: its tiles
+    // read the same rows of A and, side by side, the same columns of B; the shorter-running tiles of a last strip are units
+    // of their own.  A unit lives on one XCD -- block i of a launch runs on XCD i % 8, each with an L2 of its own.  Measured
+    // on the benchmark's 128 blocks: dealing the tiles out one by one in the order of their k, each problem spread over all
+    // eight L2s, fetches 2.82 GB for 0.68 GB of operands; units of one row panel 2.09 GB, of two 1.59 GB, of four 1.30 GB,
+    // at the same speed within 1 %.  How the units are ordered and dealt out is described where it is done, below.
+    struct Unit { std::vector<T> tiles; double cost; double tile_cost; };   // cost of the unit, of one of its tiles
     std::vector<Unit> units;
     // a 128 x 64 tile does half the multiply-adds of a full tile in about 0.63 of its time (measured on thin products)
     const double thin_cost = 0.63;
@@ -1191,12 +1189,20 @@ int32_t grouped_plan_init(tfh_plan& plan) {
                     u.tiles.push_back({gi, (int)tm, (int)tn, 0, K});
                     u.cost += kcost;
                 }
-            if (thin_n)   // column strip: tile_n counts 64-column tiles
+            if (!u.tiles.empty()) {
+                u.tile_cost = kcost;
+                units.push_back(std::move(u));
+            }
+            if (thin_n) {   // column strip, a unit of its own (its tiles are shorter): tile_n counts 64-column tiles
+                Unit v;
+                v.cost = 0;
+                v.tile_cost = thin_cost * kcost;
                 for (int64_t tm = tm0; tm < tm1; ++tm) {
-                    u.tiles.push_back({gi, (int)tm, (int)(2 * cols128), 1, K});
-                    u.cost += thin_cost * kcost;
+                    v.tiles.push_back({gi, (int)tm, (int)(2 * cols128), 1, K});
+                    v.cost += thin_cost * kcost;
                 }
-            units.push_back(std::move(u));
+                units.push_back(std::move(v));
+            }
         }
         if (thin_m) {   // row strip, transposed: the body's rows are the columns (128 per tile), its 64-wide tile_n counts rows
             Unit u;
@@ -1206,16 +1212,17 @@ int32_t grouped_plan_init(tfh_plan& plan) {
                 u.tiles.push_back({gi, (int)tn, (int)(2 * rows128 * ec), 2, K});
                 u.cost += thin_cost * kcost;
             }
+            u.tile_cost = thin_cost * kcost;
             units.push_back(std::move(u));
         }
     }
     // Workgroups are dispatched in launch order, position i to XCD i % 8, and position i does not start before position
     // i - 1 has: an XCD whose list holds longer tiles than the others' at the same depth holds all of them back.  So the
-    // units are taken in the order of their k (longest first; a lone tile with a long k that started late would also run
-    // on after everything else has finished) and each goes to the XCD with the least work so far: the eight lists then
-    // have the same k at the same depth and the same total.
+    // units are taken in the order of their tiles' duration (longest first; a lone long tile that started late would also
+    // run on after everything else has finished) and each goes to the XCD with the least work so far: the eight lists then
+    // hold tiles of the same duration at the same depth and the same total.
     std::stable_sort(units.begin(), units.end(), [](const Unit& x, const Unit& y) {
-        return x.tiles[0].k != y.tiles[0].k ? x.tiles[0].k > y.tiles[0].k : x.cost > y.cost;
+        return x.tile_cost != y.tile_cost ? x.tile_cost > y.tile_cost : x.cost > y.cost;
     });
     std::array<std::vector<T>, XCDS> per_xcd;
     std::array<double, XCDS> load{};
