@@ -442,9 +442,12 @@ __device__ __forceinline__ void gemm128_body(const GemmArgs& g, const TileCtx& t
         int64_t s = 0;
         for (; s + 2 < nstage; ++s) {
             // Two blocks share a CU.  The arbiter favours the older wave, so one block runs ahead and the other is
-            // left to finish alone; lowering a block's issue priority as it progresses keeps the one that is behind
-            // ahead in the arbitration, and the two finish together (a launch of exactly one wave of blocks gains ~2%).
-            if ((s & 3) == 0) {
+            // left to finish alone; when all blocks of a launch start together and nothing follows them, lowering a
+            // block's issue priority as it progresses keeps the one that is behind ahead in the arbitration, and the
+            // two finish together (config 1: 1 % faster).  With more tiles than resident blocks it is the other way
+            // round: blocks that end at different times overlap their epilogues and prologues with their neighbours'
+            // main loops, so nothing is done to align them (the grouped launch of config 4 lost 1.5 % to this).
+            if (g.one_round && (s & 3) == 0) {
                 const int q = (int)((4 * s) / nstage);
                 if (q == 0) __builtin_amdgcn_s_setprio(3);
                 else if (q == 1) __builtin_amdgcn_s_setprio(2);

@@ -54,6 +54,7 @@ struct GemmArgs {
     int32_t vec;                   // both operands allow 16-byte accesses along their contiguous direction
     const GroupProblem* problems;  // grouped launch when non-null
     const int4* tile_map;          // per block: (problem, tile_m, tile_n, 0)
+    int32_t one_round;             // 128x128 kernel: every block of the launch is resident at once (see the main loop)
 };
 
 // Workgroups are handed to the eight XCDs (each with its own L2) round-robin in launch order.  logical_block()

@@ -531,6 +531,21 @@ bool vec_ok(int dtype, const std::vector<Axis>& lanes, const std::vector<Axis>& 
     return other.empty() || (other.size() == 1 && (other[0].n == 1 || other[0].s[slot] >= V));
 }
 
+// Compute units of the current device (looked up once per device).
+uint32_t compute_units() {
+    static std::mutex mu;
+    static std::map<int, uint32_t> cus;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    std::lock_guard<std::mutex> lk(mu);
+    auto it = cus.find(dev);
+    if (it != cus.end()) return it->second;
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = (uint32_t)n;
+    return (uint32_t)n;
+}
+
 int bke_of(int dtype) {
     int bkr = is_double(dtype) ? 16 : 32;
     return is_complex(dtype) ? bkr / 2 : bkr;
@@ -1018,6 +1033,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     }
     if (nsplit > 1) g.partial = ws + (cached ? 0 : table_bytes);
     dim3 grid((uint32_t)((int64_t)g.tiles_m * g.tiles_n * nb * nsplit), 1, 1);
+    g.one_round = grid.x <= 2u * compute_units();   // two blocks of the 128-tile kernel fit a CU
     const int prof = prof_begin(PROF_CONTRACT, stream);
     if (skinny) {
         SkinnyArgs sk;
