@@ -110,6 +110,7 @@ struct OperandMap {
     typedef Pack<R, PN> P;
     uint32_t voff[NL];   // byte offset of load l relative to the (advancing) base
     int kq, rq;
+    int lds0;            // LDS index of this thread's first 16-byte store (unit 0); the other units derive from it
     // Last stage only.  A vector that straddles the end of its contiguous direction (k past `rem` for a k-contiguous
     // operand, rows past the matrix edge for a row-contiguous one) is loaded from a window moved back to end exactly
     // at the boundary -- nothing is read past the operand -- and its elements are moved up by the same amount when
@@ -122,6 +123,7 @@ struct OperandMap {
         if (KFAST) { kq = (t % KV) * V; rq = t / KV; }
         else { rq = (t % RVN) * V; kq = t / RVN; }
         row_shift = (!KFAST && rq < rows_valid && rq + V > rows_valid) ? rq + V - rows_valid : 0;
+        lds0 = C_::lds_idx(rq * RM, (KFAST ? kq : kq * V) * EC);
 #pragma unroll
         for (int l = 0; l < NL; ++l) {
             const int row = KFAST ? rq + l * RP : rq;
@@ -191,10 +193,11 @@ struct OperandMap {
     // store unit u = (pass p, row v of the patch): one 16-byte (V > 1) or one-element LDS store (two for a complex B)
     __device__ __forceinline__ void store_unit(R* tile, const P (&x)[NL], int u, bool mask_tail, int rem, bool conj) const {
         const int p = u / VV, v = u % VV;
-        // the LDS index is recomputed at every use (a few VALU operations): kept out of the loop-invariant set, it
-        // does not occupy a register during the MFMA phase
-        int rq_ = rq, kq_ = kq;
-        asm volatile("" : "+v"(rq_), "+v"(kq_));
+        // the thread's row and k position are recomputed from the thread index where they are needed (the last stage and
+        // the element-wise path), so that they occupy no registers during the MFMA phase
+        int t_ = threadIdx.x;
+        asm volatile("" : "+v"(t_));
+        const int rq_ = KFAST ? t_ / KV : (t_ % RVN) * V, kq_ = KFAST ? (t_ % KV) * V : t_ / RVN;
         const int row = KFAST ? rq_ + p * RP : rq_ + v;
         const int kel0 = KFAST ? kq_ : (p * KP + kq_) * V;
         R out0[PN], out1[PN];
@@ -225,7 +228,18 @@ struct OperandMap {
                 out0[j] = ok ? sre : R(0);
             }
         }
-        const int idx = C_::lds_idx(row * RM, kel0 * EC);
+        // Whole-chunk stores derive their index from unit 0's with a constant or two, because the swizzle of a row only
+        // depends on its low five bits: passes of a k-contiguous operand are RP * RM rows (a multiple of 32) apart; pass
+        // p of a row-contiguous one is KP chunks further along k (kq < KP, a power of two: an XOR), and row v of its
+        // patch is v * RM rows down with the chunk position XOR-ed by the same v * RM (rq is a multiple of V <= 4).
+        constexpr bool WHOLE = V * EC == C_::CH && (!KFAST || (RP * RM) % 32 == 0) && (KFAST || (KP & (KP - 1)) == 0);
+        int idx;
+        if constexpr (WHOLE) {
+            if constexpr (KFAST) idx = lds0 + p * RP * RM * C_::PITCH;
+            else idx = ((lds0 ^ (v * RM * C_::CH)) + v * RM * C_::PITCH) ^ (p * KP * C_::CH);
+        } else {
+            idx = C_::lds_idx(row * RM, kel0 * EC);
+        }
         lds_store_pack<R, PN>(tile + idx, out0);
         // the odd row below an even one: its swizzle differs in bit 0 only, i.e. the neighbouring chunk of the next row
         if constexpr (RM == 2) lds_store_pack<R, PN>(tile + (idx ^ C_::CH) + C_::PITCH, out1);
