@@ -61,6 +61,13 @@ __device__ __forceinline__ Pack<R, N> gload_pack(gptr base, uint32_t off) {
     }
     return out;
 }
+// x or -x by an XOR of the sign bit
+__device__ __forceinline__ double flip_sign(double x, bool flip) {
+    return __builtin_bit_cast(double, __builtin_bit_cast(uint64_t, x) ^ (flip ? 0x8000000000000000ull : 0ull));
+}
+__device__ __forceinline__ float flip_sign(float x, bool flip) {
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x) ^ (flip ? 0x80000000u : 0u));
+}
 template <class R, int N>
 __device__ __forceinline__ void lds_store_pack(R* p, const R (&x)[N]) {
     typedef typename RawVec<R, N>::type Raw;
@@ -195,8 +202,12 @@ struct OperandMap {
         const int p = u / VV, v = u % VV;
         // the thread's row and k position are recomputed from the thread index where they are needed (the last stage and
         // the element-wise path), so that they occupy no registers during the MFMA phase
-        int t_ = threadIdx.x;
-        asm volatile("" : "+v"(t_));
+        constexpr bool WHOLE = V * EC == C_::CH && (!KFAST || (RP * RM) % 32 == 0) && (KFAST || (KP & (KP - 1)) == 0);
+        int t_ = 0;
+        if (mask_tail || !WHOLE) {   // (not needed by a full stage of whole-chunk stores: nothing is emitted for those)
+            t_ = threadIdx.x;
+            asm volatile("" : "+v"(t_));
+        }
         const int rq_ = KFAST ? t_ / KV : (t_ % RVN) * V, kq_ = KFAST ? (t_ % KV) * V : t_ / RVN;
         const int row = KFAST ? rq_ + p * RP : rq_ + v;
         const int kel0 = KFAST ? kq_ : (p * KP + kq_) * V;
@@ -216,10 +227,12 @@ struct OperandMap {
                 sim = EC == 2 ? src.v[EC * e + EC - 1] : R(0);
             }
             if constexpr (CX) {
+                // conj and the minus sign of the expansion are one XOR of the sign bit each, with a mask that is uniform
+                // and constant over the tile (a select between x and -x would cost two instructions per value)
                 const R re = ok ? sre : R(0);
-                const R im = ok ? (conj ? -sim : sim) : R(0);
+                const R im = ok ? flip_sign(sim, conj) : R(0);
                 if constexpr (RM == 2) {
-                    out0[2 * j] = re; out0[2 * j + 1] = -im;
+                    out0[2 * j] = re; out0[2 * j + 1] = ok ? flip_sign(sim, !conj) : R(0);
                     out1[2 * j] = im; out1[2 * j + 1] = re;
                 } else {
                     out0[2 * j] = re; out0[2 * j + 1] = im;
@@ -232,7 +245,6 @@ struct OperandMap {
         // depends on its low five bits: passes of a k-contiguous operand are RP * RM rows (a multiple of 32) apart; pass
         // p of a row-contiguous one is KP chunks further along k (kq < KP, a power of two: an XOR), and row v of its
         // patch is v * RM rows down with the chunk position XOR-ed by the same v * RM (rq is a multiple of V <= 4).
-        constexpr bool WHOLE = V * EC == C_::CH && (!KFAST || (RP * RM) % 32 == 0) && (KFAST || (KP & (KP - 1)) == 0);
         int idx;
         if constexpr (WHOLE) {
             if constexpr (KFAST) idx = lds0 + p * RP * RM * C_::PITCH;
