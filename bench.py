@@ -12,7 +12,9 @@ contraction, one permute+reduce, one grouped launch.
 
 `roofline` describes the kernel that takes most of the step's time: `achieved` is its algorithmic flops (or bytes) per
 launch divided by its average duration, measured from the begin/end timestamps of its own dispatches on the launch
-stream inside the timed region; `kernel` is the label the library reported for those dispatches.  `traffic` is read
+stream over a second pass of the same K steps (the K timed steps themselves carry no events: launching a kernel with
+them costs 4-5 us of stream time, which is not the library's); `kernel` is the label the library reported for those
+dispatches.  `traffic` is read
 from profiles/bench_hbm_traffic_pmc.txt (a profiler cannot run inside this script) and is null when the kernel that
 ran is not the one that file was measured on.  `cpu_baseline` is the CPU oracle (a port: the reference has no CPU
 backend to time) on the host cores of this machine, on the same inputs; its result is also the parity check of the run.
