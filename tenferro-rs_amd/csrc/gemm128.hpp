@@ -497,8 +497,23 @@ __device__ __forceinline__ void gemm128_body(const GemmArgs& g, const TileCtx& t
     // ---- epilogue: real column wn0 + 16 j + lrow; for complex, column 2n+p is part p of element n ----------
     const int64_t NR = CX ? 2 * N : N;
     const int64_t n0r = CX ? 2 * n0 : n0;
+    // A tile that lies wholly inside the matrix (all but the last row and column of tiles) is written without a
+    // bounds predicate per element: one address per accumulator row, the four column blocks at constant offsets from it.
+    const bool full_tile = m0 + BM <= M && n0r + BN <= NR;
     if (g.nsplit > 1) {
         R* P = reinterpret_cast<R*>(g.partial) + ((int64_t)split * g.nbatch + batch) * M * NR;
+        if (full_tile) {
+            R* p0 = P + (m0 + wm0) * NR + n0r + wn0 + lrow;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    R* p = p0 + (int64_t)(16 * i + Mfma<R>::row(lane, r)) * NR;
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) p[16 * j] = acc[i][j][r];
+                }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -515,6 +530,24 @@ __device__ __forceinline__ void gemm128_body(const GemmArgs& g, const TileCtx& t
     }
     R* Cb = reinterpret_cast<R*>(Cp) + (t.grouped ? 0 : off_of(g.cb, batch)) * (CX ? 2 : 1);
     const R ar = (R)g.alpha_re, ai = (R)g.alpha_im, br = (R)g.beta_re, bi = (R)g.beta_im;
+    const bool real_scalars = g.alpha_im == 0.0 && g.beta_im == 0.0;
+    // C contiguous along n (the usual case; the host exchanges the operands to get it), real scalars: the same for the result
+    if (full_tile && !cn.tab && cn.stride == 1 && (!CX || real_scalars)) {
+        R* c0 = Cb + n0r + wn0 + lrow;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                R* p = c0 + off_of(cm, m0 + wm0 + 16 * i + Mfma<R>::row(lane, r)) * (CX ? 2 : 1);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    R out = ar * acc[i][j][r];
+                    if (g.use_beta) out += br * p[16 * j];
+                    p[16 * j] = out;
+                }
+            }
+        return;
+    }
     int64_t coff[TN];
     bool cok[TN];
 #pragma unroll
@@ -537,6 +570,14 @@ __device__ __forceinline__ void gemm128_body(const GemmArgs& g, const TileCtx& t
                 const bool ok = rok && cok[j];
                 R* dst = Cb + roff + coff[j];
                 if constexpr (CX) {
+                    if (real_scalars) {   // real alpha and beta act on the two parts separately: no exchange
+                        if (ok) {
+                            R out = ar * v;
+                            if (g.use_beta) out += br * *dst;
+                            *dst = out;
+                        }
+                        continue;
+                    }
                     // even lanes hold re, odd lanes hold im of the same element: exchange with the neighbour
                     R other = __shfl_xor(v, 1);
                     R old = (g.use_beta && ok) ? *dst : R(0);
