@@ -336,6 +336,8 @@ __device__ __forceinline__ void gemm128_body(const GemmArgs& g, const TileCtx& t
     const int64_t nstage = (klen + BKE - 1) / BKE;
     const int rem = (int)(klen - (nstage - 1) * BKE);   // k elements in the last stage (1..BKE)
     const bool ktab = ak.tab != nullptr;               // the host builds k tables for both operands or for none
+    // the last stage is a full one and no 16-byte access straddles the matrix edge: it is stored like any other
+    const bool plain_last = rem == BKE && (AKF || VA == 1 || rowsA % VA == 0) && (BKF || VB == 1 || rowsB % VB == 0);
 
     auto load_fast = [&]() {
         sa = uniform_ptr(sa);
@@ -454,12 +456,15 @@ __device__ __forceinline__ void gemm128_body(const GemmArgs& g, const TileCtx& t
         // prologue: stage 0 into buffer 0 and, when a full stage follows, its loads into the registers
         if (nstage == 1) {
             if (ktab) load_tab(0);
+            else if (plain_last) load_fast();
             else load_tail();
         } else {
             if (ktab) load_tab(0);
             else load_fast();
         }
-        store_stage(0, nstage == 1);
+        // (two calls: with the flag a constant, the store of a full stage carries none of the masking arithmetic)
+        if (nstage == 1 && !plain_last) store_stage(0, true);
+        else store_stage(0, false);
         if (ktab) {
             ma.fetch_tab(ka, ak.tab, kbeg + BKE, kend);
             mb.fetch_tab(kb, bk.tab, kbeg + BKE, kend);
@@ -485,9 +490,11 @@ __device__ __forceinline__ void gemm128_body(const GemmArgs& g, const TileCtx& t
         }
         if (s + 1 < nstage) {
             if (ktab) load_tab(s + 1);
+            else if (plain_last) load_fast();
             else load_tail();
             compute((int)(s & 1));
-            store_stage((int)((s + 1) & 1), true);
+            if (plain_last) store_stage((int)((s + 1) & 1), false);
+            else store_stage((int)((s + 1) & 1), true);
             __syncthreads();
             ++s;
         }
