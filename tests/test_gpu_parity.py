@@ -684,6 +684,37 @@ def test_einsum_async_chaining(tf):
     assert relerr(d.to_numpy(), a @ b @ b) < 1e-12
 
 
+@pytest.mark.parametrize("dtype", ALL)
+def test_large_tile_kernel_stage_and_tile_boundaries(tf, dtype):
+    # The 128-tile kernel treats a last k stage that is full, and a tile that lies wholly inside the matrix, like interior
+    # ones (plain loads and stores, no predicates); everything else takes the masked paths.  Extents on and around those
+    # boundaries -- k a whole number of stages or one element off, rows and columns a whole number of tiles, of 16-byte
+    # vectors, or neither -- in the four storage-order combinations of the operands and both orders of the result, with
+    # and without an old result to add, against numpy.
+    rng = np.random.default_rng(71)
+    tol = TOL[dtype]
+    stage = {np.float32: 32, np.float64: 16, np.complex64: 16, np.complex128: 8}[dtype]
+    seen = set()
+    nb = 48   # batch entries: enough tiles for the large-tile kernel at every extent below
+    for (m, n) in [(256, 256), (384, 130), (257, 255), (130, 384), (129, 131)]:
+        for k in (stage, 2 * stage, 3 * stage, 3 * stage - 1, 2 * stage + 1):
+            for a_kfast, b_kfast in [(True, True), (True, False), (False, True), (False, False)]:
+                a = rand(rng, (nb, m, k), dtype) if a_kfast else rand(rng, (nb, k, m), dtype).transpose(0, 2, 1)
+                b = rand(rng, (nb, n, k), dtype).transpose(0, 2, 1) if b_kfast else rand(rng, (nb, k, n), dtype)
+                c_row = (m * 7 + n + k) % 2 == 0
+                c0 = rand(rng, (nb, m, n), dtype) if c_row else rand(rng, (nb, n, m), dtype).transpose(0, 2, 1)
+                beta = 0.0 if (m + k) % 3 == 0 else 0.5
+                out = dev(tf, c0)
+                plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("bmk"), lab("bkn"), lab("bmn")), [a.shape, b.shape, c0.shape])
+                tf.HipBackend.execute(plan, 1.25, [dev(tf, a), dev(tf, b)], beta, out)
+                seen.add(tf.last_kernel().split("<")[0])
+                wide = np.complex128 if np.iscomplexobj(a) else np.float64
+                ref = 1.25 * np.matmul(a.astype(wide), b.astype(wide)) + beta * c0
+                err = relerr(out.to_numpy(), ref)
+                assert err < tol, (m, n, k, a_kfast, b_kfast, c_row, beta, err, tf.last_kernel())
+    assert seen == {"(gemm128_kernel"}, seen
+
+
 # ------------------------------------------------------------------------------------------------ conj on load
 def _contract_np(a, ma, b, mb, mc):
     return np.einsum(f"{ma},{mb}->{mc}", a, b, optimize=True)
