@@ -875,9 +875,30 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
                 nsplit = s_;
             }
         }
-    } else if (tiles < 256 && kstages >= 16) {
-        nsplit = (int)std::min<int64_t>((512 + tiles - 1) / tiles, kstages / 8);
-        nsplit = std::max(1, std::min(nsplit, 512));   // a single tile with a very long k still fills the chip
+    } else if (tiles < 256 && kstages >= 8) {
+        // Few small tiles: a block of the 64x64 kernel that is alone on its CU takes about 3 us plus 1.25 us per stage,
+        // whatever the type (two blocks that share a CU 1.3 times that each); splitting k shortens the blocks, and costs
+        // a second launch that reads one partial result per split.  Estimated time in us of a split count, from what
+        // those kernels measure on this device (512^3 f64: 21.5 us with 4 splits, 22.9 with 8; 256^3: 17.0 with 2,
+        // 13.0 with 4; 64 x 64 x 4096: 25 with 32, 13.3 with 64; 200 x 200 x 2000: 23 with 15, 25 with 31); the count
+        // with the least estimate is taken.
+        const double out_mb = (double)(nb * M * NR * rb) / 1e6;
+        auto estimate = [&](int64_t s_) {
+            const double stages = (double)((kstages + s_ - 1) / s_);
+            const int64_t blocks = tiles * s_;
+            double t = 1.5 + (3.0 + 1.25 * stages) * (blocks > 256 ? 1.3 : 1.0) * (double)((blocks + 511) / 512);
+            if (s_ > 1) t += 3.0 + 0.45 * (double)s_ * out_mb;
+            return t;
+        };
+        const int64_t smax = std::min<int64_t>(std::min<int64_t>((512 + tiles - 1) / tiles, kstages / 2), 512);
+        double best = estimate(1);
+        for (int64_t s_ = 2; s_ <= smax; ++s_) {
+            const double t = estimate(s_);
+            if (t < best * 0.97) {
+                best = t;
+                nsplit = (int)s_;
+            }
+        }
     }
     if (skinny) nsplit = 1;
     // many tiny products (both free extents at most 32): one wave per 32x32 tile, no LDS staging (k_gemm_wave.hip)

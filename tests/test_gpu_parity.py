@@ -715,6 +715,27 @@ def test_large_tile_kernel_stage_and_tile_boundaries(tf, dtype):
     assert seen == {"(gemm128_kernel"}, seen
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex64, np.complex128])
+def test_small_products_across_split_counts(tf, dtype):
+    # Products with fewer than 256 tiles of 64 x 64 choose their number of k splits from an estimate of the run time: from
+    # none (few stages) to hundreds (one tile with a long k).  Whatever it chooses, the result is that of the product:
+    # extents that give one tile and many, k from one stage to thousands of elements, ragged in every direction, with
+    # alpha and an old result to add, against numpy.
+    rng = np.random.default_rng(83)
+    tol = TOL[dtype]
+    for (m, n, k) in [(64, 64, 4096), (64, 64, 4099), (128, 128, 128), (256, 256, 256), (200, 200, 2000), (100, 60, 5000),
+                      (384, 384, 384), (512, 512, 512), (300, 260, 1103), (33, 47, 129), (64, 64, 33), (1000, 90, 70)]:
+        a, b, c0 = rand(rng, (m, k), dtype), rand(rng, (k, n), dtype), rand(rng, (m, n), dtype)
+        for alpha, beta in ((1.0, 0.0), (0.75, -0.5)):
+            out = dev(tf, c0)
+            plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("mk"), lab("kn"), lab("mn")), [a.shape, b.shape, c0.shape])
+            tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, out)
+            wide = np.complex128 if np.iscomplexobj(a) else np.float64
+            ref = alpha * np.matmul(a.astype(wide), b.astype(wide)) + beta * c0
+            err = relerr(out.to_numpy(), ref)
+            assert err < tol, (m, n, k, alpha, beta, err, tf.last_kernel())
+
+
 # ------------------------------------------------------------------------------------------------ conj on load
 def _contract_np(a, ma, b, mb, mc):
     return np.einsum(f"{ma},{mb}->{mc}", a, b, optimize=True)
