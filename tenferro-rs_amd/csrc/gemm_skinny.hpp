@@ -21,7 +21,8 @@ struct SkinnyArgs {
     int32_t kc;              // 16-byte chunks per row of B: K for complex128, K/2 for f64
     int32_t conj_a, conj_b, use_beta, plain;   // plain: alpha == 1 and beta == 0
     int32_t out_rows;        // C is contiguous along m (the rows of A), not along n: a unit's results are transposed in LDS
-    int64_t units;           // N / SKINNY_UNIT
+    int64_t units;           // work units: (outer extents of n) x upr
+    int32_t upr, tail;       // units per innermost run of n; n in the last unit of each run (0: every unit is full)
     OffFn am, ak, cm;        // element offsets of A's rows and k, of C's rows
     OffFn bu, cu;            // element offset of a unit's first n in B and in C
     int32_t b_in, c_in;      // element stride between consecutive n inside a unit, in B and in C

@@ -546,6 +546,10 @@ uint32_t compute_units() {
     return (uint32_t)n;
 }
 
+// An innermost run of n suits the streaming kernel's units of SKINNY_UNIT consecutive n when it is a whole number of them,
+// or long enough that a partly filled last unit costs little (500 = 31 units and a quarter).
+bool skinny_run_ok(int64_t n) { return n % SKINNY_UNIT == 0 || n >= 3 * SKINNY_UNIT; }
+
 int bke_of(int dtype) {
     int bkr = is_double(dtype) ? 16 : 32;
     return is_complex(dtype) ? bkr / 2 : bkr;
@@ -687,7 +691,15 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     {
         const int ec = is_complex(dtype) ? 2 : 1;
         // (a small operator against a long tensor keeps its orientation: the streaming kernel looks at it below)
-        const bool streamable = (dtype == TFH_F64 || dtype == TFH_C128) && M <= SKINNY_MAX_M && K * ec <= SKINNY_MAX_KR && N >= 4096;
+        bool streamable = (dtype == TFH_F64 || dtype == TFH_C128) && M <= SKINNY_MAX_M && K * ec <= SKINNY_MAX_KR && N >= 4096;
+        if (streamable) {
+            // (that kernel works on units of SKINNY_UNIT consecutive n: a long side whose innermost runs are too short
+            // for them would end on the 64x64 tiles below, at half the rate of the thin tiles)
+            std::vector<Axis> long_side = ax.N;
+            order_by(long_side, 2);
+            fuse_axes(long_side, 3);
+            if (long_side.empty() || !skinny_run_ok(long_side.back().n)) streamable = false;
+        }
         if (M < 96 && M * ec >= 33 && N * ec >= 96 && !streamable) {
             std::swap(a, b);
             std::swap(conj_a, conj_b);
@@ -765,7 +777,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     // LDS tile ("out_rows").
     bool out_rows = false;
     if ((dtype == TFH_F64 || cxd) && nb == 1 && N <= SKINNY_MAX_M && M >= 4096 && K * (cxd ? 2 : 1) <= SKINNY_MAX_KR && a_kfast &&
-        !k_by_b && !ax.K.empty() && ax.N.size() == 1 && ax.N[0].s[2] == 1 && !ax.M.empty() && ax.M.back().n % SKINNY_UNIT == 0 &&
+        !k_by_b && !ax.K.empty() && ax.N.size() == 1 && ax.N[0].s[2] == 1 && !ax.M.empty() && skinny_run_ok(ax.M.back().n) &&
         (cxd || (N % 2 == 0 && K % 2 == 0 && (uintptr_t)c % 16 == 0 && (uintptr_t)a % 16 == 0))) {
         bool ok = true;
         int64_t expect = 1;
@@ -792,7 +804,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     const bool k_rows_b = out_rows || k_by_b;   // the k modes are in the memory order of the (possibly exchanged) B
     bool skinny = (dtype == TFH_F64 || cxd) && nb == 1 && M <= SKINNY_MAX_M && K * (cxd ? 2 : 1) <= SKINNY_MAX_KR && N >= 4096 &&
                   b_kfast && !ax.K.empty() && k_rows_b && !ax.N.empty() &&
-                  ax.N.back().n % SKINNY_UNIT == 0 && (out_rows || ax.N.back().s[2] == 1);
+                  skinny_run_ok(ax.N.back().n) && (out_rows || ax.N.back().s[2] == 1);
     if (skinny) {   // a row of B is one contiguous run of k (A's k order is free: it goes through the k table)
         int64_t expect = 1;
         for (int d = (int)ax.K.size() - 1; d >= 0; --d) {
@@ -804,7 +816,8 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         skinny = K % 2 == 0 && (uintptr_t)b % 16 == 0;
         for (auto& x : ax.N) skinny = skinny && x.s[1] % 2 == 0;
     }
-    int64_t inner_b = 0, inner_c = 0;
+    int64_t inner_b = 0, inner_c = 0, skinny_upr = 1;
+    int skinny_tail = 0;
     if (skinny) {
         int64_t lo = 0, hi = 0;
         reach(ax.M, 2, lo, hi);
@@ -815,10 +828,16 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         Axis& x = ax.N.back();
         inner_b = x.s[1];
         inner_c = x.s[2];
-        x.n /= SKINNY_UNIT;
+        skinny_tail = (int)(x.n % SKINNY_UNIT);
+        x.n = (x.n + SKINNY_UNIT - 1) / SKINNY_UNIT;   // units per innermost run; the last one holds skinny_tail n (0: all)
+        skinny_upr = x.n;
         for (int slot = 0; slot < 3; ++slot) x.s[slot] *= SKINNY_UNIT;
     }
-    const int64_t Ntab = skinny ? N / SKINNY_UNIT : N;   // entries of the n tables
+    int64_t Ntab = N;   // entries of the n tables
+    if (skinny) {
+        Ntab = 1;
+        for (auto& x : ax.N) Ntab *= x.n;
+    }
 
     GemmArgs g;
     std::memset(&g, 0, sizeof g);
@@ -1067,6 +1086,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         sk.out_rows = out_rows;
         sk.plain = alpha.re == 1.0 && alpha.im == 0.0 && beta.is_zero();
         sk.units = Ntab;
+        sk.upr = (int32_t)skinny_upr; sk.tail = skinny_tail;
         sk.am = g.am; sk.ak = g.ak; sk.cm = g.cm; sk.bu = g.bn; sk.cu = g.cn;
         sk.b_in = (int32_t)inner_b; sk.c_in = (int32_t)inner_c;
         sk.alpha_re = alpha.re; sk.alpha_im = alpha.im; sk.beta_re = beta.re; sk.beta_im = beta.im;

@@ -90,12 +90,14 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
 
     // ---- this lane's share of a unit of B: chunk id = lane + 64 u -> (row, chunk of the row)
     int32_t goff[LOADS], loff[LOADS];
-    uint32_t have = 0;
+    uint32_t have = 0, lrows = 0;   // lrows: four bits per load, the row (n of the unit) it belongs to
+    static_assert(LOADS <= 8 && SKINNY_UNIT <= 16, "row numbers are packed four bits per load");
 #pragma unroll
     for (int u = 0; u < LOADS; ++u) {
         const int id = lane + 64 * u, row = id / kc, col = id - row * kc;
         const bool ok = id < SKINNY_UNIT * kc;
         have |= (ok ? 1u : 0u) << u;
+        lrows |= (ok ? (uint32_t)row : 0u) << (4 * u);
         goff[u] = ok ? row * s.b_in * (8 * NC) + col * 16 : 0;
         loff[u] = ok ? row * PITCH + col * 16 : 0;
     }
@@ -117,7 +119,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
     const double ar = s.alpha_re, ai = s.alpha_im, br = s.beta_re, bi = s.beta_im;
     // C contiguous along m: 16-byte piece id = lane + 64 u of the unit's result tile -> (n of the unit, piece of its row)
     int32_t ogoff[LOADS], oloff[LOADS];
-    uint32_t ohave = 0;
+    uint32_t ohave = 0, orows = 0;
     if (s.out_rows) {
         const int cpr = s.M * NC / 2;   // 16-byte pieces per row of C
 #pragma unroll
@@ -125,6 +127,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
             const int id = lane + 64 * u, row = id / cpr, col = id - row * cpr;
             const bool ok = id < SKINNY_UNIT * cpr;
             ohave |= (ok ? 1u : 0u) << u;
+            orows |= (ok ? (uint32_t)row : 0u) << (4 * u);
             ogoff[u] = ok ? (row * s.c_in * NC + col * 2) * 8 : 0;
             oloff[u] = ok ? (row * OUT_PITCH + col * 2) * 8 : 0;
         }
@@ -133,14 +136,26 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
     const int64_t nwaves = (int64_t)gridDim.x * (THREADS / 64);
     int64_t unit = (int64_t)blockIdx.x * (THREADS / 64) + wave;
     d2 stage[LOADS];
+    // The innermost run of n need not hold a whole number of units: the last unit of each run then has s.tail valid n.
+    // Rows past them are neither loaded (what is parked for them is whatever the registers held: their columns of the
+    // product are independent of the others and never stored) nor written.
+    auto valid_of = [&](int64_t un) -> int {
+        if (s.tail == 0) return SKINNY_UNIT;
+        return (int)(un % s.upr) == s.upr - 1 ? s.tail : SKINNY_UNIT;
+    };
     auto issue = [&](int64_t un) {
         const unsigned char* Bu = reinterpret_cast<const unsigned char*>(s.B) + off_of(s.bu, un) * (8 * NC);
+        const int valid = valid_of(un);
 #pragma unroll
         for (int u = 0; u < LOADS; ++u)
-            if ((have >> u) & 1u) stage[u] = __builtin_nontemporal_load(reinterpret_cast<const d2*>(Bu + goff[u]));
+            if (((have >> u) & 1u) && (int)((lrows >> (4 * u)) & 15u) < valid)
+                stage[u] = __builtin_nontemporal_load(reinterpret_cast<const d2*>(Bu + goff[u]));
     };
+#pragma unroll
+    for (int u = 0; u < LOADS; ++u) stage[u] = d2{0, 0};
     if (unit < s.units) issue(unit);
     while (unit < s.units) {
+        const int valid = valid_of(unit);
 #pragma unroll
         for (int u = 0; u < LOADS; ++u)
             if ((have >> u) & 1u) *reinterpret_cast<d2*>(lds + loff[u]) = stage[u];
@@ -201,7 +216,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
             wave_sync();
 #pragma unroll
             for (int u = 0; u < LOADS; ++u)
-                if ((ohave >> u) & 1u) {
+                if (((ohave >> u) & 1u) && (int)((orows >> (4 * u)) & 15u) < valid) {
                     d2 v = *reinterpret_cast<const d2*>(lds + oloff[u]);
                     d2* dst = reinterpret_cast<d2*>(reinterpret_cast<unsigned char*>(Cu) + ogoff[u]);
                     if (!s.plain) {
@@ -231,9 +246,10 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
             if (mb < nmb) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const bool ok = Mfma<double>::row(lane, r) + 16 * mb < s.M;
+                    const bool row_ok = Mfma<double>::row(lane, r) + 16 * mb < s.M;
 #pragma unroll
                     for (int nb = 0; nb < NBLK; ++nb) {
+                        const bool ok = row_ok && (CX ? 8 * nb + (j >> 1) : j) < valid;
                         double* dst = Cu + crow[mb][r] + ccol[nb];
                         double v = acc[mb][nb][r];
                         if (!s.plain) {

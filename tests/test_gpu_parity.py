@@ -1708,12 +1708,15 @@ def test_offset_tables_are_kept_per_layout_and_survive_a_release(tf, oracle):
 
 
 @pytest.mark.parametrize("dtype", [np.complex128, np.float64])
-@pytest.mark.parametrize("m,k,x,c", [(32, 32, 8, 1024), (20, 13, 64, 80), (16, 32, 1, 4096), (7, 6, 16, 512), (32, 2, 32, 160)])
+@pytest.mark.parametrize("m,k,x,c", [(32, 32, 8, 1024), (20, 13, 64, 80), (16, 32, 1, 4096), (7, 6, 16, 512), (32, 2, 32, 160),
+                                     (32, 32, 16, 500), (16, 8, 64, 100), (20, 16, 100, 50), (5, 4, 5, 1000), (8, 6, 300, 17)])
 def test_contract_small_operator_applied_to_a_long_tensor(tf, oracle, dtype, m, k, x, c):
     # T[x, c, k] . W[k, m] -> out[x, m, c]: few rows, little k, a long n = (x, c) whose fastest output axis is c -- the
     # shape of an operator applied to every fibre of a large tensor, which takes the streaming kernel.  Odd m and k,
     # general alpha/beta, and a W that is a strided view are covered; f64 needs an even k for that kernel and falls
-    # back to the tiled one otherwise (k = 13).
+    # back to the tiled one otherwise (k = 13).  The kernel works on units of 16 consecutive c: extents that are no
+    # multiple of 16 (500, 100, 50, 1000: bond dimensions are rarely powers of two) end each run on a partly filled unit;
+    # a run shorter than three units (17) is left to the tiled kernels.
     rng = np.random.default_rng(91)
     t = rand(rng, (x, c, k), dtype)
     w = rand(rng, (k, 2 * m), dtype)[:, ::2]
@@ -1726,7 +1729,7 @@ def test_contract_small_operator_applied_to_a_long_tensor(tf, oracle, dtype, m, 
         dout = dev(tf, out0)
         plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab("xmc")), [t.shape, w.shape, ref.shape])
         tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
-        streamed = cplx or k % 2 == 0
+        streamed = (cplx or k % 2 == 0) and (c % 16 == 0 or c >= 48)
         assert ("gemm_skinny_kernel" in tf.last_kernel()) == streamed, tf.last_kernel()
         assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
 
@@ -1774,10 +1777,12 @@ def test_contract_small_operator_strided_rows_and_split_k_order(tf, oracle, dtyp
 
 
 @pytest.mark.parametrize("dtype", [np.complex128, np.float64])
-@pytest.mark.parametrize("m,k,x,c", [(32, 32, 8, 1024), (20, 13, 64, 80), (16, 32, 1, 4096), (7, 6, 16, 512), (32, 2, 32, 160), (2, 64, 4, 2048)])
+@pytest.mark.parametrize("m,k,x,c", [(32, 32, 8, 1024), (20, 13, 64, 80), (16, 32, 1, 4096), (7, 6, 16, 512), (32, 2, 32, 160), (2, 64, 4, 2048),
+                                     (32, 32, 9, 500), (16, 8, 7, 700), (4, 4, 1, 4099)])
 def test_contract_small_operator_with_the_result_contiguous_along_its_columns(tf, oracle, dtype, m, k, x, c):
     # the other orientation of the same product: T[x, c, k] . W[k, m] -> out[x, c, m], the few columns m adjacent in the
     # output.  The streaming kernel then transposes each unit's results through LDS.  f64 needs even m and k for it.
+    # (x, c) is one run of x * c here: 9 * 500, 7 * 700 and 4099 leave a partly filled last unit.
     cplx = np.issubdtype(dtype, np.complexfloating)
     if k > 32 and cplx:
         k = 32
