@@ -51,7 +51,9 @@ __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <bool CX>
+// RAGGED: the innermost run of n holds no whole number of units (its own instantiation: the full-unit kernel carries
+// none of the per-unit predicates)
+template <bool CX, bool RAGGED>
 __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
     constexpr int NBLK = CX ? 2 : 1;   // column blocks (16 real columns each) per unit
     constexpr int NC = CX ? 2 : 1;     // doubles per element
@@ -140,7 +142,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
     // Rows past them are neither loaded (what is parked for them is whatever the registers held: their columns of the
     // product are independent of the others and never stored) nor written.
     auto valid_of = [&](int64_t un) -> int {
-        if (s.tail == 0) return SKINNY_UNIT;
+        if constexpr (!RAGGED) return SKINNY_UNIT;
         return (int)(un % s.upr) == s.upr - 1 ? s.tail : SKINNY_UNIT;
     };
     auto issue = [&](int64_t un) {
@@ -284,8 +286,13 @@ void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
     const int64_t blocks_wanted = (s.units + THREADS / 64 - 1) / (THREADS / 64);
     const dim3 grid((uint32_t)std::min<int64_t>(blocks_wanted, 512)), block(THREADS);
     const size_t lds = (size_t)(THREADS / 64) * WAVE_LDS;
-    if (dtype == TFH_C128) TFH_LAUNCH_TIMED((gemm_skinny_kernel<true>), grid, block, lds, st, s);
-    else TFH_LAUNCH_TIMED((gemm_skinny_kernel<false>), grid, block, lds, st, s);
+    if (s.tail != 0) {
+        if (dtype == TFH_C128) TFH_LAUNCH_TIMED((gemm_skinny_kernel<true, true>), grid, block, lds, st, s);
+        else TFH_LAUNCH_TIMED((gemm_skinny_kernel<false, true>), grid, block, lds, st, s);
+    } else {
+        if (dtype == TFH_C128) TFH_LAUNCH_TIMED((gemm_skinny_kernel<true, false>), grid, block, lds, st, s);
+        else TFH_LAUNCH_TIMED((gemm_skinny_kernel<false, false>), grid, block, lds, st, s);
+    }
 }
 
 }  // namespace tfh
