@@ -77,10 +77,11 @@ __device__ __forceinline__ void lds_store_pack(R* p, const R (&x)[N]) {
     *reinterpret_cast<Raw*>(p) = __builtin_bit_cast(Raw, t);
 }
 
-// BNV: real columns per tile, 128 or 64 (a thin right-hand side: 33..95 real columns)
-template <class R, bool CX, int BNV = 128>
+// BNV: real columns per tile, 128 or 64 (a thin right-hand side: 33..95 real columns); BMV: rows per tile, 128, or 64 for
+// products with too few large tiles to fill the device (64 x 64 tiles: wave tile 32 x 32, four blocks per CU)
+template <class R, bool CX, int BNV = 128, int BMV = 128>
 struct Cfg128 {
-    static constexpr int BM = 128, BN = BNV;
+    static constexpr int BM = BMV, BN = BNV;
     static constexpr int BKR = 128 / sizeof(R);           // real k per stage: 128 bytes per row
     static constexpr int EC = CX ? 2 : 1;                 // reals per element
     static constexpr int BKE = BKR / EC;                  // elements of k per stage
@@ -90,9 +91,9 @@ struct Cfg128 {
     static constexpr int BNE = BN / EC;                   // element columns per tile
     static constexpr int WAVES_M = 2, WAVES_N = 2, NT = 64 * WAVES_M * WAVES_N;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 16, TN = WN / 16;
-    static constexpr int MIN_WAVES = 2;   // waves per SIMD the register budget is sized for
+    static constexpr int MIN_WAVES = BMV == 64 ? 4 : 2;   // waves per SIMD the register budget is sized for
     static constexpr size_t LDS_BYTES = (size_t)2 * (BM + BN) * PITCH * sizeof(R);
-    static_assert(TM == 4 && (TN == 4 || TN == 2), "wave tiles are four or two 16-row blocks wide");
+    static_assert((TM == 4 && (TN == 4 || TN == 2)) || (TM == 2 && TN == 2), "wave tiles are four or two 16-row blocks high and wide");
     static_assert(BKR / CH == 8, "eight 16-byte chunks per row");
     // position of a row's chunks: see the layout note at the top of the file
     __device__ static __forceinline__ int swizzle(int rr) { return (rr & 7) ^ ((rr >> 3) & 3); }
@@ -271,9 +272,9 @@ struct TileCtx {
     bool grouped;   // a problem of a grouped launch: plain strided matrices, offsets relative to the problem's first element
 };
 
-template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128>
+template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128, int BMV = 128>
 __device__ __forceinline__ void gemm128_body(const GemmArgs& g, const TileCtx& t, unsigned char* smem_raw) {
-    typedef Cfg128<R, CX, BNV> C_;
+    typedef Cfg128<R, CX, BNV, BMV> C_;
     typedef typename Mfma<R>::acc_t acc_t;
     constexpr int BM = C_::BM, BN = C_::BN, BKE = C_::BKE, PITCH = C_::PITCH, BNE = C_::BNE, CH = C_::CH;
     constexpr int TM = C_::TM, TN = C_::TN;
@@ -607,8 +608,8 @@ __device__ __forceinline__ void gemm128_body(const GemmArgs& g, const TileCtx& t
 }
 
 // One tile of a uniform launch (single problem, batched, split-K) or of a grouped launch whose tiles all have this shape.
-template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128>
-__global__ void __launch_bounds__((Cfg128<R, CX, BNV>::NT), (Cfg128<R, CX, BNV>::MIN_WAVES)) gemm128_kernel(GemmArgs g) {
+template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128, int BMV = 128>
+__global__ void __launch_bounds__((Cfg128<R, CX, BNV, BMV>::NT), (Cfg128<R, CX, BNV, BMV>::MIN_WAVES)) gemm128_kernel(GemmArgs g) {
     typedef typename ElemT<R, CX>::type E;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     TileCtx t;
@@ -642,7 +643,7 @@ __global__ void __launch_bounds__((Cfg128<R, CX, BNV>::NT), (Cfg128<R, CX, BNV>:
         t.Ap += off_of(g.ab, t.batch) * (int64_t)sizeof(E);
         t.Bp += off_of(g.bb, t.batch) * (int64_t)sizeof(E);
     }
-    gemm128_body<R, CX, AKF, BKF, VA, VB, BNV>(g, t, smem_raw);
+    gemm128_body<R, CX, AKF, BKF, VA, VB, BNV, BMV>(g, t, smem_raw);
 }
 
 // Grouped launch with a tile shape per map entry (tile_map[].w): 0 = 128 x 128; 1 = 128 rows x 64 real columns (a last
@@ -690,19 +691,20 @@ __global__ void __launch_bounds__((Cfg128<R, CX, 128>::NT), (Cfg128<R, CX, 128>:
     }
 }
 
-template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128>
+template <class R, bool CX, bool AKF, bool BKF, int VA, int VB, int BNV = 128, int BMV = 128>
 inline void launch_gemm128_variant(const GemmArgs& g, dim3 grid, hipStream_t st) {
     static bool once = [] {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm128_kernel<R, CX, AKF, BKF, VA, VB, BNV>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg128<R, CX, BNV>::LDS_BYTES);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm128_kernel<R, CX, AKF, BKF, VA, VB, BNV, BMV>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)Cfg128<R, CX, BNV, BMV>::LDS_BYTES);
         return true;
     }();
     (void)once;
-    typedef Cfg128<R, CX, BNV> C_;
+    typedef Cfg128<R, CX, BNV, BMV> C_;
     const size_t lds = C_::LDS_BYTES;
     const dim3 block(C_::NT);
-    TFH_LAUNCH_TIMED((gemm128_kernel<R, CX, AKF, BKF, VA, VB, BNV>), grid, block, lds, st, g);
-    if (BNV == 64) note_kernel("(gemm128_kernel, 128x64 tiles)");
+    TFH_LAUNCH_TIMED((gemm128_kernel<R, CX, AKF, BKF, VA, VB, BNV, BMV>), grid, block, lds, st, g);
+    if (BMV == 64) note_kernel("(gemm128_kernel, 64x64 tiles)");
+    else if (BNV == 64) note_kernel("(gemm128_kernel, 128x64 tiles)");
 }
 
 template <class R, bool CX, int V, int BNV = 128>
@@ -780,6 +782,32 @@ inline void launch_gemm128x64_any(const GemmArgs& g, dim3 grid, bool akf, bool b
     launch_gemm128_layout<R, CX, 1, 64>(g, grid, akf, bkf, st);
 }
 
+// 64 x 64 tiles.  A row-contiguous operand of 4-byte reals over 64 rows is loaded with 8-byte accesses (as the thin B above).
+template <class R, bool CX>
+inline void launch_gemm64x64_any(const GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
+    constexpr int VMAX = Cfg128<R, CX>::VMAX;
+    if constexpr (VMAX > 1) {
+        if (g.vec) {
+            constexpr int VR = sizeof(R) == 8 ? VMAX : VMAX / 2;   // row-contiguous operand
+            if (akf) {
+                if (bkf) launch_gemm128_variant<R, CX, true, true, VMAX, VMAX, 64, 64>(g, grid, st);
+                else launch_gemm128_variant<R, CX, true, false, VMAX, VR, 64, 64>(g, grid, st);
+            } else {
+                if (bkf) launch_gemm128_variant<R, CX, false, true, VR, VMAX, 64, 64>(g, grid, st);
+                else launch_gemm128_variant<R, CX, false, false, VR, VR, 64, 64>(g, grid, st);
+            }
+            return;
+        }
+    }
+    if (akf) {
+        if (bkf) launch_gemm128_variant<R, CX, true, true, 1, 1, 64, 64>(g, grid, st);
+        else launch_gemm128_variant<R, CX, true, false, 1, 1, 64, 64>(g, grid, st);
+    } else {
+        if (bkf) launch_gemm128_variant<R, CX, false, true, 1, 1, 64, 64>(g, grid, st);
+        else launch_gemm128_variant<R, CX, false, false, 1, 1, 64, 64>(g, grid, st);
+    }
+}
+
 }  // namespace gemm
 
 // One translation unit per dtype instantiates its four layout variants.
@@ -792,6 +820,11 @@ void launch_gemm128x64_f32(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bk
 void launch_gemm128x64_f64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
 void launch_gemm128x64_c64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
 void launch_gemm128x64_c128(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+// ... with 64 x 64 tiles (translation units of their own)
+void launch_gemm64x64_f32(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+void launch_gemm64x64_f64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+void launch_gemm64x64_c64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
+void launch_gemm64x64_c128(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
 // ... and the grouped kernel with a tile shape per map entry
 void launch_gemm128_grouped_f32(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);
 void launch_gemm128_grouped_f64(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st);

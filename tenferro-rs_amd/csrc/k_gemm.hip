@@ -487,7 +487,16 @@ void launch_generic64(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st) {
 }  // namespace
 void launch_gemm_wave(int dtype, const gemm::GemmArgs& g, int64_t nwork, hipStream_t st);   // k_gemm_wave.hip
 namespace {
-void launch_128(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st, int bn = 128) {
+void launch_128(int dtype, const GemmArgs& g, dim3 grid, hipStream_t st, int bn = 128, int bm = 128) {
+    if (bm == 64) {
+        switch (dtype) {
+            case TFH_F32: launch_gemm64x64_f32(g, grid, g.a_kfast, g.b_kfast, st); break;
+            case TFH_F64: launch_gemm64x64_f64(g, grid, g.a_kfast, g.b_kfast, st); break;
+            case TFH_C64: launch_gemm64x64_c64(g, grid, g.a_kfast, g.b_kfast, st); break;
+            default: launch_gemm64x64_c128(g, grid, g.a_kfast, g.b_kfast, st); break;
+        }
+        return;
+    }
     if (bn == 64) {
         switch (dtype) {
             case TFH_F32: launch_gemm128x64_f32(g, grid, g.a_kfast, g.b_kfast, st); break;
@@ -946,7 +955,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     // whole extent.  Usable when the offsets of
     // an operand span less than 4 GiB: always for operands below 4 GiB, and for larger ones whose long groups have
     // a single stride (anything else takes the generic kernel with 64-bit offsets).
-    bool use128 = bm == 128 && !skinny;
+    bool use128 = !skinny && !wavek;   // the large-tile kernel family: 128x128, 128x64 and 64x64 tiles
     int64_t lo_a = 0, hi_a = 0, lo_b = 0, hi_b = 0;
     auto tile_reach = [&](const std::vector<Axis>& grp, int slot, int64_t& lo, int64_t& hi) {
         if (grp.size() == 1) {
@@ -1073,7 +1082,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     }
     if (nsplit > 1) g.partial = ws + (cached ? 0 : table_bytes);
     dim3 grid((uint32_t)((int64_t)g.tiles_m * g.tiles_n * nb * nsplit), 1, 1);
-    g.one_round = grid.x <= 2u * compute_units();   // two blocks of the 128-tile kernel fit a CU
+    g.one_round = bm == 128 && grid.x <= 2u * compute_units();   // two blocks of the 128-tile kernel fit a CU
     const int prof = prof_begin(PROF_CONTRACT, stream);
     if (skinny) {
         SkinnyArgs sk;
@@ -1092,7 +1101,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         sk.alpha_re = alpha.re; sk.alpha_im = alpha.im; sk.beta_re = beta.re; sk.beta_im = beta.im;
         launch_gemm_skinny(dtype, sk, st);
     } else if (wavek) launch_gemm_wave(dtype, g, nb * g.tiles_m * g.tiles_n, st);
-    else if (use128) launch_128(dtype, g, grid, st, bn);
+    else if (use128) launch_128(dtype, g, grid, st, bn, bm);
     else launch_generic64(dtype, g, grid, st);
     prof_end(prof, stream);
     release_packed();   // stream-ordered: the next user of these blocks is enqueued after this kernel

@@ -1,0 +1,8 @@
+// k_gemm64_c128.hip -- instantiates the 64x64-tile variants of the large-tile contraction kernel for c128.
+#include "gemm128.hpp"
+
+namespace tfh {
+void launch_gemm64x64_c128(const gemm::GemmArgs& g, dim3 grid, bool akf, bool bkf, hipStream_t st) {
+    gemm::launch_gemm64x64_any<double, true>(g, grid, akf, bkf, st);
+}
+}  // namespace tfh

@@ -755,7 +755,7 @@ def test_conj_on_load_in_every_contraction_kernel(tf, dtype):
         ("km", "nk", "mn", dict(m=1500, k=150, n=1000), ", 128>)"),             # A column-contiguous, B k-contiguous
         ("mk", "kn", "mn", dict(m=32768, k=64, n=40), "128x64 tiles"),                # thin right-hand side: 128x64 tiles
         ("mk", "kn", "mn", dict(m=40, k=64, n=32768), "128x64 tiles"),                # thin left-hand side: exchanged
-        ("mk", "kn", "mn", dict(m=40, k=30, n=50), "(gemm_kernel"),
+        ("mk", "kn", "mn", dict(m=40, k=30, n=50), "64x64 tiles"),
         ("bmk", "bkn", "bmn", dict(b=70, m=20, k=24, n=18), "gemm_wave_kernel"),
         ("xk", "mk", "xm", dict(x=4096, k=16, m=12), None),                     # small operator on a long tensor
         ("mk", "k", "m", dict(m=500, k=300), None),                              # matrix . vector: conjugated copy, then the reduction kernel
@@ -782,7 +782,26 @@ def test_conj_on_load_in_every_contraction_kernel(tf, dtype):
                 seen.add(want)
             ref = alpha * _contract_np(np.conj(a) if ca else a, ma, np.conj(b) if cb else b, mb, mc) + beta * c0
             assert relerr(out.to_numpy(), ref) < tol, (ma, mb, mc, ca, cb, label)
-    assert {", 128>)", "128x64 tiles", "(gemm_kernel", "gemm_wave_kernel"} <= seen
+    assert {", 128>)", "128x64 tiles", "64x64 tiles", "gemm_wave_kernel"} <= seen
+    # the kernel with 64-bit offsets takes what the others cannot address: rows of A 2 GiB apart (a view of a large
+    # buffer of which only those rows are ever touched; more than eight rows, or a conjugated copy would be made first)
+    import torch
+    m, k, n = 9, 30, 50
+    gap = (1 << 31) // np.dtype(dtype).itemsize
+    big = torch.empty((m - 1) * gap + k, dtype=torch.complex64 if dtype == np.complex64 else torch.complex128, device="cuda")
+    a = rand(rng, (m, k), dtype)
+    for r in range(m):
+        big[r * gap:r * gap + k] = torch.from_numpy(a[r]).cuda()
+    A = tf.Tensor(big, [m, k], [gap, 1], 0, tf.GpuMemory(0), tf.dtype_code(np.dtype(dtype)))
+    b = rand(rng, (k, n), dtype)
+    c0 = rand(rng, (m, n), dtype)
+    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("mk"), lab("kn"), lab("mn")), [[m, k], [k, n], [m, n]])
+    for ca, cb in [(True, False), (False, True), (True, True)]:
+        out = dev(tf, c0)
+        tf.HipBackend.execute(plan, alpha, [A.conj_on_load() if ca else A, dev(tf, b).conj_on_load() if cb else dev(tf, b)], beta, out)
+        assert "(gemm_kernel" in tf.last_kernel(), tf.last_kernel()
+        ref = alpha * ((np.conj(a) if ca else a) @ (np.conj(b) if cb else b)) + beta * c0
+        assert relerr(out.to_numpy(), ref) < tol, (ca, cb)
 
 
 def test_conj_on_load_views_einsum_permute_and_rejections(tf, oracle):
