@@ -1451,7 +1451,9 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
         std::memcpy(s.p, probs.data() + first, sizeof(GroupProblem) * (size_t)s.count);
         hipLaunchKernelGGL(set_problems_kernel, dim3(1), dim3(64), 0, st, problems_dev, s);
     }
-    g.vec = gs->bm == 128 && vec;
+    // 64 x 64 tiles run on the large-tile kernel as well when its 32-bit offsets suffice
+    const bool large64 = gs->bm == 64 && ok128;
+    g.vec = (gs->bm == 128 || large64) && vec;
     g.alpha_re = alpha.re; g.alpha_im = alpha.im; g.beta_re = beta.re; g.beta_im = beta.im;
     g.use_beta = !beta.is_zero();
     g.problems = problems_dev;
@@ -1467,6 +1469,7 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
             default: launch_gemm128_grouped_c128(g, grid, g.a_kfast, g.b_kfast, st); break;
         }
     } else if (gs->bm == 128) launch_128(dtype, g, grid, st);
+    else if (large64) launch_128(dtype, g, grid, st, 64, 64);
     else launch_generic64(dtype, g, grid, st);
     prof_end(prof, stream);
     return hip_check(hipGetLastError(), "grouped contraction launch");
