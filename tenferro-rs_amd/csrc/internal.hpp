@@ -80,6 +80,8 @@ namespace tfh {
 // labels; returns TFH_OK or records an error.
 int32_t make_plan(int32_t dtype, const tfh_desc* desc, const int64_t* const* shapes, const int32_t* ranks,
                   int32_t n_tensors, tfh_plan& plan);
+// Whether `stream` is recording a graph (nothing may be allocated or synchronised then).
+bool stream_is_capturing(void* stream);
 int32_t check_view_against(const std::vector<int64_t>& shape, const tfh_view& v, const char* what);
 
 // Mode classification of a binary contraction (tenferro-prims/src/lib.rs:136-138).

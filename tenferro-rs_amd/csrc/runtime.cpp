@@ -113,6 +113,8 @@ int32_t malloc_or_release(void** p, size_t bytes, void* stream, const char* what
 }
 }  // namespace
 
+bool stream_is_capturing(void* stream) { return capturing(stream); }
+
 void arena_begin(void* base, size_t bytes) { t_arena = Arena{(char*)base, bytes, 0, true}; }
 void arena_end() { t_arena = Arena{}; }
 

@@ -470,6 +470,52 @@ def test_grouped_plan_on_two_streams_with_different_operands(tf, oracle):
             tf.lib().tfh_stream_destroy(st)
 
 
+def test_grouped_records_are_kept_for_repeated_calls(tf, oracle):
+    # A grouped call whose operands, outputs and strides equal those of an earlier call of the plan reuses the problem
+    # records that call wrote to the device; new operand sets get records of their own, and once the plan holds as many
+    # sets as it keeps, further ones are written per call again.  Twelve operand sets, each run three times in an
+    # interleaved order, one of them also from a second stream, and a set whose output alone differs: every result is
+    # that of its own operands.
+    import ctypes
+    dims = [(96, 64, 80), (33, 70, 129), (128, 128, 128), (17, 5, 260)] * 3
+    rng = np.random.default_rng(84)
+    desc = tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik"))
+    plan = tf.HipBackend.plan_grouped(np.float64, desc, [[[i, j], [j, k], [i, k]] for (i, j, k) in dims])
+    sets = []
+    for s_ in range(12):
+        As = [rng.standard_normal((i, j)) for (i, j, k) in dims]
+        Bs = [rng.standard_normal((j, k)) for (i, j, k) in dims]
+        outs = [tf.Tensor.empty([i, k], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64) for (i, j, k) in dims]
+        sets.append((As, Bs, [(dev(tf, a), dev(tf, b)) for a, b in zip(As, Bs)], outs))
+    for rep in range(3):
+        for As, Bs, ins, outs in (sets if rep != 1 else sets[::-1]):
+            for o in outs:
+                o._buf.zero_()
+            tf.HipBackend.execute_grouped(plan, 1.0, ins, 0.0, outs)
+            for a, b, o in zip(As, Bs, outs):
+                assert relerr(o.to_numpy(), a @ b) < 1e-12, rep
+    # the first set again, from another stream (its records were written on the default stream), with alpha and beta
+    st = ctypes.c_void_p()
+    assert tf.lib().tfh_stream_create(ctypes.byref(st)) == 0
+    try:
+        As, Bs, ins, outs = sets[0]
+        before = [o.to_numpy() for o in outs]
+        import torch
+        torch.cuda.synchronize()
+        tf.HipBackend.execute_grouped(plan, 2.0, ins, -1.0, outs, stream=st.value)
+        assert tf.lib().tfh_stream_synchronize(st) == 0
+        for a, b, o, c0 in zip(As, Bs, outs, before):
+            assert relerr(o.to_numpy(), 2.0 * (a @ b) - c0) < 1e-12
+    finally:
+        tf.lib().tfh_stream_destroy(st)
+    # same inputs, other outputs: different records
+    As, Bs, ins, outs = sets[1]
+    outs2 = [tf.Tensor.empty([i, k], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64) for (i, j, k) in dims]
+    tf.HipBackend.execute_grouped(plan, 1.0, ins, 0.0, outs2)
+    for a, b, o in zip(As, Bs, outs2):
+        assert relerr(o.to_numpy(), a @ b) < 1e-12
+
+
 @pytest.mark.parametrize("dtype", ALL)
 def test_grouped_tiny_problems_take_the_wave_kernel(tf, oracle, dtype):
     # 300 problems with every extent between 1 and 32 (a block-sparse tensor with small blocks): one grouped launch,
