@@ -470,6 +470,25 @@ def test_grouped_plan_on_two_streams_with_different_operands(tf, oracle):
             tf.lib().tfh_stream_destroy(st)
 
 
+@pytest.mark.parametrize("ma,mb,mc", [("ij", "jk", "ik"), ("ji", "kj", "ki"), ("ij", "kj", "ki"), ("aij", "jk", "aik"), ("ijl", "jlk", "ik")])
+def test_grouped_label_orders_and_fusable_modes(tf, oracle, ma, mb, mc):
+    # The roles of a matrix product's axes come from the plan's labels, in any order (transposed operands, transposed
+    # result); operands with more than two modes are plain matrices once their modes fuse (a leading free mode, two
+    # summed modes), and go through the general classification.
+    rng = np.random.default_rng(85)
+    ext_sets = [dict(i=70, j=33, k=130, a=3, l=4), dict(i=5, j=64, k=7, a=2, l=2), dict(i=128, j=128, k=64, a=1, l=8), dict(i=1, j=9, k=257, a=4, l=1)]
+    shapes, As, Bs, outs = [], [], [], []
+    for ext in ext_sets:
+        sa, sb, sc = [ext[c] for c in ma], [ext[c] for c in mb], [ext[c] for c in mc]
+        shapes.append([sa, sb, sc])
+        As.append(rng.standard_normal(sa)); Bs.append(rng.standard_normal(sb))
+        outs.append(tf.Tensor.empty(sc, tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64))
+    plan = tf.HipBackend.plan_grouped(np.float64, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), shapes)
+    tf.HipBackend.execute_grouped(plan, 1.0, [(dev(tf, a), dev(tf, b)) for a, b in zip(As, Bs)], 0.0, outs)
+    for a, b, o in zip(As, Bs, outs):
+        assert relerr(o.to_numpy(), np.einsum(f"{ma},{mb}->{mc}", a, b)) < 1e-12, (ma, mb, mc, a.shape)
+
+
 def test_grouped_records_are_kept_for_repeated_calls(tf, oracle):
     # A grouped call whose operands, outputs and strides equal those of an earlier call of the plan reuses the problem
     # records that call wrote to the device; new operand sets get records of their own, and once the plan holds as many
