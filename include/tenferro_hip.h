@@ -169,7 +169,10 @@ int32_t tfh_execute(const tfh_plan* plan, const void* alpha,
 int32_t tfh_plan_create_grouped(int32_t dtype, const tfh_desc* desc, int32_t n_groups,
                                 const int64_t* const* shapes, const int32_t* ranks, int32_t n_tensors,
                                 tfh_plan** out);
-/* inputs: n_groups*n_inputs views, group-major; outputs: n_groups views.  One launch. */
+/* inputs: n_groups*n_inputs views, group-major; outputs: n_groups views.  One launch of the contraction; the
+ * problems' pointers, extents and strides are written to the device by small launches in front of it, and kept with
+ * the plan (up to eight sets per device), so that a call whose views equal those of an earlier call skips them.
+ * The plan must outlive the work enqueued through it (as its tile maps always had to). */
 int32_t tfh_execute_grouped(const tfh_plan* plan, const void* alpha,
                             const tfh_view* inputs, int32_t n_inputs,
                             const void* beta, tfh_view* outputs, tfh_stream stream);
