@@ -1499,8 +1499,18 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
     // the stream is being captured (nothing may be allocated then), they go into the workspace as described above.
     const size_t rec_bytes = sizeof(GroupProblem) * (size_t)plan.n_groups;
     GroupProblem* problems_dev = nullptr;
-    hipEvent_t written = nullptr;
+    auto write_records = [&](GroupProblem* dst) {
+        for (int first = 0; first < plan.n_groups; first += PROBS_PER_SET) {
+            ProblemSet s;
+            s.first = first;
+            s.count = std::min(PROBS_PER_SET, plan.n_groups - first);
+            std::memcpy(s.p, probs.data() + first, sizeof(GroupProblem) * (size_t)s.count);
+            hipLaunchKernelGGL(set_problems_kernel, dim3(1), dim3(64), 0, st, dst, s);
+        }
+    };
     if (!stream_is_capturing(stream)) {
+        // (the lock is held until a new set's writes and its event are enqueued: another thread that finds the set waits
+        // for an event that has been recorded)
         std::lock_guard<std::mutex> lk(gs->mu);
         int dev = 0;
         if (int32_t e = hip_check(hipGetDevice(&dev), "hipGetDevice")) return e;
@@ -1515,8 +1525,13 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
             GroupedState::Records r;
             if (hipMalloc((void**)&r.dev, rec_bytes) == hipSuccess && hipEventCreateWithFlags(&r.ready, hipEventDisableTiming) == hipSuccess) {
                 r.host = probs;
+                write_records(r.dev);
+                if (int32_t e = hip_check(hipEventRecord(r.ready, st), "hipEventRecord")) {
+                    (void)hipFree(r.dev);
+                    (void)hipEventDestroy(r.ready);
+                    return e;
+                }
                 problems_dev = r.dev;
-                written = r.ready;
                 dm.records.push_back(std::move(r));
             } else {
                 (void)hipGetLastError();
@@ -1524,22 +1539,11 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
             }
         }
     }
-    const bool reuse = problems_dev != nullptr && written == nullptr;
     if (!problems_dev) {
         void* ws = nullptr;
         if (int32_t e = workspace(stream, rec_bytes, &ws)) return e;
         problems_dev = (GroupProblem*)ws;
-    }
-    if (!reuse) {
-        for (int first = 0; first < plan.n_groups; first += PROBS_PER_SET) {
-            ProblemSet s;
-            s.first = first;
-            s.count = std::min(PROBS_PER_SET, plan.n_groups - first);
-            std::memcpy(s.p, probs.data() + first, sizeof(GroupProblem) * (size_t)s.count);
-            hipLaunchKernelGGL(set_problems_kernel, dim3(1), dim3(64), 0, st, problems_dev, s);
-        }
-        if (written)
-            if (int32_t e = hip_check(hipEventRecord(written, st), "hipEventRecord")) return e;
+        write_records(problems_dev);
     }
     // 64 x 64 tiles run on the large-tile kernel as well when its 32-bit offsets suffice
     const bool large64 = gs->bm == 64 && ok128;
