@@ -873,12 +873,12 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     // 64x64 kernel fills the chip better (18 us against 29 us; from 768^3 on the large tiles win)
     if (bm == 128 && bn == 128 && tiles_for(128, 128) * std::max<int64_t>(1, kstages / 8) <= 128 && tiles_for(64, 64) >= 2 * tiles_for(128, 128))
         bm = bn = 64;
-    // f64 / complex128 with less than one large tile per CU and at most 64 stages of k: split as deep as it pays, the
+    // f64 / complex128 with at most one large tile per CU and at most 64 stages of k: split as deep as it pays, the
     // large tiles' blocks are mostly prologue and epilogue, and four small blocks per CU do better (768^3 f64 35.6 ->
     // 30.7 us, 1024^3 56.3 -> 50.8, complex128 1024 x 1024 x 256 58 -> 42, 3000 x 600 x 200 75 -> 59); with a longer k
     // the large tiles win (1280^3 f64 85 against 94 us, complex128 768^3 80 against 112), and so they do for 4-byte
     // reals, whose MFMAs take half the time (1280^3 f32 48 against 63 us)
-    if (bm == 128 && bn == 128 && is_double(dtype) && tiles_for(128, 128) < 256 && kstages <= 64 && tiles_for(64, 64) >= 2 * tiles_for(128, 128))
+    if (bm == 128 && bn == 128 && is_double(dtype) && tiles_for(128, 128) <= 256 && kstages <= 64 && tiles_for(64, 64) >= 2 * tiles_for(128, 128))
         bm = bn = 64;
     // thin tiles that cannot reach one block per CU even with the deepest split: 64x64 tiles give twice the blocks
     if (bm == 128 && bn == 64 && tiles_for(128, 64) * std::max<int64_t>(1, kstages / 8) < 256 && tiles_for(64, 64) >= 2 * tiles_for(128, 64))

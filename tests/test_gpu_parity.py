@@ -749,7 +749,7 @@ def test_einsum_async_chaining(tf):
     assert relerr(d.to_numpy(), a @ b @ b) < 1e-12
 
 
-@pytest.mark.parametrize("nb,label", [(64, "(gemm128_kernel"), (6, "(gemm128_kernel, 64x64 tiles)")])
+@pytest.mark.parametrize("nb,label", [(80, "(gemm128_kernel"), (6, "(gemm128_kernel, 64x64 tiles)")])
 @pytest.mark.parametrize("dtype", ALL)
 def test_large_tile_kernel_stage_and_tile_boundaries(tf, dtype, nb, label):
     # The large-tile kernel treats a last k stage that is full, and a tile that lies wholly inside the matrix, like
