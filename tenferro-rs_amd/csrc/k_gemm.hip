@@ -873,13 +873,22 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     // 64x64 kernel fills the chip better (18 us against 29 us; from 768^3 on the large tiles win)
     if (bm == 128 && bn == 128 && tiles_for(128, 128) * std::max<int64_t>(1, kstages / 8) <= 128 && tiles_for(64, 64) >= 2 * tiles_for(128, 128))
         bm = bn = 64;
-    // f64 / complex128 with at most one large tile per CU and at most 64 stages of k: split as deep as it pays, the
-    // large tiles' blocks are mostly prologue and epilogue, and four small blocks per CU do better (768^3 f64 35.6 ->
-    // 30.7 us, 1024^3 56.3 -> 50.8, complex128 1024 x 1024 x 256 58 -> 42, 3000 x 600 x 200 75 -> 59); with a longer k
-    // the large tiles win (1280^3 f64 85 against 94 us, complex128 768^3 80 against 112), and so they do for 4-byte
-    // reals, whose MFMAs take half the time (1280^3 f32 48 against 63 us)
-    if (bm == 128 && bn == 128 && is_double(dtype) && tiles_for(128, 128) <= 256 && kstages <= 64 && tiles_for(64, 64) >= 2 * tiles_for(128, 128))
-        bm = bn = 64;
+    // f64 / complex128 with at most 64 stages of k (too short for a k split to even out the rounds): 512 large tiles
+    // are resident at a time, two per CU; a last round of up to 256 runs one block per CU in 0.62 of a full round's
+    // time, a fuller one takes a whole round.  64x64 tiles run 1024 at a time at half the rate per flop, so a round of
+    // them costs half a large round, and their last round fills in finer steps.  Estimated times in large rounds, the
+    // smaller wins (with a margin: the large tiles read less): 768^3 f64 35.6 -> 30.7 us, 1024^3 56.3 -> 50.8,
+    // 2560 x 2048 x 512 (320 large tiles) 131 -> 91, 3072^2 x 512 (576) 199 -> 156, 3584^2 x 256 (784) 138 -> 117;
+    // complex128 1024 x 1024 x 256 58 -> 42, 3072 x 1536 x 256 200 -> 156; 480, 768 and 1024 large tiles stay (133 / 138,
+    // 202 / 204, 259 / 270 us).  With a longer k the split estimate below evens out the large tiles' rounds, and for
+    // 4-byte reals, whose MFMAs take half the time, the small tiles lose (1280^3 f32 48 against 63 us).
+    if (bm == 128 && bn == 128 && is_double(dtype) && kstages <= 64 && tiles_for(128, 128) <= 1536 && tiles_for(64, 64) >= 2 * tiles_for(128, 128)) {
+        const int64_t t128 = tiles_for(128, 128), t64 = tiles_for(64, 64);
+        const int64_t r128 = t128 % 512, r64 = t64 % 1024;
+        const double time128 = (double)(t128 / 512) + (r128 == 0 ? 0.0 : (r128 <= 256 ? 0.62 : 1.0));
+        const double time64 = 0.5 * ((double)(t64 / 1024) + (r64 == 0 ? 0.0 : 0.5 + 0.5 * (double)r64 / 1024.0));
+        if (time64 < 0.9 * time128) bm = bn = 64;
+    }
     // thin tiles that cannot reach one block per CU even with the deepest split: 64x64 tiles give twice the blocks
     if (bm == 128 && bn == 64 && tiles_for(128, 64) * std::max<int64_t>(1, kstages / 8) < 256 && tiles_for(64, 64) >= 2 * tiles_for(128, 64))
         bm = 64;

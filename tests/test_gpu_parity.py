@@ -749,7 +749,7 @@ def test_einsum_async_chaining(tf):
     assert relerr(d.to_numpy(), a @ b @ b) < 1e-12
 
 
-@pytest.mark.parametrize("nb,label", [(80, "(gemm128_kernel"), (6, "(gemm128_kernel, 64x64 tiles)")])
+@pytest.mark.parametrize("nb,label", [(0, "(gemm128_kernel"), (6, "(gemm128_kernel, 64x64 tiles)")])
 @pytest.mark.parametrize("dtype", ALL)
 def test_large_tile_kernel_stage_and_tile_boundaries(tf, dtype, nb, label):
     # The large-tile kernel treats a last k stage that is full, and a tile that lies wholly inside the matrix, like
@@ -757,13 +757,19 @@ def test_large_tile_kernel_stage_and_tile_boundaries(tf, dtype, nb, label):
     # around those boundaries -- k a whole number of stages or one element off, rows and columns a whole number of tiles,
     # of 16-byte vectors, or neither -- in the four storage-order combinations of the operands and both orders of the
     # result, with and without an old result to add, against numpy.  Once with enough batch entries for its 128 x 128
-    # tiles at every extent below, once with so few that it runs with 64 x 64 tiles.
+    # tiles at every extent below (8-byte reals with so little k change to the small tiles until a launch holds more
+    # than 1536 large ones), once with so few that it runs with 64 x 64 tiles.
+    if nb == 0:
+        nb = {np.float32: 80, np.complex64: 80, np.float64: 385, np.complex128: 257}[dtype]
     rng = np.random.default_rng(71)
     tol = TOL[dtype]
     stage = {np.float32: 32, np.float64: 16, np.complex64: 16, np.complex128: 8}[dtype]
     seen = set()
-    for (m, n) in [(256, 256), (384, 130), (257, 255), (130, 384), (129, 131)]:
-        for k in (stage, 2 * stage, 3 * stage, 3 * stage - 1, 2 * stage + 1):
+    shapes, ks = [(256, 256), (384, 130), (257, 255), (130, 384), (129, 131)], (stage, 2 * stage, 3 * stage, 3 * stage - 1, 2 * stage + 1)
+    if nb > 100:   # (hundreds of batch entries: fewer combinations, the same boundaries)
+        shapes, ks = [(256, 256), (257, 255), (129, 131)], (stage, 3 * stage - 1, 2 * stage + 1)
+    for (m, n) in shapes:
+        for k in ks:
             for a_kfast, b_kfast in [(True, True), (True, False), (False, True), (False, False)]:
                 a = rand(rng, (nb, m, k), dtype) if a_kfast else rand(rng, (nb, k, m), dtype).transpose(0, 2, 1)
                 b = rand(rng, (nb, n, k), dtype).transpose(0, 2, 1) if b_kfast else rand(rng, (nb, k, n), dtype)
@@ -816,9 +822,9 @@ def test_conj_on_load_in_every_contraction_kernel(tf, dtype):
     rng = np.random.default_rng(61)
     tol = TOL[dtype]
     cases = [   # (modes a, modes b, modes c, extents, substring of the kernel label expected)
-        ("mk", "kn", "mn", dict(m=2000, k=150, n=1500), ", 128>)"),
-        ("mk", "kn", "nm", dict(m=2000, k=150, n=1500), ", 128>)"),             # C's fastest axis is m: operands exchanged
-        ("km", "nk", "mn", dict(m=2000, k=150, n=1500), ", 128>)"),             # A column-contiguous, B k-contiguous
+        ("mk", "kn", "mn", dict(m=2000, k=600, n=1500), ", 128>)"),
+        ("mk", "kn", "nm", dict(m=2000, k=600, n=1500), ", 128>)"),             # C's fastest axis is m: operands exchanged
+        ("km", "nk", "mn", dict(m=2000, k=600, n=1500), ", 128>)"),             # A column-contiguous, B k-contiguous
         ("mk", "kn", "mn", dict(m=32768, k=64, n=40), "128x64 tiles"),                # thin right-hand side: 128x64 tiles
         ("mk", "kn", "mn", dict(m=40, k=64, n=32768), "128x64 tiles"),                # thin left-hand side: exchanged
         ("mk", "kn", "mn", dict(m=40, k=30, n=50), "64x64 tiles"),
