@@ -559,6 +559,32 @@ uint32_t compute_units() {
 // or long enough that a partly filled last unit costs little (500 = 31 units and a quarter).
 bool skinny_run_ok(int64_t n) { return n % SKINNY_UNIT == 0 || n >= 3 * SKINNY_UNIT; }
 
+// A tiny operator (both of its extents at most 8) applied to the last leg of a long tensor -- the long operand's rows
+// are contiguous runs of k: the tiny-operator kernel (one thread per element of the long free index) then reads and
+// writes with a stride of one row between neighbouring lanes, while the streaming kernel of k_gemm_skinny.hip takes
+// whole rows.  Measured on 4M rows (us, tiny | streaming): complex128 8x8 566 | 208 with C contiguous along n and
+// 1959 | 203 along m, 8x4 185 | 172 and 1537 | 168, 4x4 130 | 166 and 412 | 159, 2x2 47 | 164 and 80 | 155; f64 8x8
+// 195 | 134 and 812 | 132, 4x4 65 | 117 and 167 | 119.  ms: the operator's free extent.
+bool last_leg_prefers_streaming(int dtype, const ContractAxes& ax, int64_t M, int64_t N, int64_t K) {
+    if (dtype != TFH_F64 && dtype != TFH_C128) return false;
+    const bool small_is_a = M <= N;
+    const int tslot = small_is_a ? 1 : 0;
+    const std::vector<Axis>& small = small_is_a ? ax.M : ax.N;
+    const int64_t ms = small_is_a ? M : N;
+    if (ms > 8 || K > 8) return false;
+    if (K * (dtype == TFH_C128 ? 16 : 8) < 32) return false;   // (rows under 32 bytes would be packed first)
+    std::vector<Axis> k = ax.K;
+    order_by(k, tslot);
+    int64_t expect = 1;
+    for (int d = (int)k.size() - 1; d >= 0; --d) {
+        if (k[d].n > 1 && k[d].s[tslot] != expect) return false;
+        expect *= k[d].n;
+    }
+    const bool rows = min_stride(small, 2) == 1;   // C contiguous along the operator's free index
+    if (dtype == TFH_C128) return rows ? (ms >= 3 || K >= 6) : (K >= 6 || (K >= 4 && ms >= 8));
+    return rows ? (ms >= 4 || K >= 8) : K >= 8;
+}
+
 int bke_of(int dtype) {
     int bkr = is_double(dtype) ? 16 : 32;
     return is_complex(dtype) ? bkr / 2 : bkr;
@@ -645,9 +671,13 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     // One free group empty (matrix-vector, vector-matrix, dot and batched dot products): there is nothing for a tile
     // of MFMAs to reuse -- a reduction of the elementwise product, bound by HBM (k_dot.hip)
     // a tiny operator applied to a long tensor (a gate on a leg of a state): a stream over the long operand
+    // (on the last leg of the long tensor the streaming kernel further down is usually faster: it is looked at first,
+    // and the tiny-operator kernel takes the product if that one cannot)
+    bool tiny_deferred = false;
     if (M > 1 && N > 1 && !conj_a && !conj_b) {
+        tiny_deferred = last_leg_prefers_streaming(dtype, ax, M, N, K);
         int32_t st_tiny = TFH_OK;
-        if (try_tiny_operator(dtype, a, b, c, ax, alpha, beta, stream, st_tiny)) return st_tiny;
+        if (!tiny_deferred && try_tiny_operator(dtype, a, b, c, ax, alpha, beta, stream, st_tiny)) return st_tiny;
     }
     if ((M == 1 || N == 1) && !conj_a && !conj_b) {
         std::vector<Axis> kept, red = ax.K;
@@ -841,6 +871,13 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         x.n = (x.n + SKINNY_UNIT - 1) / SKINNY_UNIT;   // units per innermost run; the last one holds skinny_tail n (0: all)
         skinny_upr = x.n;
         for (int slot = 0; slot < 3; ++slot) x.s[slot] *= SKINNY_UNIT;
+    }
+    if (!skinny && tiny_deferred) {
+        int32_t st_tiny = TFH_OK;
+        if (try_tiny_operator(dtype, a, b, c, ax, alpha, beta, stream, st_tiny)) {
+            release_packed();
+            return st_tiny;
+        }
     }
     int64_t Ntab = N;   // entries of the n tables
     if (skinny) {

@@ -41,7 +41,7 @@ constexpr int WAVE_LDS = SKINNY_UNIT * PITCH;      // each wave parks one unit
 constexpr int LOADS = SKINNY_UNIT * MAX_KC / 64;   // 16-byte loads per lane and unit at most
 constexpr int PAIRS = MAX_KC / 4;
 constexpr int OUT_PITCH = 2 * SKINNY_MAX_M + 2;   // doubles per row of the transposed result tile (complex: 32 x 2, +2 against bank conflicts)
-static_assert(SKINNY_UNIT * OUT_PITCH * 8 <= WAVE_LDS, "the result tile reuses the wave's LDS region");
+constexpr int TILE_LDS = SKINNY_UNIT * OUT_PITCH * 8;   // the transposed result tile of a wave: a region of its own
 
 // Orders the LDS accesses of one wave: lanes read what other lanes of the same wave wrote.  The LDS executes a wave's
 // instructions in order, so only the compiler has to be kept from moving accesses across this point.
@@ -52,14 +52,20 @@ __device__ __forceinline__ void wave_sync() {
 }
 
 // RAGGED: the innermost run of n holds no whole number of units (its own instantiation: the full-unit kernel carries
-// none of the per-unit predicates)
-template <bool CX, bool RAGGED>
+// none of the per-unit predicates).  OUT_ROWS: C is contiguous along m (s.out_rows).
+//
+// vmcnt counts loads and stores in one queue, in order, and the compiler waits for a register that was loaded in the
+// iteration before with vmcnt(0): whatever is stored shortly before that wait is waited for as well, acknowledgement
+// included.  With C contiguous along n a unit's results therefore stay in registers for one more iteration and leave
+// in the middle of the next unit's MFMAs: by the time the next wait comes, they have had half an iteration to drain.
+template <bool CX, bool RAGGED, bool OUT_ROWS>
 __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
     constexpr int NBLK = CX ? 2 : 1;   // column blocks (16 real columns each) per unit
     constexpr int NC = CX ? 2 : 1;     // doubles per element
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    unsigned char* lds = smem + wave * WAVE_LDS;
+    unsigned char* lds = smem + wave * (WAVE_LDS + (OUT_ROWS ? TILE_LDS : 0));
+    unsigned char* tile_lds = lds + WAVE_LDS;   // OUT_ROWS only
     const int g = lane >> 4, j = lane & 15, p = j & 1;
     const int kc = s.kc, npair = (kc + 3) >> 2, nmb = s.M > 16 ? 2 : 1;
 
@@ -104,25 +110,27 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
         loff[u] = ok ? row * PITCH + col * 16 : 0;
     }
     // ---- where this lane reads its operands and writes its results
-    int32_t roff[NBLK], ccol[NBLK], crow[2][4];
+    int32_t roff[NBLK], ccol[NBLK] = {}, crow[2][4] = {};
 #pragma unroll
     for (int nb = 0; nb < NBLK; ++nb) {
         const int nloc = CX ? 8 * nb + (j >> 1) : j;
         roff[nb] = nloc * PITCH + g * 16;
-        ccol[nb] = nloc * s.c_in * NC + (CX ? p : 0);
+        if constexpr (!OUT_ROWS) ccol[nb] = nloc * s.c_in * NC + (CX ? p : 0);
     }
+    if constexpr (!OUT_ROWS) {
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+        for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int m = Mfma<double>::row(lane, r) + 16 * mb;
-            crow[mb][r] = m < s.M ? (int32_t)(off_of(s.cm, m) * NC) : 0;
-        }
+            for (int r = 0; r < 4; ++r) {
+                const int m = Mfma<double>::row(lane, r) + 16 * mb;
+                crow[mb][r] = m < s.M ? (int32_t)(off_of(s.cm, m) * NC) : 0;
+            }
+    }
     const double ar = s.alpha_re, ai = s.alpha_im, br = s.beta_re, bi = s.beta_im;
     // C contiguous along m: 16-byte piece id = lane + 64 u of the unit's result tile -> (n of the unit, piece of its row)
-    int32_t ogoff[LOADS], oloff[LOADS];
+    int32_t ogoff[LOADS] = {}, oloff[LOADS] = {};
     uint32_t ohave = 0, orows = 0;
-    if (s.out_rows) {
+    if constexpr (OUT_ROWS) {
         const int cpr = s.M * NC / 2;   // 16-byte pieces per row of C
 #pragma unroll
         for (int u = 0; u < LOADS; ++u) {
@@ -153,6 +161,71 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
             if (((have >> u) & 1u) && (int)((lrows >> (4 * u)) & 15u) < valid)
                 stage[u] = __builtin_nontemporal_load(reinterpret_cast<const d2*>(Bu + goff[u]));
     };
+    // C contiguous along n: lane (g, j) holds rows g + 4r (+16), column j of each column block
+    auto store_direct = [&](const d4 (&res)[2][NBLK], double* Cu, int valid) {
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+            if (mb < nmb) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const bool row_ok = Mfma<double>::row(lane, r) + 16 * mb < s.M;
+#pragma unroll
+                    for (int nb = 0; nb < NBLK; ++nb) {
+                        const bool ok = row_ok && (CX ? 8 * nb + (j >> 1) : j) < valid;
+                        double* dst = Cu + crow[mb][r] + ccol[nb];
+                        double v = res[mb][nb][r];
+                        if (!s.plain) {
+                            if constexpr (CX) {
+                                // even lanes hold re, odd lanes im of one element: exchange with the neighbour
+                                const double other = __shfl_xor(v, 1);
+                                const double re_v = p ? other : v, im_v = p ? v : other;
+                                v = p ? (ar * im_v + ai * re_v) : (ar * re_v - ai * im_v);
+                                if (s.use_beta) {
+                                    const double old = ok ? *dst : 0.0;
+                                    const double old_other = __shfl_xor(old, 1);
+                                    const double re_o = p ? old_other : old, im_o = p ? old : old_other;
+                                    v += p ? (br * im_o + bi * re_o) : (br * re_o - bi * im_o);
+                                }
+                            } else {
+                                v *= ar;
+                                if (s.use_beta && ok) v += br * *dst;
+                            }
+                        }
+                        if (ok) __builtin_nontemporal_store(v, dst);
+                    }
+                }
+            }
+        }
+    };
+    // C contiguous along m: the tile of the unit before leaves as 16-byte pieces of whole rows
+    auto store_rows = [&](double* Cu, int valid) {
+#pragma unroll
+        for (int u = 0; u < LOADS; ++u)
+            if (((ohave >> u) & 1u) && (int)((orows >> (4 * u)) & 15u) < valid) {
+                d2 v = *reinterpret_cast<const d2*>(tile_lds + oloff[u]);
+                d2* dst = reinterpret_cast<d2*>(reinterpret_cast<unsigned char*>(Cu) + ogoff[u]);
+                if (!s.plain) {
+                    d2 o;
+                    if constexpr (CX) {
+                        o.x = ar * v.x - ai * v.y;
+                        o.y = ar * v.y + ai * v.x;
+                        if (s.use_beta) {
+                            const d2 old = *dst;
+                            o.x += br * old.x - bi * old.y;
+                            o.y += br * old.y + bi * old.x;
+                        }
+                    } else {
+                        o = v * ar;
+                        if (s.use_beta) o += *dst * br;
+                    }
+                    v = o;
+                }
+                __builtin_nontemporal_store(v, dst);
+            }
+    };
+    d4 held[2][NBLK];          // !OUT_ROWS: the results of the unit before, not yet stored (OUT_ROWS: they wait in the tile)
+    double* held_c = nullptr;
+    int held_valid = 0;
 #pragma unroll
     for (int u = 0; u < LOADS; ++u) stage[u] = d2{0, 0};
     if (unit < s.units) issue(unit);
@@ -162,6 +235,8 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
         for (int u = 0; u < LOADS; ++u)
             if ((have >> u) & 1u) *reinterpret_cast<d2*>(lds + loff[u]) = stage[u];
         const int64_t next = unit + nwaves;
+        // (a table lookup here finds nothing else in flight: behind the loads of the next unit it would wait for them)
+        double* Cu = reinterpret_cast<double*>(s.C) + off_of(s.cu, unit) * NC;
         if (next < s.units) issue(next);
         wave_sync();
 
@@ -196,14 +271,17 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
                     }
                 }
             }
+            if (i == 0 && held_c) {
+                if constexpr (OUT_ROWS) store_rows(held_c, held_valid);
+                else store_direct(held, held_c, held_valid);
+            }
         }
-        wave_sync();   // the next unit is parked over these rows
+        wave_sync();   // the next unit is parked over these rows, and its results are written over the tile
 
         // ---- results: lane (g, j) holds rows g + 4r (+16), column j of each column block
-        double* Cu = reinterpret_cast<double*>(s.C) + off_of(s.cu, unit) * NC;
-        if (s.out_rows) {
-            // tile[n of the unit][m][part] in LDS, then whole rows out: C[n][m] is contiguous along m
-            double* tile = reinterpret_cast<double*>(lds);
+        if constexpr (OUT_ROWS) {
+            // tile[n of the unit][m][part] in LDS; whole rows leave during the next unit's MFMAs (store_rows)
+            double* tile = reinterpret_cast<double*>(tile_lds);
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb)
                 if (mb < nmb) {
@@ -215,68 +293,26 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
                             tile[nloc * OUT_PITCH + m * NC + (CX ? p : 0)] = acc[mb][nb][r];
                         }
                 }
-            wave_sync();
-#pragma unroll
-            for (int u = 0; u < LOADS; ++u)
-                if (((ohave >> u) & 1u) && (int)((orows >> (4 * u)) & 15u) < valid) {
-                    d2 v = *reinterpret_cast<const d2*>(lds + oloff[u]);
-                    d2* dst = reinterpret_cast<d2*>(reinterpret_cast<unsigned char*>(Cu) + ogoff[u]);
-                    if (!s.plain) {
-                        d2 o;
-                        if constexpr (CX) {
-                            o.x = ar * v.x - ai * v.y;
-                            o.y = ar * v.y + ai * v.x;
-                            if (s.use_beta) {
-                                const d2 old = *dst;
-                                o.x += br * old.x - bi * old.y;
-                                o.y += br * old.y + bi * old.x;
-                            }
-                        } else {
-                            o = v * ar;
-                            if (s.use_beta) o += *dst * br;
-                        }
-                        v = o;
-                    }
-                    __builtin_nontemporal_store(v, dst);
-                }
-            wave_sync();   // the next unit is parked over the tile
-            unit = next;
-            continue;
+            held_c = Cu;
+            held_valid = valid;
         }
+        if constexpr (!OUT_ROWS) {
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-            if (mb < nmb) {
+            for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const bool row_ok = Mfma<double>::row(lane, r) + 16 * mb < s.M;
-#pragma unroll
-                    for (int nb = 0; nb < NBLK; ++nb) {
-                        const bool ok = row_ok && (CX ? 8 * nb + (j >> 1) : j) < valid;
-                        double* dst = Cu + crow[mb][r] + ccol[nb];
-                        double v = acc[mb][nb][r];
-                        if (!s.plain) {
-                            if constexpr (CX) {
-                                // even lanes hold re, odd lanes im of one element: exchange with the neighbour
-                                const double other = __shfl_xor(v, 1);
-                                const double re_v = p ? other : v, im_v = p ? v : other;
-                                v = p ? (ar * im_v + ai * re_v) : (ar * re_v - ai * im_v);
-                                if (s.use_beta) {
-                                    const double old = ok ? *dst : 0.0;
-                                    const double old_other = __shfl_xor(old, 1);
-                                    const double re_o = p ? old_other : old, im_o = p ? old : old_other;
-                                    v += p ? (br * im_o + bi * re_o) : (br * re_o - bi * im_o);
-                                }
-                            } else {
-                                v *= ar;
-                                if (s.use_beta && ok) v += br * *dst;
-                            }
-                        }
-                        if (ok) __builtin_nontemporal_store(v, dst);
-                    }
-                }
-            }
+                for (int nb = 0; nb < NBLK; ++nb) held[mb][nb] = acc[mb][nb];
+            held_c = Cu;
+            held_valid = valid;
         }
         unit = next;
+    }
+    if (held_c) {
+        if constexpr (OUT_ROWS) {
+            wave_sync();
+            store_rows(held_c, held_valid);
+        } else {
+            store_direct(held, held_c, held_valid);
+        }
     }
 }
 
@@ -285,14 +321,30 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
 void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
     const int64_t blocks_wanted = (s.units + THREADS / 64 - 1) / (THREADS / 64);
     const dim3 grid((uint32_t)std::min<int64_t>(blocks_wanted, 512)), block(THREADS);
-    const size_t lds = (size_t)(THREADS / 64) * WAVE_LDS;
-    if (s.tail != 0) {
-        if (dtype == TFH_C128) TFH_LAUNCH_TIMED((gemm_skinny_kernel<true, true>), grid, block, lds, st, s);
-        else TFH_LAUNCH_TIMED((gemm_skinny_kernel<false, true>), grid, block, lds, st, s);
-    } else {
-        if (dtype == TFH_C128) TFH_LAUNCH_TIMED((gemm_skinny_kernel<true, false>), grid, block, lds, st, s);
-        else TFH_LAUNCH_TIMED((gemm_skinny_kernel<false, false>), grid, block, lds, st, s);
+    const bool cx = dtype == TFH_C128, ragged = s.tail != 0, rows = s.out_rows != 0;
+    const size_t lds = (size_t)(THREADS / 64) * (WAVE_LDS + (rows ? TILE_LDS : 0));
+    // (more than 64 KB of dynamic LDS has to be asked for once per kernel)
+#define TFH_SKINNY_CASE(CXV, RAGV, ROWV)                                                                  \
+    if (cx == CXV && ragged == RAGV && rows == ROWV) {                                                     \
+        static bool once = [] {                                                                            \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<CXV, RAGV, ROWV>), \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize,                          \
+                                      (THREADS / 64) * (WAVE_LDS + (ROWV ? TILE_LDS : 0)));                \
+            return true;                                                                                   \
+        }();                                                                                               \
+        (void)once;                                                                                        \
+        TFH_LAUNCH_TIMED((gemm_skinny_kernel<CXV, RAGV, ROWV>), grid, block, lds, st, s);                  \
+        return;                                                                                            \
     }
+    TFH_SKINNY_CASE(true, false, false)
+    TFH_SKINNY_CASE(true, false, true)
+    TFH_SKINNY_CASE(true, true, false)
+    TFH_SKINNY_CASE(true, true, true)
+    TFH_SKINNY_CASE(false, false, false)
+    TFH_SKINNY_CASE(false, false, true)
+    TFH_SKINNY_CASE(false, true, false)
+    TFH_SKINNY_CASE(false, true, true)
+#undef TFH_SKINNY_CASE
 }
 
 }  // namespace tfh

@@ -1904,6 +1904,65 @@ def test_contract_small_operator_with_the_result_contiguous_along_its_columns(tf
     assert np.array_equal(got[:, :, m:], wide[:, :, m:])          # the padding is untouched
 
 
+@pytest.mark.parametrize("dtype", [np.complex128, np.float64])
+@pytest.mark.parametrize("out_modes", ["xmc", "xcm"])
+@pytest.mark.parametrize("m,k,c", [(32, 32, 24000), (20, 12, 24008), (12, 10, 30001)])
+def test_contract_small_operator_every_wave_streams_several_units(tf, oracle, dtype, out_modes, m, k, c):
+    # The streaming kernel launches at most 2048 waves; with more units than that (3 x 1500 and more here) a wave works
+    # through several, loads the next unit while it multiplies and stores a unit's results during the MFMAs of the
+    # following one (the last unit's after the loop).  Both output orientations, whole and partly filled last units,
+    # general alpha / beta.
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    if not cplx:
+        k *= 2
+    rng = np.random.default_rng(95)
+    x = 3
+    t = rand(rng, (x, c, k), dtype)
+    w = rand(rng, (k, m), dtype)
+    out0 = rand(rng, (x, m, c) if out_modes == "xmc" else (x, c, m), dtype)
+    for alpha, beta in [(1.0, 0.0), ((0.5 - 2j, 1.5 + 1j) if cplx else (0.5, -1.5))]:
+        ref = out0.copy()
+        oracle.contract(t, lab("xck"), w, lab("km"), ref, lab(out_modes), alpha=alpha, beta=beta)
+        dout = dev(tf, out0)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab(out_modes)), [t.shape, w.shape, ref.shape])
+        tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
+        assert "gemm_skinny_kernel" in tf.last_kernel(), tf.last_kernel()
+        assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
+
+
+@pytest.mark.parametrize("dtype", [np.complex128, np.float64])
+@pytest.mark.parametrize("out_modes", ["xmc", "xcm"])
+@pytest.mark.parametrize("m,k,c", [(8, 8, 4096), (4, 4, 4096), (2, 2, 4096), (8, 4, 4096), (3, 6, 4096), (8, 8, 17)])
+def test_contract_tiny_operator_on_the_last_leg_of_a_long_tensor(tf, oracle, dtype, out_modes, m, k, c):
+    # a gate on the last leg: T[x, c, k] . W[k, m], at most 8 x 8, the rows of T contiguous runs of k.  Two kernels can
+    # take it: the tiny-operator kernel (lanes a whole row apart) and the streaming kernel (whole rows per lane group);
+    # which one is faster depends on the extents and on the output's orientation, and a product the streaming kernel
+    # is preferred for but cannot take (runs of 17 columns) still goes to the tiny-operator kernel.
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    rows = out_modes == "xcm"
+    rng = np.random.default_rng(96)
+    x = 32 if c > 100 else 4096
+    t = rand(rng, (x, c, k), dtype)
+    w = rand(rng, (k, m), dtype)
+    out0 = rand(rng, (x, c, m) if rows else (x, m, c), dtype)
+    if cplx:
+        prefer = (m >= 3 or k >= 6) if rows else (k >= 6 or (k >= 4 and m >= 8))
+        can = True
+    else:
+        prefer = ((m >= 4 or k >= 8) if rows else k >= 8) and k >= 4
+        can = k % 2 == 0 and (m % 2 == 0 or not rows)
+    can = can and (rows or c >= 48)
+    for alpha, beta in [(1.0, 0.0), ((0.5 - 2j, 1.5 + 1j) if cplx else (0.5, -1.5))]:
+        ref = out0.copy()
+        oracle.contract(t, lab("xck"), w, lab("km"), ref, lab(out_modes), alpha=alpha, beta=beta)
+        dout = dev(tf, out0)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab(out_modes)), [t.shape, w.shape, ref.shape])
+        tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
+        want = "gemm_skinny_kernel" if prefer and can else "tiny_operator_kernel"
+        assert want in tf.last_kernel(), (tf.last_kernel(), want)
+        assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
+
+
 @pytest.mark.parametrize("dtype", ALL)
 def test_reduce_rows_and_inner_axes_take_the_butterfly_fold(tf, oracle, dtype):
     # sums over the contiguous axis (row sums) and over an inner axis next to a short kept one: nothing is left to loop
