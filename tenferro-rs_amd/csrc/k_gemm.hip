@@ -562,9 +562,10 @@ bool skinny_run_ok(int64_t n) { return n % SKINNY_UNIT == 0 || n >= 3 * SKINNY_U
 // A tiny operator (both of its extents at most 8) applied to the last leg of a long tensor -- the long operand's rows
 // are contiguous runs of k: the tiny-operator kernel (one thread per element of the long free index) then reads and
 // writes with a stride of one row between neighbouring lanes, while the streaming kernel of k_gemm_skinny.hip takes
-// whole rows.  Measured on 4M rows (us, tiny | streaming): complex128 8x8 566 | 208 with C contiguous along n and
-// 1959 | 203 along m, 8x4 185 | 172 and 1537 | 168, 4x4 130 | 166 and 412 | 159, 2x2 47 | 164 and 80 | 155; f64 8x8
-// 195 | 134 and 812 | 132, 4x4 65 | 117 and 167 | 119.  ms: the operator's free extent.
+// whole rows.  Measured on 4M rows (us, tiny | streaming): complex128 8x8 566 | 196 with C contiguous along n and
+// 1959 | 189 along m, 4x4 130 | 98 and 412 | 98, 2x4 102 | 82 and 128 | 83, 4x2 73 | 90, 3x3 81 | 85, 2x2 47 | 81 and
+// 80 | 81; f64 8x8 195 | 95 and 812 | 92, 4x6 106 | 69, 6x6 120 | 78, 4x4 64 | 69 and 167 | 72, 2x4 50 | 61 and 56 | 64.
+// ms: the operator's free extent.
 bool last_leg_prefers_streaming(int dtype, const ContractAxes& ax, int64_t M, int64_t N, int64_t K) {
     if (dtype != TFH_F64 && dtype != TFH_C128) return false;
     const bool small_is_a = M <= N;
@@ -581,8 +582,8 @@ bool last_leg_prefers_streaming(int dtype, const ContractAxes& ax, int64_t M, in
         expect *= k[d].n;
     }
     const bool rows = min_stride(small, 2) == 1;   // C contiguous along the operator's free index
-    if (dtype == TFH_C128) return rows ? (ms >= 3 || K >= 6) : (K >= 6 || (K >= 4 && ms >= 8));
-    return rows ? (ms >= 4 || K >= 8) : K >= 8;
+    if (dtype == TFH_C128) return rows ? (ms >= 3 || K >= 4) : K >= 4;
+    return rows ? (ms >= 4 || K >= 6) : K >= 6;
 }
 
 int bke_of(int dtype) {

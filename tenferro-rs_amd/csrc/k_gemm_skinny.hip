@@ -35,13 +35,22 @@ using namespace gemm;
 
 typedef double d2 __attribute__((ext_vector_type(2)));
 
-constexpr int MAX_KC = SKINNY_MAX_KR / 2;          // 16-byte chunks per row of B at most
-constexpr int PITCH = MAX_KC * 16 + 64;            // bytes per LDS row: rows 0..3 start 16 banks apart
-constexpr int WAVE_LDS = SKINNY_UNIT * PITCH;      // each wave parks one unit
-constexpr int LOADS = SKINNY_UNIT * MAX_KC / 64;   // 16-byte loads per lane and unit at most
-constexpr int PAIRS = MAX_KC / 4;
-constexpr int OUT_PITCH = 2 * SKINNY_MAX_M + 2;   // doubles per row of the transposed result tile (complex: 32 x 2, +2 against bank conflicts)
-constexpr int TILE_LDS = SKINNY_UNIT * OUT_PITCH * 8;   // the transposed result tile of a wave: a region of its own
+// Sizes of one instantiation: KCM 16-byte chunks per row of B at most, MBM blocks of 16 rows of A at most.  The general
+// kernel (32 chunks, 2 blocks) keeps 64 VGPRs of A and 32 of staging and runs two waves per SIMD; an operator of at most
+// 16 rows and 8 chunks needs a tenth of that, and twice as many waves hide twice the latency of its short units.
+template <int KCM, int MBM>
+struct SkinnyCfg {
+    static constexpr int MAX_KC = KCM;
+    static constexpr int PITCH = MAX_KC * 16 + 64;            // bytes per LDS row: rows 0..3 start 16 banks apart
+    static constexpr int WAVE_LDS = SKINNY_UNIT * PITCH;      // each wave parks one unit
+    static constexpr int LOADS = SKINNY_UNIT * MAX_KC / 64;   // 16-byte loads per lane and unit at most
+    static constexpr int PAIRS = MAX_KC / 4;
+    static constexpr int OLOADS = SKINNY_UNIT * 16 * MBM / 64;   // 16-byte pieces of the result tile per lane at most (complex)
+    static constexpr int OUT_PITCH = 2 * 16 * MBM + 2;        // doubles per row of the transposed result tile (+2 against bank conflicts)
+    static constexpr int TILE_LDS = SKINNY_UNIT * OUT_PITCH * 8;   // the transposed result tile of a wave: a region of its own
+    static constexpr int BLOCKS_PER_CU = KCM <= 8 && MBM == 1 ? 4 : 2;
+    static_assert(KCM % 4 == 0 && KCM * 2 <= SKINNY_MAX_KR && MBM * 16 <= SKINNY_MAX_M, "");
+};
 
 // Orders the LDS accesses of one wave: lanes read what other lanes of the same wave wrote.  The LDS executes a wave's
 // instructions in order, so only the compiler has to be kept from moving accesses across this point.
@@ -58,8 +67,11 @@ __device__ __forceinline__ void wave_sync() {
 // iteration before with vmcnt(0): whatever is stored shortly before that wait is waited for as well, acknowledgement
 // included.  With C contiguous along n a unit's results therefore stay in registers for one more iteration and leave
 // in the middle of the next unit's MFMAs: by the time the next wait comes, they have had half an iteration to drain.
-template <bool CX, bool RAGGED, bool OUT_ROWS>
-__global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
+template <bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM>
+__global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU)) gemm_skinny_kernel(SkinnyArgs s) {
+    typedef SkinnyCfg<KCM, MBM> Cfg;
+    constexpr int PITCH = Cfg::PITCH, WAVE_LDS = Cfg::WAVE_LDS, LOADS = Cfg::LOADS, PAIRS = Cfg::PAIRS;
+    constexpr int OUT_PITCH = Cfg::OUT_PITCH, TILE_LDS = Cfg::TILE_LDS, OLOADS = Cfg::OLOADS;
     constexpr int NBLK = CX ? 2 : 1;   // column blocks (16 real columns each) per unit
     constexpr int NC = CX ? 2 : 1;     // doubles per element
     extern __shared__ __align__(16) unsigned char smem[];
@@ -67,14 +79,14 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
     unsigned char* lds = smem + wave * (WAVE_LDS + (OUT_ROWS ? TILE_LDS : 0));
     unsigned char* tile_lds = lds + WAVE_LDS;   // OUT_ROWS only
     const int g = lane >> 4, j = lane & 15, p = j & 1;
-    const int kc = s.kc, npair = (kc + 3) >> 2, nmb = s.M > 16 ? 2 : 1;
+    const int kc = s.kc, npair = (kc + 3) >> 2, nmb = MBM > 1 && s.M > 16 ? 2 : 1;
 
     // ---- A as MFMA operands: a[mb][i][q] = A'[j + 16 mb][2 (4i + g) + q], zero outside the matrix
-    double a[2][PAIRS][2];
+    double a[MBM][PAIRS][2];
     {
         const double* Ad = reinterpret_cast<const double*>(s.A);
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
+        for (int mb = 0; mb < MBM; ++mb)
 #pragma unroll
             for (int i = 0; i < PAIRS; ++i) {
                 const int m = j + 16 * mb, c = 4 * i + g;
@@ -99,7 +111,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
     // ---- this lane's share of a unit of B: chunk id = lane + 64 u -> (row, chunk of the row)
     int32_t goff[LOADS], loff[LOADS];
     uint32_t have = 0, lrows = 0;   // lrows: four bits per load, the row (n of the unit) it belongs to
-    static_assert(LOADS <= 8 && SKINNY_UNIT <= 16, "row numbers are packed four bits per load");
+    static_assert(LOADS <= 8 && OLOADS <= 8 && SKINNY_UNIT <= 16, "row numbers are packed four bits per load or store");
 #pragma unroll
     for (int u = 0; u < LOADS; ++u) {
         const int id = lane + 64 * u, row = id / kc, col = id - row * kc;
@@ -110,7 +122,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
         loff[u] = ok ? row * PITCH + col * 16 : 0;
     }
     // ---- where this lane reads its operands and writes its results
-    int32_t roff[NBLK], ccol[NBLK] = {}, crow[2][4] = {};
+    int32_t roff[NBLK], ccol[NBLK] = {}, crow[MBM][4] = {};
 #pragma unroll
     for (int nb = 0; nb < NBLK; ++nb) {
         const int nloc = CX ? 8 * nb + (j >> 1) : j;
@@ -119,7 +131,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
     }
     if constexpr (!OUT_ROWS) {
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
+        for (int mb = 0; mb < MBM; ++mb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = Mfma<double>::row(lane, r) + 16 * mb;
@@ -128,12 +140,12 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
     }
     const double ar = s.alpha_re, ai = s.alpha_im, br = s.beta_re, bi = s.beta_im;
     // C contiguous along m: 16-byte piece id = lane + 64 u of the unit's result tile -> (n of the unit, piece of its row)
-    int32_t ogoff[LOADS] = {}, oloff[LOADS] = {};
+    int32_t ogoff[OLOADS] = {}, oloff[OLOADS] = {};
     uint32_t ohave = 0, orows = 0;
     if constexpr (OUT_ROWS) {
         const int cpr = s.M * NC / 2;   // 16-byte pieces per row of C
 #pragma unroll
-        for (int u = 0; u < LOADS; ++u) {
+        for (int u = 0; u < OLOADS; ++u) {
             const int id = lane + 64 * u, row = id / cpr, col = id - row * cpr;
             const bool ok = id < SKINNY_UNIT * cpr;
             ohave |= (ok ? 1u : 0u) << u;
@@ -162,9 +174,9 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
                 stage[u] = __builtin_nontemporal_load(reinterpret_cast<const d2*>(Bu + goff[u]));
     };
     // C contiguous along n: lane (g, j) holds rows g + 4r (+16), column j of each column block
-    auto store_direct = [&](const d4 (&res)[2][NBLK], double* Cu, int valid) {
+    auto store_direct = [&](const d4 (&res)[MBM][NBLK], double* Cu, int valid) {
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
+        for (int mb = 0; mb < MBM; ++mb) {
             if (mb < nmb) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -200,7 +212,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
     // C contiguous along m: the tile of the unit before leaves as 16-byte pieces of whole rows
     auto store_rows = [&](double* Cu, int valid) {
 #pragma unroll
-        for (int u = 0; u < LOADS; ++u)
+        for (int u = 0; u < OLOADS; ++u)
             if (((ohave >> u) & 1u) && (int)((orows >> (4 * u)) & 15u) < valid) {
                 d2 v = *reinterpret_cast<const d2*>(tile_lds + oloff[u]);
                 d2* dst = reinterpret_cast<d2*>(reinterpret_cast<unsigned char*>(Cu) + ogoff[u]);
@@ -223,7 +235,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
                 __builtin_nontemporal_store(v, dst);
             }
     };
-    d4 held[2][NBLK];          // !OUT_ROWS: the results of the unit before, not yet stored (OUT_ROWS: they wait in the tile)
+    d4 held[MBM][NBLK];          // !OUT_ROWS: the results of the unit before, not yet stored (OUT_ROWS: they wait in the tile)
     double* held_c = nullptr;
     int held_valid = 0;
 #pragma unroll
@@ -240,9 +252,9 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
         if (next < s.units) issue(next);
         wave_sync();
 
-        d4 acc[2][NBLK];
+        d4 acc[MBM][NBLK];
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
+        for (int mb = 0; mb < MBM; ++mb)
 #pragma unroll
             for (int nb = 0; nb < NBLK; ++nb) acc[mb][nb] = d4{0, 0, 0, 0};
 #pragma unroll
@@ -265,10 +277,11 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
                     b1 = kok ? b1 : 0.0;
                     acc[0][nb] = Mfma<double>::run(a[0][i][0], b0, acc[0][nb]);
                     acc[0][nb] = Mfma<double>::run(a[0][i][1], b1, acc[0][nb]);
-                    if (nmb > 1) {
-                        acc[1][nb] = Mfma<double>::run(a[1][i][0], b0, acc[1][nb]);
-                        acc[1][nb] = Mfma<double>::run(a[1][i][1], b1, acc[1][nb]);
-                    }
+                    if constexpr (MBM > 1)
+                        if (nmb > 1) {
+                            acc[1][nb] = Mfma<double>::run(a[1][i][0], b0, acc[1][nb]);
+                            acc[1][nb] = Mfma<double>::run(a[1][i][1], b1, acc[1][nb]);
+                        }
                 }
             }
             if (i == 0 && held_c) {
@@ -283,7 +296,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
             // tile[n of the unit][m][part] in LDS; whole rows leave during the next unit's MFMAs (store_rows)
             double* tile = reinterpret_cast<double*>(tile_lds);
 #pragma unroll
-            for (int mb = 0; mb < 2; ++mb)
+            for (int mb = 0; mb < MBM; ++mb)
                 if (mb < nmb) {
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
@@ -298,7 +311,7 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
         }
         if constexpr (!OUT_ROWS) {
 #pragma unroll
-            for (int mb = 0; mb < 2; ++mb)
+            for (int mb = 0; mb < MBM; ++mb)
 #pragma unroll
                 for (int nb = 0; nb < NBLK; ++nb) held[mb][nb] = acc[mb][nb];
             held_c = Cu;
@@ -318,23 +331,36 @@ __global__ void __launch_bounds__(THREADS, 2) gemm_skinny_kernel(SkinnyArgs s) {
 
 }  // namespace
 
-void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
+namespace {
+template <bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM>
+void launch_variant(const gemm::SkinnyArgs& s, hipStream_t st) {
+    typedef SkinnyCfg<KCM, MBM> Cfg;
+    constexpr int lds = (THREADS / 64) * (Cfg::WAVE_LDS + (OUT_ROWS ? Cfg::TILE_LDS : 0));
+    static bool once = [] {   // (more than 64 KB of dynamic LDS has to be asked for once per kernel)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<CX, RAGGED, OUT_ROWS, KCM, MBM>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        return true;
+    }();
+    (void)once;
     const int64_t blocks_wanted = (s.units + THREADS / 64 - 1) / (THREADS / 64);
-    const dim3 grid((uint32_t)std::min<int64_t>(blocks_wanted, 512)), block(THREADS);
+    const dim3 grid((uint32_t)std::min<int64_t>(blocks_wanted, 256 * Cfg::BLOCKS_PER_CU)), block(THREADS);
+    TFH_LAUNCH_TIMED((gemm_skinny_kernel<CX, RAGGED, OUT_ROWS, KCM, MBM>), grid, block, (size_t)lds, st, s);
+}
+
+template <bool CX, bool RAGGED, bool OUT_ROWS>
+void launch_sized(const gemm::SkinnyArgs& s, hipStream_t st) {
+    // (twice the waves pay where a unit is short: measured faster up to 8 complex or 16 real rows, even beyond)
+    if (s.kc <= 8 && s.M <= (CX ? 8 : 16)) launch_variant<CX, RAGGED, OUT_ROWS, 8, 1>(s, st);
+    else launch_variant<CX, RAGGED, OUT_ROWS, SKINNY_MAX_KR / 2, SKINNY_MAX_M / 16>(s, st);
+}
+}  // namespace
+
+void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
     const bool cx = dtype == TFH_C128, ragged = s.tail != 0, rows = s.out_rows != 0;
-    const size_t lds = (size_t)(THREADS / 64) * (WAVE_LDS + (rows ? TILE_LDS : 0));
-    // (more than 64 KB of dynamic LDS has to be asked for once per kernel)
-#define TFH_SKINNY_CASE(CXV, RAGV, ROWV)                                                                  \
-    if (cx == CXV && ragged == RAGV && rows == ROWV) {                                                     \
-        static bool once = [] {                                                                            \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<CXV, RAGV, ROWV>), \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize,                          \
-                                      (THREADS / 64) * (WAVE_LDS + (ROWV ? TILE_LDS : 0)));                \
-            return true;                                                                                   \
-        }();                                                                                               \
-        (void)once;                                                                                        \
-        TFH_LAUNCH_TIMED((gemm_skinny_kernel<CXV, RAGV, ROWV>), grid, block, lds, st, s);                  \
-        return;                                                                                            \
+#define TFH_SKINNY_CASE(CXV, RAGV, ROWV)               \
+    if (cx == CXV && ragged == RAGV && rows == ROWV) { \
+        launch_sized<CXV, RAGV, ROWV>(s, st);          \
+        return;                                        \
     }
     TFH_SKINNY_CASE(true, false, false)
     TFH_SKINNY_CASE(true, false, true)

@@ -1906,7 +1906,7 @@ def test_contract_small_operator_with_the_result_contiguous_along_its_columns(tf
 
 @pytest.mark.parametrize("dtype", [np.complex128, np.float64])
 @pytest.mark.parametrize("out_modes", ["xmc", "xcm"])
-@pytest.mark.parametrize("m,k,c", [(32, 32, 24000), (20, 12, 24008), (12, 10, 30001)])
+@pytest.mark.parametrize("m,k,c", [(32, 32, 24000), (20, 12, 24008), (12, 10, 30001), (8, 6, 30001), (4, 8, 160000)])
 def test_contract_small_operator_every_wave_streams_several_units(tf, oracle, dtype, out_modes, m, k, c):
     # The streaming kernel launches at most 2048 waves; with more units than that (3 x 1500 and more here) a wave works
     # through several, loads the next unit while it multiplies and stores a unit's results during the MFMAs of the
@@ -1932,7 +1932,7 @@ def test_contract_small_operator_every_wave_streams_several_units(tf, oracle, dt
 
 @pytest.mark.parametrize("dtype", [np.complex128, np.float64])
 @pytest.mark.parametrize("out_modes", ["xmc", "xcm"])
-@pytest.mark.parametrize("m,k,c", [(8, 8, 4096), (4, 4, 4096), (2, 2, 4096), (8, 4, 4096), (3, 6, 4096), (8, 8, 17)])
+@pytest.mark.parametrize("m,k,c", [(8, 8, 4096), (4, 4, 4096), (2, 2, 4096), (8, 4, 4096), (3, 6, 4096), (4, 2, 4096), (8, 8, 17)])
 def test_contract_tiny_operator_on_the_last_leg_of_a_long_tensor(tf, oracle, dtype, out_modes, m, k, c):
     # a gate on the last leg: T[x, c, k] . W[k, m], at most 8 x 8, the rows of T contiguous runs of k.  Two kernels can
     # take it: the tiny-operator kernel (lanes a whole row apart) and the streaming kernel (whole rows per lane group);
@@ -1946,10 +1946,10 @@ def test_contract_tiny_operator_on_the_last_leg_of_a_long_tensor(tf, oracle, dty
     w = rand(rng, (k, m), dtype)
     out0 = rand(rng, (x, c, m) if rows else (x, m, c), dtype)
     if cplx:
-        prefer = (m >= 3 or k >= 6) if rows else (k >= 6 or (k >= 4 and m >= 8))
+        prefer = (m >= 3 or k >= 4) if rows else k >= 4
         can = True
     else:
-        prefer = ((m >= 4 or k >= 8) if rows else k >= 8) and k >= 4
+        prefer = ((m >= 4 or k >= 6) if rows else k >= 6) and k >= 4
         can = k % 2 == 0 and (m % 2 == 0 or not rows)
     can = can and (rows or c >= 48)
     for alpha, beta in [(1.0, 0.0), ((0.5 - 2j, 1.5 + 1j) if cplx else (0.5, -1.5))]:
