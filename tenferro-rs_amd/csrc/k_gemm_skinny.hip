@@ -7,8 +7,8 @@
 // Here A lives in registers, already laid out as MFMA operands, for the whole kernel, and every wave streams B on
 // its own: a work unit is 16 consecutive n; the wave loads the unit's rows of B (k contiguous) with 16-byte
 // accesses into registers, parks them in its private LDS region, has the next unit's loads in flight while the
-// MFMAs of the current one run, and writes the unit's columns of C from the accumulators.  Waves never wait for
-// each other (no block barrier).
+// MFMAs of the current one run, and writes the unit's columns of C from the accumulators one unit later, among the
+// MFMAs of the next unit.  Waves never wait for each other (no block barrier).
 //
 // v_mfma_f64_16x16x4_f64: lane l = 16 g + j feeds A'[row j][k' = 4 step + g] and B'[k' = 4 step + g][col j] and
 // receives C'[row g + 4 r][col j] in accumulator register r.  One 16-byte chunk of B serves two steps:
@@ -21,8 +21,8 @@
 // under the sum.  HBM-bound: algorithmic bytes = sizeof(B) + sizeof(C) (+ C again when beta != 0).
 //
 // C may be contiguous along n (each lane stores its accumulators: 128-byte segments per row of C) or along m (the
-// other orientation of the same product, C[n][m]): then the unit's 16 x M results are transposed through the wave's
-// LDS region and leave as 16-byte stores along m.
+// other orientation of the same product, C[n][m]): then the unit's 16 x M results are transposed through an LDS tile
+// of the wave's own and leave as 16-byte stores along m.
 #include <hip/hip_runtime.h>
 
 #include "gemm_skinny.hpp"
