@@ -11,14 +11,14 @@ namespace gemm {
 
 constexpr int SKINNY_UNIT = 16;        // consecutive n (rows of B, columns of C) per work unit
 constexpr int SKINNY_MAX_M = 32;       // rows of A
-constexpr int SKINNY_MAX_KR = 64;      // real k per row of B (64 doubles = 32 chunks of 16 bytes)
+constexpr int SKINNY_MAX_CHUNKS = 32;  // 16-byte chunks per row of B: 64 doubles or 128 floats (half as many complex elements)
 
 struct SkinnyArgs {
     const void* A;
     const void* B;
     void* C;
     int32_t M, K;            // rows of A, elements of k
-    int32_t kc;              // 16-byte chunks per row of B: K for complex128, K/2 for f64
+    int32_t kc;              // 16-byte chunks per row of B: K for complex128, K/2 for f64 and complex64, K/4 for f32
     int32_t conj_a, conj_b, use_beta, plain;   // plain: alpha == 1 and beta == 0
     int32_t out_rows;        // C is contiguous along m (the rows of A), not along n: a unit's results are transposed in LDS
     int64_t units;           // work units: (outer extents of n) x upr
@@ -31,6 +31,5 @@ struct SkinnyArgs {
 
 }  // namespace gemm
 
-// dtype is TFH_F64 or TFH_C128
 void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st);
 }  // namespace tfh

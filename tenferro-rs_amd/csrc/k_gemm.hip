@@ -731,7 +731,8 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     {
         const int ec = is_complex(dtype) ? 2 : 1;
         // (a small operator against a long tensor keeps its orientation: the streaming kernel looks at it below)
-        bool streamable = (dtype == TFH_F64 || dtype == TFH_C128) && M <= SKINNY_MAX_M && K * ec <= SKINNY_MAX_KR && N >= 4096;
+        const int64_t per_chunk = 16 / ((int64_t)eb / ec);   // components per 16-byte chunk
+        bool streamable = M <= SKINNY_MAX_M && K * ec <= SKINNY_MAX_CHUNKS * per_chunk && N >= 4096;
         if (streamable) {
             // (that kernel works on units of SKINNY_UNIT consecutive n: a long side whose innermost runs are too short
             // for them would end on the 64x64 tiles below, at half the rate of the thin tiles)
@@ -812,13 +813,16 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     // A small left operand against a long n whose rows of B are contiguous in k: the streaming kernel of
     // k_gemm_skinny.hip (work units of SKINNY_UNIT consecutive n; the n tables then hold one entry per unit).
     const bool cxd = dtype == TFH_C128;
+    const int sk_nc = is_complex(dtype) ? 2 : 1;                  // components per element
+    const int64_t sk_q = 16 / ((int64_t)eb / sk_nc);               // components per 16-byte chunk: 2 doubles, 4 floats
+    auto whole_chunks = [&](int64_t elems) { return elems * sk_nc % sk_q == 0; };
     // The same product seen from the other side -- the long operand is A and C is contiguous along the few columns
     // of B (C[m][n], n = 0..N-1 adjacent): exchange the operands; the kernel then writes C through a transposing
     // LDS tile ("out_rows").
     bool out_rows = false;
-    if ((dtype == TFH_F64 || cxd) && nb == 1 && N <= SKINNY_MAX_M && M >= 4096 && K * (cxd ? 2 : 1) <= SKINNY_MAX_KR && a_kfast &&
+    if (nb == 1 && N <= SKINNY_MAX_M && M >= 4096 && K * sk_nc <= SKINNY_MAX_CHUNKS * sk_q && a_kfast &&
         !k_by_b && !ax.K.empty() && ax.N.size() == 1 && ax.N[0].s[2] == 1 && !ax.M.empty() && skinny_run_ok(ax.M.back().n) &&
-        (cxd || (N % 2 == 0 && K % 2 == 0 && (uintptr_t)c % 16 == 0 && (uintptr_t)a % 16 == 0))) {
+        (cxd || (whole_chunks(N) && whole_chunks(K) && (uintptr_t)c % 16 == 0 && (uintptr_t)a % 16 == 0))) {
         bool ok = true;
         int64_t expect = 1;
         for (int d = (int)ax.K.size() - 1; d >= 0; --d) {   // a row of A is one contiguous run of k
@@ -826,7 +830,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
             expect *= ax.K[d].n;
         }
         if (!cxd)
-            for (auto& x : ax.M) ok = ok && x.s[2] % 2 == 0 && x.s[0] % 2 == 0;
+            for (auto& x : ax.M) ok = ok && whole_chunks(x.s[2]) && whole_chunks(x.s[0]);
         const Axis& in = ax.M.back();
         ok = ok && std::llabs(in.s[0]) * SKINNY_UNIT * (int64_t)eb < ((int64_t)1 << 31) &&
              std::llabs(in.s[2]) * SKINNY_UNIT * (int64_t)eb < ((int64_t)1 << 31);
@@ -842,7 +846,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         }
     }
     const bool k_rows_b = out_rows || k_by_b;   // the k modes are in the memory order of the (possibly exchanged) B
-    bool skinny = (dtype == TFH_F64 || cxd) && nb == 1 && M <= SKINNY_MAX_M && K * (cxd ? 2 : 1) <= SKINNY_MAX_KR && N >= 4096 &&
+    bool skinny = nb == 1 && M <= SKINNY_MAX_M && K * sk_nc <= SKINNY_MAX_CHUNKS * sk_q && N >= 4096 &&
                   b_kfast && !ax.K.empty() && k_rows_b && !ax.N.empty() &&
                   skinny_run_ok(ax.N.back().n) && (out_rows || ax.N.back().s[2] == 1);
     if (skinny) {   // a row of B is one contiguous run of k (A's k order is free: it goes through the k table)
@@ -852,16 +856,16 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
             expect *= ax.K[d].n;
         }
     }
-    if (skinny && !cxd) {   // 16-byte chunks of two f64: rows of B must start on 16-byte boundaries and hold whole chunks
-        skinny = K % 2 == 0 && (uintptr_t)b % 16 == 0;
-        for (auto& x : ax.N) skinny = skinny && x.s[1] % 2 == 0;
+    if (skinny && !cxd) {   // 16-byte chunks of several elements: rows of B must start on 16-byte boundaries and hold whole chunks
+        skinny = whole_chunks(K) && (uintptr_t)b % 16 == 0;
+        for (auto& x : ax.N) skinny = skinny && whole_chunks(x.s[1]);
     }
     int64_t inner_b = 0, inner_c = 0, skinny_upr = 1;
     int skinny_tail = 0;
     if (skinny) {
         int64_t lo = 0, hi = 0;
         reach(ax.M, 2, lo, hi);
-        if (std::max(-lo, hi) * (cxd ? 2 : 1) >= ((int64_t)1 << 31)) skinny = false;
+        if (std::max(-lo, hi) * sk_nc >= ((int64_t)1 << 31)) skinny = false;
         if (std::llabs(ax.N.back().s[1]) * SKINNY_UNIT * (int64_t)eb >= ((int64_t)1 << 31)) skinny = false;
     }
     if (skinny) {
@@ -1143,7 +1147,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         std::memset(&sk, 0, sizeof sk);
         sk.A = a; sk.B = b; sk.C = c;
         sk.M = (int32_t)M; sk.K = (int32_t)K;
-        sk.kc = (int32_t)(cxd ? K : K / 2);
+        sk.kc = (int32_t)(K * sk_nc / sk_q);
         sk.use_beta = g.use_beta;
         sk.conj_a = conj_a; sk.conj_b = conj_b;
         sk.out_rows = out_rows;

@@ -33,23 +33,28 @@ namespace {
 
 using namespace gemm;
 
-typedef double d2 __attribute__((ext_vector_type(2)));
+// A 16-byte chunk: two doubles or four floats
+template <class R> struct Chunk;
+template <> struct Chunk<double> { typedef double type __attribute__((ext_vector_type(2))); };
+template <> struct Chunk<float> { typedef float type __attribute__((ext_vector_type(4))); };
 
-// Sizes of one instantiation: KCM 16-byte chunks per row of B at most, MBM blocks of 16 rows of A at most.  The general
-// kernel (32 chunks, 2 blocks) keeps 64 VGPRs of A and 32 of staging and runs two waves per SIMD; an operator of at most
-// 16 rows and 8 chunks needs a tenth of that, and twice as many waves hide twice the latency of its short units.
-template <int KCM, int MBM>
+// Sizes of one instantiation: R the component type, KCM 16-byte chunks per row of B at most, MBM blocks of 16 rows of A
+// at most.  The general kernel (32 chunks, 2 blocks) keeps 64 VGPRs of A (doubles) and 32 of staging and runs two waves
+// per SIMD; an operator of at most 16 rows and 8 chunks needs a tenth of that, and twice as many waves hide twice the
+// latency of its short units.
+template <class R, int KCM, int MBM>
 struct SkinnyCfg {
+    static constexpr int Q = 16 / (int)sizeof(R);             // components per chunk
     static constexpr int MAX_KC = KCM;
     static constexpr int PITCH = MAX_KC * 16 + 64;            // bytes per LDS row: rows 0..3 start 16 banks apart
     static constexpr int WAVE_LDS = SKINNY_UNIT * PITCH;      // each wave parks one unit
     static constexpr int LOADS = SKINNY_UNIT * MAX_KC / 64;   // 16-byte loads per lane and unit at most
     static constexpr int PAIRS = MAX_KC / 4;
-    static constexpr int OLOADS = SKINNY_UNIT * 16 * MBM / 64;   // 16-byte pieces of the result tile per lane at most (complex)
-    static constexpr int OUT_PITCH = 2 * 16 * MBM + 2;        // doubles per row of the transposed result tile (+2 against bank conflicts)
-    static constexpr int TILE_LDS = SKINNY_UNIT * OUT_PITCH * 8;   // the transposed result tile of a wave: a region of its own
+    static constexpr int OLOADS = SKINNY_UNIT * (32 * MBM / Q) / 64;   // 16-byte pieces of the result tile per lane at most (complex)
+    static constexpr int OUT_PITCH = 2 * 16 * MBM + Q;        // components per row of the transposed result tile (+16 bytes against bank conflicts)
+    static constexpr int TILE_LDS = SKINNY_UNIT * OUT_PITCH * (int)sizeof(R);   // the transposed result tile of a wave: a region of its own
     static constexpr int BLOCKS_PER_CU = KCM <= 8 && MBM == 1 ? 4 : 2;
-    static_assert(KCM % 4 == 0 && KCM * 2 <= SKINNY_MAX_KR && MBM * 16 <= SKINNY_MAX_M, "");
+    static_assert(KCM % 4 == 0 && KCM <= SKINNY_MAX_CHUNKS && MBM * 16 <= SKINNY_MAX_M, "");
 };
 
 // Orders the LDS accesses of one wave: lanes read what other lanes of the same wave wrote.  The LDS executes a wave's
@@ -67,13 +72,16 @@ __device__ __forceinline__ void wave_sync() {
 // iteration before with vmcnt(0): whatever is stored shortly before that wait is waited for as well, acknowledgement
 // included.  With C contiguous along n a unit's results therefore stay in registers for one more iteration and leave
 // in the middle of the next unit's MFMAs: by the time the next wait comes, they have had half an iteration to drain.
-template <bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM>
-__global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU)) gemm_skinny_kernel(SkinnyArgs s) {
-    typedef SkinnyCfg<KCM, MBM> Cfg;
-    constexpr int PITCH = Cfg::PITCH, WAVE_LDS = Cfg::WAVE_LDS, LOADS = Cfg::LOADS, PAIRS = Cfg::PAIRS;
+template <class R, bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM>
+__global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_CU)) gemm_skinny_kernel(SkinnyArgs s) {
+    typedef SkinnyCfg<R, KCM, MBM> Cfg;
+    typedef typename Chunk<R>::type chunk_t;
+    typedef typename Mfma<R>::acc_t acc_t;
+    constexpr int PITCH = Cfg::PITCH, WAVE_LDS = Cfg::WAVE_LDS, LOADS = Cfg::LOADS, PAIRS = Cfg::PAIRS, Q = Cfg::Q;
     constexpr int OUT_PITCH = Cfg::OUT_PITCH, TILE_LDS = Cfg::TILE_LDS, OLOADS = Cfg::OLOADS;
     constexpr int NBLK = CX ? 2 : 1;   // column blocks (16 real columns each) per unit
-    constexpr int NC = CX ? 2 : 1;     // doubles per element
+    constexpr int NC = CX ? 2 : 1;     // components per element
+    constexpr int EB = (int)sizeof(R);
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     unsigned char* lds = smem + wave * (WAVE_LDS + (OUT_ROWS ? TILE_LDS : 0));
@@ -81,30 +89,27 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU))
     const int g = lane >> 4, j = lane & 15, p = j & 1;
     const int kc = s.kc, npair = (kc + 3) >> 2, nmb = MBM > 1 && s.M > 16 ? 2 : 1;
 
-    // ---- A as MFMA operands: a[mb][i][q] = A'[j + 16 mb][2 (4i + g) + q], zero outside the matrix
-    double a[MBM][PAIRS][2];
+    // ---- A as MFMA operands: a[mb][i][q] = A'[j + 16 mb][Q (4i + g) + q], zero outside the matrix.  A' is A itself for
+    // real elements and its real form for complex ones: A'[m][2k + part] = (re, im)[part] of A[m][k].
+    R a[MBM][PAIRS][Q];
     {
-        const double* Ad = reinterpret_cast<const double*>(s.A);
+        const R* Ad = reinterpret_cast<const R*>(s.A);
 #pragma unroll
         for (int mb = 0; mb < MBM; ++mb)
 #pragma unroll
             for (int i = 0; i < PAIRS; ++i) {
                 const int m = j + 16 * mb, c = 4 * i + g;
-                double x0 = 0, x1 = 0;
-                if (m < s.M) {
-                    if constexpr (CX) {
-                        if (c < s.K) {
-                            const double* q = Ad + 2 * (off_of(s.am, m) + off_of(s.ak, c));
-                            x0 = q[0];
-                            x1 = s.conj_a ? -q[1] : q[1];
-                        }
-                    } else {
-                        if (2 * c < s.K) x0 = Ad[off_of(s.am, m) + off_of(s.ak, 2 * c)];
-                        if (2 * c + 1 < s.K) x1 = Ad[off_of(s.am, m) + off_of(s.ak, 2 * c + 1)];
+#pragma unroll
+                for (int q = 0; q < Q; ++q) {
+                    const int kk = Q * c + q;               // index into the real form
+                    const int k = kk / NC, part = kk % NC;
+                    R x = 0;
+                    if (m < s.M && k < s.K) {
+                        x = Ad[NC * (off_of(s.am, m) + off_of(s.ak, k)) + part];
+                        if (CX && part == 1 && s.conj_a) x = -x;
                     }
+                    a[mb][i][q] = x;
                 }
-                a[mb][i][0] = x0;
-                a[mb][i][1] = x1;
             }
     }
 
@@ -118,7 +123,7 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU))
         const bool ok = id < SKINNY_UNIT * kc;
         have |= (ok ? 1u : 0u) << u;
         lrows |= (ok ? (uint32_t)row : 0u) << (4 * u);
-        goff[u] = ok ? row * s.b_in * (8 * NC) + col * 16 : 0;
+        goff[u] = ok ? row * s.b_in * (EB * NC) + col * 16 : 0;
         loff[u] = ok ? row * PITCH + col * 16 : 0;
     }
     // ---- where this lane reads its operands and writes its results
@@ -134,30 +139,30 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU))
         for (int mb = 0; mb < MBM; ++mb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int m = Mfma<double>::row(lane, r) + 16 * mb;
+                const int m = Mfma<R>::row(lane, r) + 16 * mb;
                 crow[mb][r] = m < s.M ? (int32_t)(off_of(s.cm, m) * NC) : 0;
             }
     }
-    const double ar = s.alpha_re, ai = s.alpha_im, br = s.beta_re, bi = s.beta_im;
+    const R ar = (R)s.alpha_re, ai = (R)s.alpha_im, br = (R)s.beta_re, bi = (R)s.beta_im;
     // C contiguous along m: 16-byte piece id = lane + 64 u of the unit's result tile -> (n of the unit, piece of its row)
     int32_t ogoff[OLOADS] = {}, oloff[OLOADS] = {};
     uint32_t ohave = 0, orows = 0;
     if constexpr (OUT_ROWS) {
-        const int cpr = s.M * NC / 2;   // 16-byte pieces per row of C
+        const int cpr = s.M * NC / Q;   // 16-byte pieces per row of C
 #pragma unroll
         for (int u = 0; u < OLOADS; ++u) {
             const int id = lane + 64 * u, row = id / cpr, col = id - row * cpr;
             const bool ok = id < SKINNY_UNIT * cpr;
             ohave |= (ok ? 1u : 0u) << u;
             orows |= (ok ? (uint32_t)row : 0u) << (4 * u);
-            ogoff[u] = ok ? (row * s.c_in * NC + col * 2) * 8 : 0;
-            oloff[u] = ok ? (row * OUT_PITCH + col * 2) * 8 : 0;
+            ogoff[u] = ok ? (row * s.c_in * NC + col * Q) * EB : 0;
+            oloff[u] = ok ? (row * OUT_PITCH + col * Q) * EB : 0;
         }
     }
 
     const int64_t nwaves = (int64_t)gridDim.x * (THREADS / 64);
     int64_t unit = (int64_t)blockIdx.x * (THREADS / 64) + wave;
-    d2 stage[LOADS];
+    chunk_t stage[LOADS];
     // The innermost run of n need not hold a whole number of units: the last unit of each run then has s.tail valid n.
     // Rows past them are neither loaded (what is parked for them is whatever the registers held: their columns of the
     // product are independent of the others and never stored) nor written.
@@ -166,36 +171,36 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU))
         return (int)(un % s.upr) == s.upr - 1 ? s.tail : SKINNY_UNIT;
     };
     auto issue = [&](int64_t un) {
-        const unsigned char* Bu = reinterpret_cast<const unsigned char*>(s.B) + off_of(s.bu, un) * (8 * NC);
+        const unsigned char* Bu = reinterpret_cast<const unsigned char*>(s.B) + off_of(s.bu, un) * (EB * NC);
         const int valid = valid_of(un);
 #pragma unroll
         for (int u = 0; u < LOADS; ++u)
             if (((have >> u) & 1u) && (int)((lrows >> (4 * u)) & 15u) < valid)
-                stage[u] = __builtin_nontemporal_load(reinterpret_cast<const d2*>(Bu + goff[u]));
+                stage[u] = __builtin_nontemporal_load(reinterpret_cast<const chunk_t*>(Bu + goff[u]));
     };
-    // C contiguous along n: lane (g, j) holds rows g + 4r (+16), column j of each column block
-    auto store_direct = [&](const d4 (&res)[MBM][NBLK], double* Cu, int valid) {
+    // C contiguous along n: lane (g, j) holds the rows Mfma<R>::row(lane, r) (+16), column j of each column block
+    auto store_direct = [&](const acc_t (&res)[MBM][NBLK], R* Cu, int valid) {
 #pragma unroll
         for (int mb = 0; mb < MBM; ++mb) {
             if (mb < nmb) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const bool row_ok = Mfma<double>::row(lane, r) + 16 * mb < s.M;
+                    const bool row_ok = Mfma<R>::row(lane, r) + 16 * mb < s.M;
 #pragma unroll
                     for (int nb = 0; nb < NBLK; ++nb) {
                         const bool ok = row_ok && (CX ? 8 * nb + (j >> 1) : j) < valid;
-                        double* dst = Cu + crow[mb][r] + ccol[nb];
-                        double v = res[mb][nb][r];
+                        R* dst = Cu + crow[mb][r] + ccol[nb];
+                        R v = res[mb][nb][r];
                         if (!s.plain) {
                             if constexpr (CX) {
                                 // even lanes hold re, odd lanes im of one element: exchange with the neighbour
-                                const double other = __shfl_xor(v, 1);
-                                const double re_v = p ? other : v, im_v = p ? v : other;
+                                const R other = __shfl_xor(v, 1);
+                                const R re_v = p ? other : v, im_v = p ? v : other;
                                 v = p ? (ar * im_v + ai * re_v) : (ar * re_v - ai * im_v);
                                 if (s.use_beta) {
-                                    const double old = ok ? *dst : 0.0;
-                                    const double old_other = __shfl_xor(old, 1);
-                                    const double re_o = p ? old_other : old, im_o = p ? old : old_other;
+                                    const R old = ok ? *dst : R(0);
+                                    const R old_other = __shfl_xor(old, 1);
+                                    const R re_o = p ? old_other : old, im_o = p ? old : old_other;
                                     v += p ? (br * im_o + bi * re_o) : (br * re_o - bi * im_o);
                                 }
                             } else {
@@ -210,21 +215,27 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU))
         }
     };
     // C contiguous along m: the tile of the unit before leaves as 16-byte pieces of whole rows
-    auto store_rows = [&](double* Cu, int valid) {
+    auto store_rows = [&](R* Cu, int valid) {
 #pragma unroll
         for (int u = 0; u < OLOADS; ++u)
             if (((ohave >> u) & 1u) && (int)((orows >> (4 * u)) & 15u) < valid) {
-                d2 v = *reinterpret_cast<const d2*>(tile_lds + oloff[u]);
-                d2* dst = reinterpret_cast<d2*>(reinterpret_cast<unsigned char*>(Cu) + ogoff[u]);
+                chunk_t v = *reinterpret_cast<const chunk_t*>(tile_lds + oloff[u]);
+                chunk_t* dst = reinterpret_cast<chunk_t*>(reinterpret_cast<unsigned char*>(Cu) + ogoff[u]);
                 if (!s.plain) {
-                    d2 o;
+                    chunk_t o;
                     if constexpr (CX) {
-                        o.x = ar * v.x - ai * v.y;
-                        o.y = ar * v.y + ai * v.x;
+#pragma unroll
+                        for (int e = 0; e < Q; e += 2) {
+                            o[e] = ar * v[e] - ai * v[e + 1];
+                            o[e + 1] = ar * v[e + 1] + ai * v[e];
+                        }
                         if (s.use_beta) {
-                            const d2 old = *dst;
-                            o.x += br * old.x - bi * old.y;
-                            o.y += br * old.y + bi * old.x;
+                            const chunk_t old = *dst;
+#pragma unroll
+                            for (int e = 0; e < Q; e += 2) {
+                                o[e] += br * old[e] - bi * old[e + 1];
+                                o[e + 1] += br * old[e + 1] + bi * old[e];
+                            }
                         }
                     } else {
                         o = v * ar;
@@ -235,52 +246,56 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU))
                 __builtin_nontemporal_store(v, dst);
             }
     };
-    d4 held[MBM][NBLK];          // !OUT_ROWS: the results of the unit before, not yet stored (OUT_ROWS: they wait in the tile)
-    double* held_c = nullptr;
+    acc_t held[MBM][NBLK];     // !OUT_ROWS: the results of the unit before, not yet stored (OUT_ROWS: they wait in the tile)
+    R* held_c = nullptr;
     int held_valid = 0;
 #pragma unroll
-    for (int u = 0; u < LOADS; ++u) stage[u] = d2{0, 0};
+    for (int u = 0; u < LOADS; ++u)
+#pragma unroll
+        for (int e = 0; e < Q; ++e) stage[u][e] = 0;
     if (unit < s.units) issue(unit);
     while (unit < s.units) {
         const int valid = valid_of(unit);
 #pragma unroll
         for (int u = 0; u < LOADS; ++u)
-            if ((have >> u) & 1u) *reinterpret_cast<d2*>(lds + loff[u]) = stage[u];
+            if ((have >> u) & 1u) *reinterpret_cast<chunk_t*>(lds + loff[u]) = stage[u];
         const int64_t next = unit + nwaves;
         // (a table lookup here finds nothing else in flight: behind the loads of the next unit it would wait for them)
-        double* Cu = reinterpret_cast<double*>(s.C) + off_of(s.cu, unit) * NC;
+        R* Cu = reinterpret_cast<R*>(s.C) + off_of(s.cu, unit) * NC;
         if (next < s.units) issue(next);
         wave_sync();
 
-        d4 acc[MBM][NBLK];
+        acc_t acc[MBM][NBLK];
 #pragma unroll
         for (int mb = 0; mb < MBM; ++mb)
 #pragma unroll
-            for (int nb = 0; nb < NBLK; ++nb) acc[mb][nb] = d4{0, 0, 0, 0};
+            for (int nb = 0; nb < NBLK; ++nb) acc[mb][nb] = acc_t{0, 0, 0, 0};
 #pragma unroll
         for (int i = 0; i < PAIRS; ++i) {
             if (i < npair) {
                 const bool kok = 4 * i + g < kc;
 #pragma unroll
                 for (int nb = 0; nb < NBLK; ++nb) {
-                    const d2 ch = *reinterpret_cast<const d2*>(lds + roff[nb] + i * 64);
-                    double b0, b1;
-                    if constexpr (CX) {
-                        const double im = s.conj_b ? -ch.y : ch.y;
-                        b0 = p ? im : ch.x;
-                        b1 = p ? ch.x : -im;
-                    } else {
-                        b0 = ch.x;
-                        b1 = ch.y;
+                    const chunk_t ch = *reinterpret_cast<const chunk_t*>(lds + roff[nb] + i * 64);
+                    // the chunk as operands B'[Q c + q][column j]: the components themselves for real elements; for a
+                    // complex element (br, bi) the even column of its pair takes (br, -bi), the odd one (bi, br)
+                    R b[Q];
+#pragma unroll
+                    for (int q = 0; q < Q; ++q) {
+                        if constexpr (CX) {
+                            const R re = ch[q & ~1], im = s.conj_b ? -ch[q | 1] : ch[q | 1];
+                            b[q] = (q & 1) ? (p ? re : -im) : (p ? im : re);
+                        } else {
+                            b[q] = ch[q];
+                        }
+                        b[q] = kok ? b[q] : R(0);   // a row of B may be shorter than the LDS row: never multiply what was not loaded
                     }
-                    b0 = kok ? b0 : 0.0;   // a row of B may be shorter than the LDS row: never multiply what was not loaded
-                    b1 = kok ? b1 : 0.0;
-                    acc[0][nb] = Mfma<double>::run(a[0][i][0], b0, acc[0][nb]);
-                    acc[0][nb] = Mfma<double>::run(a[0][i][1], b1, acc[0][nb]);
+#pragma unroll
+                    for (int q = 0; q < Q; ++q) acc[0][nb] = Mfma<R>::run(a[0][i][q], b[q], acc[0][nb]);
                     if constexpr (MBM > 1)
                         if (nmb > 1) {
-                            acc[1][nb] = Mfma<double>::run(a[1][i][0], b0, acc[1][nb]);
-                            acc[1][nb] = Mfma<double>::run(a[1][i][1], b1, acc[1][nb]);
+#pragma unroll
+                            for (int q = 0; q < Q; ++q) acc[1][nb] = Mfma<R>::run(a[1][i][q], b[q], acc[1][nb]);
                         }
                 }
             }
@@ -291,10 +306,9 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU))
         }
         wave_sync();   // the next unit is parked over these rows, and its results are written over the tile
 
-        // ---- results: lane (g, j) holds rows g + 4r (+16), column j of each column block
         if constexpr (OUT_ROWS) {
             // tile[n of the unit][m][part] in LDS; whole rows leave during the next unit's MFMAs (store_rows)
-            double* tile = reinterpret_cast<double*>(tile_lds);
+            R* tile = reinterpret_cast<R*>(tile_lds);
 #pragma unroll
             for (int mb = 0; mb < MBM; ++mb)
                 if (mb < nmb) {
@@ -302,7 +316,7 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU))
                     for (int r = 0; r < 4; ++r)
 #pragma unroll
                         for (int nb = 0; nb < NBLK; ++nb) {
-                            const int m = Mfma<double>::row(lane, r) + 16 * mb, nloc = CX ? 8 * nb + (j >> 1) : j;
+                            const int m = Mfma<R>::row(lane, r) + 16 * mb, nloc = CX ? 8 * nb + (j >> 1) : j;
                             tile[nloc * OUT_PITCH + m * NC + (CX ? p : 0)] = acc[mb][nb][r];
                         }
                 }
@@ -329,48 +343,49 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<KCM, MBM>::BLOCKS_PER_CU))
     }
 }
 
-}  // namespace
-
-namespace {
-template <bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM>
+template <class R, bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM>
 void launch_variant(const gemm::SkinnyArgs& s, hipStream_t st) {
-    typedef SkinnyCfg<KCM, MBM> Cfg;
+    typedef SkinnyCfg<R, KCM, MBM> Cfg;
     constexpr int lds = (THREADS / 64) * (Cfg::WAVE_LDS + (OUT_ROWS ? Cfg::TILE_LDS : 0));
     static bool once = [] {   // (more than 64 KB of dynamic LDS has to be asked for once per kernel)
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<CX, RAGGED, OUT_ROWS, KCM, MBM>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<R, CX, RAGGED, OUT_ROWS, KCM, MBM>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         return true;
     }();
     (void)once;
     const int64_t blocks_wanted = (s.units + THREADS / 64 - 1) / (THREADS / 64);
     const dim3 grid((uint32_t)std::min<int64_t>(blocks_wanted, 256 * Cfg::BLOCKS_PER_CU)), block(THREADS);
-    TFH_LAUNCH_TIMED((gemm_skinny_kernel<CX, RAGGED, OUT_ROWS, KCM, MBM>), grid, block, (size_t)lds, st, s);
+    TFH_LAUNCH_TIMED((gemm_skinny_kernel<R, CX, RAGGED, OUT_ROWS, KCM, MBM>), grid, block, (size_t)lds, st, s);
 }
 
-template <bool CX, bool RAGGED, bool OUT_ROWS>
+template <class R, bool CX, bool RAGGED, bool OUT_ROWS>
 void launch_sized(const gemm::SkinnyArgs& s, hipStream_t st) {
     // (twice the waves pay where a unit is short: measured faster up to 8 complex or 16 real rows, even beyond)
-    if (s.kc <= 8 && s.M <= (CX ? 8 : 16)) launch_variant<CX, RAGGED, OUT_ROWS, 8, 1>(s, st);
-    else launch_variant<CX, RAGGED, OUT_ROWS, SKINNY_MAX_KR / 2, SKINNY_MAX_M / 16>(s, st);
+    if (s.kc <= 8 && s.M <= (CX ? 8 : 16)) launch_variant<R, CX, RAGGED, OUT_ROWS, 8, 1>(s, st);
+    else launch_variant<R, CX, RAGGED, OUT_ROWS, SKINNY_MAX_CHUNKS, SKINNY_MAX_M / 16>(s, st);
 }
+
+template <class R, bool CX>
+void launch_typed(const gemm::SkinnyArgs& s, hipStream_t st) {
+    const bool ragged = s.tail != 0, rows = s.out_rows != 0;
+    if (ragged) {
+        if (rows) launch_sized<R, CX, true, true>(s, st);
+        else launch_sized<R, CX, true, false>(s, st);
+    } else {
+        if (rows) launch_sized<R, CX, false, true>(s, st);
+        else launch_sized<R, CX, false, false>(s, st);
+    }
+}
+
 }  // namespace
 
 void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
-    const bool cx = dtype == TFH_C128, ragged = s.tail != 0, rows = s.out_rows != 0;
-#define TFH_SKINNY_CASE(CXV, RAGV, ROWV)               \
-    if (cx == CXV && ragged == RAGV && rows == ROWV) { \
-        launch_sized<CXV, RAGV, ROWV>(s, st);          \
-        return;                                        \
+    switch (dtype) {
+        case TFH_F32: launch_typed<float, false>(s, st); break;
+        case TFH_F64: launch_typed<double, false>(s, st); break;
+        case TFH_C64: launch_typed<float, true>(s, st); break;
+        default: launch_typed<double, true>(s, st); break;
     }
-    TFH_SKINNY_CASE(true, false, false)
-    TFH_SKINNY_CASE(true, false, true)
-    TFH_SKINNY_CASE(true, true, false)
-    TFH_SKINNY_CASE(true, true, true)
-    TFH_SKINNY_CASE(false, false, false)
-    TFH_SKINNY_CASE(false, false, true)
-    TFH_SKINNY_CASE(false, true, false)
-    TFH_SKINNY_CASE(false, true, true)
-#undef TFH_SKINNY_CASE
 }
 
 }  // namespace tfh

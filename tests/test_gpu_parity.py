@@ -1798,14 +1798,20 @@ def test_offset_tables_are_kept_per_layout_and_survive_a_release(tf, oracle):
             assert tf.lib().tfh_release_workspaces() == 0
 
 
-@pytest.mark.parametrize("dtype", [np.complex128, np.float64])
+def whole_chunks(dtype, n):
+    # n elements fill a whole number of 16-byte chunks
+    return (n * np.dtype(dtype).itemsize) % 16 == 0
+
+
+@pytest.mark.parametrize("dtype", ALL)
 @pytest.mark.parametrize("m,k,x,c", [(32, 32, 8, 1024), (20, 13, 64, 80), (16, 32, 1, 4096), (7, 6, 16, 512), (32, 2, 32, 160),
                                      (32, 32, 16, 500), (16, 8, 64, 100), (20, 16, 100, 50), (5, 4, 5, 1000), (8, 6, 300, 17)])
 def test_contract_small_operator_applied_to_a_long_tensor(tf, oracle, dtype, m, k, x, c):
     # T[x, c, k] . W[k, m] -> out[x, m, c]: few rows, little k, a long n = (x, c) whose fastest output axis is c -- the
     # shape of an operator applied to every fibre of a large tensor, which takes the streaming kernel.  Odd m and k,
-    # general alpha/beta, and a W that is a strided view are covered; f64 needs an even k for that kernel and falls
-    # back to the tiled one otherwise (k = 13).  The kernel works on units of 16 consecutive c: extents that are no
+    # general alpha/beta, and a W that is a strided view are covered; a row of k must fill whole 16-byte chunks for that
+    # kernel (any k for complex128, even k for f64 and complex64, k a multiple of 4 for f32), otherwise the tiled ones
+    # take the product (k = 13).  The kernel works on units of 16 consecutive c: extents that are no
     # multiple of 16 (500, 100, 50, 1000: bond dimensions are rarely powers of two) end each run on a partly filled unit;
     # a run shorter than three units (17) is left to the tiled kernels.
     rng = np.random.default_rng(91)
@@ -1820,9 +1826,9 @@ def test_contract_small_operator_applied_to_a_long_tensor(tf, oracle, dtype, m, 
         dout = dev(tf, out0)
         plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab("xmc")), [t.shape, w.shape, ref.shape])
         tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
-        streamed = (cplx or k % 2 == 0) and (c % 16 == 0 or c >= 48)
+        streamed = whole_chunks(dtype, k) and (c % 16 == 0 or c >= 48)
         assert ("gemm_skinny_kernel" in tf.last_kernel()) == streamed, tf.last_kernel()
-        assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
+        assert relerr(dout.to_numpy(), ref) < TOL[dtype], (alpha, beta)
 
 
 def test_contract_small_operator_exact_on_integer_inputs(tf):
@@ -1838,7 +1844,7 @@ def test_contract_small_operator_exact_on_integer_inputs(tf):
     assert np.array_equal(out.to_numpy(), np.einsum("xck,km->xmc", t, w))
 
 
-@pytest.mark.parametrize("dtype", [np.complex128, np.float64])
+@pytest.mark.parametrize("dtype", ALL)
 def test_contract_small_operator_strided_rows_and_split_k_order(tf, oracle, dtype):
     # the streaming kernel's addressing: rows of the long operand reversed along c and padded (a view of a larger buffer),
     # its k split over two modes that the small operand holds in the opposite order (its k goes through the offset table),
@@ -1853,7 +1859,7 @@ def test_contract_small_operator_strided_rows_and_split_k_order(tf, oracle, dtyp
     plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xcsw"), lab("wstv"), lab("xvtc")), [t1.shape, wop.shape, ref.shape])
     tf.HipBackend.execute(plan, 1.0, [dev(tf, t1), dev(tf, wop)], 0.0, out)
     assert "gemm_skinny_kernel" in tf.last_kernel()
-    assert relerr(out.to_numpy(), ref) < 1e-12
+    assert relerr(out.to_numpy(), ref) < TOL[dtype]
     # padded rows: each (x, c) row is the first 16 elements of a 24-element row of a larger buffer
     bigk = rand(rng, (x, c, 24), dtype)
     t2 = bigk[:, :, :16]
@@ -1864,15 +1870,16 @@ def test_contract_small_operator_strided_rows_and_split_k_order(tf, oracle, dtyp
     plan2 = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab("xmc")), [t2.shape, w2.shape, ref2.shape])
     tf.HipBackend.execute(plan2, 1.0, [dev(tf, t2), dev(tf, w2)], 0.0, out2)
     assert "gemm_skinny_kernel" in tf.last_kernel()
-    assert relerr(out2.to_numpy(), ref2) < 1e-12
+    assert relerr(out2.to_numpy(), ref2) < TOL[dtype]
 
 
-@pytest.mark.parametrize("dtype", [np.complex128, np.float64])
+@pytest.mark.parametrize("dtype", ALL)
 @pytest.mark.parametrize("m,k,x,c", [(32, 32, 8, 1024), (20, 13, 64, 80), (16, 32, 1, 4096), (7, 6, 16, 512), (32, 2, 32, 160), (2, 64, 4, 2048),
                                      (32, 32, 9, 500), (16, 8, 7, 700), (4, 4, 1, 4099)])
 def test_contract_small_operator_with_the_result_contiguous_along_its_columns(tf, oracle, dtype, m, k, x, c):
     # the other orientation of the same product: T[x, c, k] . W[k, m] -> out[x, c, m], the few columns m adjacent in the
-    # output.  The streaming kernel then transposes each unit's results through LDS.  f64 needs even m and k for it.
+    # output.  The streaming kernel then transposes each unit's results through LDS.  Rows of k and of m must fill
+    # whole 16-byte chunks for it.
     # (x, c) is one run of x * c here: 9 * 500, 7 * 700 and 4099 leave a partly filled last unit.
     cplx = np.issubdtype(dtype, np.complexfloating)
     if k > 32 and cplx:
@@ -1887,9 +1894,9 @@ def test_contract_small_operator_with_the_result_contiguous_along_its_columns(tf
         dout = dev(tf, out0)
         plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab("xcm")), [t.shape, w.shape, ref.shape])
         tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
-        streamed = cplx or (k % 2 == 0 and m % 2 == 0)
+        streamed = whole_chunks(dtype, k) and whole_chunks(dtype, m)
         assert ("gemm_skinny_kernel" in tf.last_kernel()) == streamed, tf.last_kernel()
-        assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
+        assert relerr(dout.to_numpy(), ref) < TOL[dtype], (alpha, beta)
     # the same with the output rows padded (a view of a wider buffer) and the long operand's rows reversed
     wide = rand(rng, (x, c, m + 2), dtype)
     view = wide[:, :, :m]
@@ -1900,11 +1907,11 @@ def test_contract_small_operator_with_the_result_contiguous_along_its_columns(tf
     dview = tf.Tensor(dwide._buf, [x, c, m], dwide.strides(), 0, tf.GpuMemory(0), tf.dtype_code(dtype))
     tf.HipBackend.execute(plan, 1.0, [dev(tf, tr), dev(tf, w)], 0.0, dview)
     got = dwide.to_numpy()
-    assert relerr(got[:, :, :m], ref) < 1e-12
+    assert relerr(got[:, :, :m], ref) < TOL[dtype]
     assert np.array_equal(got[:, :, m:], wide[:, :, m:])          # the padding is untouched
 
 
-@pytest.mark.parametrize("dtype", [np.complex128, np.float64])
+@pytest.mark.parametrize("dtype", ALL)
 @pytest.mark.parametrize("out_modes", ["xmc", "xcm"])
 @pytest.mark.parametrize("m,k,c", [(32, 32, 24000), (20, 12, 24008), (12, 10, 30001), (8, 6, 30001), (4, 8, 160000)])
 def test_contract_small_operator_every_wave_streams_several_units(tf, oracle, dtype, out_modes, m, k, c):
@@ -1915,6 +1922,10 @@ def test_contract_small_operator_every_wave_streams_several_units(tf, oracle, dt
     cplx = np.issubdtype(dtype, np.complexfloating)
     if not cplx:
         k *= 2
+    if np.dtype(dtype).itemsize <= 8 and dtype != np.float64:
+        k *= 2          # whole chunks of four f32 / two complex64
+    if dtype == np.float32 and out_modes == "xcm":
+        m = (m + 3) // 4 * 4
     rng = np.random.default_rng(95)
     x = 3
     t = rand(rng, (x, c, k), dtype)
@@ -1927,7 +1938,7 @@ def test_contract_small_operator_every_wave_streams_several_units(tf, oracle, dt
         plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("xck"), lab("km"), lab(out_modes)), [t.shape, w.shape, ref.shape])
         tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
         assert "gemm_skinny_kernel" in tf.last_kernel(), tf.last_kernel()
-        assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
+        assert relerr(dout.to_numpy(), ref) < TOL[dtype], (alpha, beta)
 
 
 @pytest.mark.parametrize("dtype", [np.complex128, np.float64])
