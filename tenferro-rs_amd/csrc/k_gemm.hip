@@ -564,16 +564,16 @@ bool skinny_run_ok(int64_t n) { return n % SKINNY_UNIT == 0 || n >= 3 * SKINNY_U
 // writes with a stride of one row between neighbouring lanes, while the streaming kernel of k_gemm_skinny.hip takes
 // whole rows.  Measured on 4M rows (us, tiny | streaming): complex128 8x8 566 | 196 with C contiguous along n and
 // 1959 | 189 along m, 4x4 130 | 98 and 412 | 98, 2x4 102 | 82 and 128 | 83, 4x2 73 | 90, 3x3 81 | 85, 2x2 47 | 81 and
-// 80 | 81; f64 8x8 195 | 95 and 812 | 92, 4x6 106 | 69, 6x6 120 | 78, 4x4 64 | 69 and 167 | 72, 2x4 50 | 61 and 56 | 64.
-// ms: the operator's free extent.
+// 80 | 81; f64 8x8 195 | 95 and 812 | 92, 4x6 106 | 69, 6x6 120 | 78, 4x4 64 | 69 and 167 | 72, 2x4 50 | 61 and 56 | 64;
+// complex64 8x8 193 | 115 and 838 | 100, 4x4 63 | 94 and 187 | 82; f32 8x8 103 | 78 and 333 | 68, 4x4 39 | 69 and
+// 76 | 61.  ms: the operator's free extent.
 bool last_leg_prefers_streaming(int dtype, const ContractAxes& ax, int64_t M, int64_t N, int64_t K) {
-    if (dtype != TFH_F64 && dtype != TFH_C128) return false;
     const bool small_is_a = M <= N;
     const int tslot = small_is_a ? 1 : 0;
     const std::vector<Axis>& small = small_is_a ? ax.M : ax.N;
     const int64_t ms = small_is_a ? M : N;
-    if (ms > 8 || K > 8) return false;
-    if (K * (dtype == TFH_C128 ? 16 : 8) < 32) return false;   // (rows under 32 bytes would be packed first)
+    if (ms > 8 || K > 8 || K < 2) return false;
+    if (K * (int64_t)dtype_size(dtype) % 16 != 0) return false;   // rows of whole 16-byte chunks
     std::vector<Axis> k = ax.K;
     order_by(k, tslot);
     int64_t expect = 1;
@@ -582,8 +582,12 @@ bool last_leg_prefers_streaming(int dtype, const ContractAxes& ax, int64_t M, in
         expect *= k[d].n;
     }
     const bool rows = min_stride(small, 2) == 1;   // C contiguous along the operator's free index
-    if (dtype == TFH_C128) return rows ? (ms >= 3 || K >= 4) : K >= 4;
-    return rows ? (ms >= 4 || K >= 6) : K >= 6;
+    switch (dtype) {
+        case TFH_C128: return rows ? (ms >= 3 || K >= 4) : K >= 4;
+        case TFH_F64: return rows ? (ms >= 4 || K >= 6) : K >= 6;
+        case TFH_C64: return rows ? (ms >= 4 || K >= 6) : K >= 6;
+        default: return rows ? (ms >= 4 || K >= 8) : K >= 8;
+    }
 }
 
 int bke_of(int dtype) {
@@ -772,6 +776,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         const bool kfast = slot == 0 ? a_kfast : b_kfast;
         const std::vector<Axis>& lanes = kfast ? ax.K : rows;
         if (lanes.empty() || lanes.back().n == 1) continue;
+        if (tiny_deferred) continue;   // (the streaming kernel loads 16-byte chunks, the tiny-operator kernel elements: neither wants a copy)
         const Axis& inner = lanes.back();
         const int64_t run = std::llabs(inner.s[slot]) == 1 ? inner.n * (int64_t)eb : (int64_t)eb;
         if (run >= 32) continue;

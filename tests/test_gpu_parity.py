@@ -1941,7 +1941,7 @@ def test_contract_small_operator_every_wave_streams_several_units(tf, oracle, dt
         assert relerr(dout.to_numpy(), ref) < TOL[dtype], (alpha, beta)
 
 
-@pytest.mark.parametrize("dtype", [np.complex128, np.float64])
+@pytest.mark.parametrize("dtype", ALL)
 @pytest.mark.parametrize("out_modes", ["xmc", "xcm"])
 @pytest.mark.parametrize("m,k,c", [(8, 8, 4096), (4, 4, 4096), (2, 2, 4096), (8, 4, 4096), (3, 6, 4096), (4, 2, 4096), (8, 8, 17)])
 def test_contract_tiny_operator_on_the_last_leg_of_a_long_tensor(tf, oracle, dtype, out_modes, m, k, c):
@@ -1956,13 +1956,14 @@ def test_contract_tiny_operator_on_the_last_leg_of_a_long_tensor(tf, oracle, dty
     t = rand(rng, (x, c, k), dtype)
     w = rand(rng, (k, m), dtype)
     out0 = rand(rng, (x, c, m) if rows else (x, m, c), dtype)
-    if cplx:
+    if dtype == np.complex128:
         prefer = (m >= 3 or k >= 4) if rows else k >= 4
-        can = True
+    elif dtype == np.float32:
+        prefer = (m >= 4 or k >= 8) if rows else k >= 8
     else:
-        prefer = ((m >= 4 or k >= 6) if rows else k >= 6) and k >= 4
-        can = k % 2 == 0 and (m % 2 == 0 or not rows)
-    can = can and (rows or c >= 48)
+        prefer = (m >= 4 or k >= 6) if rows else k >= 6
+    prefer = prefer and k >= 2 and whole_chunks(dtype, k)
+    can = (whole_chunks(dtype, m) or not rows) and (rows or c >= 48)
     for alpha, beta in [(1.0, 0.0), ((0.5 - 2j, 1.5 + 1j) if cplx else (0.5, -1.5))]:
         ref = out0.copy()
         oracle.contract(t, lab("xck"), w, lab("km"), ref, lab(out_modes), alpha=alpha, beta=beta)
@@ -1971,7 +1972,7 @@ def test_contract_tiny_operator_on_the_last_leg_of_a_long_tensor(tf, oracle, dty
         tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
         want = "gemm_skinny_kernel" if prefer and can else "tiny_operator_kernel"
         assert want in tf.last_kernel(), (tf.last_kernel(), want)
-        assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
+        assert relerr(dout.to_numpy(), ref) < TOL[dtype], (alpha, beta)
 
 
 @pytest.mark.parametrize("dtype", ALL)
