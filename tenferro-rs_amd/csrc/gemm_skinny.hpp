@@ -25,6 +25,8 @@ struct SkinnyArgs {
     int32_t upr, tail;       // units per innermost run of n; n in the last unit of each run (0: every unit is full)
     OffFn am, ak, cm;        // element offsets of A's rows and k, of C's rows
     OffFn bu, cu;            // element offset of a unit's first n in B and in C
+    OffFn bk;                // nfast: element offset of k in B
+    int32_t nfast;           // B is contiguous along n instead of k (complex128, C along n)
     int32_t b_in, c_in;      // element stride between consecutive n inside a unit, in B and in C
     double alpha_re, alpha_im, beta_re, beta_im;
 };

@@ -865,6 +865,16 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         skinny = whole_chunks(K) && (uintptr_t)b % 16 == 0;
         for (auto& x : ax.N) skinny = skinny && whole_chunks(x.s[1]);
     }
+    // The same operator on a leg that is not the long tensor's last: B is contiguous along n (as is C), its k strides
+    // are whatever they are.  complex128 only (one element per 16-byte chunk): the kernel parks a unit as [k][16 n].
+    bool skinny_nfast = false;
+    if (!skinny && cxd && nb == 1 && !out_rows && M <= SKINNY_MAX_M && K <= SKINNY_MAX_CHUNKS && N >= 4096 && !b_kfast &&
+        !ax.K.empty() && !ax.N.empty() && ax.N.back().s[1] == 1 && ax.N.back().s[2] == 1 && skinny_run_ok(ax.N.back().n)) {
+        int64_t lo = 0, hi = 0;
+        reach(ax.K, 1, lo, hi);
+        skinny_nfast = std::max(-lo, hi) * (int64_t)eb < ((int64_t)1 << 30);
+        skinny = skinny_nfast;
+    }
     int64_t inner_b = 0, inner_c = 0, skinny_upr = 1;
     int skinny_tail = 0;
     if (skinny) {
@@ -1160,6 +1170,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         sk.units = Ntab;
         sk.upr = (int32_t)skinny_upr; sk.tail = skinny_tail;
         sk.am = g.am; sk.ak = g.ak; sk.cm = g.cm; sk.bu = g.bn; sk.cu = g.cn;
+        sk.bk = g.bk; sk.nfast = skinny_nfast;
         sk.b_in = (int32_t)inner_b; sk.c_in = (int32_t)inner_c;
         sk.alpha_re = alpha.re; sk.alpha_im = alpha.im; sk.beta_re = beta.re; sk.beta_im = beta.im;
         launch_gemm_skinny(dtype, sk, st);

@@ -54,6 +54,9 @@ struct SkinnyCfg {
     static constexpr int OUT_PITCH = 2 * 16 * MBM + Q;        // components per row of the transposed result tile (+16 bytes against bank conflicts)
     static constexpr int TILE_LDS = SKINNY_UNIT * OUT_PITCH * (int)sizeof(R);   // the transposed result tile of a wave: a region of its own
     static constexpr int BLOCKS_PER_CU = KCM <= 8 && MBM == 1 ? 4 : 2;
+    // B contiguous along n instead of k (complex128 only): the unit is parked as [k][16 n], one element per chunk
+    static constexpr int KPITCH = SKINNY_UNIT * 16 + 64;      // bytes per k row: lane groups g = 0..3 start 16 banks apart
+    static constexpr int WAVE_LDS_NFAST = MAX_KC * KPITCH;
     static_assert(KCM % 4 == 0 && KCM <= SKINNY_MAX_CHUNKS && MBM * 16 <= SKINNY_MAX_M, "");
 };
 
@@ -66,18 +69,23 @@ __device__ __forceinline__ void wave_sync() {
 }
 
 // RAGGED: the innermost run of n holds no whole number of units (its own instantiation: the full-unit kernel carries
-// none of the per-unit predicates).  OUT_ROWS: C is contiguous along m (s.out_rows).
+// none of the per-unit predicates).  OUT_ROWS: C is contiguous along m (s.out_rows).  NFAST (complex128, C along n):
+// B is contiguous along n, not along k -- the operator acts on a leg that is not the tensor's last: a unit is then K
+// segments of 16 consecutive n (256 bytes each), parked as [k][n]; the operands come out of LDS by the same 16-byte
+// reads, from other addresses.
 //
 // vmcnt counts loads and stores in one queue, in order, and the compiler waits for a register that was loaded in the
 // iteration before with vmcnt(0): whatever is stored shortly before that wait is waited for as well, acknowledgement
 // included.  With C contiguous along n a unit's results therefore stay in registers for one more iteration and leave
 // in the middle of the next unit's MFMAs: by the time the next wait comes, they have had half an iteration to drain.
-template <class R, bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM>
+template <class R, bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM, bool NFAST = false>
 __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_CU)) gemm_skinny_kernel(SkinnyArgs s) {
     typedef SkinnyCfg<R, KCM, MBM> Cfg;
+    static_assert(!NFAST || (CX && sizeof(R) == 8 && !OUT_ROWS), "one element per chunk");
     typedef typename Chunk<R>::type chunk_t;
     typedef typename Mfma<R>::acc_t acc_t;
-    constexpr int PITCH = Cfg::PITCH, WAVE_LDS = Cfg::WAVE_LDS, LOADS = Cfg::LOADS, PAIRS = Cfg::PAIRS, Q = Cfg::Q;
+    constexpr int PITCH = Cfg::PITCH, WAVE_LDS = NFAST ? Cfg::WAVE_LDS_NFAST : Cfg::WAVE_LDS, LOADS = Cfg::LOADS, PAIRS = Cfg::PAIRS, Q = Cfg::Q;
+    constexpr int KPITCH = Cfg::KPITCH;
     constexpr int OUT_PITCH = Cfg::OUT_PITCH, TILE_LDS = Cfg::TILE_LDS, OLOADS = Cfg::OLOADS;
     constexpr int NBLK = CX ? 2 : 1;   // column blocks (16 real columns each) per unit
     constexpr int NC = CX ? 2 : 1;     // components per element
@@ -115,23 +123,30 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_C
 
     // ---- this lane's share of a unit of B: chunk id = lane + 64 u -> (row, chunk of the row)
     int32_t goff[LOADS], loff[LOADS];
-    uint32_t have = 0, lrows = 0;   // lrows: four bits per load, the row (n of the unit) it belongs to
+    uint32_t have = 0, lrows = 0;   // lrows: four bits per load, the n of the unit it belongs to
     static_assert(LOADS <= 8 && OLOADS <= 8 && SKINNY_UNIT <= 16, "row numbers are packed four bits per load or store");
 #pragma unroll
     for (int u = 0; u < LOADS; ++u) {
-        const int id = lane + 64 * u, row = id / kc, col = id - row * kc;
+        const int id = lane + 64 * u;
         const bool ok = id < SKINNY_UNIT * kc;
+        // (row, col) = (n, chunk of its k); NFAST: (k, n)
+        const int row = NFAST ? id % SKINNY_UNIT : id / kc, col = NFAST ? id / SKINNY_UNIT : id - row * kc;
         have |= (ok ? 1u : 0u) << u;
         lrows |= (ok ? (uint32_t)row : 0u) << (4 * u);
-        goff[u] = ok ? row * s.b_in * (EB * NC) + col * 16 : 0;
-        loff[u] = ok ? row * PITCH + col * 16 : 0;
+        if constexpr (NFAST) {
+            goff[u] = ok ? (int32_t)(off_of(s.bk, col) * 16) + row * 16 : 0;
+            loff[u] = ok ? col * KPITCH + row * 16 : 0;
+        } else {
+            goff[u] = ok ? row * s.b_in * (EB * NC) + col * 16 : 0;
+            loff[u] = ok ? row * PITCH + col * 16 : 0;
+        }
     }
     // ---- where this lane reads its operands and writes its results
     int32_t roff[NBLK], ccol[NBLK] = {}, crow[MBM][4] = {};
 #pragma unroll
     for (int nb = 0; nb < NBLK; ++nb) {
         const int nloc = CX ? 8 * nb + (j >> 1) : j;
-        roff[nb] = nloc * PITCH + g * 16;
+        roff[nb] = NFAST ? g * KPITCH + nloc * 16 : nloc * PITCH + g * 16;
         if constexpr (!OUT_ROWS) ccol[nb] = nloc * s.c_in * NC + (CX ? p : 0);
     }
     if constexpr (!OUT_ROWS) {
@@ -276,7 +291,7 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_C
                 const bool kok = 4 * i + g < kc;
 #pragma unroll
                 for (int nb = 0; nb < NBLK; ++nb) {
-                    const chunk_t ch = *reinterpret_cast<const chunk_t*>(lds + roff[nb] + i * 64);
+                    const chunk_t ch = *reinterpret_cast<const chunk_t*>(lds + roff[nb] + i * (NFAST ? 4 * KPITCH : 64));
                     // the chunk as operands B'[Q c + q][column j]: the components themselves for real elements; for a
                     // complex element (br, bi) the even column of its pair takes (br, -bi), the odd one (bi, br)
                     R b[Q];
@@ -343,19 +358,19 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_C
     }
 }
 
-template <class R, bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM>
+template <class R, bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM, bool NFAST = false>
 void launch_variant(const gemm::SkinnyArgs& s, hipStream_t st) {
     typedef SkinnyCfg<R, KCM, MBM> Cfg;
-    constexpr int lds = (THREADS / 64) * (Cfg::WAVE_LDS + (OUT_ROWS ? Cfg::TILE_LDS : 0));
+    constexpr int lds = (THREADS / 64) * ((NFAST ? Cfg::WAVE_LDS_NFAST : Cfg::WAVE_LDS) + (OUT_ROWS ? Cfg::TILE_LDS : 0));
     static bool once = [] {   // (more than 64 KB of dynamic LDS has to be asked for once per kernel)
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<R, CX, RAGGED, OUT_ROWS, KCM, MBM>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<R, CX, RAGGED, OUT_ROWS, KCM, MBM, NFAST>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         return true;
     }();
     (void)once;
     const int64_t blocks_wanted = (s.units + THREADS / 64 - 1) / (THREADS / 64);
     const dim3 grid((uint32_t)std::min<int64_t>(blocks_wanted, 256 * Cfg::BLOCKS_PER_CU)), block(THREADS);
-    TFH_LAUNCH_TIMED((gemm_skinny_kernel<R, CX, RAGGED, OUT_ROWS, KCM, MBM>), grid, block, (size_t)lds, st, s);
+    TFH_LAUNCH_TIMED((gemm_skinny_kernel<R, CX, RAGGED, OUT_ROWS, KCM, MBM, NFAST>), grid, block, (size_t)lds, st, s);
 }
 
 template <class R, bool CX, bool RAGGED, bool OUT_ROWS>
@@ -380,6 +395,17 @@ void launch_typed(const gemm::SkinnyArgs& s, hipStream_t st) {
 }  // namespace
 
 void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
+    if (s.nfast) {   // complex128, C along n (the host's conditions)
+        const bool small = s.kc <= 8 && s.M <= 8;
+        if (s.tail != 0) {
+            if (small) launch_variant<double, true, true, false, 8, 1, true>(s, st);
+            else launch_variant<double, true, true, false, SKINNY_MAX_CHUNKS, SKINNY_MAX_M / 16, true>(s, st);
+        } else {
+            if (small) launch_variant<double, true, false, false, 8, 1, true>(s, st);
+            else launch_variant<double, true, false, false, SKINNY_MAX_CHUNKS, SKINNY_MAX_M / 16, true>(s, st);
+        }
+        return;
+    }
     switch (dtype) {
         case TFH_F32: launch_typed<float, false>(s, st); break;
         case TFH_F64: launch_typed<double, false>(s, st); break;
