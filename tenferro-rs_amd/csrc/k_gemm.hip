@@ -866,13 +866,19 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         for (auto& x : ax.N) skinny = skinny && whole_chunks(x.s[1]);
     }
     // The same operator on a leg that is not the long tensor's last: B is contiguous along n (as is C), its k strides
-    // are whatever they are.  complex128 only (one element per 16-byte chunk): the kernel parks a unit as [k][16 n].
+    // are whatever they are: the kernel parks a unit as [k][16 n].  The 16-byte loads run along n there: runs of n and
+    // the strides above them hold whole chunks.
     bool skinny_nfast = false;
-    if (!skinny && cxd && nb == 1 && !out_rows && M <= SKINNY_MAX_M && K <= SKINNY_MAX_CHUNKS && N >= 4096 && !b_kfast &&
+    if (!skinny && nb == 1 && !out_rows && M <= SKINNY_MAX_M && K <= SKINNY_MAX_CHUNKS && N >= 4096 && !b_kfast &&
         !ax.K.empty() && !ax.N.empty() && ax.N.back().s[1] == 1 && ax.N.back().s[2] == 1 && skinny_run_ok(ax.N.back().n)) {
         int64_t lo = 0, hi = 0;
         reach(ax.K, 1, lo, hi);
         skinny_nfast = std::max(-lo, hi) * (int64_t)eb < ((int64_t)1 << 30);
+        if (!cxd) {
+            skinny_nfast = skinny_nfast && (uintptr_t)b % 16 == 0 && whole_chunks(ax.N.back().n);
+            for (size_t d = 0; d + 1 < ax.N.size(); ++d) skinny_nfast = skinny_nfast && whole_chunks(ax.N[d].s[1]);
+            for (auto& x : ax.K) skinny_nfast = skinny_nfast && whole_chunks(x.s[1]);
+        }
         skinny = skinny_nfast;
     }
     int64_t inner_b = 0, inner_c = 0, skinny_upr = 1;

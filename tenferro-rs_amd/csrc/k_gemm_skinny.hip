@@ -37,6 +37,13 @@ using namespace gemm;
 template <class R> struct Chunk;
 template <> struct Chunk<double> { typedef double type __attribute__((ext_vector_type(2))); };
 template <> struct Chunk<float> { typedef float type __attribute__((ext_vector_type(4))); };
+// N components read from LDS at once
+template <class R, int N> struct Comps { typedef R type __attribute__((ext_vector_type(N))); };
+template <class R> struct Comps<R, 1> { typedef R type; };
+template <int Q, class V> __device__ __forceinline__ auto comp_of(const V& v, int q) {
+    if constexpr (Q == 1) return v;
+    else return v[q];
+}
 
 // Sizes of one instantiation: R the component type, KCM 16-byte chunks per row of B at most, MBM blocks of 16 rows of A
 // at most.  The general kernel (32 chunks, 2 blocks) keeps 64 VGPRs of A (doubles) and 32 of staging and runs two waves
@@ -54,9 +61,15 @@ struct SkinnyCfg {
     static constexpr int OUT_PITCH = 2 * 16 * MBM + Q;        // components per row of the transposed result tile (+16 bytes against bank conflicts)
     static constexpr int TILE_LDS = SKINNY_UNIT * OUT_PITCH * (int)sizeof(R);   // the transposed result tile of a wave: a region of its own
     static constexpr int BLOCKS_PER_CU = KCM <= 8 && MBM == 1 ? 4 : 2;
-    // B contiguous along n instead of k (complex128 only): the unit is parked as [k][16 n], one element per chunk
-    static constexpr int KPITCH = SKINNY_UNIT * 16 + 64;      // bytes per k row: lane groups g = 0..3 start 16 banks apart
-    static constexpr int WAVE_LDS_NFAST = MAX_KC * KPITCH;
+    // B contiguous along n instead of k: the unit is parked as [k][16 n], at most MAX_KC rows of k
+    template <bool CX> struct Nfast {
+        static constexpr int ELEM = (CX ? 2 : 1) * (int)sizeof(R);      // bytes per element
+        static constexpr int ROW_CHUNKS = SKINNY_UNIT * ELEM / 16;      // 16-byte chunks per k row
+        // bytes per k row: the lane groups g = 0..3 (four consecutive k) start on different banks
+        static constexpr int KPITCH = SKINNY_UNIT * ELEM + (ELEM == 4 ? 16 : 64);
+        static constexpr int WAVE_LDS = MAX_KC * KPITCH;
+        static constexpr int LOADS = (MAX_KC * ROW_CHUNKS + 63) / 64;
+    };
     static_assert(KCM % 4 == 0 && KCM <= SKINNY_MAX_CHUNKS && MBM * 16 <= SKINNY_MAX_M, "");
 };
 
@@ -69,10 +82,10 @@ __device__ __forceinline__ void wave_sync() {
 }
 
 // RAGGED: the innermost run of n holds no whole number of units (its own instantiation: the full-unit kernel carries
-// none of the per-unit predicates).  OUT_ROWS: C is contiguous along m (s.out_rows).  NFAST (complex128, C along n):
-// B is contiguous along n, not along k -- the operator acts on a leg that is not the tensor's last: a unit is then K
-// segments of 16 consecutive n (256 bytes each), parked as [k][n]; the operands come out of LDS by the same 16-byte
-// reads, from other addresses.
+// none of the per-unit predicates).  OUT_ROWS: C is contiguous along m (s.out_rows).  NFAST (C along n): B is
+// contiguous along n, not along k -- the operator acts on a leg that is not the tensor's last: a unit is then K
+// segments of 16 consecutive n, parked as [k][n]; an MFMA operand is one element of it (lane group g takes k = 4t + g
+// in step t), where the k-contiguous form reads a 16-byte chunk of one row for several steps.
 //
 // vmcnt counts loads and stores in one queue, in order, and the compiler waits for a register that was loaded in the
 // iteration before with vmcnt(0): whatever is stored shortly before that wait is waited for as well, acknowledgement
@@ -81,11 +94,13 @@ __device__ __forceinline__ void wave_sync() {
 template <class R, bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM, bool NFAST = false>
 __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_CU)) gemm_skinny_kernel(SkinnyArgs s) {
     typedef SkinnyCfg<R, KCM, MBM> Cfg;
-    static_assert(!NFAST || (CX && sizeof(R) == 8 && !OUT_ROWS), "one element per chunk");
+    static_assert(!NFAST || !OUT_ROWS, "");
+    typedef typename Cfg::template Nfast<CX> Nf;
     typedef typename Chunk<R>::type chunk_t;
     typedef typename Mfma<R>::acc_t acc_t;
-    constexpr int PITCH = Cfg::PITCH, WAVE_LDS = NFAST ? Cfg::WAVE_LDS_NFAST : Cfg::WAVE_LDS, LOADS = Cfg::LOADS, PAIRS = Cfg::PAIRS, Q = Cfg::Q;
-    constexpr int KPITCH = Cfg::KPITCH;
+    constexpr int PITCH = Cfg::PITCH, WAVE_LDS = NFAST ? Nf::WAVE_LDS : Cfg::WAVE_LDS, LOADS = NFAST ? Nf::LOADS : Cfg::LOADS;
+    constexpr int PAIRS = Cfg::PAIRS, Q = Cfg::Q, KPITCH = Nf::KPITCH;
+    constexpr int QB = NFAST ? (CX ? 2 : 1) : Q;   // components per LDS read = MFMA steps per read
     constexpr int OUT_PITCH = Cfg::OUT_PITCH, TILE_LDS = Cfg::TILE_LDS, OLOADS = Cfg::OLOADS;
     constexpr int NBLK = CX ? 2 : 1;   // column blocks (16 real columns each) per unit
     constexpr int NC = CX ? 2 : 1;     // components per element
@@ -95,11 +110,11 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_C
     unsigned char* lds = smem + wave * (WAVE_LDS + (OUT_ROWS ? TILE_LDS : 0));
     unsigned char* tile_lds = lds + WAVE_LDS;   // OUT_ROWS only
     const int g = lane >> 4, j = lane & 15, p = j & 1;
-    const int kc = s.kc, npair = (kc + 3) >> 2, nmb = MBM > 1 && s.M > 16 ? 2 : 1;
+    const int kc = s.kc, npair = ((NFAST ? s.K : kc) + 3) >> 2, nmb = MBM > 1 && s.M > 16 ? 2 : 1;
 
-    // ---- A as MFMA operands: a[mb][i][q] = A'[j + 16 mb][Q (4i + g) + q], zero outside the matrix.  A' is A itself for
+    // ---- A as MFMA operands: a[mb][i][q] = A'[j + 16 mb][QB (4i + g) + q], zero outside the matrix.  A' is A itself for
     // real elements and its real form for complex ones: A'[m][2k + part] = (re, im)[part] of A[m][k].
-    R a[MBM][PAIRS][Q];
+    R a[MBM][PAIRS][QB];
     {
         const R* Ad = reinterpret_cast<const R*>(s.A);
 #pragma unroll
@@ -108,8 +123,8 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_C
             for (int i = 0; i < PAIRS; ++i) {
                 const int m = j + 16 * mb, c = 4 * i + g;
 #pragma unroll
-                for (int q = 0; q < Q; ++q) {
-                    const int kk = Q * c + q;               // index into the real form
+                for (int q = 0; q < QB; ++q) {
+                    const int kk = QB * c + q;              // index into the real form
                     const int k = kk / NC, part = kk % NC;
                     R x = 0;
                     if (m < s.M && k < s.K) {
@@ -128,17 +143,23 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_C
 #pragma unroll
     for (int u = 0; u < LOADS; ++u) {
         const int id = lane + 64 * u;
+        if constexpr (NFAST) {
+            // chunk id -> (k, chunk of the 16 n); the first n of the chunk goes into lrows
+            const bool ok = id < s.K * Nf::ROW_CHUNKS;
+            const int krow = id / Nf::ROW_CHUNKS, ch = id % Nf::ROW_CHUNKS;
+            have |= (ok ? 1u : 0u) << u;
+            lrows |= (ok ? (uint32_t)(ch * (16 / Nf::ELEM)) : 0u) << (4 * u);
+            goff[u] = ok ? (int32_t)(off_of(s.bk, krow) * Nf::ELEM) + ch * 16 : 0;
+            loff[u] = ok ? krow * KPITCH + ch * 16 : 0;
+        } else {
         const bool ok = id < SKINNY_UNIT * kc;
-        // (row, col) = (n, chunk of its k); NFAST: (k, n)
-        const int row = NFAST ? id % SKINNY_UNIT : id / kc, col = NFAST ? id / SKINNY_UNIT : id - row * kc;
+        const int row = id / kc, col = id - row * kc;   // (n, chunk of its k)
         have |= (ok ? 1u : 0u) << u;
         lrows |= (ok ? (uint32_t)row : 0u) << (4 * u);
-        if constexpr (NFAST) {
-            goff[u] = ok ? (int32_t)(off_of(s.bk, col) * 16) + row * 16 : 0;
-            loff[u] = ok ? col * KPITCH + row * 16 : 0;
-        } else {
+        {
             goff[u] = ok ? row * s.b_in * (EB * NC) + col * 16 : 0;
             loff[u] = ok ? row * PITCH + col * 16 : 0;
+        }
         }
     }
     // ---- where this lane reads its operands and writes its results
@@ -146,7 +167,7 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_C
 #pragma unroll
     for (int nb = 0; nb < NBLK; ++nb) {
         const int nloc = CX ? 8 * nb + (j >> 1) : j;
-        roff[nb] = NFAST ? g * KPITCH + nloc * 16 : nloc * PITCH + g * 16;
+        roff[nb] = NFAST ? g * KPITCH + nloc * Nf::ELEM : nloc * PITCH + g * 16;
         if constexpr (!OUT_ROWS) ccol[nb] = nloc * s.c_in * NC + (CX ? p : 0);
     }
     if constexpr (!OUT_ROWS) {
@@ -288,29 +309,30 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_C
 #pragma unroll
         for (int i = 0; i < PAIRS; ++i) {
             if (i < npair) {
-                const bool kok = 4 * i + g < kc;
+                const bool kok = 4 * i + g < (NFAST ? s.K : kc);
 #pragma unroll
                 for (int nb = 0; nb < NBLK; ++nb) {
-                    const chunk_t ch = *reinterpret_cast<const chunk_t*>(lds + roff[nb] + i * (NFAST ? 4 * KPITCH : 64));
+                    typedef typename Comps<R, QB>::type read_t;
+                    const read_t ch = *reinterpret_cast<const read_t*>(lds + roff[nb] + i * (NFAST ? 4 * KPITCH : 64));
                     // the chunk as operands B'[Q c + q][column j]: the components themselves for real elements; for a
                     // complex element (br, bi) the even column of its pair takes (br, -bi), the odd one (bi, br)
-                    R b[Q];
+                    R b[QB];
 #pragma unroll
-                    for (int q = 0; q < Q; ++q) {
+                    for (int q = 0; q < QB; ++q) {
                         if constexpr (CX) {
                             const R re = ch[q & ~1], im = s.conj_b ? -ch[q | 1] : ch[q | 1];
                             b[q] = (q & 1) ? (p ? re : -im) : (p ? im : re);
                         } else {
-                            b[q] = ch[q];
+                            b[q] = comp_of<QB>(ch, q);
                         }
                         b[q] = kok ? b[q] : R(0);   // a row of B may be shorter than the LDS row: never multiply what was not loaded
                     }
 #pragma unroll
-                    for (int q = 0; q < Q; ++q) acc[0][nb] = Mfma<R>::run(a[0][i][q], b[q], acc[0][nb]);
+                    for (int q = 0; q < QB; ++q) acc[0][nb] = Mfma<R>::run(a[0][i][q], b[q], acc[0][nb]);
                     if constexpr (MBM > 1)
                         if (nmb > 1) {
 #pragma unroll
-                            for (int q = 0; q < Q; ++q) acc[1][nb] = Mfma<R>::run(a[1][i][q], b[q], acc[1][nb]);
+                            for (int q = 0; q < QB; ++q) acc[1][nb] = Mfma<R>::run(a[1][i][q], b[q], acc[1][nb]);
                         }
                 }
             }
@@ -361,7 +383,7 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_C
 template <class R, bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM, bool NFAST = false>
 void launch_variant(const gemm::SkinnyArgs& s, hipStream_t st) {
     typedef SkinnyCfg<R, KCM, MBM> Cfg;
-    constexpr int lds = (THREADS / 64) * ((NFAST ? Cfg::WAVE_LDS_NFAST : Cfg::WAVE_LDS) + (OUT_ROWS ? Cfg::TILE_LDS : 0));
+    constexpr int lds = (THREADS / 64) * ((NFAST ? Cfg::template Nfast<CX>::WAVE_LDS : Cfg::WAVE_LDS) + (OUT_ROWS ? Cfg::TILE_LDS : 0));
     static bool once = [] {   // (more than 64 KB of dynamic LDS has to be asked for once per kernel)
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_kernel<R, CX, RAGGED, OUT_ROWS, KCM, MBM, NFAST>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -392,17 +414,25 @@ void launch_typed(const gemm::SkinnyArgs& s, hipStream_t st) {
     }
 }
 
-}  // namespace
+template <class R, bool CX>
+void launch_nfast(const gemm::SkinnyArgs& s, hipStream_t st) {
+    const bool small = s.K <= 8 && s.M <= (CX ? 8 : 16);
+    if (s.tail != 0) {
+        if (small) launch_variant<R, CX, true, false, 8, 1, true>(s, st);
+        else launch_variant<R, CX, true, false, SKINNY_MAX_CHUNKS, SKINNY_MAX_M / 16, true>(s, st);
+    } else {
+        if (small) launch_variant<R, CX, false, false, 8, 1, true>(s, st);
+        else launch_variant<R, CX, false, false, SKINNY_MAX_CHUNKS, SKINNY_MAX_M / 16, true>(s, st);
+    }
+}
 
-void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
-    if (s.nfast) {   // complex128, C along n (the host's conditions)
-        const bool small = s.kc <= 8 && s.M <= 8;
-        if (s.tail != 0) {
-            if (small) launch_variant<double, true, true, false, 8, 1, true>(s, st);
-            else launch_variant<double, true, true, false, SKINNY_MAX_CHUNKS, SKINNY_MAX_M / 16, true>(s, st);
-        } else {
-            if (small) launch_variant<double, true, false, false, 8, 1, true>(s, st);
-            else launch_variant<double, true, false, false, SKINNY_MAX_CHUNKS, SKINNY_MAX_M / 16, true>(s, st);
+void launch_gemm_skinny_impl(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
+    if (s.nfast) {   // C along n, at most SKINNY_MAX_CHUNKS k (the host's conditions)
+        switch (dtype) {
+            case TFH_F32: launch_nfast<float, false>(s, st); break;
+            case TFH_F64: launch_nfast<double, false>(s, st); break;
+            case TFH_C64: launch_nfast<float, true>(s, st); break;
+            default: launch_nfast<double, true>(s, st); break;
         }
         return;
     }
@@ -413,5 +443,9 @@ void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
         default: launch_typed<double, true>(s, st); break;
     }
 }
+
+}  // namespace
+
+void launch_gemm_skinny(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) { launch_gemm_skinny_impl(dtype, s, st); }
 
 }  // namespace tfh

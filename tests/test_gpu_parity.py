@@ -1975,26 +1975,30 @@ def test_contract_tiny_operator_on_the_last_leg_of_a_long_tensor(tf, oracle, dty
         assert relerr(dout.to_numpy(), ref) < TOL[dtype], (alpha, beta)
 
 
+@pytest.mark.parametrize("dtype", ALL)
 @pytest.mark.parametrize("a_,k,m,c", [(64, 16, 16, 1024), (33, 12, 8, 2000), (3, 20, 12, 30001), (100, 32, 20, 777), (9, 32, 32, 4000),
-                                      (6, 3, 5, 48 * 16)])
-def test_contract_small_operator_on_a_middle_leg_complex128(tf, oracle, a_, k, m, c):
+                                      (6, 3, 5, 48 * 16), (5, 10, 9, 30002)])
+def test_contract_small_operator_on_a_middle_leg(tf, oracle, dtype, a_, k, m, c):
     # T[a, k, c] . W[m, k] -> out[a, m, c]: the operator acts on a leg that is not the last, so the long operand is
-    # contiguous along n = c like the output, and its k is strided.  The streaming kernel parks such a unit as [k][16 c]
-    # (complex128: one element per 16-byte chunk).  Whole and partly filled last units, several units per wave (30001),
-    # general alpha / beta; then k split over two modes that the operator holds in the other order, and c reversed.
-    dtype = np.complex128
+    # contiguous along n = c like the output, and its k is strided.  The streaming kernel parks such a unit as [k][16 c];
+    # its 16-byte loads run along c, so the runs of c must hold whole chunks (any c for complex128, even c for f64 and
+    # complex64, multiples of 4 for f32), otherwise the tiled kernels take the product.  Whole and partly filled last
+    # units, several units per wave (30001, 30002), general alpha / beta; then k split over two modes that the operator
+    # holds in the other order, and a view of every second a with a conjugated operator.
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    streamed = whole_chunks(dtype, c)
     rng = np.random.default_rng(97)
     t = rand(rng, (a_, k, c), dtype)
     w = rand(rng, (m, k), dtype)
     out0 = rand(rng, (a_, m, c), dtype)
-    for alpha, beta in [(1.0, 0.0), (0.5 - 2j, 1.5 + 1j)]:
+    for alpha, beta in [(1.0, 0.0), ((0.5 - 2j, 1.5 + 1j) if cplx else (0.5, -1.5))]:
         ref = out0.copy()
         oracle.contract(t, lab("akc"), w, lab("mk"), ref, lab("amc"), alpha=alpha, beta=beta)
         dout = dev(tf, out0)
         plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("akc"), lab("mk"), lab("amc")), [t.shape, w.shape, ref.shape])
         tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
-        assert "gemm_skinny_kernel" in tf.last_kernel() and ", true>" in tf.last_kernel(), tf.last_kernel()
-        assert relerr(dout.to_numpy(), ref) < 1e-12, (alpha, beta)
+        assert ("gemm_skinny_kernel" in tf.last_kernel() and ", true>" in tf.last_kernel()) == streamed, tf.last_kernel()
+        assert relerr(dout.to_numpy(), ref) < TOL[dtype], (alpha, beta)
     if k % 4 == 0:
         s_, w_ = 4, k // 4
         t4 = rand(rng, (a_, s_, w_, c), dtype)
@@ -2004,8 +2008,8 @@ def test_contract_small_operator_on_a_middle_leg_complex128(tf, oracle, a_, k, m
         out = tf.Tensor.empty([a_, m, c], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
         plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("aswc"), lab("wms"), lab("amc")), [t4.shape, wop.shape, ref.shape])
         tf.HipBackend.execute(plan, 1.0, [dev(tf, t4), dev(tf, wop)], 0.0, out)
-        assert "gemm_skinny_kernel" in tf.last_kernel(), tf.last_kernel()
-        assert relerr(out.to_numpy(), ref) < 1e-12
+        assert ("gemm_skinny_kernel" in tf.last_kernel()) == streamed, tf.last_kernel()
+        assert relerr(out.to_numpy(), ref) < TOL[dtype]
     # a view of every second a and a conjugated operator
     tv = t[::2]
     ref = np.empty((tv.shape[0], m, c), dtype)
@@ -2013,7 +2017,7 @@ def test_contract_small_operator_on_a_middle_leg_complex128(tf, oracle, a_, k, m
     out = tf.Tensor.empty(list(ref.shape), tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
     plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("akc"), lab("mk"), lab("amc")), [tv.shape, w.shape, ref.shape])
     tf.HipBackend.execute(plan, 1.0, [dev(tf, tv), dev(tf, w).conj_on_load()], 0.0, out)
-    assert relerr(out.to_numpy(), ref) < 1e-12
+    assert relerr(out.to_numpy(), ref) < TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", ALL)
