@@ -24,6 +24,7 @@ struct TinyArgs {
     void* C;
     int32_t ms, ks;  // free and contracted extent of the operator (fused), each <= TINY_MAX
     int32_t nax, use_beta;
+    int32_t rows;                                          // C[n][m] with the rows m packed: results leave through an LDS tile
     int64_t total;                                         // vectors of the long free index
     int64_t next[TINY_NAX], nst[TINY_NAX], nsc[TINY_NAX];  // its axes, innermost first: extent (axis 0 in vectors), T and C strides
     int64_t s_off[TINY_MAX * TINY_MAX];                    // element offset of S[m][k]
@@ -37,9 +38,17 @@ template <> struct Raw<8> { typedef uint32_t type __attribute__((ext_vector_type
 template <> struct Raw<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
 
 // R: component type; CX: complex elements; VEC: elements per access; KM: unroll bound of both small extents.
-template <class R, bool CX, int VEC, int KM>
+// ROWS (VEC = 1): the output is C[n][m] with the operator's rows m adjacent and packed (the acted-on leg comes last in
+// the result).  A thread's ms results are then ms adjacent elements and neighbouring lanes are ms elements apart: stored
+// directly, every store instruction touches 64 separate lines.  The block's 256 x ms results are one contiguous piece
+// of C instead: they go through an LDS tile and leave as 16-byte stores in address order.
+template <class R, bool CX, int VEC, int KM, bool ROWS = false>
 __global__ void __launch_bounds__(TINY_THREADS) tiny_operator_kernel(TinyArgs a) {
     constexpr int NC = CX ? 2 : 1, W = VEC * NC;   // components per element, per access
+    static_assert(!ROWS || VEC == 1, "");
+    constexpr int ES = NC * (int)sizeof(R);         // bytes per element
+    constexpr int TILE_PITCH = KM * ES + 16;        // bytes per thread's row of the tile (+16: lanes on different banks)
+    __shared__ __align__(16) unsigned char tile[ROWS ? TINY_THREADS * TILE_PITCH : 16];
     typedef typename Raw<W * sizeof(R)>::type RawT;
     struct alignas(W * sizeof(R)) Vals { R v[W]; };
     __shared__ R s_op[TINY_MAX * TINY_MAX * NC];
@@ -89,6 +98,10 @@ __global__ void __launch_bounds__(TINY_THREADS) tiny_operator_kernel(TinyArgs a)
                     }
                 }
             }
+        if constexpr (ROWS) {
+            *reinterpret_cast<Vals*>(tile + tid * TILE_PITCH + m * ES) = acc;
+            continue;
+        }
         RawT* dst = reinterpret_cast<RawT*>(C + a.c_moff[m] * NC);
         Vals out, old;
         if (a.use_beta) old = __builtin_bit_cast(Vals, *dst);
@@ -108,6 +121,37 @@ __global__ void __launch_bounds__(TINY_THREADS) tiny_operator_kernel(TinyArgs a)
         }
         __builtin_nontemporal_store(__builtin_bit_cast(RawT, out), dst);
     }
+    if constexpr (ROWS) {
+        __syncthreads();
+        // the block's piece of C starts at thread 0's first element; 16-byte pieces of it in address order
+        constexpr int PW = 16 / (int)sizeof(R);   // components per piece
+        typedef typename Raw<16>::type Raw16;
+        struct alignas(16) Piece { R v[PW]; };
+        unsigned char* Cblk = reinterpret_cast<unsigned char*>(C) - (size_t)tid * a.ms * ES;
+        const int row_bytes = a.ms * ES, pieces = TINY_THREADS * row_bytes / 16;
+        for (int pc = tid; pc < pieces; pc += TINY_THREADS) {
+            const int byte = pc * 16, row = byte / row_bytes, within = byte - row * row_bytes;
+            const Piece x = *reinterpret_cast<const Piece*>(tile + row * TILE_PITCH + within);
+            Raw16* dst = reinterpret_cast<Raw16*>(Cblk + byte);
+            Piece out, old;
+            if (a.use_beta) old = __builtin_bit_cast(Piece, *dst);
+#pragma unroll
+            for (int e = 0; e < PW; e += NC) {
+                if constexpr (CX) {
+                    out.v[e] = ar * x.v[e] - ai * x.v[e + 1];
+                    out.v[e + 1] = ar * x.v[e + 1] + ai * x.v[e];
+                    if (a.use_beta) {
+                        out.v[e] += br * old.v[e] - bi * old.v[e + 1];
+                        out.v[e + 1] += br * old.v[e + 1] + bi * old.v[e];
+                    }
+                } else {
+                    out.v[e] = ar * x.v[e];
+                    if (a.use_beta) out.v[e] += br * old.v[e];
+                }
+            }
+            __builtin_nontemporal_store(__builtin_bit_cast(Raw16, out), dst);
+        }
+    }
 }
 
 template <class R, bool CX, int VEC>
@@ -119,7 +163,10 @@ void launch_km(const TinyArgs& ta, int km, dim3 grid, hipStream_t st) {
 template <class R, bool CX>
 void launch_vec(const TinyArgs& ta, bool vec, int km, dim3 grid, hipStream_t st) {
     constexpr int VMAX = 16 / (int)(sizeof(R) * (CX ? 2 : 1));
-    if (vec && VMAX > 1) launch_km<R, CX, VMAX>(ta, km, grid, st);
+    if (ta.rows) {
+        if (km <= 4) TFH_LAUNCH_TIMED((tiny_operator_kernel<R, CX, 1, 4, true>), grid, dim3(TINY_THREADS), 0, st, ta);
+        else TFH_LAUNCH_TIMED((tiny_operator_kernel<R, CX, 1, 8, true>), grid, dim3(TINY_THREADS), 0, st, ta);
+    } else if (vec && VMAX > 1) launch_km<R, CX, VMAX>(ta, km, grid, st);
     else launch_km<R, CX, 1>(ta, km, grid, st);
 }
 
@@ -184,6 +231,12 @@ bool try_tiny_operator(int dtype, const void* a, const void* b, void* c, const C
     for (size_t d = 1; d < nx.size(); ++d) vec = vec && nx[d].s[0] % vmax == 0 && nx[d].s[1] % vmax == 0;
     for (int k = 0; k < ta.ks; ++k) vec = vec && ta.t_koff[k] % vmax == 0;
     for (int m = 0; m < ta.ms; ++m) vec = vec && ta.c_moff[m] % vmax == 0;
+    // C[n][m] with packed rows of m: whole blocks of 256 n inside the innermost long axis, rows of whole 16-byte pieces
+    bool rows = !vec && ta.ms >= 3 && nx[0].s[1] == ta.ms && nx[0].n % TINY_THREADS == 0 && (uintptr_t)c % 16 == 0 &&
+                (int64_t)ta.ms * ebytes % 16 == 0;
+    for (int m = 0; m < ta.ms; ++m) rows = rows && ta.c_moff[m] == m;
+    for (size_t d = 1; d < nx.size(); ++d) rows = rows && nx[d].s[1] * ebytes % 16 == 0;
+    ta.rows = rows;
     const int v = vec ? vmax : 1;
     ta.nax = (int32_t)nx.size();
     ta.total = 1;

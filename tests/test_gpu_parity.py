@@ -2021,6 +2021,33 @@ def test_contract_small_operator_on_a_middle_leg(tf, oracle, dtype, a_, k, m, c)
 
 
 @pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("a_,k,m,c", [(64, 8, 8, 1024), (300, 2, 8, 256), (33, 3, 4, 2048), (5, 8, 6, 25600), (70, 4, 3, 1024), (66, 8, 8, 1000)])
+def test_contract_tiny_operator_with_the_acted_leg_moved_last(tf, oracle, dtype, a_, k, m, c):
+    # T[a, k, c] . W[m, k] -> out[a, c, m]: a gate on a middle leg whose result carries that leg last.  A thread of the
+    # tiny-operator kernel then holds m adjacent output elements and its neighbours are m elements away; where the rows
+    # of m are packed, fill whole 16-byte pieces and the innermost long axis holds whole blocks of 256, the block's
+    # results leave through an LDS tile in address order (the kernel's last template argument); elsewhere the direct
+    # stores remain (c = 1000; three f64 per row) or another kernel takes the product.
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    rng = np.random.default_rng(98)
+    t = rand(rng, (a_, k, c), dtype)
+    w = rand(rng, (m, k), dtype)
+    out0 = rand(rng, (a_, c, m), dtype)
+    tiled = m >= 3 and c % 256 == 0 and whole_chunks(dtype, m)
+    for alpha, beta in [(1.0, 0.0), ((0.5 - 2j, 1.5 + 1j) if cplx else (0.5, -1.5))]:
+        ref = out0.copy()
+        oracle.contract(t, lab("akc"), w, lab("mk"), ref, lab("acm"), alpha=alpha, beta=beta)
+        dout = dev(tf, out0)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("akc"), lab("mk"), lab("acm")), [t.shape, w.shape, ref.shape])
+        tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
+        if "tiny_operator_kernel" in tf.last_kernel():
+            assert tf.last_kernel().rstrip(")").endswith(", true>") == tiled, tf.last_kernel()
+        else:
+            assert not tiled, tf.last_kernel()
+        assert relerr(dout.to_numpy(), ref) < TOL[dtype], (alpha, beta)
+
+
+@pytest.mark.parametrize("dtype", ALL)
 def test_reduce_rows_and_inner_axes_take_the_butterfly_fold(tf, oracle, dtype):
     # sums over the contiguous axis (row sums) and over an inner axis next to a short kept one: nothing is left to loop
     # over, so a block handles eight outputs per lane group and folds them with the transposing butterfly.  Exact
