@@ -850,9 +850,36 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
             out_rows = true;
         }
     }
+    // ... and with the long operand contiguous along its free index instead of k (the operator on a leg that is not the
+    // last, the result carrying that leg last): the same exchange; the kernel parks [k][16 n] and writes through the tile.
+    bool out_rows_nfast = false;
+    if (!out_rows && nb == 1 && N <= SKINNY_MAX_M && M >= 4096 && K <= SKINNY_MAX_CHUNKS && !a_kfast && !ax.K.empty() &&
+        ax.N.size() == 1 && ax.N[0].s[2] == 1 && !ax.M.empty() && ax.M.back().s[0] == 1 && skinny_run_ok(ax.M.back().n) &&
+        (cxd || (whole_chunks(N) && (uintptr_t)c % 16 == 0 && (uintptr_t)a % 16 == 0 && whole_chunks(ax.M.back().n)))) {
+        bool ok = true;
+        if (!cxd) {
+            for (size_t d = 0; d + 1 < ax.M.size(); ++d) ok = ok && whole_chunks(ax.M[d].s[0]);
+            for (auto& x : ax.M) ok = ok && whole_chunks(x.s[2]);
+            for (auto& x : ax.K) ok = ok && whole_chunks(x.s[0]);
+        }
+        int64_t lo = 0, hi = 0;
+        reach(ax.K, 0, lo, hi);
+        ok = ok && std::max(-lo, hi) * (int64_t)eb < ((int64_t)1 << 30) &&
+             std::llabs(ax.M.back().s[2]) * SKINNY_UNIT * (int64_t)eb < ((int64_t)1 << 31);
+        if (ok) {
+            std::swap(a, b);
+            std::swap(conj_a, conj_b);
+            std::swap(ax.M, ax.N);
+            std::swap(M, N);
+            std::swap(a_kfast, b_kfast);
+            for (auto* grp : {&ax.batch, &ax.M, &ax.N, &ax.K})
+                for (auto& x : *grp) std::swap(x.s[0], x.s[1]);
+            out_rows = out_rows_nfast = true;
+        }
+    }
     const bool k_rows_b = out_rows || k_by_b;   // the k modes are in the memory order of the (possibly exchanged) B
     bool skinny = nb == 1 && M <= SKINNY_MAX_M && K * sk_nc <= SKINNY_MAX_CHUNKS * sk_q && N >= 4096 &&
-                  b_kfast && !ax.K.empty() && k_rows_b && !ax.N.empty() &&
+                  b_kfast && !out_rows_nfast && !ax.K.empty() && k_rows_b && !ax.N.empty() &&
                   skinny_run_ok(ax.N.back().n) && (out_rows || ax.N.back().s[2] == 1);
     if (skinny) {   // a row of B is one contiguous run of k (A's k order is free: it goes through the k table)
         int64_t expect = 1;
@@ -881,6 +908,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         }
         skinny = skinny_nfast;
     }
+    if (out_rows_nfast) skinny = skinny_nfast = true;
     int64_t inner_b = 0, inner_c = 0, skinny_upr = 1;
     int skinny_tail = 0;
     if (skinny) {

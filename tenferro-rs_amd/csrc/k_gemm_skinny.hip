@@ -82,7 +82,7 @@ __device__ __forceinline__ void wave_sync() {
 }
 
 // RAGGED: the innermost run of n holds no whole number of units (its own instantiation: the full-unit kernel carries
-// none of the per-unit predicates).  OUT_ROWS: C is contiguous along m (s.out_rows).  NFAST (C along n): B is
+// none of the per-unit predicates).  OUT_ROWS: C is contiguous along m (s.out_rows).  NFAST (either output): B is
 // contiguous along n, not along k -- the operator acts on a leg that is not the tensor's last: a unit is then K
 // segments of 16 consecutive n, parked as [k][n]; an MFMA operand is one element of it (lane group g takes k = 4t + g
 // in step t), where the k-contiguous form reads a 16-byte chunk of one row for several steps.
@@ -94,7 +94,6 @@ __device__ __forceinline__ void wave_sync() {
 template <class R, bool CX, bool RAGGED, bool OUT_ROWS, int KCM, int MBM, bool NFAST = false>
 __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_CU)) gemm_skinny_kernel(SkinnyArgs s) {
     typedef SkinnyCfg<R, KCM, MBM> Cfg;
-    static_assert(!NFAST || !OUT_ROWS, "");
     typedef typename Cfg::template Nfast<CX> Nf;
     typedef typename Chunk<R>::type chunk_t;
     typedef typename Mfma<R>::acc_t acc_t;
@@ -414,20 +413,26 @@ void launch_typed(const gemm::SkinnyArgs& s, hipStream_t st) {
     }
 }
 
+template <class R, bool CX, bool RAGGED, bool OUT_ROWS>
+void launch_nfast_sized(const gemm::SkinnyArgs& s, hipStream_t st) {
+    if (s.K <= 8 && s.M <= (CX ? 8 : 16)) launch_variant<R, CX, RAGGED, OUT_ROWS, 8, 1, true>(s, st);
+    else launch_variant<R, CX, RAGGED, OUT_ROWS, SKINNY_MAX_CHUNKS, SKINNY_MAX_M / 16, true>(s, st);
+}
+
 template <class R, bool CX>
 void launch_nfast(const gemm::SkinnyArgs& s, hipStream_t st) {
-    const bool small = s.K <= 8 && s.M <= (CX ? 8 : 16);
-    if (s.tail != 0) {
-        if (small) launch_variant<R, CX, true, false, 8, 1, true>(s, st);
-        else launch_variant<R, CX, true, false, SKINNY_MAX_CHUNKS, SKINNY_MAX_M / 16, true>(s, st);
+    const bool ragged = s.tail != 0, rows = s.out_rows != 0;
+    if (ragged) {
+        if (rows) launch_nfast_sized<R, CX, true, true>(s, st);
+        else launch_nfast_sized<R, CX, true, false>(s, st);
     } else {
-        if (small) launch_variant<R, CX, false, false, 8, 1, true>(s, st);
-        else launch_variant<R, CX, false, false, SKINNY_MAX_CHUNKS, SKINNY_MAX_M / 16, true>(s, st);
+        if (rows) launch_nfast_sized<R, CX, false, true>(s, st);
+        else launch_nfast_sized<R, CX, false, false>(s, st);
     }
 }
 
 void launch_gemm_skinny_impl(int dtype, const gemm::SkinnyArgs& s, hipStream_t st) {
-    if (s.nfast) {   // C along n, at most SKINNY_MAX_CHUNKS k (the host's conditions)
+    if (s.nfast) {   // at most SKINNY_MAX_CHUNKS k (the host's conditions)
         switch (dtype) {
             case TFH_F32: launch_nfast<float, false>(s, st); break;
             case TFH_F64: launch_nfast<double, false>(s, st); break;

@@ -2048,6 +2048,29 @@ def test_contract_tiny_operator_with_the_acted_leg_moved_last(tf, oracle, dtype,
 
 
 @pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("a_,k,m,c", [(64, 16, 16, 1024), (30, 12, 32, 2000), (3, 20, 12, 30001), (100, 32, 20, 776), (9, 32, 32, 4000),
+                                      (5, 10, 9, 30002), (64, 8, 8, 1000)])
+def test_contract_small_operator_on_a_middle_leg_with_that_leg_moved_last(tf, oracle, dtype, a_, k, m, c):
+    # T[a, k, c] . W[m, k] -> out[a, c, m]: the long operand contiguous along c, the result along the operator's rows.
+    # The streaming kernel parks [k][16 c] and writes through its transposing tile; runs of c and rows of m must hold
+    # whole 16-byte chunks (any for complex128).
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    streamed = whole_chunks(dtype, c) and whole_chunks(dtype, m)
+    rng = np.random.default_rng(99)
+    t = rand(rng, (a_, k, c), dtype)
+    w = rand(rng, (m, k), dtype)
+    out0 = rand(rng, (a_, c, m), dtype)
+    for alpha, beta in [(1.0, 0.0), ((0.5 - 2j, 1.5 + 1j) if cplx else (0.5, -1.5))]:
+        ref = out0.copy()
+        oracle.contract(t, lab("akc"), w, lab("mk"), ref, lab("acm"), alpha=alpha, beta=beta)
+        dout = dev(tf, out0)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("akc"), lab("mk"), lab("acm")), [t.shape, w.shape, ref.shape])
+        tf.HipBackend.execute(plan, alpha, [dev(tf, t), dev(tf, w)], beta, dout)
+        assert ("gemm_skinny_kernel" in tf.last_kernel() and ", true>" in tf.last_kernel()) == streamed, tf.last_kernel()
+        assert relerr(dout.to_numpy(), ref) < TOL[dtype], (alpha, beta)
+
+
+@pytest.mark.parametrize("dtype", ALL)
 def test_reduce_rows_and_inner_axes_take_the_butterfly_fold(tf, oracle, dtype):
     # sums over the contiguous axis (row sums) and over an inner axis next to a short kept one: nothing is left to loop
     # over, so a block handles eight outputs per lane group and folds them with the transposing butterfly.  Exact
