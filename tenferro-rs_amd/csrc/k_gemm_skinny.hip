@@ -1,6 +1,7 @@
 // k_gemm_skinny.hip -- contraction with a small left operand: C[m, n] = alpha * sum_k A[m, k] * B[n, k] + beta * C
-// with at most 32 rows m, at most 64 real k, and a long n (the "apply a small operator to every fibre of a large
-// tensor" step of a tensor-network contraction, PrimDescriptor::Contract, tenferro-prims/src/lib.rs:227-239).
+// with at most 32 rows m, at most 32 16-byte chunks of k (64 real k in double, 128 in single precision), and a long n
+// (the "apply a small operator to every fibre of a large tensor" step of a tensor-network contraction,
+// PrimDescriptor::Contract, tenferro-prims/src/lib.rs:227-239).  All four dtypes.
 //
 // Such a product is bound by HBM (B is read once, C written once, a few flops per byte), and a tiled GEMM kernel
 // spends it in per-tile latency: with so little k there is no main loop to hide the loads and the stores behind.
@@ -11,7 +12,8 @@
 // MFMAs of the next unit.  Waves never wait for each other (no block barrier).
 //
 // v_mfma_f64_16x16x4_f64: lane l = 16 g + j feeds A'[row j][k' = 4 step + g] and B'[k' = 4 step + g][col j] and
-// receives C'[row g + 4 r][col j] in accumulator register r.  One 16-byte chunk of B serves two steps:
+// receives C'[row g + 4 r][col j] in accumulator register r (v_mfma_f32_16x16x4_f32: row 4 g + r).  One 16-byte chunk
+// of B serves two steps in double precision (four in single: twice the components per chunk, otherwise alike):
 //   complex128: chunk c of row n is the element B[n][k = c] = (br, bi).  Real form of the product: A'[m][2k + q] =
 //     (re, im)[q] of A[m][k]; B'[2k][2n] = br, B'[2k+1][2n] = -bi, B'[2k][2n+1] = bi, B'[2k+1][2n+1] = br; C'[m][2n + p]
 //     is the interleaved complex C.  Column j is (n = j / 2, p = j % 2): the lane turns its chunk into the operands
@@ -19,6 +21,9 @@
 //   f64: chunk c of row n holds B[n][2c], B[n][2c+1], the operands of q = 0, 1.  Column j is n.  One column block.
 // Pair i of steps (2i, 2i+1) uses chunk 4i + g in lane group g: a permutation of k shared by A' and B', harmless
 // under the sum.  HBM-bound: algorithmic bytes = sizeof(B) + sizeof(C) (+ C again when beta != 0).
+//
+// B may also be contiguous along n instead of k (the operator acts on a leg that is not the tensor's last): the unit
+// is then parked as [k][16 n] and an MFMA operand is one element of the park (see NFAST below).
 //
 // C may be contiguous along n (each lane stores its accumulators: 128-byte segments per row of C) or along m (the
 // other orientation of the same product, C[n][m]): then the unit's 16 x M results are transposed through an LDS tile
