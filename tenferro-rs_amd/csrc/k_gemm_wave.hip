@@ -73,6 +73,9 @@ __global__ void __launch_bounds__(THREADS) gemm_wave_kernel(GemmArgs g, int64_t 
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int jb = 0; jb < 2; ++jb) acc[i][jb] = acc_t{0, 0, 0, 0};
+    // a problem of at most 16 rows or 16 real columns leaves the second block of that side empty: its MFMAs are skipped
+    // (the same for every lane of the wave; 8x8x8 f64 issues four of the sixteen)
+    const bool rows2 = m0 + 16 < M, cols2 = n0r + 16 < NR;
 
     // four k steps (16 real k) per iteration: their loads are issued together, then the sixteen MFMAs
     for (int64_t k0 = 0; k0 < KR; k0 += 16) {
@@ -110,7 +113,8 @@ __global__ void __launch_bounds__(THREADS) gemm_wave_kernel(GemmArgs g, int64_t 
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int jb = 0; jb < 2; ++jb) acc[i][jb] = Mfma<R>::run(av[u][i], bv[u][jb], acc[i][jb]);
+                for (int jb = 0; jb < 2; ++jb)
+                    if ((i == 0 || rows2) && (jb == 0 || cols2)) acc[i][jb] = Mfma<R>::run(av[u][i], bv[u][jb], acc[i][jb]);
     }
 
     // ---- epilogue: the same arithmetic as the tiled kernels; real column n0r + 16 jb + j
