@@ -82,6 +82,7 @@ __global__ void __launch_bounds__(THREADS) gemm_wave_kernel(GemmArgs g, int64_t 
         R av[4][2], bv[4][2];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
+            if (k0 + 4 * u >= KR) break;   // (the same for every lane: a short k ends the iteration early)
             const int64_t kk = k0 + 4 * u + gq;
             const bool kok = kk < KR;
             const int64_t ke = kok ? (CX ? kk >> 1 : kk) : 0;
@@ -109,12 +110,14 @@ __global__ void __launch_bounds__(THREADS) gemm_wave_kernel(GemmArgs g, int64_t 
             }
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < 4; ++u) {
+            if (k0 + 4 * u >= KR) break;
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int jb = 0; jb < 2; ++jb)
                     if ((i == 0 || rows2) && (jb == 0 || cols2)) acc[i][jb] = Mfma<R>::run(av[u][i], bv[u][jb], acc[i][jb]);
+        }
     }
 
     // ---- epilogue: the same arithmetic as the tiled kernels; real column n0r + 16 jb + j
