@@ -212,28 +212,45 @@ def run_c2(h):
     shape = (16,) * 6
     perm = [5, 2, 0, 4, 1, 3]
     X = inputs.uniform(1002, 0, shape)
-    nset = 3   # 3 x (134 MB in + 134 MB out) > 256 MB last-level cache: every pass misses
-    Xs = [h.gpu(X) for _ in range(nset)]
+    nset = 6   # permuted buffers in rotation: the reduce of step i reads the one written FOUR steps earlier
+    lag = 4    # 4 x (134 MB read + 134 MB written by the permutes between) = 1.07 GB through the 256 MB last-level cache
+    Xs = [h.gpu(X) for _ in range(3)]
     Ps = [h.empty(shape, np.float64) for _ in range(nset)]
     Rs = [h.empty((16,) * 4, np.float64) for _ in range(nset)]
     pplan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute(list(range(6)), perm), [shape, shape])
     modes_a, modes_c = perm, [5, 0, 4, 3]          # sum over output axes 1 and 4 of the permuted tensor
     rplan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Reduce(modes_a, modes_c, tf.ReduceOp.Sum), [shape, (16,) * 4])
-    pcalls = [h.bound_execute(pplan, [Xs[i]], Ps[i]) for i in range(nset)]
+    pcalls = [h.bound_execute(pplan, [Xs[i % 3]], Ps[i]) for i in range(nset)]
     rcalls = [h.bound_execute(rplan, [Ps[i]], Rs[i]) for i in range(nset)]
     pbytes = 2.0 * X.nbytes
     rbytes = float(X.nbytes + 16 ** 4 * 8)
+    for c in pcalls:    # every permuted buffer holds the permuted tensor before anything is timed
+        c()
 
-    def step(i):
+    def step_cold(i):
+        # the reduce reads a buffer that no kernel has touched for `lag` steps: its input comes from HBM
+        pcalls[i % nset]()
+        rcalls[(i - lag) % nset]()
+
+    def step_chained(i):
+        # the reduce reads what the permute has just written (part of it still sits in the last-level cache)
         pcalls[i % nset]()
         rcalls[i % nset]()
-    ms, prof = h.timed(step, [tf.PROF_COPY, tf.PROF_REDUCE])
+    ms_chained, prof_chained = h.timed(step_chained, [tf.PROF_COPY, tf.PROF_REDUCE])
+    ms_chained_events = h.last_ms_with_events
+    ms, prof = h.timed(step_cold, [tf.PROF_COPY, tf.PROF_REDUCE])
     prec, rrec = dominant(prof[tf.PROF_COPY]), dominant(prof[tf.PROF_REDUCE])
+    rrec_chained = dominant(prof_chained[tf.PROF_REDUCE])
     res = {
-        "workload": "f64 16^6 tensor: permute to (5,2,0,4,1,3), then sum over output axes 1 and 4",
+        "workload": "f64 16^6 tensor: permute to (5,2,0,4,1,3), then sum over output axes 1 and 4 "
+                    "(six permuted buffers in rotation; the timed reduce reads the one written four steps earlier, i.e. from HBM)",
         "dtype": "f64", "ms_per_step": ms, "ms_per_step_with_kernel_events": h.last_ms_with_events, "value": (pbytes + rbytes) / (ms * 1e-3) / 1e9, "unit": "GB/s",
         "permute": {"roofline": roofline("hbm", "hbm", pbytes, prec, "c2_permute"), "algorithmic_bytes": pbytes},
-        "reduce": {"roofline": roofline("hbm", "hbm", rbytes, rrec, "c2_reduce"), "algorithmic_bytes": rbytes},
+        "reduce": {"roofline": roofline("hbm", "hbm", rbytes, rrec, "c2_reduce"), "algorithmic_bytes": rbytes,
+                   "input": "cold: written four steps (1.07 GB of other traffic) before it is read"},
+        "reduce_chained": {"roofline": roofline("hbm", "hbm", rbytes, rrec_chained, "c2_reduce"), "algorithmic_bytes": rbytes,
+                           "ms_per_step": ms_chained, "ms_per_step_with_kernel_events": ms_chained_events,
+                           "input": "warm: the buffer the preceding permute has just written (not the roofline figure)"},
     }
     if h.cpu:
         P = np.empty(shape)
