@@ -912,9 +912,20 @@ class Tensor:
     def to_numpy(self):
         """Host copy with this tensor's dims (waits for pending work)."""
         self.wait()
-        flat = self._buf if self.logical_memory_space_.kind == 0 else self._buf.cpu().numpy().ravel()
+        off = self._offset
+        if self.logical_memory_space_.kind == 0:
+            flat = self._buf
+        else:
+            # the elements as they lie in memory from the lowest to the highest address this view reaches (a wrapped
+            # torch tensor may have any strides: its own .numpy() would hand back the logical order, not the memory order)
+            import torch
+            lo = off + sum((d - 1) * s for d, s in zip(self._dims, self._strides) if s < 0 and d > 0)
+            hi = off + sum((d - 1) * s for d, s in zip(self._dims, self._strides) if s > 0 and d > 0)
+            span = 0 if 0 in self._dims else hi - lo + 1
+            flat = torch.as_strided(self._buf, (span,), (1,), self._buf.storage_offset() + lo).cpu().numpy()
+            off -= lo
         isz = flat.dtype.itemsize
-        out = np.lib.stride_tricks.as_strided(flat[self._offset:], self._dims, [s * isz for s in self._strides]).copy()
+        out = np.lib.stride_tricks.as_strided(flat[off:], self._dims, [s * isz for s in self._strides]).copy()
         return np.conj(out) if self._conj else out
 
 

@@ -124,6 +124,11 @@ bool try_tiny_operator(int dtype, const void* a, const void* b, void* c, const C
 // false when the shape is not one it tiles; true when it launched (status holds the outcome).  Axis strides: A, B, C.
 bool try_dot(int dtype, const void* a, const void* b, void* c, std::vector<Axis> kept, std::vector<Axis> red, Scalar alpha,
              Scalar beta, void* stream, int32_t& status);
+// Batched products whose batch index is the contiguous one in all three tensors (column-major "bij,bjk->bik"): the kernel
+// of k_gemm_bfirst.hip, whose blocks take all the batch entries of a 128-byte line at once.  Returns false when the shape
+// is not one it takes; true when it launched (status holds the outcome).
+bool try_batch_first(int dtype, const void* a, const void* b, void* c, const ContractAxes& ax, Scalar alpha, Scalar beta,
+                     void* stream, bool conj_a, bool conj_b, int32_t& status);
 int32_t grouped_plan_init(tfh_plan& plan);
 int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* inputs, Scalar beta, tfh_view* outputs,
                        void* stream);

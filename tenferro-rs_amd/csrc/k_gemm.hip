@@ -721,6 +721,11 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
             return TFH_OK;
         clear_error();
     }
+    // the batch index contiguous in all three tensors (column-major "bij,bjk->bik"): a kernel of its own, no packing
+    if (M > 1 && N > 1 && nb > 1) {
+        int32_t st_bf = TFH_OK;
+        if (try_batch_first(dtype, a, b, c, ax, alpha, beta, stream, conj_a, conj_b, st_bf)) return st_bf;
+    }
     // lanes of the epilogue run along n: put C's fastest axis in the N group (swap operands if needed)
     if (min_stride(ax.M, 2) < min_stride(ax.N, 2)) {
         std::swap(a, b);

@@ -2,6 +2,7 @@
 inputs.  Bit-exact for data movement; relative Frobenius error <= 1e-12 for f64/complex128 and
 <= 1e-5 for f32/complex64 (the tolerances the backend is specified to)."""
 import itertools
+import os
 
 import numpy as np
 import pytest
@@ -19,6 +20,15 @@ def tf():
     import tenferro_rs_amd as tf
     tf.lib()
     return tf
+
+
+# Every randomized test draws from seeded_rng(n): n is the test's own number, TFH_TEST_SEED (default 0: the inputs these
+# tests have always run on) is added to it, so another set of inputs can be tried without editing this file.
+SEED_OFFSET = int(os.environ.get("TFH_TEST_SEED", "0"))
+
+
+def seeded_rng(n):
+    return np.random.default_rng(n + SEED_OFFSET)
 
 
 def rand(rng, shape, dtype):
@@ -93,7 +103,7 @@ def lab(s):
 # ------------------------------------------------------------------------------------------------ permute
 @pytest.mark.parametrize("dtype", ALL)
 def test_permute_all_rank4_perms_bit_exact(tf, oracle, dtype):
-    rng = np.random.default_rng(21)
+    rng = seeded_rng(21)
     a = rand(rng, (5, 12, 7, 9), dtype)
     da = dev(tf, a)
     for perm in itertools.permutations(range(4)):
@@ -110,7 +120,7 @@ def test_permute_all_rank4_perms_bit_exact(tf, oracle, dtype):
                                         ((4, 4, 4, 4, 4, 4, 4), (6, 2, 4, 0, 5, 1, 3)), ((2000,), (0,)), ((3, 1000), (1, 0)),
                                         ((0, 5), (1, 0)), ((), ())])
 def test_permute_shapes_bit_exact(tf, oracle, shape, perm):
-    rng = np.random.default_rng(22)
+    rng = seeded_rng(22)
     a = rng.standard_normal(shape)
     oshape = [shape[p] for p in perm]
     out = tf.Tensor.empty(oshape, tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float64)
@@ -133,7 +143,7 @@ def test_permute_special_values_bitwise(tf):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex128])
 def test_permute_strided_negative_alpha_beta_and_column_major(tf, oracle, dtype):
-    rng = np.random.default_rng(23)
+    rng = seeded_rng(23)
     big = rand(rng, (16, 18, 20), dtype)
     a = big[::2, ::-1, 1:19:3]
     b0 = np.asfortranarray(rand(rng, (a.shape[2], a.shape[0], a.shape[1]), dtype))   # column-major output
@@ -170,7 +180,7 @@ def test_permute_config2_full_size_bit_exact(tf, oracle):
 # ------------------------------------------------------------------------------------------------ reduce
 @pytest.mark.parametrize("dtype", ALL)
 def test_reduce_sum_keep_sets(tf, oracle, dtype):
-    rng = np.random.default_rng(24)
+    rng = seeded_rng(24)
     a = rand(rng, (6, 17, 5, 33), dtype)
     da = dev(tf, a)
     for keep in [(0,), (1, 3), (3, 0), (2, 1, 0), (), (0, 1, 2, 3), (3,), (2,)]:
@@ -207,7 +217,7 @@ def test_reduce_closed_forms_exact_and_long_reductions(tf):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_reduce_max_min_alpha_beta_strided(tf, oracle, dtype):
-    rng = np.random.default_rng(25)
+    rng = seeded_rng(25)
     big = rand(rng, (14, 40, 18), dtype)
     a = big[::2, ::-1, ::3]
     da = dev(tf, a)
@@ -266,7 +276,7 @@ CASES = [
 @pytest.mark.parametrize("case", CASES, ids=[c[0] + "," + c[1] + "->" + c[2] + str(i) for i, c in enumerate(CASES)])
 def test_contract_against_oracle(tf, oracle, dtype, case):
     ma, mb, mc, ext = case
-    rng = np.random.default_rng(26)
+    rng = seeded_rng(26)
     a = rand(rng, [ext[l] for l in ma], dtype)
     b = rand(rng, [ext[l] for l in mb], dtype)
     cshape = [ext[l] for l in mc]
@@ -281,7 +291,7 @@ def test_contract_against_oracle(tf, oracle, dtype, case):
 @pytest.mark.parametrize("dtype", ALL)
 def test_contract_integer_inputs_exact(tf, dtype):
     # small integers: products and sums are exact, so MFMA accumulation order cannot matter
-    rng = np.random.default_rng(27)
+    rng = seeded_rng(27)
 
     def ints(shape):
         x = rng.integers(-3, 4, shape).astype(np.float64)
@@ -298,7 +308,7 @@ def test_contract_integer_inputs_exact(tf, dtype):
 
 @pytest.mark.parametrize("dtype", [np.float64, np.complex128, np.float32])
 def test_contract_alpha_beta_strided_views(tf, oracle, dtype):
-    rng = np.random.default_rng(28)
+    rng = seeded_rng(28)
     alpha, beta = (0.7 - 1.1j, -0.3 + 0.2j) if np.issubdtype(dtype, np.complexfloating) else (0.7, -0.3)
     big = rand(rng, (140, 90), dtype)
     av = big[::2, ::-2]                       # 70 x 45, negative stride
@@ -325,7 +335,7 @@ def test_contract_alpha_beta_strided_views(tf, oracle, dtype):
 
 @pytest.mark.parametrize("dtype", ALL)
 def test_batched_gemm(tf, oracle, dtype):
-    rng = np.random.default_rng(29)
+    rng = seeded_rng(29)
     a, b = rand(rng, (2, 3, 50, 70), dtype), rand(rng, (2, 3, 70, 40), dtype)
     ref = np.empty((2, 3, 50, 40), dtype)
     oracle.batched_gemm(a, b, ref, n_batch=2)
@@ -333,6 +343,88 @@ def test_batched_gemm(tf, oracle, dtype):
     plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.BatchedGemm([2, 3], 50, 40, 70), [a.shape, b.shape, ref.shape])
     tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
     assert relerr(out.to_numpy(), ref) < TOL[dtype]
+
+
+def colmajor(x):
+    """The values of x laid out column-major (first index contiguous): a numpy view that dev() uploads as it is."""
+    return np.ascontiguousarray(x.transpose()).transpose()
+
+
+# the batched patterns of the reference's einsum documentation (tenferro-einsum/src/lib.rs:74-93) in the layout its
+# examples allocate (MemoryOrder::ColumnMajor): the batch index is the contiguous one in all three tensors
+BATCH_FIRST = [
+    ("bij,bjk->bik", lambda b: dict(b=b, i=3, j=4, k=5)),
+    ("abij,abjk->abik", lambda b: dict(a=2, b=b, i=4, j=5, k=6)),
+    ("bij,jk->bik", lambda b: dict(b=b, i=3, j=4, k=5)),
+    ("bij,bjk->bik", lambda b: dict(b=b, i=33, j=7, k=45)),      # ragged tiles, a partial k stage
+    ("bij,bkj->bki", lambda b: dict(b=b, i=40, j=13, k=50)),     # k innermost of the free axes, output transposed
+    ("bij,bjk->bik", lambda b: dict(b=b, i=64, j=64, k=64)),
+]
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("nb", [10, 1023, 1024, 1100])
+@pytest.mark.parametrize("case", range(len(BATCH_FIRST)))
+def test_column_major_batched_products(tf, oracle, dtype, nb, case):
+    sub, ext_of = BATCH_FIRST[case]
+    ext = ext_of(nb)
+    if case == 5 and nb > 100:
+        ext["b"] = 136 if nb % 2 == 0 else 135
+    rng = seeded_rng(201 + case)
+    terms, out_l = sub.split("->")[0].split(","), sub.split("->")[1]
+    hs = [colmajor(rand(rng, [ext[l] for l in t], dtype)) for t in terms]
+    cshape = [ext[l] for l in out_l]
+    ref = np.empty(cshape, dtype)
+    oracle.contract(hs[0], lab(terms[0]), hs[1], lab(terms[1]), ref, lab(out_l))
+    out = dev(tf, colmajor(np.full(cshape, np.nan, dtype)))      # beta == 0 must not read the NaNs
+    tf.einsum_into(sub, [dev(tf, h) for h in hs], 1.0, 0.0, out)
+    kernel = tf.last_kernel()
+    assert relerr(out.to_numpy(), ref) < TOL[dtype]
+    # the batch-first kernel takes whole 16-byte chunks of batch entries and at least two 128-byte lines of them
+    nbf = int(np.prod([ext[l] for l in out_l if l in terms[0] and l in terms[1]]))
+    per_chunk = 16 // np.dtype(dtype).itemsize
+    batch_first = nbf % per_chunk == 0 and nbf >= 16 * per_chunk
+    assert kernel.startswith("(gemm_bfirst_kernel") == batch_first, (kernel, nbf)
+    # alpha and beta (complex for complex dtypes) on top of an existing output
+    cx = np.issubdtype(dtype, np.complexfloating)
+    alpha, beta = (0.5 - 0.25j, 2.0 + 1.0j) if cx else (0.5, 2.0)
+    c0 = colmajor(rand(rng, cshape, dtype))
+    out = dev(tf, c0)
+    tf.einsum_into(sub, [dev(tf, h) for h in hs], alpha, beta, out)
+    ref2 = (alpha * ref.astype(np.complex128 if cx else np.float64) + beta * c0).astype(dtype)
+    scale = np.abs(alpha) * np.einsum(sub, np.abs(hs[0]).astype(np.float64), np.abs(hs[1]).astype(np.float64)) + np.abs(beta) * np.abs(c0)
+    assert contraction_within_tolerance(out.to_numpy(), ref2, dtype, scale, ext["j"])
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_batch_first_kernel_exact_on_integers_with_views_and_conj(tf, dtype):
+    """Small integers (exact products and sums): the batch-first kernel against numpy on operands that are views -- an
+    outer batch axis that does not fuse with the contiguous one, row and k strides that skip elements, a conjugated
+    operand -- and on a batch extent that leaves the last group of lines partly filled."""
+    rng = seeded_rng(207)
+    cx = np.issubdtype(dtype, np.complexfloating)
+
+    def ints(shape):
+        x = rng.integers(-3, 4, shape).astype(np.float64)
+        if cx:
+            x = x + 1j * rng.integers(-3, 4, shape)
+        return x.astype(dtype)
+
+    nb, no = 72, 3
+    # buffers [k or n][m or k][outer][batch] with the batch contiguous; views take every second row / k
+    abuf, bbuf = ints((2 * 9, 2 * 21, no, nb)), ints((no, 37, 2 * 9, nb))
+    a = abuf[::2, ::2].transpose(2, 3, 1, 0)          # [o, b, m=21, k=9]: (o, b) would fuse here ...
+    b = bbuf[:, :, ::2].transpose(0, 3, 2, 1)         # [o, b, k=9, n=37]: ... but not here, where o is the outermost axis
+    cbuf = ints((37, 21, no, nb))
+    c = cbuf.transpose(2, 3, 1, 0)                    # [o, b, m, n]
+    out = dev(tf, c)
+    ops = [dev(tf, a), dev(tf, b)]
+    if cx:
+        ops[1] = ops[1].conj_on_load()
+    tf.einsum_into("obmk,obkn->obmn", ops, 2.0, -1.0, out)
+    assert tf.last_kernel().startswith("(gemm_bfirst_kernel"), tf.last_kernel()
+    expect = 2.0 * np.einsum("obmk,obkn->obmn", a, np.conj(b)) - c
+    assert np.array_equal(out.to_numpy(), expect.astype(dtype))
 
 
 def test_config0_matmul_512_f64(tf, oracle):
@@ -415,7 +507,7 @@ def test_grouped_tile_shapes_for_last_strips(tf, oracle, dtype):
 def test_grouped_column_major_operands_and_views(tf, oracle):
     # column-major blocks (A contiguous along its rows, B along k) and blocks cut out of larger buffers: the other
     # loader layouts of the grouped kernel, with last strips in both directions
-    rng = np.random.default_rng(82)
+    rng = seeded_rng(82)
     dims = [(192, 70, 320), (320, 130, 192), (256, 64, 200), (200, 90, 256)]
     As = [np.asfortranarray(rng.standard_normal((i, j))) for (i, j, k) in dims]
     Bs = [np.asfortranarray(rng.standard_normal((j, k))) for (i, j, k) in dims]
@@ -441,7 +533,7 @@ def test_grouped_plan_on_two_streams_with_different_operands(tf, oracle):
     import ctypes
     import torch
     dims = [(192, 256, 320), (320, 192, 192), (256, 128, 256), (128, 320, 448)] * 6
-    rng = np.random.default_rng(83)
+    rng = seeded_rng(83)
     sets = []
     for s in range(2):
         As = [rng.standard_normal((i, j)) for (i, j, k) in dims]
@@ -475,7 +567,7 @@ def test_grouped_label_orders_and_fusable_modes(tf, oracle, ma, mb, mc):
     # The roles of a matrix product's axes come from the plan's labels, in any order (transposed operands, transposed
     # result); operands with more than two modes are plain matrices once their modes fuse (a leading free mode, two
     # summed modes), and go through the general classification.
-    rng = np.random.default_rng(85)
+    rng = seeded_rng(85)
     ext_sets = [dict(i=70, j=33, k=130, a=3, l=4), dict(i=5, j=64, k=7, a=2, l=2), dict(i=128, j=128, k=64, a=1, l=8), dict(i=1, j=9, k=257, a=4, l=1)]
     shapes, As, Bs, outs = [], [], [], []
     for ext in ext_sets:
@@ -497,7 +589,7 @@ def test_grouped_records_are_kept_for_repeated_calls(tf, oracle):
     # that of its own operands.
     import ctypes
     dims = [(96, 64, 80), (33, 70, 129), (128, 128, 128), (17, 5, 260)] * 3
-    rng = np.random.default_rng(84)
+    rng = seeded_rng(84)
     desc = tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik"))
     plan = tf.HipBackend.plan_grouped(np.float64, desc, [[[i, j], [j, k], [i, k]] for (i, j, k) in dims])
     sets = []
@@ -539,7 +631,7 @@ def test_grouped_records_are_kept_for_repeated_calls(tf, oracle):
 def test_grouped_tiny_problems_take_the_wave_kernel(tf, oracle, dtype):
     # 300 problems with every extent between 1 and 32 (a block-sparse tensor with small blocks): one grouped launch,
     # one wave per 32x32 tile
-    rng = np.random.default_rng(79)
+    rng = seeded_rng(79)
     dims = [tuple(int(v) for v in rng.integers(1, 33, 3)) for _ in range(300)]
     assert _grouped_case(tf, oracle, dims, dtype, 79) < TOL[dtype]
     assert "gemm_wave_kernel" in tf.last_kernel(), tf.last_kernel()
@@ -555,7 +647,7 @@ def test_config4_grouped_full_size(tf, oracle):
 # ------------------------------------------------------------------------------------------------ elementwise, conj, fill, trace family
 @pytest.mark.parametrize("dtype", ALL)
 def test_elementwise_mul_conj_fill(tf, oracle, dtype):
-    rng = np.random.default_rng(30)
+    rng = seeded_rng(30)
     a, b = rand(rng, (9, 40, 21), dtype), rand(rng, (21, 40, 9), dtype).transpose(2, 1, 0)
     c0 = rand(rng, (9, 40, 21), dtype)
     ref = c0.copy()
@@ -577,7 +669,7 @@ def test_elementwise_mul_second_operand_in_another_axis_order(tf, oracle, dtype)
     # the second operand's contiguous axis is neither A's nor the output's: it is brought into the output's axis order
     # first (a pool block, released in stream order); strided / reversed / broadcast operands and an output that is
     # a view are covered, and the operands must come out unchanged
-    rng = np.random.default_rng(130)
+    rng = seeded_rng(130)
     shape = (70, 50, 60)
     a = rand(rng, shape, dtype)
     cases = {
@@ -611,7 +703,7 @@ def test_conj_reference_doc_example(tf):
 
 @pytest.mark.parametrize("dtype", [np.float64, np.complex128])
 def test_trace_anti_trace_anti_diag(tf, oracle, dtype):
-    rng = np.random.default_rng(31)
+    rng = seeded_rng(31)
     a = rand(rng, (14, 5, 14, 3), dtype)
     ref = np.empty((3, 5), dtype)
     oracle.trace(a, [0, 1, 2, 3], ref, [3, 1], pairs=[(0, 2)])
@@ -642,7 +734,7 @@ PATTERNS = ["ij,jk->ik", "ii->", "i,j->ij", "i,i->", "ij,j->i", "ii->i", "ijk->"
 @pytest.mark.parametrize("pattern", PATTERNS)
 def test_einsum_pattern_catalogue(tf, oracle, dtype, pattern):
     # tenferro-einsum/src/lib.rs:37-93, against the brute-force einsum of the oracle
-    rng = np.random.default_rng(32)
+    rng = seeded_rng(32)
     ext = dict(i=13, j=14, k=15, l=6, a=2, b=3, x=4)
     ins, out = pattern.replace("(", "").replace(")", "").split("->")
     terms = ins.split(",")
@@ -669,7 +761,7 @@ def test_einsum_reference_doc_examples(tf):
 
 @pytest.mark.parametrize("dtype", [np.float64, np.complex128])
 def test_einsum_every_tree_of_a_small_network_agrees(tf, oracle, dtype):
-    rng = np.random.default_rng(33)
+    rng = seeded_rng(33)
     ext = dict(a=9, c=8, x=7, y=6, w=3, v=4, s=2, t=2)
     terms, out = ["awc", "asx", "wstv", "cty"], "xvy"
     ops = [rand(rng, [ext[l] for l in t], dtype) for t in terms]
@@ -717,7 +809,7 @@ def _random_network(rng):
 def test_einsum_random_networks(tf, oracle, dtype):
     # the executor end to end (parser, optimiser, layouts of intermediates, diagonal views, reductions, output
     # diagonals, alpha/beta into a strided output) against the oracle's single-loop-nest einsum
-    rng = np.random.default_rng(59)
+    rng = seeded_rng(59)
     for case in range(60):
         terms, out, ext = _random_network(rng)
         ops = [_random_view(rng, [ext[l] for l in t], dtype) for t in terms]
@@ -738,7 +830,7 @@ def test_einsum_random_networks(tf, oracle, dtype):
 
 def test_einsum_async_chaining(tf):
     # tenferro-einsum/src/lib.rs:158-177: the second call chains on the first result's event
-    rng = np.random.default_rng(34)
+    rng = seeded_rng(34)
     a, b = rng.standard_normal((300, 400)), rng.standard_normal((400, 400))
     da, db = dev(tf, a), dev(tf, b)
     c = tf.einsum("ij,jk->ik", [da, db])
@@ -761,7 +853,7 @@ def test_large_tile_kernel_stage_and_tile_boundaries(tf, dtype, nb, label):
     # than 1536 large ones), once with so few that it runs with 64 x 64 tiles.
     if nb == 0:
         nb = {np.float32: 80, np.complex64: 80, np.float64: 385, np.complex128: 257}[dtype]
-    rng = np.random.default_rng(71)
+    rng = seeded_rng(71)
     tol = TOL[dtype]
     stage = {np.float32: 32, np.float64: 16, np.complex64: 16, np.complex128: 8}[dtype]
     seen = set()
@@ -793,7 +885,7 @@ def test_small_products_across_split_counts(tf, dtype):
     # none (few stages) to hundreds (one tile with a long k).  Whatever it chooses, the result is that of the product:
     # extents that give one tile and many, k from one stage to thousands of elements, ragged in every direction, with
     # alpha and an old result to add, against numpy.
-    rng = np.random.default_rng(83)
+    rng = seeded_rng(83)
     tol = TOL[dtype]
     for (m, n, k) in [(64, 64, 4096), (64, 64, 4099), (128, 128, 128), (256, 256, 256), (200, 200, 2000), (100, 60, 5000),
                       (384, 384, 384), (512, 512, 512), (300, 260, 1103), (33, 47, 129), (64, 64, 33), (1000, 90, 70)]:
@@ -819,7 +911,7 @@ def test_conj_on_load_in_every_contraction_kernel(tf, dtype):
     # contraction kernels; shapes that go to the other kernels get a conjugated copy first.  Each shape with the flag on
     # A, on B and on both, alpha and beta complex, against numpy on explicitly conjugated operands; the routing is
     # checked so that every kernel's sign flip is exercised, including the paths that exchange the operands.
-    rng = np.random.default_rng(61)
+    rng = seeded_rng(61)
     tol = TOL[dtype]
     cases = [   # (modes a, modes b, modes c, extents, substring of the kernel label expected)
         ("mk", "kn", "mn", dict(m=2000, k=600, n=1500), ", 128>)"),
@@ -877,7 +969,7 @@ def test_conj_on_load_in_every_contraction_kernel(tf, dtype):
 
 
 def test_conj_on_load_views_einsum_permute_and_rejections(tf, oracle):
-    rng = np.random.default_rng(62)
+    rng = seeded_rng(62)
     a = rand(rng, (12, 2, 14), np.complex128)
     L = rand(rng, (12, 5, 12), np.complex128)
     W = rand(rng, (5, 2, 2, 5), np.complex128)
@@ -931,7 +1023,7 @@ def test_chaining_across_two_streams_through_the_completion_event(tf):
     # is long (2 x 2048^3 f64 per call, four calls queued) and the consumer is enqueued at once: without the wait it
     # would read a half-written operand.  Both the einsum path and TensorPrims::execute.
     import torch
-    rng = np.random.default_rng(35)
+    rng = seeded_rng(35)
     n = 2048
     a = rng.standard_normal((n, n)) / 32
     b = rng.standard_normal((n, n)) / 32
@@ -973,7 +1065,7 @@ def test_host_transfers_pageable_and_pinned_round_trip(tf):
     import torch
     L = tf.lib()
     (st,) = _new_streams(tf, 1)
-    rng = np.random.default_rng(36)
+    rng = seeded_rng(36)
     try:
         for nbytes in [1, 4097, (16 << 20) - 3, 16 << 20, (16 << 20) + 5, (40 << 20) + 1]:
             src = rng.integers(0, 256, nbytes, dtype=np.uint8)
@@ -1097,7 +1189,7 @@ def test_permute_large_tiles_for_far_apart_rows_bit_exact(tf, oracle, dtype, sha
     # an axis that is contiguous on one side and the slowest on the other: every tile touches rows megabytes apart,
     # and the copy takes the large-tile variant (512 threads, four times the tile, the longer run on the scattered
     # side).  Bit-exact against numpy's transpose; the identity and a near-identity stay on the ordinary tiles.
-    rng = np.random.default_rng(44)
+    rng = seeded_rng(44)
     a = rand(rng, shape, dtype)
     da = dev(tf, a)
     large = 0
@@ -1118,7 +1210,7 @@ def test_permute_large_tiles_for_far_apart_rows_bit_exact(tf, oracle, dtype, sha
 @pytest.mark.parametrize("dtype", ALL)
 def test_permute_power_of_two_shapes_take_the_vector_path(tf, oracle, dtype):
     # every tile full, contiguous fastest axes on both sides: 16-byte accesses, no bounds checks
-    rng = np.random.default_rng(41)
+    rng = seeded_rng(41)
     a = rand(rng, (32, 8, 64, 16), dtype)
     for perm in [(3, 1, 0, 2), (0, 1, 2, 3), (2, 3, 0, 1), (1, 0, 3, 2)]:
         got, ref = _permute_check(tf, oracle, a, perm)
@@ -1132,7 +1224,7 @@ def test_permute_power_of_two_shapes_take_the_vector_path(tf, oracle, dtype):
 
 def test_permute_misaligned_base_and_odd_inner_extent(tf, oracle):
     # a view that starts one element into its buffer is only 8-byte aligned: the scalar path must be used
-    rng = np.random.default_rng(42)
+    rng = seeded_rng(42)
     big = rng.standard_normal(64 * 64 * 16 + 1)
     a = big[1:].reshape(64, 64, 16)
     got, ref = _permute_check(tf, oracle, a, (2, 0, 1))
@@ -1156,7 +1248,7 @@ def _reduce_check(tf, oracle, a, modes_a, modes_c, op_tf, op_or, alpha=1.0, beta
 
 @pytest.mark.parametrize("dtype", ALL)
 def test_reduce_fast_path_variants(tf, oracle, dtype):
-    rng = np.random.default_rng(43)
+    rng = seeded_rng(43)
     a = rand(rng, (8, 16, 4, 16, 32), dtype)
     m = [0, 1, 2, 3, 4]
     cases = [[0, 1, 2, 3],          # contiguous axis reduced, few addends: block-serial kept indices
@@ -1184,7 +1276,7 @@ def test_reduce_fast_path_variants(tf, oracle, dtype):
 
 
 def test_reduce_misaligned_base_and_split_reductions(tf, oracle):
-    rng = np.random.default_rng(44)
+    rng = seeded_rng(44)
     big = rng.standard_normal(16 * 16 * 64 + 1)
     a = big[1:].reshape(16, 16, 64)                   # 8-byte aligned only
     got, ref = _reduce_check(tf, oracle, a, [0, 1, 2], [0, 2], tf.ReduceOp.Sum, oracle.SUM)
@@ -1219,7 +1311,7 @@ def test_contract_128_tile_kernel(tf, oracle, dtype, case):
     pattern, ext = case
     ins, mc = pattern.split("->")
     ma, mb = ins.split(",")
-    rng = np.random.default_rng(45)
+    rng = seeded_rng(45)
     a = rand(rng, [ext[l] for l in ma], dtype)
     b = rand(rng, [ext[l] for l in mb], dtype)
     cshape = [ext[l] for l in mc]
@@ -1237,7 +1329,7 @@ def test_contract_128_tile_kernel(tf, oracle, dtype, case):
 @pytest.mark.parametrize("dtype", [np.float64, np.complex128])
 def test_contract_128_tile_negative_strides_and_offsets(tf, oracle, dtype):
     # reversed views: the kernel rebases each operand to its lowest address
-    rng = np.random.default_rng(46)
+    rng = seeded_rng(46)
     abig, bbig = rand(rng, (400, 310), dtype), rand(rng, (310, 280), dtype)
     av, bv = abig[::-2, ::-1][:, 5:], bbig[::-1, ::-2][5:, :]      # 200 x 305, 305 x 140
     ref = np.empty((200, 140), dtype)
@@ -1281,7 +1373,7 @@ def test_contract_odd_extents_take_the_straddling_vector_path(tf, oracle, dtype,
     # extents that are not multiples of the 16-byte vector length: the last vector of a row or column straddles the
     # end of the operand and is loaded from a window moved back inside it (k smaller than one vector: scalar path)
     ma, mb = layout
-    rng = np.random.default_rng(47)
+    rng = seeded_rng(47)
     for m, k, n in ODD_SIZES:
         ext = dict(m=m, k=k, n=n)
         a = rand(rng, [ext[l] for l in ma], dtype)
@@ -1307,7 +1399,7 @@ def test_contract_thin_side_takes_128x64_tiles(tf, oracle, dtype, layout):
     # one free group of 33..95 real columns and a long other side: 128x64 tiles of the large-tile kernel, whichever
     # operand is the thin one (the operands are exchanged so that it becomes the right-hand side)
     ma, mb = layout
-    rng = np.random.default_rng(147)
+    rng = seeded_rng(147)
     ec = 2 if np.issubdtype(dtype, np.complexfloating) else 1
     for m, k, n in THIN_SIZES:
         ext = dict(m=m, k=k, n=n)
@@ -1331,7 +1423,7 @@ def test_contract_thin_side_takes_128x64_tiles(tf, oracle, dtype, layout):
 def test_contract_odd_extents_few_tiles(tf, oracle, dtype, layout):
     # the same kind of extents with so few tiles that the 64x64 kernel (or, for complex128, the large-tile one) is chosen
     ma, mb = layout
-    rng = np.random.default_rng(148)
+    rng = seeded_rng(148)
     for m, k, n in [(129, 1031, 133), (255, 1077, 257), (193, 1058, 97), (257, 1025, 129), (130, 1027, 131), (131, 37, 129), (300, 5, 310)]:
         ext = dict(m=m, k=k, n=n)
         a = rand(rng, [ext[l] for l in ma], dtype)
@@ -1346,7 +1438,7 @@ def test_contract_odd_extents_few_tiles(tf, oracle, dtype, layout):
 
 def test_contract_operand_ending_at_the_end_of_its_allocation(tf, oracle):
     # the operands are the tail of exactly-sized device buffers: a read past the last element would leave the buffer
-    rng = np.random.default_rng(48)
+    rng = seeded_rng(48)
     for dtype, m, k, n in [(np.float32, 643, 1033, 641), (np.float64, 641, 523, 643)]:
         for ma, mb in LAYOUTS:
             ext = dict(m=m, k=k, n=n)
@@ -1364,7 +1456,7 @@ def test_contract_operand_ending_at_the_end_of_its_allocation(tf, oracle):
 @pytest.mark.parametrize("dtype", ALL)
 def test_permute_extents_with_divisor_tiles(tf, oracle, dtype):
     # extents that are not powers of two but have useful divisors (15, 50, 60, 250): tiled without partial tiles
-    rng = np.random.default_rng(49)
+    rng = seeded_rng(49)
     for shape, perm in [((15, 15, 15, 15), (3, 1, 0, 2)), ((60, 50, 70), (2, 0, 1)), ((250, 130), (1, 0)), ((6, 250, 9, 20), (1, 3, 0, 2)),
                         ((33, 257), (1, 0)), ((12, 100, 35), (0, 2, 1))]:
         a = rand(rng, shape, dtype)
@@ -1395,7 +1487,7 @@ def test_permute_extents_with_divisor_tiles(tf, oracle, dtype):
 def test_permute_large_ragged_tensors_split_into_interior_and_border(tf, oracle, dtype):
     # more than 2^20 elements with extents just off the tile grid: whole tiles go through the fast path, the border
     # slabs are copied separately; every element must be written exactly once
-    rng = np.random.default_rng(50)
+    rng = seeded_rng(50)
     for shape, perm in [((1030, 1100), (1, 0)), ((101, 103, 107), (2, 0, 1)), ((65, 129, 131), (1, 2, 0)), ((3, 1025, 515), (2, 1, 0))]:
         a = rand(rng, shape, dtype)
         got, ref = _permute_check(tf, oracle, a, perm)
@@ -1457,7 +1549,7 @@ def _random_view(rng, shape, dtype):
 @pytest.mark.parametrize("dtype", ALL)
 @pytest.mark.parametrize("big", [False, True], ids=["small", "large"])
 def test_contract_random_label_patterns_and_views(tf, oracle, dtype, big):
-    rng = np.random.default_rng(51 + (7 if big else 0))
+    rng = seeded_rng(51 + (7 if big else 0))
     for case in range(25 if big else 40):
         ma, mb, mc, ext = _random_contraction(rng, big)
         while not ma or not mb:   # rank-0 operands are not views of anything
@@ -1528,7 +1620,7 @@ def test_contract_random_layouts_on_the_128_tile_kernel(tf, oracle, dtype):
     # random shapes sized for the 128x128 kernel (both free products >= 700, k of a thousand or more: enough tiles and stages):
     # one or two modes per group, random axis orders, random strided / reversed / offset views, odd extents.  Most
     # cases are contiguous along some operand direction (16-byte loads with their tail handling), the stepped views are not.
-    rng = np.random.default_rng(58)
+    rng = seeded_rng(58)
     on128 = 0
     for case in range(14):
         labels = list("abcdefgh")
@@ -1565,7 +1657,7 @@ def test_contract_random_layouts_on_the_128_tile_kernel(tf, oracle, dtype):
 
 @pytest.mark.parametrize("dtype", ALL)
 def test_permute_and_reduce_random_shapes_and_views(tf, oracle, dtype):
-    rng = np.random.default_rng(52)
+    rng = seeded_rng(52)
     for case in range(30):
         rank = int(rng.integers(1, 6))
         shape = [int(rng.integers(1, 24)) for _ in range(rank)]
@@ -1596,7 +1688,7 @@ def test_calls_are_capturable_in_a_hip_graph_and_replay_correctly(tf, oracle):
     # permute, a reduction and a three-operand einsum are captured into one graph and replayed on new input contents,
     # with eager work and synchronisation between the replays; every replay must equal the eager result.
     import torch
-    rng = np.random.default_rng(53)
+    rng = seeded_rng(53)
     ext = dict(a=8, j=32, b=16, k=48, c=64)
     A = rand(rng, [ext[l] for l in "ajbk"], np.float64)
     B = rand(rng, [ext[l] for l in "kcj"], np.float64)
@@ -1661,7 +1753,7 @@ def test_graph_replays_after_the_workspace_grew_and_the_caches_were_released(tf,
     # those buffers alone (they are retired or passed over, never freed): the graph is replayed afterwards on new
     # contents and must still give the eager result.
     import torch
-    rng = np.random.default_rng(55)
+    rng = seeded_rng(55)
     A = rand(rng, (8, 32, 16, 48), np.float64)        # "ajbk,kcj->abc": packing, offset tables, split-K partials
     B = rand(rng, (48, 64, 32), np.float64)
     E1, E2, E3 = rand(rng, (40, 50), np.float64), rand(rng, (50, 30), np.float64), rand(rng, (30, 20), np.float64)
@@ -1720,7 +1812,7 @@ def test_owned_variant_keeps_intermediates_in_donated_operand_buffers(tf, oracle
     # ends up overwritten; the borrowing variant leaves its operands intact; a buffer that another tensor shares, or
     # that the caller wrapped from their own torch tensor, is never written.
     import torch
-    rng = np.random.default_rng(54)
+    rng = seeded_rng(54)
     host = [rand(rng, (64, 64), np.float64) for _ in range(4)]
     subs = tf.Subscripts.parse("ij,jk,kl,lm->im")
     tree = tf.ContractionTree.from_pairs(subs, [h.shape for h in host], [(0, 1), (4, 2), (5, 3)])
@@ -1776,7 +1868,7 @@ def test_offset_tables_are_kept_per_layout_and_survive_a_release(tf, oracle):
     # The offset tables of a multi-mode contraction are built once per (dims, strides) and stream and reused by later
     # calls.  Two layouts of the same shapes alternate through one plan: each call must use its own layout's tables;
     # releasing the library's scratch memory in between drops them and the next call builds them again.
-    rng = np.random.default_rng(77)
+    rng = seeded_rng(77)
     sa, sb, sc = (16, 40, 8, 24), (24, 130, 40), (16, 8, 130)                  # "ajbk,kcj->abc": 128x128 tiles
     a1, b1 = rand(rng, sa, np.float64), rand(rng, sb, np.float64)
     a2 = np.ascontiguousarray(rand(rng, (24, 8, 40, 16), np.float64)).transpose(3, 2, 1, 0)      # same dims, reversed strides
@@ -1814,7 +1906,7 @@ def test_contract_small_operator_applied_to_a_long_tensor(tf, oracle, dtype, m, 
     # take the product (k = 13).  The kernel works on units of 16 consecutive c: extents that are no
     # multiple of 16 (500, 100, 50, 1000: bond dimensions are rarely powers of two) end each run on a partly filled unit;
     # a run shorter than three units (17) is left to the tiled kernels.
-    rng = np.random.default_rng(91)
+    rng = seeded_rng(91)
     t = rand(rng, (x, c, k), dtype)
     w = rand(rng, (k, 2 * m), dtype)[:, ::2]
     ref = rand(rng, (x, m, c), dtype)
@@ -1834,7 +1926,7 @@ def test_contract_small_operator_applied_to_a_long_tensor(tf, oracle, dtype, m, 
 def test_contract_small_operator_exact_on_integer_inputs(tf):
     # small integers: every product and sum is exact, so the streaming kernel must agree with numpy to the bit, and a
     # wrong sign in the complex expansion or a misplaced k would show
-    rng = np.random.default_rng(92)
+    rng = seeded_rng(92)
     t = (rng.integers(-4, 5, (4, 1024, 32)) + 1j * rng.integers(-4, 5, (4, 1024, 32))).astype(np.complex128)
     w = (rng.integers(-4, 5, (32, 32)) + 1j * rng.integers(-4, 5, (32, 32))).astype(np.complex128)
     out = tf.Tensor.empty([4, 32, 1024], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.complex128)
@@ -1849,7 +1941,7 @@ def test_contract_small_operator_strided_rows_and_split_k_order(tf, oracle, dtyp
     # the streaming kernel's addressing: rows of the long operand reversed along c and padded (a view of a larger buffer),
     # its k split over two modes that the small operand holds in the opposite order (its k goes through the offset table),
     # the small operand's rows split over two modes of the output
-    rng = np.random.default_rng(93)
+    rng = seeded_rng(93)
     x, c, s_, w_, t_, v_ = 16, 320, 2, 8, 2, 7
     t1 = rand(rng, (x, c, s_, w_), dtype)[:, ::-1]                                        # contiguous k per row, rows reversed
     wop = rand(rng, (w_, s_, t_, v_), dtype)
@@ -1884,7 +1976,7 @@ def test_contract_small_operator_with_the_result_contiguous_along_its_columns(tf
     cplx = np.issubdtype(dtype, np.complexfloating)
     if k > 32 and cplx:
         k = 32
-    rng = np.random.default_rng(94)
+    rng = seeded_rng(94)
     t = rand(rng, (x, c, k), dtype)
     w = rand(rng, (k, m), dtype)
     out0 = rand(rng, (x, c, m), dtype)
@@ -1926,7 +2018,7 @@ def test_contract_small_operator_every_wave_streams_several_units(tf, oracle, dt
         k *= 2          # whole chunks of four f32 / two complex64
     if dtype == np.float32 and out_modes == "xcm":
         m = (m + 3) // 4 * 4
-    rng = np.random.default_rng(95)
+    rng = seeded_rng(95)
     x = 3
     t = rand(rng, (x, c, k), dtype)
     w = rand(rng, (k, m), dtype)
@@ -1951,7 +2043,7 @@ def test_contract_tiny_operator_on_the_last_leg_of_a_long_tensor(tf, oracle, dty
     # is preferred for but cannot take (runs of 17 columns) still goes to the tiny-operator kernel.
     cplx = np.issubdtype(dtype, np.complexfloating)
     rows = out_modes == "xcm"
-    rng = np.random.default_rng(96)
+    rng = seeded_rng(96)
     x = 32 if c > 100 else 4096
     t = rand(rng, (x, c, k), dtype)
     w = rand(rng, (k, m), dtype)
@@ -1987,7 +2079,7 @@ def test_contract_small_operator_on_a_middle_leg(tf, oracle, dtype, a_, k, m, c)
     # holds in the other order, and a view of every second a with a conjugated operator.
     cplx = np.issubdtype(dtype, np.complexfloating)
     streamed = whole_chunks(dtype, c)
-    rng = np.random.default_rng(97)
+    rng = seeded_rng(97)
     t = rand(rng, (a_, k, c), dtype)
     w = rand(rng, (m, k), dtype)
     out0 = rand(rng, (a_, m, c), dtype)
@@ -2029,7 +2121,7 @@ def test_contract_tiny_operator_with_the_acted_leg_moved_last(tf, oracle, dtype,
     # results leave through an LDS tile in address order (the kernel's last template argument); elsewhere the direct
     # stores remain (c = 1000; three f64 per row) or another kernel takes the product.
     cplx = np.issubdtype(dtype, np.complexfloating)
-    rng = np.random.default_rng(98)
+    rng = seeded_rng(98)
     t = rand(rng, (a_, k, c), dtype)
     w = rand(rng, (m, k), dtype)
     out0 = rand(rng, (a_, c, m), dtype)
@@ -2056,7 +2148,7 @@ def test_contract_small_operator_on_a_middle_leg_with_that_leg_moved_last(tf, or
     # whole 16-byte chunks (any for complex128).
     cplx = np.issubdtype(dtype, np.complexfloating)
     streamed = whole_chunks(dtype, c) and whole_chunks(dtype, m)
-    rng = np.random.default_rng(99)
+    rng = seeded_rng(99)
     t = rand(rng, (a_, k, c), dtype)
     w = rand(rng, (m, k), dtype)
     out0 = rand(rng, (a_, c, m), dtype)
@@ -2075,7 +2167,7 @@ def test_reduce_rows_and_inner_axes_take_the_butterfly_fold(tf, oracle, dtype):
     # sums over the contiguous axis (row sums) and over an inner axis next to a short kept one: nothing is left to loop
     # over, so a block handles eight outputs per lane group and folds them with the transposing butterfly.  Exact
     # integer inputs make a misrouted accumulator visible; max/min and alpha/beta go the same way.
-    rng = np.random.default_rng(95)
+    rng = seeded_rng(95)
     cplx = np.issubdtype(dtype, np.complexfloating)
     def ints(shape):
         x = rng.integers(-9, 10, shape).astype(np.float64)
@@ -2105,7 +2197,7 @@ def test_reduce_rows_and_inner_axes_take_the_butterfly_fold(tf, oracle, dtype):
 def test_reduce_few_outputs_split_over_blocks(tf, oracle, dtype):
     # few outputs and a long reduction: the serial range is split over blocks (raw partials) and a second launch folds
     # the partials in a fixed order.  Exact integer inputs: any lost or doubled chunk changes the sum.
-    rng = np.random.default_rng(96)
+    rng = seeded_rng(96)
     cplx = np.issubdtype(dtype, np.complexfloating)
     def ints(shape):
         x = rng.integers(-9, 10, shape).astype(np.float64)
@@ -2138,7 +2230,7 @@ def test_contract_one_tile_with_a_very_long_k_and_many_batches(tf, oracle, dtype
     # a single output tile under a k of several hundred thousand: the range is split hundreds of ways and the partials
     # are folded by the many-splits kernel (fixed order: two runs give the same bits); and a batch count above 65535
     # (more (batch, split) pairs than one grid dimension holds)
-    rng = np.random.default_rng(97)
+    rng = seeded_rng(97)
     m, n, k = 40, 24, 300000
     a, b = rand(rng, (m, k), dtype), rand(rng, (n, k), dtype)
     ref = np.empty((m, n), dtype)
@@ -2187,7 +2279,7 @@ def test_contract_with_an_empty_free_group_takes_the_product_reduction_kernel(tf
     pattern, ext = case
     ins, mc = pattern.split("->")
     ma, mb = ins.split(",")
-    rng = np.random.default_rng(98)
+    rng = seeded_rng(98)
     a = rand(rng, [ext[l] for l in ma], dtype)
     b = rand(rng, [ext[l] for l in mb], dtype)
     cshape = [ext[l] for l in mc]
@@ -2212,7 +2304,7 @@ def test_contract_with_an_empty_free_group_takes_the_product_reduction_kernel(tf
 @pytest.mark.parametrize("dtype", [np.float64, np.complex128, np.float32])
 def test_product_reduction_on_strided_and_reversed_views(tf, oracle, dtype):
     # operands seen through stepped, reversed and offset views: scalar loads, negative strides
-    rng = np.random.default_rng(99)
+    rng = seeded_rng(99)
     big = rand(rng, (256, 2 * 512 + 3), dtype)
     a = big[::-1, 1:1025:2]                       # [256, 512], rows reversed, every other column
     x = rand(rng, (3 * 512,), dtype)[::3]
@@ -2245,7 +2337,7 @@ def test_product_reduction_random_shapes(tf, oracle, dtype):
     # random contractions with one free group empty, over extents the product-reduction kernel tiles: random mode
     # structure (batch modes, modes only one operand has, several contracted modes), random axis orders, dense or
     # stepped / reversed views, alpha/beta.  Most cases must reach that kernel.
-    rng = np.random.default_rng(101)
+    rng = seeded_rng(101)
     hits = 0
     ncase = 40
     for case in range(ncase):
@@ -2292,7 +2384,7 @@ def test_reduce_random_shapes_that_tile(tf, oracle, dtype):
     # random reductions over power-of-two-friendly extents: every variant of the fast kernel (vector / scalar loads,
     # contiguous axis kept or reduced, eight block-serial outputs with the butterfly fold, the serial range split over
     # blocks) is reached by some case; sums, max/min, alpha/beta, dense and strided views
-    rng = np.random.default_rng(102)
+    rng = seeded_rng(102)
     kernels = set()
     cplx = np.issubdtype(dtype, np.complexfloating)
     for case in range(60):
@@ -2326,7 +2418,7 @@ def test_reduce_random_shapes_that_tile(tf, oracle, dtype):
 def test_batches_of_tiny_products_take_the_wave_kernel(tf, oracle, dtype, m, k, n, nbatch):
     # many products with both free extents at most 32: one wave per 32x32 tile, operands loaded straight into the MFMA
     # layout with bounds masks.  Odd extents, k that is not a multiple of the step, alpha/beta, operand orders.
-    rng = np.random.default_rng(103)
+    rng = seeded_rng(103)
     cplx = np.issubdtype(dtype, np.complexfloating)
     for ma, mb, mc in [("bmk", "bkn", "bmn"), ("kbm", "nbk", "bnm")]:
         ext = dict(b=nbatch, m=m, k=k, n=n)
@@ -2357,7 +2449,7 @@ def test_calls_from_several_host_threads_on_their_own_streams(tf, oracle):
     # (tables, split-K, packing), einsum trees, permutes and reductions at once; every result is checked
     import threading
     import torch
-    rng = np.random.default_rng(104)
+    rng = seeded_rng(104)
     work = []
     for t in range(4):
         a, b = rand(rng, (24, 8, 20, 12 + t), np.float64), rand(rng, (12 + t, 30, 8), np.float64)      # "ajbk,kcj->abc"
@@ -2419,7 +2511,7 @@ def test_operand_above_4_gib(tf, oracle):
     X = tf.Tensor.from_torch(x)
     rows = [0, 1, 63, 64, 127, 128, 20011, 35791, 35792, 39935, 39936, 39999]
     xs = x[rows].cpu().numpy()
-    rng = np.random.default_rng(111)
+    rng = seeded_rng(111)
 
     t = tf.Tensor.empty([k, m], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
     back = tf.Tensor.empty([m, k], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, np.float32)
@@ -2475,7 +2567,7 @@ def test_operand_above_4_gib(tf, oracle):
 
 def test_long_grids_and_high_rank(tf, oracle):
     # extents past the 65535 limit of a grid's y and z dimensions, many small outputs, a rank-12 permutation
-    rng = np.random.default_rng(112)
+    rng = seeded_rng(112)
     x = rand(rng, (70000, 3, 5), np.float64)
     out = dev(tf, np.zeros((5, 70000, 3)))
     tf.HipBackend.execute(tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute([0, 1, 2], [2, 0, 1]), [x.shape, out.dims()]), 1.0, [dev(tf, x)], 0.0, out)
@@ -2504,7 +2596,7 @@ def test_long_grids_and_high_rank(tf, oracle):
 def test_tensor_view_materialises_on_the_device(tf, oracle):
     # TensorView (tenferro-tensor/src/lib.rs:183-300) over device memory: zero-copy permute / diagonal / broadcast, then
     # to_tensor / contiguous / conj run the copy kernels; bit-exact against the oracle's permute
-    rng = np.random.default_rng(120)
+    rng = seeded_rng(120)
     x = rand(rng, (6, 5, 6, 4), np.complex128)
     v = dev(tf, x).tensor_view()
     assert v.logical_memory_space() == tf.GpuMemory(0) and v.dims() == [6, 5, 6, 4]
@@ -2528,7 +2620,7 @@ def test_contract_tiny_operator_applied_to_a_long_tensor(tf):
     # the streaming kernel, against numpy's einsum in double precision.  Legs at the front, in the middle and at the end,
     # extents 2, 3 and 8, either operand order, two-leg gates, alpha/beta, a sliced long operand, an output whose
     # contiguous axis is not the long operand's (scalar accesses), all four dtypes; exact on small integers.
-    rng = np.random.default_rng(134)
+    rng = seeded_rng(134)
     lab = lambda t: [ord(ch) for ch in t]
 
     def run(sub, sa, sb, dtype, alpha=1.0, beta=0.0, views=None, out_order="C", exact=False):
@@ -2579,7 +2671,7 @@ def test_contract_without_a_summed_index_scales_through_the_elementwise_kernel(t
     # "asx,x->asx", "ij,i->ij": a tensor scaled along some of its axes.  One free group is empty and nothing is summed, so
     # the elementwise kernel does it with the missing axes as broadcast axes; extents that tile and extents that do not,
     # alpha/beta, all dtypes (4-byte elements keep the product-reduction kernel where the extents tile).
-    rng = np.random.default_rng(135)
+    rng = seeded_rng(135)
     lab = lambda t: [ord(ch) for ch in t]
     for dtype in ALL:
         for sub, sa, sb in (("asx,x->asx", (100, 3, 1000), (1000,)), ("asx,a->asx", (128, 2, 1024), (128,)), ("ij,j->ij", (1021, 1031), (1031,)),
@@ -2601,7 +2693,7 @@ def test_permute_tensors_of_many_short_axes(tf):
     # come from cached tables.  Bit-exact against numpy for reversals, a cyclic shift and neighbour exchanges, extents that
     # are and are not powers of two, 4-, 8- and 16-byte elements, a sliced operand (strides that are not the dense ones),
     # the second call on a layout (tables from the cache) and a call after the caches were released.
-    rng = np.random.default_rng(133)
+    rng = seeded_rng(133)
     cases = [((3,) * 14, tuple(reversed(range(14))), np.float64), ((3,) * 12, tuple(reversed(range(12))), np.complex128),
              ((3,) * 13, (0, 2, 1, 3, 5, 4, 6, 8, 7, 9, 11, 10, 12), np.float32), ((5,) * 8, tuple(reversed(range(8))), np.float64),
              ((3, 4) * 5, tuple(reversed(range(10))), np.float64), ((2, 3) * 7, tuple(reversed(range(14))), np.float64),
@@ -2641,7 +2733,7 @@ def test_reduce_over_short_contiguous_rows(tf, oracle):
     # under an odd row count): 256 rows per block go through LDS and every thread adds up its own row.  Sum (exact on
     # small integers, and against the oracle on random data), max/min, alpha/beta on a permuted output, a sliced operand
     # whose outer axes do not merge, both real dtypes; complex and rows longer than 32 stay on the general kernel.
-    rng = np.random.default_rng(132)
+    rng = seeded_rng(132)
     for dtype in (np.float64, np.float32):
         for shape, red in (((100, 100, 100, 17), (3,)), ((15, 17, 33, 65, 31), (4,)), ((4097, 333, 3), (2,)), ((1001, 1025, 6), (2,)),
                            ((3000, 32), (1,)), ((70000, 2), (1,))):
@@ -2684,7 +2776,7 @@ def test_rotated_serial_starts_sum_every_index_exactly_once(tf):
     # serial index that is skipped or taken twice -- counts that are not powers of two, a last chunk shorter than the
     # others -- shows as an inequality.  Shapes: a middle axis of 12 and of 7 with serial steps of 128 KB under >= 512
     # blocks (rotation by block group), 1000 and 777 rows summed into few outputs (rotation by chunk).
-    rng = np.random.default_rng(131)
+    rng = seeded_rng(131)
     lab = lambda t: [ord(ch) for ch in t]
 
     def ints(shape, dtype):
@@ -2731,7 +2823,7 @@ def test_intermediates_cached_for_reuse_are_given_back_when_the_device_runs_out_
     except RuntimeError:
         pytest.skip("one allocation of all but 6 GiB of the free device memory is not available")
     try:
-        rng = np.random.default_rng(130)
+        rng = seeded_rng(130)
         subs = tf.Subscripts.parse("ij,jk,kl->il")
         for step, n in enumerate((16384, 18688, 21376)):
             a, b, c = rand(rng, (n, 2), np.float64), rand(rng, (2, n), np.float64), rand(rng, (n, 3), np.float64)
