@@ -99,11 +99,16 @@ class Harness:
             self.tfo = tfo
             self.cores = tfo.num_threads()
 
-    def gpu(self, arr):
-        return self.tf.Tensor.from_torch(self.torch.from_numpy(np.ascontiguousarray(arr)).cuda())
+    def gpu(self, arr, cm=False):
+        """Device tensor with the values of arr, row-major, or column-major (first index contiguous) when cm."""
+        if not cm:
+            return self.tf.Tensor.from_torch(self.torch.from_numpy(np.ascontiguousarray(arr)).cuda())
+        t = self.torch.from_numpy(np.ascontiguousarray(arr.transpose())).cuda()
+        return self.tf.Tensor.from_torch(t.permute(*reversed(range(arr.ndim))))
 
-    def empty(self, shape, dtype):
-        return self.tf.Tensor.empty(list(shape), self.tf.GpuMemory(0), self.tf.MemoryOrder.RowMajor, dtype)
+    def empty(self, shape, dtype, cm=False):
+        order = self.tf.MemoryOrder.ColumnMajor if cm else self.tf.MemoryOrder.RowMajor
+        return self.tf.Tensor.empty(list(shape), self.tf.GpuMemory(0), order, dtype)
 
     def timed(self, step, kinds):
         """step(i) enqueues one pass.  Returns (ms per step, {kind: [(kernel label, ms per launch, launches per step)]})."""
@@ -173,7 +178,7 @@ class Harness:
 
 
 # ------------------------------------------------------------------------------------------------- config 1
-def run_c1(h):
+def run_c1(h, cm=False, ref_out=None):
     tf, inputs = h.tf, h.inputs
     a, j, b, k, c = 64, 128, 64, 96, 256
     A = inputs.normal(1001, 0, (a, j, b, k), np.float32)
@@ -181,23 +186,26 @@ def run_c1(h):
     flops = 2.0 * a * b * c * j * k
     algo_bytes = 4.0 * (A.size + B.size + a * b * c)
     nset = 3   # rotate operand sets so the 201 MB operand is not served from the 256 MB last-level cache
-    As = [h.gpu(A) for _ in range(nset)]
-    Bd = h.gpu(B)
-    outs = [h.empty((a, b, c), np.float32) for _ in range(nset)]
+    As = [h.gpu(A, cm) for _ in range(nset)]
+    Bd = h.gpu(B, cm)
+    outs = [h.empty((a, b, c), np.float32, cm) for _ in range(nset)]
     plan = tf.HipBackend.plan(np.float32, tf.PrimDescriptor.Contract(lab("ajbk"), lab("kcj"), lab("abc")),
                               [A.shape, B.shape, (a, b, c)])
     calls = [h.bound_execute(plan, [As[i], Bd], outs[i]) for i in range(nset)]
     ms, prof = h.timed(lambda i: calls[i % nset](), [tf.PROF_CONTRACT, tf.PROF_COPY])
     rec = dominant(prof[tf.PROF_CONTRACT])
     res = {
-        "workload": "einsum ajbk,kcj->abc f32 a=64 j=128 b=64 k=96 c=256 (GEMM view M=4096 N=256 K=12288)",
+        "workload": "einsum ajbk,kcj->abc f32 a=64 j=128 b=64 k=96 c=256 (GEMM view M=4096 N=256 K=12288)" + LAYOUT_NOTE[cm],
         "dtype": "f32", "ms_per_step": ms, "ms_per_step_with_kernel_events": h.last_ms_with_events, "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
         "whole_step_frac_of_peak": flops / (ms * 1e-3) / 1e12 / PEAK["f32"],
         "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
         "roofline": roofline("mfma", "f32", flops, rec, "c1"),
         "other_kernels": [r for kind in prof.values() for r in kind if r is not rec],
     }
-    if h.cpu:
+    res["_out"] = outs[0].to_numpy()
+    if ref_out is not None:
+        res["parity"] = {"vs_row_major_rel_frobenius": relerr(res["_out"].astype(np.float64), ref_out.astype(np.float64)), "tolerance": 1e-5}
+    elif h.cpu:
         ref = np.empty((a, b, c), np.float32)
         t = h.cpu_time(lambda: h.tfo.contract(A, lab("ajbk"), B, lab("kcj"), ref, lab("abc")), 20)
         res["cpu_baseline"] = {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": h.cores, "kind": "port",
@@ -266,7 +274,7 @@ def run_c2(h):
 
 
 # ------------------------------------------------------------------------------------------------- config 3
-def run_c3(h):
+def run_c3(h, cm=False, ref_out=None):
     tf, inputs = h.tf, h.inputs
     chi, D, d = 1024, 16, 2
     sig = 1.0 / np.sqrt(chi)
@@ -286,7 +294,7 @@ def run_c3(h):
             labels, dims = tree.node(node)
             ext.update(zip(labels, dims))
         step_flops.append(8.0 * float(np.prod([float(v) for v in ext.values()])))
-    Ld, Ad, Wd = h.gpu(Lh), h.gpu(Ah), h.gpu(Wh)
+    Ld, Ad, Wd = h.gpu(Lh, cm), h.gpu(Ah, cm), h.gpu(Wh, cm)
     # 4th operand: A itself behind the conjugate-on-load flag (no conjugated copy is made; the contraction kernel that
     # reads it flips the sign of the imaginary parts as it stages them).  The explicit copy (Tensor::conj) is timed
     # beside it, and one pass over it, for comparison.
@@ -297,7 +305,7 @@ def run_c3(h):
         Acd = Ad.conj()
     h.torch.cuda.synchronize()
     conj_ms = (time.perf_counter() - t0) * 1e3 / 20
-    res_t = h.empty((chi, D, chi), np.complex128)
+    res_t = h.empty((chi, D, chi), np.complex128, cm)
     ops_copy = [Ld, Ad, Wd, Acd]
     ms_copy, _ = h.timed(lambda i: tf.einsum_with_plan_into(tree, ops_copy, 1.0, 0.0, res_t), [tf.PROF_CONTRACT])
     copy_result = res_t.to_numpy()
@@ -311,7 +319,7 @@ def run_c3(h):
     dom_flops = sorted(step_flops, reverse=True)[:n_dom]
     res = {
         "workload": "einsum awc,asx,wstv,cty->xvy complex128 chi=1024 D=16 d=2 via einsum_with_plan_into (tree from the optimiser; "
-                    "4th operand is A behind the conjugate-on-load flag: no conjugated copy exists)",
+                    "4th operand is A behind the conjugate-on-load flag: no conjugated copy exists)" + LAYOUT_NOTE[cm],
         "dtype": "c128", "ms_per_step": ms, "ms_per_step_with_kernel_events": h.last_ms_with_events, "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
         "whole_step_frac_of_peak": flops / (ms * 1e-3) / 1e12 / PEAK["f64"],
         "flops_per_step": flops, "tree_steps": tree.steps, "step_flops": step_flops, "min_flop_tree": bool(abs(flops - 558.3e9) < 0.1e9),
@@ -322,7 +330,10 @@ def run_c3(h):
         "all_kernels": {"kernel_ms_per_step": total_kms, "frac_of_peak": flops / (total_kms * 1e-3) / 1e12 / PEAK["f64"],
                         "kernels": recs},
     }
-    if h.cpu:
+    res["_out"] = res_t.to_numpy()
+    if ref_out is not None:
+        res["parity"] = {"vs_row_major_rel_frobenius": relerr(res["_out"], ref_out), "tolerance": 1e-12}
+    elif h.cpu:
         host = [Lh, Ah, Wh, np.conj(Ah)]
         ref = np.empty((chi, D, chi), np.complex128)
         t = h.cpu_time(lambda: h.tfo.einsum_pairs(host, [lab(t_) for t_ in terms], ref, lab(out), tree.steps), 3)
@@ -334,27 +345,30 @@ def run_c3(h):
 
 
 # ------------------------------------------------------------------------------------------------- config 4
-def run_c4(h):
+def run_c4(h, cm=False, ref_out=None):
     tf, inputs = h.tf, h.inputs
     dims = inputs.draw_block_dims(1004, 128)
     As = [inputs.uniform(1004, 3 * g, (i, j)) for g, (i, j, k) in enumerate(dims)]
     Bs = [inputs.uniform(1004, 3 * g + 1, (j, k)) for g, (i, j, k) in enumerate(dims)]
     flops = float(sum(2 * i * j * k for i, j, k in dims))
     algo_bytes = float(sum(8 * (i * j + j * k + i * k) for i, j, k in dims))
-    dA, dB = [h.gpu(x) for x in As], [h.gpu(x) for x in Bs]
-    outs = [h.empty((i, k), np.float64) for i, j, k in dims]
+    dA, dB = [h.gpu(x, cm) for x in As], [h.gpu(x, cm) for x in Bs]
+    outs = [h.empty((i, k), np.float64, cm) for i, j, k in dims]
     plan = tf.HipBackend.plan_grouped(np.float64, tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik")),
                                       [[[i, j], [j, k], [i, k]] for i, j, k in dims])
     pairs = list(zip(dA, dB))
     ms, prof = h.timed(lambda i: tf.HipBackend.execute_grouped(plan, 1.0, pairs, 0.0, outs), [tf.PROF_CONTRACT])
     rec = dominant(prof[tf.PROF_CONTRACT])
     res = {
-        "workload": "128 independent ij,jk->ik f64 blocks, i,j,k iid from {64,...,1024}, one grouped launch",
+        "workload": "128 independent ij,jk->ik f64 blocks, i,j,k iid from {64,...,1024}, one grouped launch" + LAYOUT_NOTE[cm],
         "dtype": "f64", "ms_per_step": ms, "ms_per_step_with_kernel_events": h.last_ms_with_events, "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
         "flops_per_step": flops, "algorithmic_bytes": algo_bytes,
         "roofline": roofline("mfma", "f64", flops, rec, "c4"),
     }
-    if h.cpu:
+    res["_out"] = [o.to_numpy() for o in outs]
+    if ref_out is not None:
+        res["parity"] = {"vs_row_major_max_rel_frobenius": max(relerr(o, r) for o, r in zip(res["_out"], ref_out)), "tolerance": 1e-12}
+    elif h.cpu:
         refs = [np.empty((i, k)) for i, j, k in dims]
 
         def cpu():
@@ -367,7 +381,71 @@ def run_c4(h):
     return res
 
 
-RUNNERS = {"c1": run_c1, "c2": run_c2, "c3": run_c3, "c4": run_c4}
+# ------------------------------------------------------------------------------------------------- config 0 and batched products
+def run_matmul(h, cm=False, ref_out=None):
+    """Configuration 0 (the CPU-runnable plumbing case, 512^3 f64 through einsum) on the GPU, for the layout comparison."""
+    tf, inputs = h.tf, h.inputs
+    A, B = inputs.uniform(1000, 0, (512, 512)), inputs.uniform(1000, 1, (512, 512))
+    Ad, Bd = h.gpu(A, cm), h.gpu(B, cm)
+    out = h.empty((512, 512), np.float64, cm)
+    tree = tf.ContractionTree.optimize(tf.Subscripts.parse("ij,jk->ik"), [A.shape, B.shape])
+    ms, prof = h.timed(lambda i: tf.einsum_with_plan_into(tree, [Ad, Bd], 1.0, 0.0, out), [tf.PROF_CONTRACT])
+    rec = dominant(prof[tf.PROF_CONTRACT])
+    flops = 2.0 * 512 ** 3
+    res = {"workload": "einsum ij,jk->ik f64 512^3" + LAYOUT_NOTE[cm], "dtype": "f64", "ms_per_step": ms, "value": flops / (ms * 1e-3) / 1e12,
+           "unit": "TFLOP/s", "roofline": roofline("mfma", "f64", flops, rec, "c0"), "_out": out.to_numpy()}
+    if ref_out is not None:
+        res["parity"] = {"vs_row_major_rel_frobenius": relerr(res["_out"], ref_out), "tolerance": 1e-12}
+    elif h.cpu:
+        ref = np.empty((512, 512))
+        t = h.cpu_time(lambda: h.tfo.contract(A, lab("ij"), B, lab("jk"), ref, lab("ik")), 20)
+        res["cpu_baseline"] = {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": h.cores, "kind": "port", "sample": "the full product, best of 20", "seconds": t}
+        res["parity"] = {"rel_frobenius": relerr(res["_out"], ref), "tolerance": 1e-12}
+    return res
+
+
+def run_batched(h, dtype, nb, n, cm=False, ref_out=None):
+    """einsum bij,bjk->bik, nb products of n^3 (the batched pattern of the reference's einsum documentation); column-major
+    is the layout the reference's examples allocate: the batch index is then the contiguous one in all three tensors."""
+    tf = h.tf
+    rng = np.random.default_rng(1005)
+    cx = np.dtype(dtype).kind == "c"
+
+    def draw(shape):
+        x = rng.standard_normal(shape)
+        return (x + 1j * rng.standard_normal(shape)).astype(dtype) if cx else x.astype(dtype)
+    A, B = draw((nb, n, n)), draw((nb, n, n))
+    Ad, Bd = h.gpu(A, cm), h.gpu(B, cm)
+    out = h.empty((nb, n, n), dtype, cm)
+    tree = tf.ContractionTree.optimize(tf.Subscripts.parse("bij,bjk->bik"), [A.shape, B.shape])
+    ms, prof = h.timed(lambda i: tf.einsum_with_plan_into(tree, [Ad, Bd], 1.0, 0.0, out), [tf.PROF_CONTRACT, tf.PROF_COPY])
+    rec = dominant(prof[tf.PROF_CONTRACT])
+    flops = (8.0 if cx else 2.0) * nb * n ** 3
+    nbytes = 3.0 * A.nbytes
+    res = {"workload": "einsum bij,bjk->bik %s b=%d i=j=k=%d" % (np.dtype(dtype).name, nb, n) + LAYOUT_NOTE[cm],
+           "dtype": "c128" if cx else "f64", "ms_per_step": ms, "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
+           "algorithmic_bytes": nbytes, "effective_GBps": nbytes / (ms * 1e-3) / 1e9,
+           "roofline": roofline("mfma", "f64", flops, rec, "batched"),
+           "operand_pack_kernels": [r for r in prof[tf.PROF_COPY]], "_out": out.to_numpy()}
+    if ref_out is not None:
+        res["parity"] = {"vs_row_major_rel_frobenius": relerr(res["_out"], ref_out), "tolerance": 1e-12}
+    elif h.cpu:
+        # a bounded sample of the batch on the CPU: the first 64 products
+        m = min(nb, 64)
+        ref = np.empty((m, n, n), dtype)
+        As, Bs = np.ascontiguousarray(A[:m]), np.ascontiguousarray(B[:m])
+        t = h.cpu_time(lambda: h.tfo.contract(As, lab("bij"), Bs, lab("bjk"), ref, lab("bik")), 5)
+        res["cpu_baseline"] = {"value": flops * m / nb / t / 1e12, "unit": "TFLOP/s", "cores": h.cores, "kind": "port",
+                               "sample": "the first %d of the %d products, best of 5" % (m, nb), "seconds": t}
+        res["parity"] = {"rel_frobenius": relerr(res["_out"][:m], ref), "tolerance": 1e-12}
+    return res
+
+
+LAYOUT_NOTE = {False: "; operands and result row-major", True: "; operands and result column-major (MemoryOrder::ColumnMajor, the order of the reference's examples)"}
+RUNNERS = {"c1": run_c1, "c2": run_c2, "c3": run_c3, "c4": run_c4, "c0": run_matmul,
+           "b64": lambda h, cm=False, ref_out=None: run_batched(h, np.float64, 4096, 64, cm, ref_out),
+           "b128": lambda h, cm=False, ref_out=None: run_batched(h, np.complex128, 1024, 128, cm, ref_out)}
+HAS_LAYOUTS = ("c0", "c1", "c3", "c4", "b64", "b128")   # configurations that are also run column-major
 HEADLINE = "c3"   # the largest configuration that fits one GPU
 
 
@@ -376,7 +454,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--configs", default="c3,c1,c2,c4")
+    ap.add_argument("--configs", default="c3,c1,c2,c4,c0,b64,b128")
+    ap.add_argument("--no-colmajor", action="store_true", help="skip the column-major variants of the configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also launch three plain 1 GiB device-to-device copies (torch's elementwise copy kernel): under "
@@ -397,11 +476,24 @@ def main():
     if HEADLINE not in wanted:
         wanted.insert(0, HEADLINE)
     results = {}
-    for name in wanted:
-        results[name] = RUNNERS[name](h)
+    def release():
         h.torch.cuda.synchronize()
         h.torch.cuda.empty_cache()
         h.tf.lib().tfh_release_workspaces()
+    for name in wanted:
+        results[name] = RUNNERS[name](h)
+        release()
+        if name in HAS_LAYOUTS and not args.no_colmajor:
+            # the same configuration with every operand and the result column-major; its result is checked against the
+            # row-major run's (which the CPU oracle has checked), its fraction of the roofline is reported beside it
+            r = RUNNERS[name](h, True, results[name]["_out"])
+            base = results[name]
+            r["vs_row_major"] = {"ms_per_step_ratio": r["ms_per_step"] / base["ms_per_step"],
+                                 "roofline_frac": r["roofline"]["frac"], "row_major_roofline_frac": base["roofline"]["frac"]}
+            r.pop("_out", None)
+            results[name + "_colmajor"] = r
+            release()
+        results[name].pop("_out", None)
     top = results[HEADLINE]
     line = {
         "metric": METRIC, "value": top["value"], "unit": top["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
