@@ -120,22 +120,33 @@ __global__ void __launch_bounds__(THREADS, (SkinnyCfg<R, KCM, MBM>::BLOCKS_PER_C
     // real elements and its real form for complex ones: A'[m][2k + part] = (re, im)[part] of A[m][k].
     R a[MBM][PAIRS][QB];
     {
+        // (indices past the matrix are redirected to its last row and last k and the values dropped afterwards: without a
+        // branch per element all of a lane's loads are in flight together -- with 32 units per wave at a million columns
+        // this prologue is not small; a complex element is one load of both parts)
         const R* Ad = reinterpret_cast<const R*>(s.A);
+        typedef R Pair __attribute__((ext_vector_type(2), aligned(sizeof(R))));
 #pragma unroll
         for (int mb = 0; mb < MBM; ++mb)
 #pragma unroll
             for (int i = 0; i < PAIRS; ++i) {
                 const int m = j + 16 * mb, c = 4 * i + g;
+                const int64_t mo = off_of(s.am, m < s.M ? m : s.M - 1);
+                if constexpr (CX) {
 #pragma unroll
-                for (int q = 0; q < QB; ++q) {
-                    const int kk = QB * c + q;              // index into the real form
-                    const int k = kk / NC, part = kk % NC;
-                    R x = 0;
-                    if (m < s.M && k < s.K) {
-                        x = Ad[NC * (off_of(s.am, m) + off_of(s.ak, k)) + part];
-                        if (CX && part == 1 && s.conj_a) x = -x;
+                    for (int e = 0; e < QB / 2; ++e) {
+                        const int k = (QB / 2) * c + e;
+                        const bool ok = m < s.M && k < s.K;
+                        const Pair v = *reinterpret_cast<const Pair*>(Ad + 2 * (mo + off_of(s.ak, k < s.K ? k : s.K - 1)));
+                        a[mb][i][2 * e] = ok ? v[0] : R(0);
+                        a[mb][i][2 * e + 1] = ok ? (s.conj_a ? -v[1] : v[1]) : R(0);
                     }
-                    a[mb][i][q] = x;
+                } else {
+#pragma unroll
+                    for (int q = 0; q < QB; ++q) {
+                        const int k = QB * c + q;
+                        const R x = Ad[mo + off_of(s.ak, k < s.K ? k : s.K - 1)];
+                        a[mb][i][q] = (m < s.M && k < s.K) ? x : R(0);
+                    }
                 }
             }
     }
