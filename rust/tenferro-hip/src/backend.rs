@@ -190,6 +190,14 @@ impl TensorPrims<Standard> for HipBackend {
     /// tenferro-prims/src/lib.rs:300-320.  The views look into DEVICE memory (`HipBuffer::as_device_slice`); the
     /// kernels are enqueued on the calling thread's current stream ([`HipBackend::set_current_stream`]) and the call
     /// does not wait for them.
+    ///
+    /// # Device memory
+    /// The trait's signature cannot say where a `StridedView` lives.  This backend takes the ADDRESSES of the views'
+    /// slices as device addresses: every view handed to it must have been built over
+    /// [`HipBuffer::as_device_slice`] / [`HipBuffer::as_device_slice_mut`] (both `unsafe`, which is where the caller
+    /// takes on that obligation).  A view over ordinary host memory makes the kernels dereference host pointers.  The
+    /// tensor and einsum layers never go through this method: they call [`HipBackend::execute_on`] with [`HipView`]s,
+    /// which can only be made from a `HipBuffer`.
     fn execute<T: ScalarBase>(
         plan: &HipPlan<T>,
         alpha: T,

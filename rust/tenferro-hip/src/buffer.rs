@@ -220,7 +220,10 @@ impl<'a, T: ScalarBase> HipView<'a, T> {
 
     /// From the `StridedView` that `TensorPrims::execute` is handed: the slice under it is device memory
     /// ([`HipBuffer::as_device_slice`]); only its address, dims, strides and offset are read.
-    pub fn from_strided(view: &'a StridedView<'a, T>) -> Result<Self> {
+    pub fn from_strided<'v>(view: &'a StridedView<'v, T>) -> Result<Self>
+    where
+        'v: 'a,
+    {
         check_rank(view.dims().len())?;
         Ok(Self {
             base: view.data().as_ptr(),
@@ -284,8 +287,13 @@ impl<'a, T: ScalarBase> HipViewMut<'a, T> {
         Self { base: buffer.as_device_ptr(), dims: dims.to_vec(), strides: row_major(dims), offset: 0, _buffer: PhantomData }
     }
 
-    /// From the `StridedViewMut` that `TensorPrims::execute` is handed (device memory underneath).
-    pub fn from_strided(view: &'a mut StridedViewMut<'a, T>) -> Result<Self> {
+    /// From the `StridedViewMut` that `TensorPrims::execute` is handed (device memory underneath).  The borrow of the
+    /// view (`'a`) is separate from, and outlived by, the lifetime of the data it views (`'v`): `execute` passes
+    /// `&mut StridedViewMut<T>` whose own lifetime parameter is invariant and unrelated to the borrow.
+    pub fn from_strided<'v>(view: &'a mut StridedViewMut<'v, T>) -> Result<Self>
+    where
+        'v: 'a,
+    {
         check_rank(view.dims().len())?;
         Ok(Self {
             base: view.data().as_ptr() as *mut T,

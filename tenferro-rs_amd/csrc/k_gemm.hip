@@ -1591,8 +1591,14 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
         int4*& slot = (shaped || gs->bm != 128) ? dm.shaped : dm.uniform;
         if (!slot) {
             const size_t nb = map_host.size() * sizeof(int4);
-            if (int32_t e = hip_check(hipMalloc((void**)&slot, std::max<size_t>(nb, 16)), "hipMalloc(tile map)")) return e;
-            if (int32_t e = hip_check(hipMemcpy(slot, map_host.data(), nb, hipMemcpyHostToDevice), "upload tile map")) return e;
+            // (into a local pointer first: the slot must never name a map that was not filled)
+            int4* fresh = nullptr;
+            if (int32_t e = hip_check(hipMalloc((void**)&fresh, std::max<size_t>(nb, 16)), "hipMalloc(tile map)")) return e;
+            if (int32_t e = hip_check(hipMemcpy(fresh, map_host.data(), nb, hipMemcpyHostToDevice), "upload tile map")) {
+                (void)hipFree(fresh);
+                return e;
+            }
+            slot = fresh;
         }
         map_dev = slot;
     }
@@ -1633,6 +1639,8 @@ int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* input
                 r.host = probs;
                 write_records(r.dev);
                 if (int32_t e = hip_check(hipEventRecord(r.ready, st), "hipEventRecord")) {
+                    // the kernels that write the records are enqueued already: they must finish before the block goes
+                    (void)hipStreamSynchronize(st);
                     (void)hipFree(r.dev);
                     (void)hipEventDestroy(r.ready);
                     return e;

@@ -39,10 +39,15 @@ struct StreamScratch {
     std::map<std::string, Tables> tables;
     size_t table_bytes = 0;
     // two pinned host buffers for transfers from and to pageable host memory (allocated on first use)
+    // One staged transfer at a time uses them: bounce_mu is held from a transfer's first chunk to its last, so two host
+    // threads that copy pageable memory on one stream take turns instead of filling each other's staging buffers.
+    std::mutex bounce_mu;
     void* bounce[2] = {nullptr, nullptr};
     hipEvent_t bounce_ev[2] = {nullptr, nullptr};
     bool bounce_busy[2] = {false, false};   // a copy recorded in bounce_ev may still be using the buffer
 };
+// Buffers that a captured graph may still use when their stream is destroyed: kept until the process ends.
+std::vector<void*> g_orphans;
 constexpr size_t BOUNCE_BYTES = (size_t)16 << 20;
 bool capturing(void* stream) {
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
@@ -236,19 +241,36 @@ bool is_pinned_host(const void* p) {
     return attr.type == hipMemoryTypeHost;
 }
 
-int32_t bounce_buffers(void* stream, StreamScratch** out) {
+// The stream's scratch entry (entries of the map stay where they are until their stream is destroyed).
+int32_t bounce_scratch(void* stream, StreamScratch** out) {
     std::lock_guard<std::mutex> lk(g_mu);
     int32_t err;
     StreamScratch* s = scratch_for(stream, &err);
     if (!s) return err;
+    *out = s;
+    return TFH_OK;
+}
+// The two staging buffers, allocated on first use; bounce_mu is held.
+int32_t bounce_buffers(StreamScratch* s) {
     for (int i = 0; i < 2; ++i) {
         if (!s->bounce[i]) {
             if (int32_t e = hip_check(hipHostMalloc(&s->bounce[i], BOUNCE_BYTES, hipHostMallocDefault), "hipHostMalloc(staging buffer)")) return e;
             if (int32_t e = hip_check(hipEventCreateWithFlags(&s->bounce_ev[i], hipEventDisableTiming), "hipEventCreate")) return e;
+            s->bounce_busy[i] = false;
         }
     }
-    *out = s;   // (entries of the map stay where they are: the buffers can be used without the lock)
     return TFH_OK;
+}
+// Frees the staging buffers of a scratch entry; no copy may be using them (the caller has synchronised).
+void free_bounce(StreamScratch& sc) {
+    std::lock_guard<std::mutex> lk(sc.bounce_mu);
+    for (int i = 0; i < 2; ++i) {
+        if (sc.bounce[i]) (void)hipHostFree(sc.bounce[i]);
+        if (sc.bounce_ev[i]) (void)hipEventDestroy(sc.bounce_ev[i]);
+        sc.bounce[i] = nullptr;
+        sc.bounce_ev[i] = nullptr;
+        sc.bounce_busy[i] = false;
+    }
 }
 
 // Pageable host memory cannot be the source or target of an asynchronous copy: the transfer goes through two pinned
@@ -263,7 +285,9 @@ int32_t wait_bounce(StreamScratch* s, int b) {
 }
 int32_t staged_h2d(void* dst, const void* src, size_t bytes, void* stream) {
     StreamScratch* s = nullptr;
-    if (int32_t e = bounce_buffers(stream, &s)) return e;
+    if (int32_t e = bounce_scratch(stream, &s)) return e;
+    std::lock_guard<std::mutex> turn(s->bounce_mu);
+    if (int32_t e = bounce_buffers(s)) return e;
     size_t done = 0;
     for (int i = 0; done < bytes; ++i) {
         const int b = i & 1;
@@ -279,7 +303,9 @@ int32_t staged_h2d(void* dst, const void* src, size_t bytes, void* stream) {
 }
 int32_t staged_d2h(void* dst, const void* src, size_t bytes, void* stream) {
     StreamScratch* s = nullptr;
-    if (int32_t e = bounce_buffers(stream, &s)) return e;
+    if (int32_t e = bounce_scratch(stream, &s)) return e;
+    std::lock_guard<std::mutex> turn(s->bounce_mu);
+    if (int32_t e = bounce_buffers(s)) return e;
     const size_t nchunks = (bytes + BOUNCE_BYTES - 1) / BOUNCE_BYTES;
     auto issue = [&](size_t c) {
         const int b = (int)(c & 1);
@@ -463,6 +489,7 @@ int32_t tfh_release_workspaces(void) {
             sc.table_bytes -= it->second.bytes;
             it = sc.tables.erase(it);
         }
+        tfh::free_bounce(sc);   // (the device is idle: no copy is using the staging buffers)
     }
     return TFH_OK;
 }
@@ -547,7 +574,45 @@ int32_t tfh_stream_create(tfh_stream* out) {
     *out = s;
     return TFH_OK;
 }
-int32_t tfh_stream_destroy(tfh_stream s) { return hip_check(hipStreamDestroy((hipStream_t)s), "hipStreamDestroy"); }
+// The stream's scratch goes with it: workspace, cached intermediates, offset tables and the pinned staging buffers are
+// freed once the stream's work has finished, so that a later stream that happens to get the same handle value starts
+// clean.  Buffers that were handed out during a graph capture stay alive (the graph may be replayed on another stream).
+int32_t tfh_stream_destroy(tfh_stream s) {
+    if (int32_t e = hip_check(hipStreamSynchronize((hipStream_t)s), "hipStreamSynchronize")) return e;
+    {
+        std::lock_guard<std::mutex> lk(tfh::g_mu);
+        int dev = 0;
+        if (hipGetDevice(&dev) == hipSuccess) {
+            auto it = tfh::g_scratch.find({dev, (void*)s});
+            if (it != tfh::g_scratch.end()) {
+                auto& sc = it->second;
+                if (sc.ws) {
+                    if (sc.ws_pinned) tfh::g_orphans.push_back(sc.ws);
+                    else (void)hipFree(sc.ws);
+                }
+                for (void* p : sc.retired) tfh::g_orphans.push_back(p);
+                for (auto& fb : sc.free_blocks) {
+                    if (sc.pinned_blocks.count(fb.second)) tfh::g_orphans.push_back(fb.second);
+                    else (void)hipFree(fb.second);
+                }
+                for (auto& t : sc.tables) {
+                    if (t.second.pinned) tfh::g_orphans.push_back(t.second.dev);
+                    else (void)hipFree(t.second.dev);
+                }
+                tfh::free_bounce(sc);
+                // (blocks still handed out belong to their holders: the entry stays until they are back)
+                if (sc.live.empty()) tfh::g_scratch.erase(it);
+                else {
+                    sc.ws = nullptr; sc.ws_bytes = 0; sc.ws_pinned = false;
+                    sc.retired.clear(); sc.free_blocks.clear(); sc.tables.clear(); sc.table_bytes = 0;
+                }
+            }
+        } else {
+            (void)hipGetLastError();
+        }
+    }
+    return hip_check(hipStreamDestroy((hipStream_t)s), "hipStreamDestroy");
+}
 int32_t tfh_stream_synchronize(tfh_stream s) { return hip_check(hipStreamSynchronize((hipStream_t)s), "hipStreamSynchronize"); }
 
 int32_t tfh_event_create(tfh_event* out) {

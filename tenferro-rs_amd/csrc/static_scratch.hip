@@ -13,6 +13,7 @@
 // race on it.
 #include <hip/hip_runtime.h>
 
+#include <exception>
 #include <mutex>
 
 #include "internal.hpp"
@@ -50,10 +51,19 @@ int32_t tfh_execute_static(const tfh_plan* plan, const void* alpha, const tfh_vi
                            tfh_view* output, tfh_stream stream) {
     void* base = nullptr;
     if (int32_t e = scratch_address(&base)) return e;
-    tfh::arena_begin(base, TFH_STATIC_SCRATCH_BYTES);
-    const int32_t e = tfh_execute(plan, alpha, inputs, n_inputs, beta, output, stream);
-    tfh::arena_end();
-    return e;
+    // (the arena ends with this scope whatever happens inside: an exception out of the host code below -- an allocation
+    // failure of a std::vector, say -- must not leave later calls of this thread carving from the shared array)
+    struct ArenaScope {
+        ArenaScope(void* b, size_t n) { tfh::arena_begin(b, n); }
+        ~ArenaScope() { tfh::arena_end(); }
+    } scope(base, TFH_STATIC_SCRATCH_BYTES);
+    try {
+        return tfh_execute(plan, alpha, inputs, n_inputs, beta, output, stream);
+    } catch (const std::exception& ex) {
+        return tfh::set_error(TFH_ERR_DEVICE, "tfh_execute_static: %s", ex.what());
+    } catch (...) {
+        return tfh::set_error(TFH_ERR_DEVICE, "tfh_execute_static: unknown exception");
+    }
 }
 
 }  // extern "C"

@@ -1092,6 +1092,43 @@ def test_host_transfers_pageable_and_pinned_round_trip(tf):
         L.tfh_stream_destroy(st)
 
 
+def test_two_host_threads_copy_pageable_memory_on_one_stream(tf):
+    # both threads stage through the stream's two pinned buffers: a transfer holds them from its first chunk to its last,
+    # so neither carries the other's bytes; uploads and downloads, several chunks each, on the null stream and on a created one
+    import threading
+    import torch
+    L = tf.lib()
+    (st,) = _new_streams(tf, 1)
+    rng = seeded_rng(136)
+    try:
+        for stream in (None, st):
+            nbytes = [(40 << 20) + 3, (33 << 20) + 1]
+            srcs = [rng.integers(0, 256, n, dtype=np.uint8) for n in nbytes]
+            dbufs = [torch.empty(n, dtype=torch.uint8, device="cuda") for n in nbytes]
+            backs = [np.zeros(n, np.uint8) for n in nbytes]
+            rcs = [[], []]
+
+            def work(i):
+                for _ in range(3):
+                    rcs[i].append(L.tfh_memcpy_h2d(dbufs[i].data_ptr(), srcs[i].ctypes.data, nbytes[i], stream))
+                    rcs[i].append(L.tfh_memcpy_d2h(backs[i].ctypes.data, dbufs[i].data_ptr(), nbytes[i], stream))
+            threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+            for t in threads:
+                t.start()
+            for t in threads:
+                t.join()
+            assert L.tfh_stream_synchronize(stream) == 0
+            for i in range(2):
+                assert rcs[i] == [0] * 6
+                assert np.array_equal(backs[i], srcs[i]), i
+                assert np.array_equal(dbufs[i].cpu().numpy(), srcs[i]), i
+    finally:
+        assert L.tfh_stream_destroy(st) == 0
+    # a destroyed stream leaves no staging buffers behind, and the null stream's go with tfh_release_workspaces
+    torch.cuda.synchronize()
+    assert L.tfh_release_workspaces() == 0
+
+
 def test_host_to_device_copy_runs_beside_a_contraction_on_another_stream(tf):
     # a staged transfer from pageable memory on stream A and contractions on stream B, each alone and then together
     # (the transfer from a second host thread, because its host side is busy copying into the staging buffers): together
