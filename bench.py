@@ -441,6 +441,102 @@ def run_batched(h, dtype, nb, n, cm=False, ref_out=None):
     return res
 
 
+# ------------------------------------------------------------------------------------------------- host cost of a call
+def host_overhead(h):
+    """Microseconds of host time per enqueue (python bench.py --host-overhead): the first execute of a plan (routing, table
+    build, workspace growth) against repeated ones (the plan keeps the routed launch per set of view strides), for a small
+    contraction that is one launch, 128^3 f64 (split-K: two launches), configuration 1 (an operand pack, offset tables,
+    split-K: not replayed) and a grouped plan of 1024 small problems.  Bursts of 200 calls on an idle stream, so that the
+    launch queue never fills; every figure includes the ctypes call itself, measured beside them on tfh_version()."""
+    tf, inputs, torch = h.tf, h.inputs, h.torch
+    L = tf.lib()
+    lines = []
+
+    def measure(name, make_call, n=200, first_note=""):
+        call = make_call()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        call()
+        t_first = (time.perf_counter() - t0) * 1e6
+        torch.cuda.synchronize()
+        for _ in range(20):
+            call()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(5):
+            t0 = time.perf_counter()
+            for _ in range(n):
+                call()
+            t1 = time.perf_counter()
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            rep = ((t1 - t0) * 1e6 / n, (t2 - t0) * 1e6 / n)
+            best = rep if best is None or rep[0] < best[0] else best
+        lines.append("%-58s first call %8.1f us   repeated enqueue %5.2f us   with drain %6.2f us   %s%s" %
+                     (name, t_first, best[0], best[1], tf.last_kernel()[:44], first_note))
+
+    t0 = time.perf_counter()
+    for _ in range(20000):
+        L.tfh_version()
+    floor = (time.perf_counter() - t0) * 1e6 / 20000
+    lines.append("measured from Python through ctypes (a call of a function that does nothing, tfh_version: %.2f us; marshalling the" % floor)
+    lines.append("seven arguments of tfh_execute costs about a microsecond more):")
+
+    def contraction(ma, mb, mc, ext, dtype):
+        def make():
+            rng = np.random.default_rng(3)
+            A = rng.standard_normal([ext[c] for c in ma]).astype(dtype)
+            B = rng.standard_normal([ext[c] for c in mb]).astype(dtype)
+            out = h.empty([ext[c] for c in mc], dtype)
+            plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), [A.shape, B.shape, [ext[c] for c in mc]])
+            call = h.bound_execute(plan, [h.gpu(A), h.gpu(B)], out)
+            make.plan = plan
+            return call
+        return make
+    m = contraction("ij", "jk", "ik", dict(i=64, j=64, k=64), np.float64)
+    measure("Contract ij,jk->ik f64 64^3 (one launch)", m)
+    lines.append("    plan.cache_stats() (hits, misses, routes kept): %r" % (m.plan.cache_stats(),))
+    m = contraction("ij", "jk", "ik", dict(i=128, j=128, k=128), np.float64)
+    measure("Contract ij,jk->ik f64 128^3 (split-K + fold: two launches)", m)
+    lines.append("    plan.cache_stats(): %r" % (m.plan.cache_stats(),))
+    m = contraction("ajbk", "kcj", "abc", dict(a=64, j=128, b=64, k=96, c=256), np.float32)
+    measure("configuration 1 (pack of B, tables, split-K 8)", m)
+    lines.append("    plan.cache_stats(): %r  (a route with an operand pack is not kept: every call routes)" % (m.plan.cache_stats(),))
+
+    def grouped():
+        rng = np.random.default_rng(4)
+        dims = [(int(rng.integers(8, 40)), int(rng.integers(8, 40)), int(rng.integers(8, 40))) for _ in range(1024)]
+        As = [h.gpu(rng.standard_normal((i, j))) for i, j, k in dims]
+        Bs = [h.gpu(rng.standard_normal((j, k))) for i, j, k in dims]
+        outs = [h.empty((i, k), np.float64) for i, j, k in dims]
+        plan = tf.HipBackend.plan_grouped(np.float64, tf.PrimDescriptor.Contract(lab("ij"), lab("jk"), lab("ik")),
+                                          [[[i, j], [j, k], [i, k]] for i, j, k in dims])
+        pairs = list(zip(As, Bs))
+        # marshalled once: the views of all 1024 problems
+        views = (tf.tfh_view * (2 * len(dims)))(*[tf.view_of(t) for pr in pairs for t in pr])
+        vouts = (tf.tfh_view * len(dims))(*[tf.view_of(t) for t in outs])
+        al, be = tf._scalar_c(plan.dtype, 1.0), tf._scalar_c(plan.dtype, 0.0)
+        st = tf.current_stream()
+
+        def call():
+            rc = L.tfh_execute_grouped(plan._h, al, views, 2, be, vouts, st)
+            if rc:
+                tf._check(rc)
+        call.keep = (views, vouts, al, be, pairs, outs, plan)
+        return call
+    measure("grouped plan, 1024 problems of 8..40 (f64)", grouped, n=100)
+    print("\n".join(lines))
+    # the same from C, without the interpreter and ctypes between the calls (tests/cpp/host_overhead.cpp, built by
+    # __graft_entry__.build())
+    prog = os.path.join(ROOT, "tests", "cpp", "host_overhead")
+    if os.path.exists(prog):
+        import subprocess
+        torch.cuda.synchronize()
+        print("\nfrom C (tests/cpp/host_overhead):")
+        sys.stdout.flush()
+        subprocess.run([prog], check=False)
+
+
 LAYOUT_NOTE = {False: "; operands and result row-major", True: "; operands and result column-major (MemoryOrder::ColumnMajor, the order of the reference's examples)"}
 RUNNERS = {"c1": run_c1, "c2": run_c2, "c3": run_c3, "c4": run_c4, "c0": run_matmul,
            "b64": lambda h, cm=False, ref_out=None: run_batched(h, np.float64, 4096, 64, cm, ref_out),
@@ -457,6 +553,8 @@ def main():
     ap.add_argument("--configs", default="c3,c1,c2,c4,c0,b64,b128")
     ap.add_argument("--no-colmajor", action="store_true", help="skip the column-major variants of the configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--host-overhead", action="store_true",
+                    help="print the host cost of tfh_execute per call (first against repeated) instead of running the benchmark")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also launch three plain 1 GiB device-to-device copies (torch's elementwise copy kernel): under "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE their readings give the counter's scale for known traffic")
@@ -464,7 +562,10 @@ def main():
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus %d is not supported\n" % args.gpus)
         sys.exit(2)
-    h = Harness(args.steps, args.warmup, not args.no_cpu)
+    h = Harness(args.steps, args.warmup, not args.no_cpu and not args.host_overhead)
+    if args.host_overhead:
+        host_overhead(h)
+        return
     if args.pmc_calibration:
         src = h.torch.ones(1 << 28, dtype=h.torch.float32, device="cuda")
         dst = h.torch.empty_like(src)

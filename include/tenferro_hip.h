@@ -150,8 +150,15 @@ int32_t tfh_plan_create(int32_t dtype, const tfh_desc* desc,
                         tfh_plan** out);
 void tfh_plan_destroy(tfh_plan* plan);
 
-/* One-line description of what a plan will launch (kernel family, GEMM view M/N/K/batch). */
+/* One-line description of a plan: operation, dtype, and -- for a Contract / BatchedGemm plan that has been executed -- the
+ * kernels of the routes it keeps (one per set of view strides it has seen, see tfh_plan_cache_stats). */
 int32_t tfh_plan_describe(const tfh_plan* plan, char* buf, size_t cap);
+/* "The plan pre-computes kernel selection" (tenferro-prims/src/lib.rs:8, :284): what the route of a contraction depends on
+ * besides the extents -- the views' strides -- only shows at execute, so a Contract / BatchedGemm plan keeps the routed
+ * launch of the first execute with each set of strides (up to eight) and later executes with the same strides enqueue it
+ * again on their buffers without routing.  This reads the plan's counters: executes that found their route, executes
+ * that had to route, routes kept (any pointer may be null; all zero for other operations). */
+int32_t tfh_plan_cache_stats(const tfh_plan* plan, int64_t* hits, int64_t* misses, int32_t* entries);
 
 /* TensorPrims::execute(plan, alpha, inputs, beta, output)  (tenferro-prims/src/lib.rs:300-320).
  * output = alpha*op(inputs) + beta*output; beta == 0 overwrites without reading the output.

@@ -150,6 +150,7 @@ extern "C" {
         n_tensors: i32, out: *mut *mut tfh_plan) -> i32;
     pub fn tfh_plan_destroy(plan: *mut tfh_plan);
     pub fn tfh_plan_describe(plan: *const tfh_plan, buf: *mut c_char, cap: usize) -> i32;
+    pub fn tfh_plan_cache_stats(plan: *const tfh_plan, hits: *mut i64, misses: *mut i64, entries: *mut i32) -> i32;
     pub fn tfh_execute(plan: *const tfh_plan, alpha: *const c_void, inputs: *const tfh_view, n_inputs: i32,
         beta: *const c_void, output: *mut tfh_view, stream: tfh_stream) -> i32;
     pub fn tfh_plan_create_grouped(dtype: i32, desc: *const tfh_desc, n_groups: i32, shapes: *const *const i64,

@@ -41,6 +41,13 @@ impl<T> HipPlan<T> {
         unsafe { sys::tfh_plan_describe(self.raw, buf.as_mut_ptr(), buf.len()) };
         unsafe { CStr::from_ptr(buf.as_ptr()) }.to_string_lossy().into_owned()
     }
+    /// (executes that found their routed launch in the plan, executes that had to route, routes kept): the plan keeps
+    /// the kernel selection of the first execute with each set of view strides (tenferro-prims/src/lib.rs:8, :284).
+    pub fn cache_stats(&self) -> (i64, i64, i32) {
+        let (mut h, mut m, mut e) = (0i64, 0i64, 0i32);
+        unsafe { sys::tfh_plan_cache_stats(self.raw, &mut h, &mut m, &mut e) };
+        (h, m, e)
+    }
     pub(crate) fn raw(&self) -> *const sys::tfh_plan {
         self.raw
     }

@@ -79,6 +79,7 @@ def lib():
         L.tfh_execute.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
         L.tfh_execute_grouped.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
         L.tfh_execute_static.argtypes = L.tfh_execute.argtypes
+        L.tfh_plan_cache_stats.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.tfh_static_scratch_bytes.restype = C.c_size_t
         L.tfh_static_scratch_bytes.argtypes = []
         L.tfh_einsum_execute.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p,
@@ -413,6 +414,12 @@ class HipPlan:
 
     def __init__(self, handle, dtype, n_inputs, grouped=0):
         self._h, self.dtype, self.n_inputs, self.n_groups = handle, dtype, n_inputs, grouped
+
+    def cache_stats(self):
+        """(executes that found their routed launch in the plan, executes that had to route, routes kept)."""
+        h, m, e = C.c_int64(), C.c_int64(), C.c_int32()
+        _check(lib().tfh_plan_cache_stats(self._h, C.byref(h), C.byref(m), C.byref(e)))
+        return h.value, m.value, e.value
 
     def describe(self):
         buf = C.create_string_buffer(256)

@@ -53,6 +53,14 @@ struct tfh_tree {
     std::vector<TreeStep> steps;
     double macs = 0, peak = 0;
     std::atomic<int> refs{1};   // the creator's reference; the tree cache and each of its hits hold one more
+    // One cache of routed launches per step (contract_cache.cpp): executions of the tree on operands with the strides of
+    // an earlier execution enqueue that execution's kernels again without routing.  Made on first use (under step_mu);
+    // an entry that could not be made stays null and its step routes every time.
+    mutable std::mutex step_mu;
+    mutable std::vector<tfh::ContractCache*> step_cache;
+    ~tfh_tree() {
+        for (tfh::ContractCache* c : step_cache) tfh::contract_cache_destroy(c);
+    }
 };
 
 namespace {
@@ -867,6 +875,15 @@ int32_t tfh_einsum_execute(int32_t dtype, const tfh_tree* tree, const tfh_view* 
         if (!alone) continue;
         donated.push_back(Donated{view_ptr(v, dtype), (size_t)count * eb, consumed, false});
     }
+    ContractCache* const* step_caches = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(t.step_mu);
+        if (t.step_cache.empty() && ns > 0) {
+            t.step_cache.resize((size_t)ns, nullptr);
+            for (auto& c : t.step_cache) c = contract_cache_create();
+        }
+        step_caches = t.step_cache.data();   // (the vector is sized once and never touched again)
+    }
     for (int s = 0; s < ns; ++s) {
         const bool last = s == ns - 1;
         const Operand& A = nodes[t.steps[s].lhs];
@@ -901,10 +918,9 @@ int32_t tfh_einsum_execute(int32_t dtype, const tfh_tree* tree, const tfh_view* 
                 C.owned = p;
             }
         }
-        ContractAxes ax;
-        int32_t e = classify_contract(A.labels, A.dims.data(), A.strides.data(), B.labels, B.dims.data(), B.strides.data(), C.labels,
-                                      C.dims.data(), C.strides.data(), ax);
-        if (!e) e = launch_contract(dtype, A.ptr, B.ptr, C.ptr, ax, last ? al : one, last ? be_final : zero, stream, (A.conj ? 1 : 0) | (B.conj ? 2 : 0));
+        int32_t e = execute_contract(step_caches[s], dtype, A.labels, A.dims.data(), A.strides.data(), A.ptr, B.labels, B.dims.data(),
+                                     B.strides.data(), B.ptr, C.labels, C.dims.data(), C.strides.data(), C.ptr, last ? al : one,
+                                     last ? be_final : zero, stream, (A.conj ? 1 : 0) | (B.conj ? 2 : 0));
         // operands of this step are dead once its kernels are enqueued (stream order protects them)
         for (int side = 0; side < 2; ++side) {
             Operand& o = nodes[side ? t.steps[s].rhs : t.steps[s].lhs];

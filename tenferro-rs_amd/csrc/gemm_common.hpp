@@ -34,6 +34,21 @@ struct GroupProblem {   // one problem of a grouped launch (plain strided matric
     int64_t sam, sak, sbk, sbn, scm, scn;
 };
 
+// One launch of the batch-first kernel (k_gemm_bfirst.hip): batched products whose batch index is the contiguous one.
+struct BfArgs {
+    const void* A;
+    const void* B;
+    void* C;
+    int64_t nb;                              // extent of the contiguous batch axis
+    int64_t nbo;                             // extent of an outer batch axis (1: none)
+    int64_t M, N, K;
+    int64_t sam, sak, sbk, sbn, scm, scn;    // element strides of the row, column and k axes
+    int64_t sao, sbo, sco;                   // element strides of the outer batch axis
+    int32_t tiles_m, tiles_n, groups;        // groups of NB batch entries
+    int32_t conj_a, conj_b, use_beta;
+    double alpha_re, alpha_im, beta_re, beta_im;
+};
+
 struct GemmArgs {
     const void* A;
     const void* B;

@@ -3,6 +3,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <memory>
 #include <string>
 #include <utility>
 #include <vector>
@@ -58,6 +59,7 @@ struct Axis {
 
 // ---- plan ----------------------------------------------------------------------------------------
 struct GroupedState;  // device tables of a grouped plan (gemm.cpp)
+struct ContractCache;  // routed launches of earlier calls of a Contract / BatchedGemm plan (contract_cache.cpp)
 }  // namespace tfh
 
 struct tfh_plan {
@@ -71,6 +73,10 @@ struct tfh_plan {
     std::vector<std::vector<int64_t>> shapes;
     int32_t n_groups = 0;  // 0 = not grouped
     tfh::GroupedState* grouped = nullptr;
+    // Kernel selection is part of the plan (tenferro-prims/src/lib.rs:8, :284): the first execute with a given set of view
+    // strides routes the contraction and keeps the routed launch here; later executes with the same strides only patch
+    // the buffer addresses and scalars into it.  Guarded by its own lock: the plan stays shareable between threads.
+    tfh::ContractCache* contract_cache = nullptr;
     ~tfh_plan();
 };
 
@@ -112,10 +118,36 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
 // two operands read at the same coordinates (sum only).  Axis slots here: 0 = A, 1 = C, 2 = B.
 int32_t launch_reduce_general(int dtype, const void* a, const void* b, void* c, std::vector<Axis> kept, std::vector<Axis> red,
                               int reduce_op, Scalar alpha, Scalar beta, void* stream);
+// What a contraction's launcher leaves behind for a repeated call: the routed launch (kernel, tile and split choice,
+// operand exchange, table handles) with the buffer addresses and scalars taken out.  Defined by the launcher.
+struct ContractRecord {
+    std::string label;   // the kernel the route ends in, as tfh_last_kernel names it
+    virtual ~ContractRecord() = default;
+};
 // C = alpha*A*B + beta*C over classified axes
 // conj: bit 0 = conj(A), bit 1 = conj(B) (see k_gemm.hip)
+// record: when non-null and the route is one that can be enqueued again without routing (no operand pack, no per-call
+// table build), *record receives it.
 int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes axes, Scalar alpha,
-                        Scalar beta, void* stream, int conj = 0);
+                        Scalar beta, void* stream, int conj = 0, std::shared_ptr<ContractRecord>* record = nullptr);
+// Enqueues a recorded launch on new buffers (a, b: the first and second input as the caller passes them).  Returns false
+// when the record no longer applies (the offset tables it names were released, another device is current): the caller
+// routes the call again.
+bool replay_contract(const ContractRecord& rec, int dtype, const void* a, const void* b, void* c, Scalar alpha, Scalar beta,
+                     void* stream, int32_t& status);
+// A contraction through a cache of routed launches (null: no cache).  The key is everything the route depends on besides
+// the extents, which are fixed where the cache lives (a plan, a step of an einsum tree): the element type (a tree serves
+// every type), the three views' strides, the 16-byte alignment classes of their addresses, the conj flags, whether beta
+// is zero, the stream.
+ContractCache* contract_cache_create();
+void contract_cache_destroy(ContractCache* c);
+void contract_cache_stats(const ContractCache* c, int64_t* hits, int64_t* misses, int32_t* entries);
+// "<kernel label>; <kernel label>; ..." of the routes kept, oldest first (empty: none yet).
+std::string contract_cache_routes(const ContractCache* c);
+int32_t execute_contract(ContractCache* cache, int dtype, const std::vector<uint32_t>& ma, const int64_t* dims_a, const int64_t* str_a,
+                         const void* a, const std::vector<uint32_t>& mb, const int64_t* dims_b, const int64_t* str_b, const void* b,
+                         const std::vector<uint32_t>& mc, const int64_t* dims_c, const int64_t* str_c, void* c, Scalar alpha,
+                         Scalar beta, void* stream, int conj);
 // A tiny operator (<= 8 free and <= 8 contracted indices) applied to a long tensor: the streaming kernel of
 // k_gemm_tiny.hip.  Returns false when the shape is not one it takes; true when it launched (status holds the outcome).
 bool try_tiny_operator(int dtype, const void* a, const void* b, void* c, const ContractAxes& ax, Scalar alpha, Scalar beta,
@@ -124,11 +156,9 @@ bool try_tiny_operator(int dtype, const void* a, const void* b, void* c, const C
 // false when the shape is not one it tiles; true when it launched (status holds the outcome).  Axis strides: A, B, C.
 bool try_dot(int dtype, const void* a, const void* b, void* c, std::vector<Axis> kept, std::vector<Axis> red, Scalar alpha,
              Scalar beta, void* stream, int32_t& status);
-// Batched products whose batch index is the contiguous one in all three tensors (column-major "bij,bjk->bik"): the kernel
-// of k_gemm_bfirst.hip, whose blocks take all the batch entries of a 128-byte line at once.  Returns false when the shape
-// is not one it takes; true when it launched (status holds the outcome).
-bool try_batch_first(int dtype, const void* a, const void* b, void* c, const ContractAxes& ax, Scalar alpha, Scalar beta,
-                     void* stream, bool conj_a, bool conj_b, int32_t& status);
+// Counts the releases of cached offset tables (tfh_release_workspaces, a destroyed stream, the out-of-memory path): a
+// recorded launch that names such tables is valid only while the count stands where it stood when the record was made.
+uint64_t table_epoch();
 int32_t grouped_plan_init(tfh_plan& plan);
 int32_t launch_grouped(const tfh_plan& plan, Scalar alpha, const tfh_view* inputs, Scalar beta, tfh_view* outputs,
                        void* stream);

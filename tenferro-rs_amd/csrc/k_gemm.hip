@@ -597,9 +597,41 @@ int bke_of(int dtype) {
 
 }  // namespace
 
+// k_gemm_bfirst.hip: batched products whose batch index is the contiguous one in all three tensors (column-major
+// "bij,bjk->bik").  try_batch_first returns false when the shape is not one that kernel takes; true when it launched
+// (status holds the outcome; *routed, when given, the arguments it launched with).
+bool try_batch_first(int dtype, const void* a, const void* b, void* c, const ContractAxes& ax, Scalar alpha, Scalar beta,
+                     void* stream, bool conj_a, bool conj_b, int32_t& status, gemm::BfArgs* routed);
+int32_t launch_batch_first(int dtype, const gemm::BfArgs& g, void* stream);
+
 namespace {
+// A routed launch, kept for repeated calls (ContractRecord): the kernel's argument block as the router built it, with
+// what changes from call to call noted beside it -- which input each kernel operand is (the router may have exchanged
+// them), the byte distance from a view's first element to the rebased operand base of the large-tile kernel, the size
+// of the split-K partials (the workspace is asked for again on every call) and which fold kernel follows.
+struct GemmRecord : ContractRecord {
+    enum Kind { TILES, BATCH_FIRST } kind = TILES;
+    GemmArgs g;
+    BfArgs bf;
+    uint32_t grid = 0;
+    int bn = 0, bm = 0;
+    bool use128 = false;
+    int src_a = 0, src_b = 1;          // input index of the kernel's A and B
+    int64_t d_a32 = 0, d_b32 = 0;      // g.A32 - A, g.B32 - B in bytes
+    size_t partial_bytes = 0;
+    int fold = 0;                      // 0: none, 1: many splits, 2: 16-byte fold, 3: element-wise fold
+    uint32_t fold_grid = 0;
+    bool has_tables = false;           // g points into the stream's cache of offset tables
+    uint64_t epoch = 0;                // table_epoch() when the record was made
+    int device = 0;
+};
+// The record the router fills while launch_contract runs on this thread (null: none wanted, or the route took a turn
+// that cannot be replayed: an operand pack, a conjugated copy, tables built into the workspace).
+thread_local GemmRecord* t_record = nullptr;
+
 int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, ContractAxes ax, Scalar alpha, Scalar beta,
                              void* stream, bool conj_a, bool conj_b);
+void launch_fold(int dtype, int fold, uint32_t fold_grid, const GemmArgs& g, hipStream_t st);
 }
 
 // conj: bit 0 = use conj(A), bit 1 = use conj(B) (complex dtypes; ignored for real ones).  The tiled and the streaming
@@ -608,11 +640,22 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
 // indices: the tiny-operator, product-reduction and elementwise kernels -- get a conjugated copy of the flagged operand
 // first (one pass of the copy kernel over it).
 int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes ax, Scalar alpha, Scalar beta,
-                        void* stream, int conj) {
+                        void* stream, int conj, std::shared_ptr<ContractRecord>* record) {
     bool ca = (conj & 1) != 0 && is_complex(dtype), cb = (conj & 2) != 0 && is_complex(dtype);
-    if (!ca && !cb) return launch_contract_impl(dtype, a, b, c, ax, alpha, beta, stream, false, false);
     const int64_t M = prod(ax.M), N = prod(ax.N);
-    if (M > 8 && N > 8) return launch_contract_impl(dtype, a, b, c, ax, alpha, beta, stream, ca, cb);
+    if ((!ca && !cb) || (M > 8 && N > 8)) {
+        if (!record) return launch_contract_impl(dtype, a, b, c, ax, alpha, beta, stream, ca, cb);
+        // the router fills the record when the route it takes can be replayed; it stays empty (grid 0) otherwise
+        auto rec = std::make_shared<GemmRecord>();
+        t_record = rec.get();
+        const int32_t e = launch_contract_impl(dtype, a, b, c, ax, alpha, beta, stream, ca, cb);
+        t_record = nullptr;
+        if (!e && rec->grid) {
+            rec->label = tfh_last_kernel();
+            *record = std::move(rec);
+        }
+        return e;
+    }
     const size_t eb = dtype_size(dtype);
     void* copies[2] = {nullptr, nullptr};
     auto release = [&]() {
@@ -660,6 +703,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     if (((uintptr_t)a % eb) || ((uintptr_t)b % eb) || ((uintptr_t)c % rb))
         return set_error(TFH_ERR_STRIDED, "view base is not aligned to the element size");
     hipStream_t st = (hipStream_t)stream;
+    int src_a = 0, src_b = 1;   // which of the caller's inputs the kernel's A and B are (they may be exchanged below)
     int64_t nb = prod(ax.batch), M = prod(ax.M), N = prod(ax.N), K = prod(ax.K);
     if (nb == 0 || M == 0 || N == 0) return TFH_OK;
     for (auto* grp : {&ax.batch, &ax.M, &ax.N})
@@ -724,11 +768,21 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     // the batch index contiguous in all three tensors (column-major "bij,bjk->bik"): a kernel of its own, no packing
     if (M > 1 && N > 1 && nb > 1) {
         int32_t st_bf = TFH_OK;
-        if (try_batch_first(dtype, a, b, c, ax, alpha, beta, stream, conj_a, conj_b, st_bf)) return st_bf;
+        GemmRecord* rec = t_record;
+        if (try_batch_first(dtype, a, b, c, ax, alpha, beta, stream, conj_a, conj_b, st_bf, rec ? &rec->bf : nullptr)) {
+            if (rec && !st_bf) {
+                rec->kind = GemmRecord::BATCH_FIRST;
+                rec->grid = 1;
+                rec->epoch = table_epoch();
+                (void)hipGetDevice(&rec->device);
+            }
+            return st_bf;
+        }
     }
     // lanes of the epilogue run along n: put C's fastest axis in the N group (swap operands if needed)
     if (min_stride(ax.M, 2) < min_stride(ax.N, 2)) {
         std::swap(a, b);
+        std::swap(src_a, src_b);
         std::swap(conj_a, conj_b);
         std::swap(ax.M, ax.N);
         std::swap(M, N);
@@ -752,6 +806,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
         }
         if (M < 96 && M * ec >= 33 && N * ec >= 96 && !streamable) {
             std::swap(a, b);
+            std::swap(src_a, src_b);
             std::swap(conj_a, conj_b);
             std::swap(ax.M, ax.N);
             std::swap(M, N);
@@ -846,6 +901,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
              std::llabs(in.s[2]) * SKINNY_UNIT * (int64_t)eb < ((int64_t)1 << 31);
         if (ok) {
             std::swap(a, b);
+            std::swap(src_a, src_b);
             std::swap(conj_a, conj_b);
             std::swap(ax.M, ax.N);
             std::swap(M, N);
@@ -873,6 +929,7 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
              std::llabs(ax.M.back().s[2]) * SKINNY_UNIT * (int64_t)eb < ((int64_t)1 << 31);
         if (ok) {
             std::swap(a, b);
+            std::swap(src_a, src_b);
             std::swap(conj_a, conj_b);
             std::swap(ax.M, ax.N);
             std::swap(M, N);
@@ -1195,6 +1252,26 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     if (nsplit > 1) g.partial = ws + (cached ? 0 : table_bytes);
     dim3 grid((uint32_t)((int64_t)g.tiles_m * g.tiles_n * nb * nsplit), 1, 1);
     g.one_round = bm == 128 && grid.x <= 2u * compute_units();   // two blocks of the 128-tile kernel fit a CU
+    // what a repeated call needs to enqueue this launch again: kept when the route used neither an operand pack nor
+    // tables of its own in the workspace (the cached tables stay where they are until they are released)
+    GemmRecord* rec = t_record;
+    if (rec && (skinny || wavek || packed[0] || packed[1] || (njobs && !cached))) rec = nullptr;
+    if (rec) {
+        rec->kind = GemmRecord::TILES;
+        rec->g = g;
+        rec->grid = grid.x;
+        rec->bn = bn;
+        rec->bm = bm;
+        rec->use128 = use128;
+        rec->src_a = src_a;
+        rec->src_b = src_b;
+        rec->d_a32 = use128 ? lo_a * (int64_t)eb : 0;
+        rec->d_b32 = use128 ? lo_b * (int64_t)eb : 0;
+        rec->partial_bytes = partial_bytes;
+        rec->has_tables = njobs != 0;
+        rec->epoch = table_epoch();
+        (void)hipGetDevice(&rec->device);
+    }
     const int prof = prof_begin(PROF_CONTRACT, stream);
     if (skinny) {
         SkinnyArgs sk;
@@ -1219,47 +1296,106 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
     prof_end(prof, stream);
     release_packed();   // stream-ordered: the next user of these blocks is enqueued after this kernel
     if (int32_t e = hip_check(hipGetLastError(), "contraction kernel launch")) return e;
+    // the fold of the split-K partials (fixed order: deterministic)
+    int fold = 0;
+    uint32_t fold_grid = 0;
     if (nsplit > 32) {
-        const int64_t total = nb * M * N;
-        dim3 g2((uint32_t)((total + 15) / 16));
-        switch (dtype) {
-            case TFH_F32: hipLaunchKernelGGL((splitk_finalize_deep_kernel<float, false>), g2, dim3(THREADS), 0, st, g); break;
-            case TFH_F64: hipLaunchKernelGGL((splitk_finalize_deep_kernel<double, false>), g2, dim3(THREADS), 0, st, g); break;
-            case TFH_C64: hipLaunchKernelGGL((splitk_finalize_deep_kernel<float, true>), g2, dim3(THREADS), 0, st, g); break;
-            default: hipLaunchKernelGGL((splitk_finalize_deep_kernel<double, true>), g2, dim3(THREADS), 0, st, g); break;
-        }
-        return hip_check(hipGetLastError(), "split-K finalize launch");
-    }
-    if (nsplit > 1) {
+        fold = 1;
+        fold_grid = (uint32_t)((nb * M * N + 15) / 16);
+    } else if (nsplit > 1) {
         // 16-byte fold: C contiguous along n, whole vectors per row, every row of C on a 16-byte boundary
         const int64_t vec = 16 / rb, ncx = cx ? 2 : 1;
         bool fold_vec = !g.cn.tab && g.cn.stride == 1 && NR % vec == 0 && (uintptr_t)c % 16 == 0;
         for (auto* grp : {&ax.M, &ax.batch})
             for (auto& x : *grp) fold_vec = fold_vec && (x.n == 1 || (x.s[2] * ncx) % vec == 0);
-        if (fold_vec) {
-            const int64_t total = nb * M * (NR / vec);
-            dim3 g2((uint32_t)((total + THREADS - 1) / THREADS));
-            switch (dtype) {
-                case TFH_F32: hipLaunchKernelGGL((splitk_finalize_vec_kernel<float, false>), g2, dim3(THREADS), 0, st, g); break;
-                case TFH_F64: hipLaunchKernelGGL((splitk_finalize_vec_kernel<double, false>), g2, dim3(THREADS), 0, st, g); break;
-                case TFH_C64: hipLaunchKernelGGL((splitk_finalize_vec_kernel<float, true>), g2, dim3(THREADS), 0, st, g); break;
-                default: hipLaunchKernelGGL((splitk_finalize_vec_kernel<double, true>), g2, dim3(THREADS), 0, st, g); break;
-            }
-            return hip_check(hipGetLastError(), "split-K finalize launch");
-        }
-        int64_t total = nb * M * N;
-        dim3 g2((uint32_t)((total + THREADS - 1) / THREADS));
-        switch (dtype) {
-            case TFH_F32: hipLaunchKernelGGL((splitk_finalize_kernel<float, false>), g2, dim3(THREADS), 0, st, g); break;
-            case TFH_F64: hipLaunchKernelGGL((splitk_finalize_kernel<double, false>), g2, dim3(THREADS), 0, st, g); break;
-            case TFH_C64: hipLaunchKernelGGL((splitk_finalize_kernel<float, true>), g2, dim3(THREADS), 0, st, g); break;
-            default: hipLaunchKernelGGL((splitk_finalize_kernel<double, true>), g2, dim3(THREADS), 0, st, g); break;
-        }
+        fold = fold_vec ? 2 : 3;
+        fold_grid = fold_vec ? (uint32_t)((nb * M * (NR / vec) + THREADS - 1) / THREADS) : (uint32_t)((nb * M * N + THREADS - 1) / THREADS);
+    }
+    if (rec) {
+        rec->fold = fold;
+        rec->fold_grid = fold_grid;
+    }
+    if (fold) {
+        launch_fold(dtype, fold, fold_grid, g, st);
         if (int32_t e = hip_check(hipGetLastError(), "split-K finalize launch")) return e;
     }
     return TFH_OK;
 }
+
+void launch_fold(int dtype, int fold, uint32_t fold_grid, const GemmArgs& g, hipStream_t st) {
+    const dim3 g2(fold_grid), blk(THREADS);
+    if (fold == 1) {
+        switch (dtype) {
+            case TFH_F32: hipLaunchKernelGGL((splitk_finalize_deep_kernel<float, false>), g2, blk, 0, st, g); break;
+            case TFH_F64: hipLaunchKernelGGL((splitk_finalize_deep_kernel<double, false>), g2, blk, 0, st, g); break;
+            case TFH_C64: hipLaunchKernelGGL((splitk_finalize_deep_kernel<float, true>), g2, blk, 0, st, g); break;
+            default: hipLaunchKernelGGL((splitk_finalize_deep_kernel<double, true>), g2, blk, 0, st, g); break;
+        }
+    } else if (fold == 2) {
+        switch (dtype) {
+            case TFH_F32: hipLaunchKernelGGL((splitk_finalize_vec_kernel<float, false>), g2, blk, 0, st, g); break;
+            case TFH_F64: hipLaunchKernelGGL((splitk_finalize_vec_kernel<double, false>), g2, blk, 0, st, g); break;
+            case TFH_C64: hipLaunchKernelGGL((splitk_finalize_vec_kernel<float, true>), g2, blk, 0, st, g); break;
+            default: hipLaunchKernelGGL((splitk_finalize_vec_kernel<double, true>), g2, blk, 0, st, g); break;
+        }
+    } else {
+        switch (dtype) {
+            case TFH_F32: hipLaunchKernelGGL((splitk_finalize_kernel<float, false>), g2, blk, 0, st, g); break;
+            case TFH_F64: hipLaunchKernelGGL((splitk_finalize_kernel<double, false>), g2, blk, 0, st, g); break;
+            case TFH_C64: hipLaunchKernelGGL((splitk_finalize_kernel<float, true>), g2, blk, 0, st, g); break;
+            default: hipLaunchKernelGGL((splitk_finalize_kernel<double, true>), g2, blk, 0, st, g); break;
+        }
+    }
+}
 }  // namespace
+
+// A repeated call: the recorded argument block with this call's addresses and scalars, enqueued as the router
+// enqueued it.  Nothing is classified, fused, chosen or allocated on the host (the split-K partials come out of the
+// stream's workspace, which has the size from the first call).
+bool replay_contract(const ContractRecord& base, int dtype, const void* a, const void* b, void* c, Scalar alpha, Scalar beta,
+                     void* stream, int32_t& status) {
+    const GemmRecord& r = static_cast<const GemmRecord&>(base);
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev != r.device) return false;
+    if (r.kind == GemmRecord::BATCH_FIRST) {
+        BfArgs g = r.bf;
+        g.A = a; g.B = b; g.C = c;
+        g.alpha_re = alpha.re; g.alpha_im = alpha.im; g.beta_re = beta.re; g.beta_im = beta.im;
+        status = launch_batch_first(dtype, g, stream);
+        return true;
+    }
+    if (r.has_tables) {
+        // the tables the arguments name live in the stream's cache: gone after a release, and a graph that is being
+        // captured must pin them, which the router does
+        if (r.epoch != table_epoch() || stream_is_capturing(stream)) return false;
+    }
+    GemmArgs g = r.g;
+    const void* in[2] = {a, b};
+    g.A = in[r.src_a];
+    g.B = in[r.src_b];
+    g.C = c;
+    if (r.use128) {
+        g.A32 = (const char*)g.A + r.d_a32;
+        g.B32 = (const char*)g.B + r.d_b32;
+    }
+    g.alpha_re = alpha.re; g.alpha_im = alpha.im; g.beta_re = beta.re; g.beta_im = beta.im;
+    if (r.partial_bytes) {
+        void* p = nullptr;
+        if ((status = workspace(stream, r.partial_bytes, &p)) != TFH_OK) return true;
+        g.partial = p;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int prof = prof_begin(PROF_CONTRACT, stream);
+    if (r.use128) launch_128(dtype, g, dim3(r.grid), st, r.bn, r.bm);
+    else launch_generic64(dtype, g, dim3(r.grid), st);
+    prof_end(prof, stream);
+    if ((status = hip_check(hipGetLastError(), "contraction kernel launch")) != TFH_OK) return true;
+    if (r.fold) {
+        launch_fold(dtype, r.fold, r.fold_grid, g, st);
+        status = hip_check(hipGetLastError(), "split-K finalize launch");
+    }
+    return true;
+}
 
 // ---- grouped launch ------------------------------------------------------------------------------------------
 struct GroupedState {

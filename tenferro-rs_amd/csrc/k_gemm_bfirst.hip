@@ -33,19 +33,6 @@
 namespace tfh {
 namespace gemm {
 
-struct BfArgs {
-    const void* A;
-    const void* B;
-    void* C;
-    int64_t nb;                              // extent of the contiguous batch axis
-    int64_t nbo;                             // extent of an outer batch axis (1: none)
-    int64_t M, N, K;
-    int64_t sam, sak, sbk, sbn, scm, scn;    // element strides of the row, column and k axes
-    int64_t sao, sbo, sco;                   // element strides of the outer batch axis
-    int32_t tiles_m, tiles_n, groups;        // groups of NB batch entries
-    int32_t conj_a, conj_b, use_beta;
-    double alpha_re, alpha_im, beta_re, beta_im;
-};
 
 template <class R, bool CX>
 struct BfCfg {
@@ -399,8 +386,22 @@ void sort_by_c(std::vector<Axis>& ax) {
 }  // namespace
 
 // Returns false when the shape is not one this kernel takes; true when it launched (status holds the outcome).
+int32_t launch_batch_first(int dtype, const gemm::BfArgs& g, void* stream) {
+    using namespace gemm;
+    hipStream_t st = (hipStream_t)stream;
+    const int prof = prof_begin(PROF_CONTRACT, stream);
+    switch (dtype) {
+        case TFH_F32: launch_bfirst_t<float, false, 2>(g, st); break;
+        case TFH_F64: launch_bfirst_t<double, false, 2>(g, st); break;
+        case TFH_C64: launch_bfirst_t<float, true, 2>(g, st); break;
+        default: launch_bfirst_t<double, true, 2>(g, st); break;
+    }
+    prof_end(prof, stream);
+    return hip_check(hipGetLastError(), "batch-first contraction kernel");
+}
+
 bool try_batch_first(int dtype, const void* a, const void* b, void* c, const ContractAxes& ax0, Scalar alpha, Scalar beta,
-                     void* stream, bool conj_a, bool conj_b, int32_t& status) {
+                     void* stream, bool conj_a, bool conj_b, int32_t& status, gemm::BfArgs* routed) {
     using namespace gemm;
     if (ax0.batch.empty() || ax0.M.empty() || ax0.N.empty() || ax0.K.empty()) return false;
     const int64_t eb = (int64_t)dtype_size(dtype);
@@ -444,16 +445,8 @@ bool try_batch_first(int dtype, const void* a, const void* b, void* c, const Con
     g.conj_a = conj_a; g.conj_b = conj_b;
     g.use_beta = !beta.is_zero();
     g.alpha_re = alpha.re; g.alpha_im = alpha.im; g.beta_re = beta.re; g.beta_im = beta.im;
-    hipStream_t st = (hipStream_t)stream;
-    const int prof = prof_begin(PROF_CONTRACT, stream);
-    switch (dtype) {
-        case TFH_F32: launch_bfirst_t<float, false, 2>(g, st); break;
-        case TFH_F64: launch_bfirst_t<double, false, 2>(g, st); break;
-        case TFH_C64: launch_bfirst_t<float, true, 2>(g, st); break;
-        default: launch_bfirst_t<double, true, 2>(g, st); break;
-    }
-    prof_end(prof, stream);
-    status = hip_check(hipGetLastError(), "batch-first contraction kernel");
+    if (routed) *routed = g;
+    status = launch_batch_first(dtype, g, stream);
     return true;
 }
 

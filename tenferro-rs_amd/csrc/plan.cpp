@@ -9,6 +9,7 @@
 
 tfh_plan::~tfh_plan() {
     if (grouped) tfh::grouped_state_destroy(grouped);
+    if (contract_cache) tfh::contract_cache_destroy(contract_cache);
 }
 
 namespace tfh {
@@ -272,6 +273,9 @@ int32_t tfh_plan_create(int32_t dtype, const tfh_desc* desc, const int64_t* cons
         delete p;
         return e;
     }
+    // kernel selection happens at the first execute with a given set of view strides and is kept here (a plan that
+    // could not get the cache still works: every execute then routes afresh)
+    if (p->op == TFH_OP_CONTRACT || p->op == TFH_OP_BATCHED_GEMM) p->contract_cache = tfh::contract_cache_create();
     *out = p;
     tfh::clear_error();
     return TFH_OK;

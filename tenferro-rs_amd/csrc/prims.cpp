@@ -135,10 +135,9 @@ int32_t tfh_execute(const tfh_plan* plan, const void* alpha, const tfh_view* inp
         }
         case TFH_OP_CONTRACT:
         case TFH_OP_BATCHED_GEMM: {
-            ContractAxes ax;
-            e = classify_contract(plan->modes_a, inputs[0].dims, inputs[0].strides, plan->modes_b, inputs[1].dims, inputs[1].strides,
-                                  plan->modes_c, output->dims, output->strides, ax);
-            if (!e) e = launch_contract(dt, view_ptr(inputs[0], dt), view_ptr(inputs[1], dt), view_ptr(*output, dt), ax, al, be, stream, conj);
+            e = execute_contract(plan->contract_cache, dt, plan->modes_a, inputs[0].dims, inputs[0].strides, view_ptr(inputs[0], dt),
+                                 plan->modes_b, inputs[1].dims, inputs[1].strides, view_ptr(inputs[1], dt), plan->modes_c, output->dims,
+                                 output->strides, view_ptr(*output, dt), al, be, stream, conj);
             break;
         }
         default: e = set_error(TFH_ERR_INVALID_ARGUMENT, "unknown operation %d", plan->op);
@@ -160,11 +159,20 @@ int32_t tfh_execute_grouped(const tfh_plan* plan, const void* alpha, const tfh_v
     return e;
 }
 
+int32_t tfh_plan_cache_stats(const tfh_plan* plan, int64_t* hits, int64_t* misses, int32_t* entries) {
+    if (!plan) return set_error(TFH_ERR_INVALID_ARGUMENT, "null plan");
+    contract_cache_stats(plan->contract_cache, hits, misses, entries);
+    return TFH_OK;
+}
+
 int32_t tfh_plan_describe(const tfh_plan* plan, char* buf, size_t cap) {
     if (!plan || !buf || !cap) return set_error(TFH_ERR_INVALID_ARGUMENT, "null argument");
     static const char* ops[] = {"BatchedGemm", "Reduce", "Trace", "Permute", "AntiTrace", "AntiDiag", "Contract", "ElementwiseMul"};
     static const char* dts[] = {"f32", "f64", "c64", "c128"};
-    snprintf(buf, cap, "%s<%s> inputs=%d groups=%d", ops[plan->op], dts[plan->dtype], plan->n_inputs, plan->n_groups);
+    // kernel selection is kept per set of view strides from the first execute on: the routes the plan holds so far
+    const std::string routes = contract_cache_routes(plan->contract_cache);
+    snprintf(buf, cap, "%s<%s> inputs=%d groups=%d%s%s", ops[plan->op], dts[plan->dtype], plan->n_inputs, plan->n_groups,
+             routes.empty() ? "" : " routes: ", routes.c_str());
     return TFH_OK;
 }
 

@@ -5,6 +5,7 @@
 
 #include <algorithm>
 #include <cstring>
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <set>
@@ -61,6 +62,7 @@ constexpr size_t TABLE_CACHE_BYTES = (size_t)64 << 20;   // per stream; beyond i
 constexpr size_t TABLE_CACHE_ENTRIES = 256;
 std::mutex g_mu;
 std::map<std::pair<int, void*>, StreamScratch> g_scratch;   // (device, stream)
+std::atomic<uint64_t> g_table_epoch{0};   // see table_epoch()
 
 // While a call made through tfh_execute_static is running on this thread, every piece of device scratch it asks for
 // (workspace, packed operands, offset tables) is carved out of a fixed region handed in by arena_begin(); nothing is
@@ -183,6 +185,8 @@ int32_t table_cache_get(void* stream, const std::string& key, size_t bytes, void
     *fresh = true;
     return TFH_OK;
 }
+
+uint64_t table_epoch() { return g_table_epoch.load(std::memory_order_acquire); }
 
 void table_cache_commit(void* stream, const std::string& key) {
     std::lock_guard<std::mutex> lk(g_mu);
@@ -464,6 +468,7 @@ const char* tfh_last_kernel(void) { return tfh::last_kernel(); }
 
 int32_t tfh_release_workspaces(void) {
     std::lock_guard<std::mutex> lk(tfh::g_mu);
+    tfh::g_table_epoch.fetch_add(1, std::memory_order_acq_rel);   // recorded launches that name cached tables are void from here on
     if (int32_t e = hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize")) return e;
     for (auto& kv : tfh::g_scratch) {
         auto& sc = kv.second;
@@ -586,6 +591,7 @@ int32_t tfh_stream_destroy(tfh_stream s) {
             auto it = tfh::g_scratch.find({dev, (void*)s});
             if (it != tfh::g_scratch.end()) {
                 auto& sc = it->second;
+                if (!sc.tables.empty()) tfh::g_table_epoch.fetch_add(1, std::memory_order_acq_rel);
                 if (sc.ws) {
                     if (sc.ws_pinned) tfh::g_orphans.push_back(sc.ws);
                     else (void)hipFree(sc.ws);

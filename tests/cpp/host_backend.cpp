@@ -9,6 +9,7 @@
 // arithmetic, so a whole call -- views in, result out -- runs on the CPU with every host-side index, stride table and
 // buffer lifetime under the sanitizers, and its result can be compared with the oracle's.
 // Test infrastructure only: nothing here is linked into libtenferro_hip.so.
+#include <atomic>
 #include <complex>
 #include <cstdlib>
 #include <cstring>
@@ -117,7 +118,26 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
     return TFH_OK;
 }
 
-int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes ax, Scalar alpha, Scalar beta, void*, int conj) {
+// The stand-in's routed launch: the classified axes.  A repeated call with the same strides (contract_cache.cpp) runs the
+// loop nest over them again on the new buffers.
+namespace {
+struct HostRecord : ContractRecord {
+    ContractAxes ax;
+    int conj = 0;
+};
+std::atomic<int64_t> g_replays{0};
+}  // namespace
+int64_t host_backend_replays() { return g_replays.load(); }
+
+int32_t launch_contract(int dtype, const void* a, const void* b, void* c, ContractAxes ax, Scalar alpha, Scalar beta, void*, int conj,
+                        std::shared_ptr<ContractRecord>* record) {
+    if (record) {
+        auto r = std::make_shared<HostRecord>();
+        r->ax = ax;
+        r->conj = conj;
+        r->label = "(host loop nest)";
+        *record = std::move(r);
+    }
     std::vector<Axis> free_axes = ax.batch;
     free_axes.insert(free_axes.end(), ax.M.begin(), ax.M.end());
     free_axes.insert(free_axes.end(), ax.N.begin(), ax.N.end());
@@ -132,6 +152,14 @@ int32_t launch_contract(int dtype, const void* a, const void* b, void* c, Contra
         store(dtype, c, ic, combine(dtype, alpha, acc, beta, c, ic));
     });
     return TFH_OK;
+}
+
+bool replay_contract(const ContractRecord& rec, int dtype, const void* a, const void* b, void* c, Scalar alpha, Scalar beta, void* stream,
+                     int32_t& status) {
+    const HostRecord& r = static_cast<const HostRecord&>(rec);
+    ++g_replays;
+    status = launch_contract(dtype, a, b, c, r.ax, alpha, beta, stream, r.conj, nullptr);
+    return true;
 }
 
 // Grouped plans keep device tables; they are outside what the sanitizer build covers.

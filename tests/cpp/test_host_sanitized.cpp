@@ -1,6 +1,6 @@
 // test_host_sanitized.cpp -- the host code of the backend and the oracle under AddressSanitizer + UndefinedBehaviorSanitizer.
 //
-// Linked from: tenferro-rs_amd/csrc/{errors,plan,prims,einsum}.cpp (unchanged), tests/cpp/host_backend.cpp (stand-ins for the
+// Linked from: tenferro-rs_amd/csrc/{errors,plan,prims,einsum,contract_cache}.cpp (unchanged), tests/cpp/host_backend.cpp (stand-ins for the
 // device launchers over host memory) and oracle/tfo_oracle.cpp, all compiled with -fsanitize=address,undefined.  Every
 // operand and result is a heap block of exactly its size, so an index or stride mistake anywhere between the C entry point
 // and the innermost loop is a sanitizer report; results are compared with the oracle's, which is itself checked here
@@ -22,6 +22,7 @@
 
 namespace tfh {
 size_t host_backend_live_blocks();
+int64_t host_backend_replays();   // contractions that ran from a routed launch kept in a plan (host_backend.cpp)
 int32_t set_no_compatible_device(int32_t space_kind, int64_t space_id, int32_t op_kind);   // errors.cpp
 }
 
@@ -375,6 +376,81 @@ static void prims_against_oracle(Rng& rng) {
     }
 }
 
+// ------------------------------------------------------------------------------------------------ routed launches kept in the plan
+// A Contract plan keeps the routed launch of the first execute with each set of view strides (contract_cache.cpp): executes
+// with strides it has seen run from the kept record, new strides route and are kept (eight sets, the oldest makes room),
+// every result equals the oracle's, and threads that share one plan may execute it at the same time.
+static void plan_keeps_routed_launches(Rng& rng) {
+    const int dt = TFH_C128;
+    const std::vector<uint32_t> ma = {0, 1, 2}, mb = {2, 3, 0}, mc = {0, 1, 3};   // batch 0, M 1, K 2, N 3
+    const std::vector<int64_t> da = {3, 5, 4}, db = {4, 6, 3}, dc = {3, 5, 6};
+    tfh_desc d;
+    std::memset(&d, 0, sizeof d);
+    d.op = TFH_OP_CONTRACT;
+    d.modes_a = ma.data(); d.n_modes_a = 3;
+    d.modes_b = mb.data(); d.n_modes_b = 3;
+    d.modes_c = mc.data(); d.n_modes_c = 3;
+    const int64_t* shapes[3] = {da.data(), db.data(), dc.data()};
+    const int32_t ranks[3] = {3, 3, 3};
+    tfh_plan* plan = nullptr;
+    CHECK(tfh_plan_create(dt, &d, shapes, ranks, 3, &plan) == TFH_OK);
+    if (!plan) return;
+    const ScalarBytes alpha = scalar(dt, 0.75, -0.5), beta = scalar(dt, 0.25, 1.0);
+    auto run = [&](int la, int lb, int lc, Rng& r) {
+        HostTensor A, B, C, Cref;
+        A.init(dt, da, la, r);
+        B.init(dt, db, lb, r);
+        Rng copy = r;
+        C.init(dt, dc, lc, r);
+        Cref.init(dt, dc, lc, copy);
+        Cref.copy_data_from(C);
+        tfh_view in[2] = {A.view(), B.view()};
+        tfh_view out = C.view();
+        CHECK(tfh_execute(plan, alpha.ptr(dt), in, 2, beta.ptr(dt), &out, nullptr) == TFH_OK);
+        tfo_view oa = A.oview(), ob = B.oview(), oc = Cref.oview();
+        CHECK(tfo_contract(dt, alpha.ptr(dt), &oa, ma.data(), &ob, mb.data(), beta.ptr(dt), &oc, mc.data()) == 0);
+        CHECK(rel_err(C, Cref) < 1e-12);
+    };
+    int64_t hits = 0, misses = 0;
+    int32_t entries = 0;
+    const int64_t replays0 = tfh::host_backend_replays();
+    // row-major everywhere, three times: one route, two replays (fresh buffers every time: only the strides are the key)
+    for (int i = 0; i < 3; ++i) run(0, 0, 0, rng);
+    CHECK(tfh_plan_cache_stats(plan, &hits, &misses, &entries) == TFH_OK && hits == 2 && misses == 1 && entries == 1);
+    CHECK(tfh::host_backend_replays() - replays0 == 2);
+    // column-major operands: new strides, a route of their own
+    for (int i = 0; i < 2; ++i) run(1, 1, 0, rng);
+    CHECK(tfh_plan_cache_stats(plan, &hits, &misses, &entries) == TFH_OK && hits == 3 && misses == 2 && entries == 2);
+    // many random layouts: never more than eight routes kept, every result right, old routes make room
+    for (int i = 0; i < 60; ++i) run(2 + rng.below(3), 2 + rng.below(3), rng.below(4), rng);
+    CHECK(tfh_plan_cache_stats(plan, &hits, &misses, &entries) == TFH_OK && entries <= 8 && hits + misses == 65);
+    // another alpha / beta class (beta == 0 overwrites) is a route of its own
+    {
+        HostTensor A, B, C;
+        A.init(dt, da, 0, rng); B.init(dt, db, 0, rng); C.init(dt, dc, 0, rng);
+        const ScalarBytes one = scalar(dt, 1, 0), zero = scalar(dt, 0, 0);
+        tfh_view in[2] = {A.view(), B.view()};
+        tfh_view out = C.view();
+        int64_t m0 = 0, m1 = 0;
+        tfh_plan_cache_stats(plan, nullptr, &m0, nullptr);
+        CHECK(tfh_execute(plan, one.ptr(dt), in, 2, zero.ptr(dt), &out, nullptr) == TFH_OK);
+        tfh_plan_cache_stats(plan, nullptr, &m1, nullptr);
+        CHECK(m1 == m0 + 1);
+    }
+    // four threads on the one plan, each alternating between two layouts
+    std::vector<std::thread> th;
+    for (int t = 0; t < 4; ++t)
+        th.emplace_back([&, t]() {
+            Rng mine(1000 + t);
+            for (int i = 0; i < 40; ++i) run((i + t) & 1, (i >> 1) & 1, 0, mine);
+        });
+    for (auto& x : th) x.join();
+    CHECK(tfh_plan_cache_stats(plan, &hits, &misses, &entries) == TFH_OK && entries <= 8 && hits > 100);
+    // no cache for other operations; null pointers are taken
+    CHECK(tfh_plan_cache_stats(plan, nullptr, nullptr, nullptr) == TFH_OK && tfh_plan_cache_stats(nullptr, &hits, &misses, &entries) != TFH_OK);
+    tfh_plan_destroy(plan);
+}
+
 // ------------------------------------------------------------------------------------------------ einsum executor vs the oracle
 static void einsum_against_oracle(Rng& rng) {
     for (int iter = 0; iter < 300; ++iter) {
@@ -620,6 +696,7 @@ int main() {
     plan_validation(rng);
     trees(rng);
     prims_against_oracle(rng);
+    plan_keeps_routed_launches(rng);
     einsum_against_oracle(rng);
     oracle_blocked_against_brute_force(rng);
     tfh_tree_cache_clear();

@@ -427,6 +427,56 @@ def test_batch_first_kernel_exact_on_integers_with_views_and_conj(tf, dtype):
     assert np.array_equal(out.to_numpy(), expect.astype(dtype))
 
 
+@pytest.mark.parametrize("dtype", ALL)
+def test_plan_keeps_the_routed_launch_per_stride_set(tf, oracle, dtype):
+    """Kernel selection lives in the plan (tenferro-prims/src/lib.rs:8, :284): the first execute with a set of view strides
+    routes, later ones replay the routed launch on their own buffers -- bit-identical results, also for a route with
+    offset tables and split-K partials, and after tfh_release_workspaces has taken the tables away."""
+    rng = seeded_rng(211)
+    cases = [("ij", "jk", "ik", dict(i=200, j=96, k=180)),                       # one launch
+             ("ij", "jk", "ik", dict(i=128, j=4096, k=128)),                     # split-K: partials + fold
+             ("ajbk", "kcj", "abc", dict(a=12, j=16, b=10, k=20, c=150)),        # multi-axis groups: offset tables (and a pack)
+             ("awc", "asx", "wcsx", dict(a=40, w=4, c=24, s=2, x=36))]
+    for ma, mb, mc, ext in cases:
+        shapes = [[ext[l] for l in m] for m in (ma, mb, mc)]
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(ma), lab(mb), lab(mc)), shapes)
+        results = []
+        for rep in range(4):
+            a, b = rand(rng, shapes[0], dtype), rand(rng, shapes[1], dtype)
+            ref = np.empty(shapes[2], dtype)
+            oracle.contract(a, lab(ma), b, lab(mb), ref, lab(mc))
+            out = dev(tf, np.full(shapes[2], np.nan, dtype))
+            tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out)
+            if rep == 0:
+                first_kernel = tf.last_kernel()
+            assert tf.last_kernel() == first_kernel
+            assert relerr(out.to_numpy(), ref) < TOL[dtype], (ma, rep)
+            # the same operands once more: the replayed launch gives the same bits
+            out2 = dev(tf, np.full(shapes[2], np.nan, dtype))
+            tf.HipBackend.execute(plan, 1.0, [dev(tf, a), dev(tf, b)], 0.0, out2)
+            assert out.to_numpy().tobytes() == out2.to_numpy().tobytes()
+            results.append(out2)
+            if rep == 1:
+                import torch
+                torch.cuda.synchronize()
+                assert tf.lib().tfh_release_workspaces() == 0      # a record that names cached tables goes stale here
+        hits, misses, entries = plan.cache_stats()
+        assert hits + misses == 8 and entries <= 2
+        assert (entries == 0) == ("routes:" not in plan.describe()), plan.describe()
+        if entries:
+            assert first_kernel in plan.describe(), plan.describe()
+        if "kernel" in first_kernel and ma != "ajbk":
+            assert hits >= 5, (ma, hits, misses)
+        # column-major views of the same extents are a second route in the same plan
+        a, b = rand(rng, shapes[0], dtype), rand(rng, shapes[1], dtype)
+        ref = np.empty(shapes[2], dtype)
+        oracle.contract(a, lab(ma), b, lab(mb), ref, lab(mc))
+        for rep in range(2):
+            out = dev(tf, colmajor(np.zeros(shapes[2], dtype)))
+            tf.HipBackend.execute(plan, 1.0, [dev(tf, colmajor(a)), dev(tf, colmajor(b))], 0.0, out)
+            assert relerr(out.to_numpy(), ref) < TOL[dtype]
+
+
 def test_config0_matmul_512_f64(tf, oracle):
     from tenferro_rs_amd import inputs
     a, b = inputs.uniform(1000, 0, (512, 512)), inputs.uniform(1000, 1, (512, 512))
@@ -1608,6 +1658,11 @@ def test_contract_random_label_patterns_and_views(tf, oracle, dtype, big):
                         alpha=abs(alpha), beta=abs(beta) if use_beta else 0.0)
         k = int(np.prod([ext[l] for l in set(ma) & set(mb) - set(mc)], dtype=np.int64))
         assert contraction_within_tolerance(out.to_numpy(), ref, dtype, scale, k), (case, ma, mb, mc, ext, relerr(out.to_numpy(), ref))
+        # once more through the same plan on fresh device buffers: where the plan kept the routed launch this is its
+        # replay (operands exchanged, tables, split-K and all), and it must give the same bits
+        out2 = dev(tf, c0) if cshape else tf.Tensor.empty([], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, out2)
+        assert out.to_numpy().tobytes() == out2.to_numpy().tobytes(), (case, ma, mb, mc, ext, plan.cache_stats())
 
 
 def _cancelling():
