@@ -441,6 +441,83 @@ def run_batched(h, dtype, nb, n, cm=False, ref_out=None):
     return res
 
 
+# ------------------------------------------------------------------------------------------------- permutes and reductions of general shapes
+def random_shape(rng, rank, elems):
+    """`rank` extents, none a power of two on purpose, whose product is close to `elems`."""
+    w = rng.uniform(0.3, 1.0, rank)
+    ext = np.maximum(2, np.round(np.exp(np.log(elems) * w / w.sum()))).astype(np.int64)
+    for d in range(rank):      # nudge powers of two to their odd neighbours: the tile grid of the fast paths must not fit by luck
+        if ext[d] & (ext[d] - 1) == 0:
+            ext[d] += 1
+    order = np.argsort(-ext)
+    k = 0
+    while np.prod(ext.astype(np.float64)) < elems:      # grow the largest extents until the tensor is large enough
+        ext[order[k % rank]] += max(1, ext[order[k % rank]] // 16)
+        k += 1
+    return [int(x) for x in ext]
+
+
+def shape_sweep(h, n_shapes=24, min_bytes=128 << 20):
+    """python bench.py --shape-sweep: permutes (random axis orders) and sum-reductions (random sets of reduced axes) of
+    seeded random tensors of rank 3..7 and at least 128 MB, whose extents are not powers of two, for all four dtypes, as
+    the fraction of the HBM peak that the bytes each must move (in + out) reach.  One line per shape, then min / median
+    per dtype and operation."""
+    tf, torch = h.tf, h.torch
+    names = {np.float32: "f32", np.float64: "f64", np.complex64: "c64", np.complex128: "c128"}
+    print("%-5s %-8s %-34s %-22s %9s %8s %6s  %s" % ("dtype", "op", "shape", "perm / reduced axes", "MB moved", "us", "% HBM", "kernel"))
+    summary = []
+    for dtype in (np.float32, np.float64, np.complex64, np.complex128):
+        rng = np.random.default_rng(1006)      # the same shapes for every dtype (scaled to the element size)
+        fr = {"permute": [], "reduce": []}
+        for i in range(n_shapes):
+            rank = 3 + i % 5
+            shape = random_shape(rng, rank, min_bytes // np.dtype(dtype).itemsize)
+            perm = [int(x) for x in rng.permutation(rank)]
+            while perm == list(range(rank)):
+                perm = [int(x) for x in rng.permutation(rank)]
+            nred = int(rng.integers(1, rank))
+            red = sorted(int(x) for x in rng.choice(rank, nred, replace=False))
+            n = int(np.prod(shape))
+            src = torch.empty(n, dtype={np.float32: torch.float32, np.float64: torch.float64, np.complex64: torch.complex64,
+                                        np.complex128: torch.complex128}[dtype], device="cuda")
+            src.view(torch.float32 if np.dtype(dtype).itemsize % 8 else torch.float64).uniform_(-1.0, 1.0)
+            X = tf.Tensor(src, shape, tf._contig_strides(shape, tf.MemoryOrder.RowMajor), 0, tf.GpuMemory(0), tf.dtype_code(dtype))
+            for op in ("permute", "reduce"):
+                if op == "permute":
+                    oshape = [shape[p] for p in perm]
+                    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Permute(list(range(rank)), perm), [shape, oshape])
+                    what, kind = str(tuple(perm)), tf.PROF_COPY
+                else:
+                    kept = [d for d in range(rank) if d not in red]
+                    oshape = [shape[d] for d in kept]
+                    plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Reduce(list(range(rank)), kept, tf.ReduceOp.Sum), [shape, oshape])
+                    what, kind = "sum over " + str(tuple(red)), tf.PROF_REDUCE
+                out = h.empty(oshape, dtype)
+                call = h.bound_execute(plan, [X], out)
+                for _ in range(3):
+                    call()
+                torch.cuda.synchronize()
+                reps = 10
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    call()
+                torch.cuda.synchronize()
+                us = (time.perf_counter() - t0) * 1e6 / reps
+                nbytes = (n + int(np.prod(oshape))) * np.dtype(dtype).itemsize
+                frac = nbytes / (us * 1e-6) / 1e9 / PEAK["hbm"]
+                fr[op].append(frac)
+                print("%-5s %-8s %-34s %-22s %9.1f %8.1f %6.1f  %s" % (names[dtype], op, "x".join(map(str, shape)), what, nbytes / 1e6, us,
+                                                                       100 * frac, tf.last_kernel()[:60]), flush=True)
+                del out
+            del X, src
+            torch.cuda.empty_cache()
+        for op in ("permute", "reduce"):
+            summary.append("%-5s %-8s %2d shapes: min %5.1f %%  median %5.1f %%  max %5.1f %% of the 8 TB/s HBM peak" %
+                           (names[dtype], op, len(fr[op]), 100 * min(fr[op]), 100 * float(np.median(fr[op])), 100 * max(fr[op])))
+    print()
+    print("\n".join(summary))
+
+
 # ------------------------------------------------------------------------------------------------- host cost of a call
 def host_overhead(h):
     """Microseconds of host time per enqueue (python bench.py --host-overhead): the first execute of a plan (routing, table
@@ -553,6 +630,8 @@ def main():
     ap.add_argument("--configs", default="c3,c1,c2,c4,c0,b64,b128")
     ap.add_argument("--no-colmajor", action="store_true", help="skip the column-major variants of the configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--shape-sweep", action="store_true",
+                    help="permutes and reductions of seeded random tensors (rank 3..7, >= 128 MB, extents that are no powers of two)")
     ap.add_argument("--host-overhead", action="store_true",
                     help="print the host cost of tfh_execute per call (first against repeated) instead of running the benchmark")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -562,7 +641,10 @@ def main():
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus %d is not supported\n" % args.gpus)
         sys.exit(2)
-    h = Harness(args.steps, args.warmup, not args.no_cpu and not args.host_overhead)
+    h = Harness(args.steps, args.warmup, not args.no_cpu and not args.host_overhead and not args.shape_sweep)
+    if args.shape_sweep:
+        shape_sweep(h)
+        return
     if args.host_overhead:
         host_overhead(h)
         return
