@@ -457,16 +457,19 @@ def random_shape(rng, rank, elems):
     return [int(x) for x in ext]
 
 
-def shape_sweep(h, n_shapes=24, min_bytes=128 << 20):
+def shape_sweep(h, n_shapes=24, min_bytes=128 << 20, ops=("permute", "reduce"), dtypes=("f32", "f64", "c64", "c128")):
     """python bench.py --shape-sweep: permutes (random axis orders) and sum-reductions (random sets of reduced axes) of
     seeded random tensors of rank 3..7 and at least 128 MB, whose extents are not powers of two, for all four dtypes, as
     the fraction of the HBM peak that the bytes each must move (in + out) reach.  One line per shape, then min / median
     per dtype and operation."""
     tf, torch = h.tf, h.torch
     names = {np.float32: "f32", np.float64: "f64", np.complex64: "c64", np.complex128: "c128"}
-    print("%-5s %-8s %-34s %-22s %9s %8s %6s  %s" % ("dtype", "op", "shape", "perm / reduced axes", "MB moved", "us", "% HBM", "kernel"))
+    print("%-5s %-8s %-34s %-22s %9s %8s %8s %6s  %s" % ("dtype", "op", "shape", "perm / reduced axes", "MB moved", "us", "kernel us", "% HBM",
+                                                         "last kernel"))
     summary = []
     for dtype in (np.float32, np.float64, np.complex64, np.complex128):
+        if names[dtype] not in dtypes:
+            continue
         rng = np.random.default_rng(1006)      # the same shapes for every dtype (scaled to the element size)
         fr = {"permute": [], "reduce": []}
         for i in range(n_shapes):
@@ -482,7 +485,7 @@ def shape_sweep(h, n_shapes=24, min_bytes=128 << 20):
                                         np.complex128: torch.complex128}[dtype], device="cuda")
             src.view(torch.float32 if np.dtype(dtype).itemsize % 8 else torch.float64).uniform_(-1.0, 1.0)
             X = tf.Tensor(src, shape, tf._contig_strides(shape, tf.MemoryOrder.RowMajor), 0, tf.GpuMemory(0), tf.dtype_code(dtype))
-            for op in ("permute", "reduce"):
+            for op in ops:
                 if op == "permute":
                     oshape = [shape[p] for p in perm]
                     plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Permute(list(range(rank)), perm), [shape, oshape])
@@ -494,24 +497,18 @@ def shape_sweep(h, n_shapes=24, min_bytes=128 << 20):
                     what, kind = "sum over " + str(tuple(red)), tf.PROF_REDUCE
                 out = h.empty(oshape, dtype)
                 call = h.bound_execute(plan, [X], out)
-                for _ in range(3):
-                    call()
-                torch.cuda.synchronize()
-                reps = 10
-                t0 = time.perf_counter()
-                for _ in range(reps):
-                    call()
-                torch.cuda.synchronize()
-                us = (time.perf_counter() - t0) * 1e6 / reps
+                ms, prof = h.timed(lambda i: call(), [kind])
+                us = ms * 1e3
+                kus = sum(m * c for (_, m, c) in prof[kind]) * 1e3      # the kernels alone, from HIP events around each
                 nbytes = (n + int(np.prod(oshape))) * np.dtype(dtype).itemsize
                 frac = nbytes / (us * 1e-6) / 1e9 / PEAK["hbm"]
                 fr[op].append(frac)
-                print("%-5s %-8s %-34s %-22s %9.1f %8.1f %6.1f  %s" % (names[dtype], op, "x".join(map(str, shape)), what, nbytes / 1e6, us,
-                                                                       100 * frac, tf.last_kernel()[:60]), flush=True)
+                print("%-5s %-8s %-34s %-22s %9.1f %8.1f %8.1f %6.1f  %s" % (names[dtype], op, "x".join(map(str, shape)), what, nbytes / 1e6, us,
+                                                                             kus, 100 * frac, tf.last_kernel()[:60]), flush=True)
                 del out
             del X, src
             torch.cuda.empty_cache()
-        for op in ("permute", "reduce"):
+        for op in ops:
             summary.append("%-5s %-8s %2d shapes: min %5.1f %%  median %5.1f %%  max %5.1f %% of the 8 TB/s HBM peak" %
                            (names[dtype], op, len(fr[op]), 100 * min(fr[op]), 100 * float(np.median(fr[op])), 100 * max(fr[op])))
     print()
@@ -630,6 +627,8 @@ def main():
     ap.add_argument("--configs", default="c3,c1,c2,c4,c0,b64,b128")
     ap.add_argument("--no-colmajor", action="store_true", help="skip the column-major variants of the configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
+    ap.add_argument("--sweep-ops", default="permute,reduce", help="operations of --shape-sweep (permute, reduce)")
+    ap.add_argument("--sweep-dtypes", default="f32,f64,c64,c128", help="dtypes of --shape-sweep")
     ap.add_argument("--shape-sweep", action="store_true",
                     help="permutes and reductions of seeded random tensors (rank 3..7, >= 128 MB, extents that are no powers of two)")
     ap.add_argument("--host-overhead", action="store_true",
@@ -643,7 +642,7 @@ def main():
         sys.exit(2)
     h = Harness(args.steps, args.warmup, not args.no_cpu and not args.host_overhead and not args.shape_sweep)
     if args.shape_sweep:
-        shape_sweep(h)
+        shape_sweep(h, ops=tuple(args.sweep_ops.split(",")), dtypes=tuple(args.sweep_dtypes.split(",")))
         return
     if args.host_overhead:
         host_overhead(h)

@@ -942,6 +942,776 @@ bool try_shortrow_reduce(int dtype, const void* a, void* c, std::vector<Axis> ke
 }
 }  // namespace
 
+namespace {
+// ---- dense runs of any extent -------------------------------------------------------------------------------------
+// For an operand whose fastest axes are dense in memory (any contiguous tensor), whatever the extents are.  A tile is
+// a contiguous run of memory: the innermost axes whole, kept and reduced alike, and a range of the next axis, so it
+// has one ragged edge at most (the last range of that axis) and no lane idles at an extent that is not a power of
+// two.  Thread t owns the 16-byte vectors t, t + 256, ... of the run, whatever coordinates they have, and adds up the
+// tiles that the reduced axes outside the tile step through (an odometer of scalar offsets, several tiles' loads in
+// flight).  Only when the walk is over do coordinates matter: the accumulators go to LDS and every reduced axis inside
+// the tile is folded there, a pass per axis, wide axes in rounds of sixteen so that all threads take part; what is
+// left are the tile's outputs in memory order.  A complex element is a kept innermost axis of two reals.  When the
+// kept axes outside the tile give too few blocks, the walk is split over blockIdx.y into partial results that a
+// second kernel folds in a fixed order.  The loads need only the alignment of a real: a tile starts wherever the
+// extents put it.  A vector never reaches past the end of its tile (the last odd reals are read one by one), so
+// nothing is read outside the operand.
+constexpr int RUN_AXES = 6;        // tile axes, the pair of reals of a complex element included
+constexpr int RUN_REALS = 2048;    // accumulators of a tile, parked in LDS as doubles
+struct RunArgs {
+    const void* in;
+    void* out;
+    double* partial;               // [nsplit][blocks][kept_per_tile] (complex: 2 doubles each)
+    int32_t nf;                    // tile axes in reals, innermost first; the last one is the ranged axis
+    int32_t f_ext[RUN_AXES], f_red[RUN_AXES];
+    int64_t f_so[RUN_AXES];        // C stride of a kept tile axis, in elements
+    int32_t tile_reals;            // product of f_ext
+    int32_t row_reals;             // reals per index of the ranged axis
+    int32_t kept_per_tile;         // outputs of a full tile
+    int32_t range, x_n;            // indices of the ranged axis per tile, and its extent
+    int32_t g0_is_range, r0_is_range;   // the tile index along the ranged axis is g[0] (kept) or r[0] (reduced)
+    int32_t all_reduced;           // no kept tile axis (a complex element's pair of reals aside)
+    int32_t ng, nr;
+    int64_t g_count[MAXG], g_si[MAXG], g_so[MAXG];   // kept axes outside the tile (A strides in reals, C in elements)
+    int64_t r_count[MAXR], r_si[MAXR];               // reduced axes outside the tile, innermost first
+    int64_t r_total, per_split, blocks;
+    int32_t nsplit, op, use_beta;
+    double alpha_re, alpha_im, beta_re, beta_im;
+};
+
+// value known to be the same in every lane -> scalar registers
+__device__ __forceinline__ int64_t uniform64(int64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+struct RunOdometer {
+    int64_t c[MAXR];
+    int64_t off;
+};
+__device__ __forceinline__ void run_advance(const RunArgs& a, RunOdometer& o) {
+    o.off += a.r_si[0];
+    if (++o.c[0] == a.r_count[0]) {
+        o.off -= a.r_si[0] * a.r_count[0];
+        o.c[0] = 0;
+#pragma unroll
+        for (int r = 1; r < MAXR; ++r) {
+            if (r < a.nr) {
+                o.off += a.r_si[r];
+                if (++o.c[r] < a.r_count[r]) break;
+                o.off -= a.r_si[r] * a.r_count[r];
+                o.c[r] = 0;
+            }
+        }
+    }
+}
+
+template <class R, int NV> struct RunVec { typedef R type __attribute__((ext_vector_type(NV), aligned(sizeof(R)))); };
+
+// UU tiles: all their loads first, then the adds.  A tile of `len` reals is len / NV whole vectors, vector v in slot v
+// (thread v % 256, register set v / 256), and up to NV - 1 odd reals behind them, real i of which lane i of the first
+// wave adds up in `odd`.  Slots past the tile read the tile's last vector again (an address inside the operand) and
+// what they add up is never used.  RAGGED: some of the tiles are shorter than the block's tile (the last range of a
+// reduced axis): their slots past the end must stay out of the sums, and their odd reals belong to the accumulators
+// of a whole slot.
+template <class R, int J, int UU, bool SUM, bool RAGGED>
+__device__ __forceinline__ void run_tiles(const RunArgs& a, const R* A, RunOdometer& odo, const int (&own)[J], int len_blk, int op,
+                                          double (&acc)[J][16 / sizeof(R)], double& odd) {
+    constexpr int NV = 16 / sizeof(R);
+    typedef typename RunVec<R, NV>::type V;
+    int64_t offs[UU];
+    int lens[UU];
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+        offs[u] = uniform64(odo.off);
+        lens[u] = len_blk;
+        if (RAGGED) {
+            const int64_t left = (int64_t)a.x_n - odo.c[0] * a.range;
+            lens[u] = (int)(left < a.range ? left : a.range) * a.row_reals;
+        }
+        run_advance(a, odo);
+    }
+    V v[UU][J];
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+        const int last = lens[u] / NV - 1;   // (a tile shorter than a vector: no slot reads anything it may use)
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const int at = own[j] < last * NV ? own[j] : last * NV;
+            v[u][j] = V{};
+            if (last >= 0) v[u][j] = __builtin_nontemporal_load(reinterpret_cast<const V*>(A + offs[u] + at));
+        }
+    }
+    // the odd reals behind the block's whole vectors: lane i of the first wave reads real i of them
+    const int whole_blk = len_blk / NV * NV, rest_blk = len_blk - whole_blk;
+    const bool odd_wave = rest_blk > 0 && threadIdx.x < 64;
+    R vo[UU];
+    if (odd_wave) {
+        const int at = whole_blk + ((int)threadIdx.x < rest_blk ? (int)threadIdx.x : rest_blk - 1);
+#pragma unroll
+        for (int u = 0; u < UU; ++u) {
+            vo[u] = R(0);
+            if (!RAGGED || lens[u] == len_blk) vo[u] = __builtin_nontemporal_load(A + offs[u] + at);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+        const int whole = lens[u] / NV * NV;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const bool in = !RAGGED || own[j] < whole;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const double x = (double)v[u][j][i];
+                const double y = SUM ? acc[j][i] + x : combine(acc[j][i], x, op);
+                acc[j][i] = in ? y : acc[j][i];
+            }
+        }
+        if (odd_wave && (!RAGGED || lens[u] == len_blk)) odd = SUM ? odd + (double)vo[u] : combine(odd, (double)vo[u], op);
+        if (RAGGED && lens[u] != len_blk && lens[u] != whole) {
+            // the odd reals of a shorter tile lie in a whole slot of the block's tile: its owner reads them one by one
+#pragma unroll
+            for (int j = 0; j < J; ++j)
+                if (own[j] == whole) {
+#pragma unroll
+                    for (int i = 0; i < NV - 1; ++i)
+                        if (i < lens[u] - whole) acc[j][i] = combine(acc[j][i], (double)A[offs[u] + whole + i], op);
+                }
+        }
+    }
+}
+
+// Kept coordinates of output q of a tile -> C offset in elements; false when q lies past the ragged edge.
+template <bool CX>
+__device__ __forceinline__ bool run_output(const RunArgs& a, int q, int x_here, int64_t& off) {
+    off = 0;
+    bool ok = true;
+#pragma unroll
+    for (int f = CX ? 1 : 0; f < RUN_AXES; ++f) {
+        if (f < a.nf && !a.f_red[f]) {
+            const int n = a.f_ext[f], h = q / n, c = q - h * n;
+            q = h;
+            off += (int64_t)c * a.f_so[f];
+            if (f == a.nf - 1) ok = c < x_here;
+        }
+    }
+    return ok;
+}
+
+template <class R, bool CX>
+__device__ __forceinline__ void run_finish(const RunArgs& a, R* C, double re, double im) {
+    if (CX) {
+        double rr = a.alpha_re * re - a.alpha_im * im, ri = a.alpha_re * im + a.alpha_im * re;
+        if (a.use_beta) {
+            const double cr = C[0], ci = C[1];
+            rr += a.beta_re * cr - a.beta_im * ci;
+            ri += a.beta_re * ci + a.beta_im * cr;
+        }
+        C[0] = (R)rr;
+        C[1] = (R)ri;
+    } else {
+        double r = a.alpha_re * re;
+        if (a.use_beta) r += a.beta_re * (double)C[0];
+        C[0] = (R)r;
+    }
+}
+
+// Block b of a split -> origins in A (reals) and C (elements), and the indices of the ranged axis inside the tensor.
+__device__ __forceinline__ void run_origin(const RunArgs& a, uint32_t bid, int64_t& org_in, int64_t& org_out, int& x_here) {
+    org_in = org_out = 0;
+    x_here = a.range;
+    for (int g = 0; g < a.ng; ++g) {   // (the grid, and so every count, is below 2^31)
+        const uint32_t n = (uint32_t)a.g_count[g], q = bid / n;
+        const int64_t c = (int64_t)(bid - q * n);
+        bid = q;
+        org_in += c * a.g_si[g];
+        org_out += c * a.g_so[g];
+        if (g == 0 && a.g0_is_range) {
+            const int64_t left = (int64_t)a.x_n - c * a.range;
+            if (left < x_here) x_here = (int)left;
+        }
+    }
+}
+
+template <class R, bool CX, int J, bool SUM>
+__global__ void __launch_bounds__(THREADS) reduce_run_kernel(RunArgs a) {
+    prefetch_kernel_arguments<sizeof(RunArgs)>();
+    constexpr int NV = 16 / sizeof(R);
+    constexpr int NC = CX ? 2 : 1;
+    constexpr int U = 8 / J;
+    __shared__ double lds[RUN_REALS];
+    const int tid = threadIdx.x;
+    const int op = SUM ? (int)TFH_REDUCE_SUM : a.op;
+    int64_t org_in, org_out;
+    int x_here;
+    run_origin(a, blockIdx.x, org_in, org_out, x_here);
+    org_in = uniform64(org_in);
+    const R* A = reinterpret_cast<const R*>(a.in) + org_in;
+    // this block's tile: shorter than the others at the ragged edge of a kept ranged axis
+    const int full = a.g0_is_range ? x_here * a.row_reals : a.tile_reals;
+    const int whole = full / NV * NV, tail = full - whole;
+    const int64_t it0 = (int64_t)blockIdx.y * a.per_split;
+    const int64_t it1 = it0 + a.per_split < a.r_total ? it0 + a.per_split : a.r_total;
+    RunOdometer odo;
+    odo.off = 0;
+    if (a.r_total < 0x7fffffff) {
+        uint32_t lin = (uint32_t)it0;
+#pragma unroll
+        for (int r = 0; r < MAXR; ++r) {
+            odo.c[r] = 0;
+            if (r < a.nr) {
+                const uint32_t n = (uint32_t)a.r_count[r], q = lin / n;
+                odo.c[r] = lin - q * n;
+                lin = q;
+                odo.off += odo.c[r] * a.r_si[r];
+            }
+        }
+    } else {
+        int64_t lin = it0;
+#pragma unroll
+        for (int r = 0; r < MAXR; ++r) {
+            odo.c[r] = 0;
+            if (r < a.nr) {
+                const int64_t q = lin / a.r_count[r];
+                odo.c[r] = lin - q * a.r_count[r];
+                lin = q;
+                odo.off += odo.c[r] * a.r_si[r];
+            }
+        }
+    }
+    int own[J];   // first real of the thread's vector slots
+#pragma unroll
+    for (int j = 0; j < J; ++j) own[j] = (tid + THREADS * j) * NV;
+    double acc[J][NV], odd = identity(op);
+#pragma unroll
+    for (int j = 0; j < J; ++j)
+#pragma unroll
+        for (int i = 0; i < NV; ++i) acc[j][i] = identity(op);
+    // a shorter tile among the reduced ones: the last index of r[0]
+    const bool ragged_r = a.r0_is_range && (int64_t)a.x_n % a.range != 0;
+    int64_t it = it0;
+    for (; it + U <= it1; it += U) {
+        if (ragged_r && odo.c[0] + U >= a.r_count[0]) run_tiles<R, J, U, SUM, true>(a, A, odo, own, full, op, acc, odd);
+        else run_tiles<R, J, U, SUM, false>(a, A, odo, own, full, op, acc, odd);
+    }
+    for (; it < it1; ++it) {
+        if (ragged_r) run_tiles<R, J, 1, SUM, true>(a, A, odo, own, full, op, acc, odd);
+        else run_tiles<R, J, 1, SUM, false>(a, A, odo, own, full, op, acc, odd);
+    }
+    // accumulators -> LDS in tile order
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        if (own[j] < whole) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) lds[own[j] + i] = acc[j][i];
+        }
+    }
+    if (tid < tail) lds[whole + tid] = odd;
+    // (positions from the block's tile length to the full tile's hold nothing: they are coordinates past the ragged
+    // edge of a kept axis, folded into outputs that are not written)
+    __syncthreads();
+    // fold the reduced tile axes, innermost first; a folded axis keeps extent 1
+    int ext[RUN_AXES];
+#pragma unroll
+    for (int f = 0; f < RUN_AXES; ++f) ext[f] = f < a.nf ? a.f_ext[f] : 1;
+#pragma unroll
+    for (int f = 0; f < RUN_AXES; ++f) {
+        if (f >= a.nf || !a.f_red[f]) continue;
+        int inner = 1, outer = 1;
+#pragma unroll
+        for (int k = 0; k < RUN_AXES; ++k) {
+            if (k < f) inner *= ext[k];
+            if (k > f) outer *= ext[k];
+        }
+        const int count = inner * outer;
+        int n = ext[f];
+        while (n > 1) {
+            int groups = THREADS / count;
+            if (groups > (n + 15) / 16) groups = (n + 15) / 16;
+            if (groups < 1) groups = 1;
+            const int each = (n + groups - 1) / groups;
+            groups = (n + each - 1) / each;
+            const int total = count * groups;   // at most RUN_REALS
+            double s[RUN_REALS / THREADS];
+#pragma unroll
+            for (int k = 0; k < RUN_REALS / THREADS; ++k) {
+                const int o = tid + THREADS * k;
+                s[k] = identity(op);
+                if (o < total) {
+                    const int in = o % inner, rest = o / inner, g = rest % groups, ou = rest / groups;
+                    const int k0 = g * each, k1 = k0 + each < n ? k0 + each : n;
+                    const double* p = lds + ((int64_t)ou * n + k0) * inner + in;
+                    for (int x = k0; x < k1; ++x, p += inner) s[k] = combine(s[k], *p, op);
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < RUN_REALS / THREADS; ++k) {
+                const int o = tid + THREADS * k;
+                if (o < total) lds[o] = s[k];
+            }
+            __syncthreads();
+            n = groups;
+        }
+        ext[f] = 1;
+    }
+    // the tile's outputs
+    const int nq = a.kept_per_tile;
+    for (int q = tid; q < nq; q += THREADS) {
+        int64_t off;
+        if (!run_output<CX>(a, q, x_here, off)) continue;
+        const double re = lds[q * NC], im = CX ? lds[q * NC + 1] : 0.0;
+        if (a.nsplit > 1) {
+            double* P = a.partial + (((int64_t)blockIdx.y * a.blocks + blockIdx.x) * nq + q) * NC;
+            P[0] = re;
+            if (CX) P[1] = im;
+        } else {
+            run_finish<R, CX>(a, reinterpret_cast<R*>(a.out) + (org_out + off) * NC, re, im);
+        }
+    }
+}
+
+// Every tile axis reduced (rows summed whole, a full reduction): a tile has no coordinates worth keeping, so a thread
+// adds everything it reads into one accumulator, and a block takes KS outputs that are neighbours along the kept axes
+// outside the tile, in step, so that rows of a few KB still give every thread eight loads in flight and one
+// exchange through LDS serves KS outputs.
+template <class R, bool CX, int J, int KS, bool SUM>
+__global__ void __launch_bounds__(THREADS) reduce_run_rows_kernel(RunArgs a) {
+    prefetch_kernel_arguments<sizeof(RunArgs)>();
+    constexpr int NV = 16 / sizeof(R);
+    constexpr int NC = CX ? 2 : 1;
+    constexpr int U = J * KS >= 8 ? 1 : 8 / (J * KS);
+    typedef typename RunVec<R, NV>::type V;
+    __shared__ double lds[KS * 4 * 2];
+    const int tid = threadIdx.x;
+    const int op = SUM ? (int)TFH_REDUCE_SUM : a.op;
+    const uint32_t item0 = blockIdx.x * KS, items = (uint32_t)a.blocks;
+    int64_t org[KS];
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+        int64_t org_out;
+        int x_here;
+        run_origin(a, item0 + k < items ? item0 + k : items - 1, org[k], org_out, x_here);
+        org[k] = uniform64(org[k]);
+    }
+    const R* A = reinterpret_cast<const R*>(a.in);
+    const int full = a.tile_reals;
+    const int64_t it0 = (int64_t)blockIdx.y * a.per_split;
+    const int64_t it1 = it0 + a.per_split < a.r_total ? it0 + a.per_split : a.r_total;
+    RunOdometer odo;
+    odo.off = 0;
+    {
+        int64_t lin = it0;
+#pragma unroll
+        for (int r = 0; r < MAXR; ++r) {
+            odo.c[r] = 0;
+            if (r < a.nr) {
+                const int64_t q = lin / a.r_count[r];
+                odo.c[r] = lin - q * a.r_count[r];
+                lin = q;
+                odo.off += odo.c[r] * a.r_si[r];
+            }
+        }
+    }
+    int own[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) own[j] = (tid + THREADS * j) * NV;
+    double re[KS], im[KS];
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+        re[k] = identity(op);
+        im[k] = 0.0;
+    }
+    const bool ragged_r = a.r0_is_range && (int64_t)a.x_n % a.range != 0;
+    for (int64_t it = it0; it < it1; it += U) {
+        int64_t offs[U];
+        int lens[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            offs[u] = uniform64(odo.off);
+            lens[u] = full;
+            if (ragged_r) {
+                const int64_t left = (int64_t)a.x_n - odo.c[0] * a.range;
+                lens[u] = (int)(left < a.range ? left : a.range) * a.row_reals;
+            }
+            if (it + u >= it1) lens[u] = 0;
+            else run_advance(a, odo);
+        }
+        V v[U][KS][J];
+        R vo[U][KS];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int last = lens[u] / NV - 1, whole = (last + 1) * NV, rest = lens[u] - whole;
+#pragma unroll
+            for (int k = 0; k < KS; ++k) {
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+                    const int at = own[j] < last * NV ? own[j] : last * NV;
+                    v[u][k][j] = V{};
+                    if (last >= 0) v[u][k][j] = __builtin_nontemporal_load(reinterpret_cast<const V*>(A + org[k] + offs[u] + at));
+                }
+                vo[u][k] = R(0);
+                if (rest > 0 && tid < 64) vo[u][k] = __builtin_nontemporal_load(A + org[k] + offs[u] + whole + (tid < rest ? tid : rest - 1));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int whole = lens[u] / NV * NV, rest = lens[u] - whole;
+#pragma unroll
+            for (int k = 0; k < KS; ++k) {
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+                    const bool in = own[j] < whole;
+#pragma unroll
+                    for (int i = 0; i < NV; ++i) {
+                        const double x = (double)v[u][k][j][i];
+                        if (CX && (i & 1)) {
+                            im[k] = in ? im[k] + x : im[k];
+                        } else {
+                            const double y = SUM ? re[k] + x : combine(re[k], x, op);
+                            re[k] = in ? y : re[k];
+                        }
+                    }
+                }
+                if (tid < rest) {
+                    const double x = (double)vo[u][k];
+                    if (CX && (tid & 1)) im[k] += x;
+                    else re[k] = combine(re[k], x, op);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            re[k] = combine(re[k], __shfl_xor(re[k], d), op);
+            if (CX) im[k] += __shfl_xor(im[k], d);
+        }
+        if ((tid & 63) == 0) {
+            lds[(k * 4 + (tid >> 6)) * 2] = re[k];
+            lds[(k * 4 + (tid >> 6)) * 2 + 1] = im[k];
+        }
+    }
+    __syncthreads();
+    if (tid >= KS || item0 + tid >= items) return;
+    const double* w = lds + tid * 8;
+    const double sre = combine(combine(w[0], w[2], op), combine(w[4], w[6], op), op), sim = (w[1] + w[3]) + (w[5] + w[7]);
+    if (a.nsplit > 1) {
+        double* P = a.partial + ((int64_t)blockIdx.y * a.blocks + item0 + tid) * NC;
+        P[0] = sre;
+        if (CX) P[1] = sim;
+    } else {
+        int64_t org_in, org_out;
+        int x_here;
+        run_origin(a, item0 + tid, org_in, org_out, x_here);
+        run_finish<R, CX>(a, reinterpret_cast<R*>(a.out) + org_out * NC, sre, sim);
+    }
+}
+
+// Second pass of a split walk: `team` threads (a power of two) per output add the partial results split, split +
+// team, ... and meet in an LDS tree.
+template <class R, bool CX>
+__global__ void __launch_bounds__(THREADS) reduce_run_fold_kernel(RunArgs a, int team) {
+    constexpr int NC = CX ? 2 : 1;
+    __shared__ double lds[THREADS * NC];
+    const int tid = threadIdx.x, per = THREADS / team, g = tid / per;
+    const int64_t outputs = a.blocks * a.kept_per_tile;
+    const int64_t o = (int64_t)blockIdx.x * per + tid % per;
+    const int op = a.op;
+    double re = identity(op), im = 0.0;
+    if (o < outputs) {
+        for (int s = g; s < a.nsplit; s += team) {
+            const double* P = a.partial + ((int64_t)s * outputs + o) * NC;
+            re = combine(re, P[0], op);
+            if (CX) im += P[1];
+        }
+    }
+    if (team > 1) {
+        lds[tid * NC] = re;
+        if (CX) lds[tid * NC + 1] = im;
+        __syncthreads();
+        for (int stride = THREADS / 2; stride >= per; stride >>= 1) {
+            if (tid < stride) {
+                lds[tid * NC] = combine(lds[tid * NC], lds[(tid + stride) * NC], op);
+                if (CX) lds[tid * NC + 1] += lds[(tid + stride) * NC + 1];
+            }
+            __syncthreads();
+        }
+        re = lds[tid * NC];
+        if (CX) im = lds[tid * NC + 1];
+    }
+    if (g != 0 || o >= outputs) return;
+    const int64_t b = o / a.kept_per_tile;
+    const int q = (int)(o - b * a.kept_per_tile);
+    int64_t org_in, org_out, off;
+    int x_here;
+    run_origin(a, (uint32_t)b, org_in, org_out, x_here);
+    if (!run_output<CX>(a, q, x_here, off)) return;
+    run_finish<R, CX>(a, reinterpret_cast<R*>(a.out) + (org_out + off) * NC, re, im);
+}
+
+template <class R, bool CX, int J>
+void launch_run_j(const RunArgs& ra, dim3 grid, hipStream_t st) {
+    if (ra.op == TFH_REDUCE_SUM) TFH_LAUNCH_TIMED((reduce_run_kernel<R, CX, J, true>), grid, dim3(THREADS), 0, st, ra);
+    else TFH_LAUNCH_TIMED((reduce_run_kernel<R, CX, J, false>), grid, dim3(THREADS), 0, st, ra);
+}
+template <class R, bool CX>
+void launch_run(const RunArgs& ra, int j, dim3 grid, hipStream_t st) {
+    if (j == 1) launch_run_j<R, CX, 1>(ra, grid, st);
+    else if (j == 2) launch_run_j<R, CX, 2>(ra, grid, st);
+    else if constexpr (sizeof(R) == 8) launch_run_j<R, CX, 4>(ra, grid, st);
+}
+template <class R, bool CX, int J, int KS>
+void launch_rows_jk(const RunArgs& ra, dim3 grid, hipStream_t st) {
+    if (ra.op == TFH_REDUCE_SUM) TFH_LAUNCH_TIMED((reduce_run_rows_kernel<R, CX, J, KS, true>), grid, dim3(THREADS), 0, st, ra);
+    else TFH_LAUNCH_TIMED((reduce_run_rows_kernel<R, CX, J, KS, false>), grid, dim3(THREADS), 0, st, ra);
+}
+template <class R, bool CX>
+void launch_rows(const RunArgs& ra, int j, int ks, dim3 grid, hipStream_t st) {
+    if (j == 1) {
+        if (ks == 8) launch_rows_jk<R, CX, 1, 8>(ra, grid, st);
+        else if (ks == 4) launch_rows_jk<R, CX, 1, 4>(ra, grid, st);
+        else if (ks == 2) launch_rows_jk<R, CX, 1, 2>(ra, grid, st);
+        else launch_rows_jk<R, CX, 1, 1>(ra, grid, st);
+    } else if (j == 2) {
+        if (ks == 4) launch_rows_jk<R, CX, 2, 4>(ra, grid, st);
+        else if (ks == 2) launch_rows_jk<R, CX, 2, 2>(ra, grid, st);
+        else launch_rows_jk<R, CX, 2, 1>(ra, grid, st);
+    } else if constexpr (sizeof(R) == 8) {
+        if (ks == 2) launch_rows_jk<R, CX, 4, 2>(ra, grid, st);
+        else launch_rows_jk<R, CX, 4, 1>(ra, grid, st);
+    }
+}
+}  // namespace
+
+namespace {
+// Returns true when the dense-run kernel was launched.
+bool try_run_reduce(int dtype, const void* a, void* c, const std::vector<Axis>& kept, const std::vector<Axis>& red, int reduce_op,
+                    Scalar alpha, Scalar beta, void* stream, int32_t& status) {
+    status = TFH_OK;
+    const bool cx = is_complex(dtype), dbl = is_double(dtype);
+    const int nc = cx ? 2 : 1, nv = dbl ? 2 : 4;
+    if (cx && reduce_op != TFH_REDUCE_SUM) return false;
+    struct Ax {
+        int64_t n, si, so;
+        bool red;
+    };
+    std::vector<Ax> all;
+    int64_t total = 1;
+    for (auto& x : kept) {
+        if (x.n == 1) continue;
+        if (x.s[0] <= 0 || x.s[1] == 0) return false;
+        all.push_back({x.n, x.s[0], x.s[1], false});
+        total *= x.n;
+    }
+    for (auto& x : red) {
+        if (x.n == 1) continue;
+        if (x.s[0] <= 0) return false;
+        all.push_back({x.n, x.s[0], 0, true});
+        total *= x.n;
+    }
+    if (total < 65536) return false;
+    std::stable_sort(all.begin(), all.end(), [](const Ax& x, const Ax& y) { return x.si < y.si; });
+    // neighbours of one kind that are dense in A (and in C, when kept) are one axis
+    std::vector<Ax> ax;
+    for (auto& x : all) {
+        if (!ax.empty() && ax.back().red == x.red && x.si == ax.back().si * ax.back().n &&
+            (x.red || x.so == ax.back().so * ax.back().n)) {
+            ax.back().n *= x.n;
+        } else {
+            ax.push_back(x);
+        }
+    }
+    // the dense prefix, and a tile in it
+    size_t np = 0;
+    for (int64_t run = 1; np < ax.size() && ax[np].si == run; ++np) run *= ax[np].n;
+    if (np == 0) return false;
+    RunArgs ra;
+    std::memset(&ra, 0, sizeof ra);
+    if (cx) {
+        ra.f_ext[0] = 2;
+        ra.nf = 1;
+    }
+    auto plan_tile = [&](int64_t cap, size_t& whole, int64_t& range) {   // axes [0, whole) whole, `range` indices of axis `whole`
+        int64_t w = nc;
+        whole = 0;
+        range = 0;
+        while (whole < np && (int)whole + (cx ? 1 : 0) < RUN_AXES - 1 && w * ax[whole].n <= cap) w *= ax[whole++].n;
+        if (whole < np && w <= cap) {
+            const int64_t t0 = std::max<int64_t>(1, cap / w), pieces = (ax[whole].n + t0 - 1) / t0;
+            if (t0 >= 2 || whole == 0) range = (ax[whole].n + pieces - 1) / pieces;   // (one index per tile: an axis outside the tile)
+        }
+        return w * std::max<int64_t>(1, range);
+    };
+    // The tile: as large as the vector slots of a block hold, unless that leaves the chip short of blocks.  Blocks come
+    // from the kept axes outside the tile and from splitting the walk, which is bounded by the size of the partial
+    // results (a share of A's) -- so with few outputs per tile a smaller tile is what gives more blocks.
+    constexpr int64_t target = 1280;   // blocks of a split walk: five per CU, all resident at once
+    constexpr int64_t minper = 2;      // tiles per block at least
+    struct Choice {
+        size_t whole;
+        int64_t range, tile_reals, kept_blocks, nsplit;
+    };
+    auto evaluate = [&](int64_t cap) {
+        Choice ch;
+        ch.tile_reals = plan_tile(cap, ch.whole, ch.range);
+        ch.kept_blocks = 1;
+        int64_t walk = 1, kept_in_tile = 1;
+        for (size_t i = 0; i < ax.size(); ++i) {
+            const bool ranged = i == ch.whole && ch.range > 0;
+            const int64_t outside = i < ch.whole ? 1 : (ranged ? (ax[i].n + ch.range - 1) / ch.range : ax[i].n);
+            const int64_t inside = i < ch.whole ? ax[i].n : (ranged ? ch.range : 1);
+            if (ax[i].red) walk *= outside;
+            else ch.kept_blocks *= outside, kept_in_tile *= inside;
+        }
+        ch.nsplit = 1;
+        if (ch.kept_blocks < 768 && walk >= 2 * minper) {
+            const int64_t outputs = ch.kept_blocks * kept_in_tile;
+            ch.nsplit = std::min<int64_t>(target / ch.kept_blocks, walk / minper);
+            ch.nsplit = std::min<int64_t>(ch.nsplit, std::max<int64_t>(1, total / (outputs * 48)));
+            ch.nsplit = std::max<int64_t>(1, std::min<int64_t>(ch.nsplit, 65535));
+        }
+        return ch;
+    };
+    Choice best = evaluate(RUN_REALS);
+    for (int64_t cap = RUN_REALS / 2; cap >= (int64_t)THREADS * nv && best.kept_blocks * best.nsplit < 1024; cap >>= 1) {
+        const Choice ch = evaluate(cap);
+        if (ch.kept_blocks * ch.nsplit > best.kept_blocks * best.nsplit) best = ch;
+    }
+    size_t whole = best.whole;
+    int64_t range = best.range;
+    const int64_t tile_reals = best.tile_reals;
+    if (tile_reals < 256) return false;   // a short dense prefix: most lanes would idle
+    int j = dbl ? 4 : 2;
+    while (j > 1 && (tile_reals + nv - 1) / nv <= (int64_t)THREADS * (j / 2)) j >>= 1;
+    // tile axes
+    int64_t kept_per_tile = 1;
+    for (size_t i = 0; i < whole + (range ? 1 : 0); ++i) {
+        const int f = ra.nf++;
+        const int64_t e = (i == whole) ? range : ax[i].n;
+        ra.f_ext[f] = (int32_t)e;
+        ra.f_red[f] = ax[i].red;
+        ra.f_so[f] = ax[i].so;
+        if (!ax[i].red) kept_per_tile *= e;
+    }
+    if (!range) {   // the tile is the whole prefix: its outermost axis is the ranged one, with a single range
+        if (whole == 0) return false;
+        range = ax[whole - 1].n;
+        --whole;
+    }
+    ra.tile_reals = (int32_t)tile_reals;
+    ra.range = (int32_t)range;
+    ra.x_n = (int32_t)ax[whole].n;
+    if (ax[whole].n > 0x7fffffff) {
+        // (the extent of the ranged axis is kept in 32 bits)
+        return false;
+    }
+    ra.row_reals = (int32_t)(tile_reals / range);
+    ra.kept_per_tile = (int32_t)kept_per_tile;
+    ra.all_reduced = 1;
+    for (int f = cx ? 1 : 0; f < ra.nf; ++f) ra.all_reduced &= ra.f_red[f];
+    const int64_t pieces = (ax[whole].n + range - 1) / range;
+    int64_t blocks = 1;
+    ra.r_total = 1;
+    if (pieces > 1) {
+        if (ax[whole].red) {
+            ra.r0_is_range = 1;
+            ra.r_count[0] = pieces;
+            ra.r_si[0] = ax[whole].si * range * nc;
+            ra.nr = 1;
+            ra.r_total = pieces;
+        } else {
+            ra.g0_is_range = 1;
+            ra.g_count[0] = pieces;
+            ra.g_si[0] = ax[whole].si * range * nc;
+            ra.g_so[0] = ax[whole].so * range;
+            ra.ng = 1;
+            blocks = pieces;
+        }
+    }
+    for (size_t i = whole + 1; i < ax.size(); ++i) {
+        if (ax[i].red) {
+            if (ra.nr == MAXR) return false;
+            ra.r_count[ra.nr] = ax[i].n;
+            ra.r_si[ra.nr] = ax[i].si * nc;
+            ++ra.nr;
+            ra.r_total *= ax[i].n;
+        } else {
+            if (ra.ng == MAXG) return false;
+            ra.g_count[ra.ng] = ax[i].n;
+            ra.g_si[ra.ng] = ax[i].si * nc;
+            ra.g_so[ra.ng] = ax[i].so;
+            ++ra.ng;
+            blocks *= ax[i].n;
+            if (blocks > 0x7fffffffll) return false;
+        }
+    }
+    if (ra.nr == 0) {
+        ra.nr = 1;
+        ra.r_count[0] = 1;
+    }
+    ra.blocks = blocks;
+    int64_t nsplit = best.nsplit;
+    ra.per_split = (ra.r_total + nsplit - 1) / nsplit;
+    nsplit = (ra.r_total + ra.per_split - 1) / ra.per_split;
+    ra.nsplit = (int32_t)nsplit;
+    ra.in = a;
+    ra.out = c;
+    ra.op = reduce_op;
+    ra.alpha_re = alpha.re;
+    ra.alpha_im = alpha.im;
+    ra.beta_re = beta.re;
+    ra.beta_im = beta.im;
+    ra.use_beta = !beta.is_zero();
+    if (nsplit > 1) {
+        void* ws = nullptr;
+        const size_t bytes = (size_t)nsplit * (size_t)blocks * (size_t)kept_per_tile * nc * sizeof(double);
+        if ((status = workspace(stream, bytes, &ws)) != TFH_OK) return true;
+        ra.partial = (double*)ws;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int prof = prof_begin(PROF_REDUCE, stream);
+    if (ra.all_reduced) {
+        // several outputs per block when each has a short walk
+        int ks = 8 / j;
+        while (ks > 1 && ((int64_t)ks * ra.per_split > 16 || blocks / ks < 1024)) ks >>= 1;
+        const dim3 grid((uint32_t)((blocks + ks - 1) / ks), (uint32_t)nsplit, 1);
+        switch (dtype) {
+            case TFH_F32: launch_rows<float, false>(ra, j, ks, grid, st); break;
+            case TFH_F64: launch_rows<double, false>(ra, j, ks, grid, st); break;
+            case TFH_C64: launch_rows<float, true>(ra, j, ks, grid, st); break;
+            default: launch_rows<double, true>(ra, j, ks, grid, st); break;
+        }
+    } else {
+        const dim3 grid((uint32_t)blocks, (uint32_t)nsplit, 1);
+        switch (dtype) {
+            case TFH_F32: launch_run<float, false>(ra, j, grid, st); break;
+            case TFH_F64: launch_run<double, false>(ra, j, grid, st); break;
+            case TFH_C64: launch_run<float, true>(ra, j, grid, st); break;
+            default: launch_run<double, true>(ra, j, grid, st); break;
+        }
+    }
+    prof_end(prof, stream);
+    if ((status = hip_check(hipGetLastError(), "reduce kernel launch")) != TFH_OK) return true;
+    if (nsplit > 1) {
+        const int64_t outputs = blocks * kept_per_tile;
+        int team = 1;
+        while (team < THREADS && team * 2 <= nsplit && outputs * team < 65536) team *= 2;
+        const int per = THREADS / team;
+        const dim3 g2((uint32_t)((outputs + per - 1) / per));
+        switch (dtype) {
+            case TFH_F32: hipLaunchKernelGGL((reduce_run_fold_kernel<float, false>), g2, dim3(THREADS), 0, st, ra, team); break;
+            case TFH_F64: hipLaunchKernelGGL((reduce_run_fold_kernel<double, false>), g2, dim3(THREADS), 0, st, ra, team); break;
+            case TFH_C64: hipLaunchKernelGGL((reduce_run_fold_kernel<float, true>), g2, dim3(THREADS), 0, st, ra, team); break;
+            default: hipLaunchKernelGGL((reduce_run_fold_kernel<double, true>), g2, dim3(THREADS), 0, st, ra, team); break;
+        }
+        status = hip_check(hipGetLastError(), "reduce fold launch");
+    }
+    return true;
+}
+}  // namespace
+
 int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, std::vector<Axis> red, int reduce_op,
                       Scalar alpha, Scalar beta, void* stream) {
     const int rb = is_double(dtype) ? 8 : 4;
@@ -964,6 +1734,7 @@ int32_t launch_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept,
         int32_t st_fast = TFH_OK;
         if (try_fast_reduce(dtype, a, c, kept, red, reduce_op, alpha, beta, stream, st_fast)) return st_fast;
         if (try_shortrow_reduce(dtype, a, c, kept, red, reduce_op, alpha, beta, stream, st_fast)) return st_fast;
+        if (try_run_reduce(dtype, a, c, kept, red, reduce_op, alpha, beta, stream, st_fast)) return st_fast;
     }
     for (auto& x : kept) x.s[2] = 0;
     for (auto& x : red) x.s[1] = x.s[2] = 0;

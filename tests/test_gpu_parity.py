@@ -2936,3 +2936,58 @@ def test_intermediates_cached_for_reuse_are_given_back_when_the_device_runs_out_
         del ballast
         assert tf.lib().tfh_release_workspaces() == 0
         torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_reduce_dense_runs_of_any_extent(tf, oracle, dtype):
+    # Extents that are no powers of two on a contiguous operand: the tiles are contiguous runs of memory with one ragged
+    # edge, folded over the reduced axes inside the tile in LDS.  Integer inputs: every sum is exact, so a dropped or
+    # doubled element (a ragged last range, the odd reals behind the last 16-byte vector, a split walk) changes the result.
+    rng = seeded_rng(131)
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    def ints(shape):
+        x = rng.integers(-9, 10, shape).astype(np.float64)
+        return (x + 1j * rng.integers(-9, 10, shape)).astype(dtype) if cplx else x.astype(dtype)
+    cases = [((37, 141, 147), [2]),            # kept innermost axis under one long fused reduced axis: split walk
+             ((41, 83, 1891), [0, 1]),         # long reduced rows, a tile per row
+             ((53, 42, 19, 79), [1, 2, 3]),    # outermost axis reduced, a range of the fused kept axis per tile
+             ((27, 90, 5, 21, 13), [0, 1, 3, 4]),   # a short reduced axis between kept ones
+             ((9, 25, 26, 11, 6, 9), [4]),     # nearly everything reduced, kept axis inside the tile
+             ((12, 10, 9, 7, 17, 5, 5), [0, 1, 4, 5, 6]),
+             ((5, 9, 33, 10, 21, 7), [3, 4, 5]),
+             ((358, 481, 3), [0, 2]),          # reduced middle axis, short kept rows
+             ((101, 29, 141, 9), [0]),
+             ((11, 139, 46, 3, 7), [2, 4]),
+             ((7, 37, 17, 19, 9, 3), [5]),
+             ((70001,), []),                   # one output
+             ((3, 70001), [0]),
+             ((66000, 3), [1])]
+    ran = 0
+    for shape, keep in cases:
+        a = ints(shape)
+        m = list(range(len(shape)))
+        got, ref = _reduce_check(tf, oracle, a, m, keep, tf.ReduceOp.Sum, oracle.SUM)
+        ran += "reduce_run_kernel" in tf.last_kernel()
+        assert np.array_equal(got, ref), (shape, keep, tf.last_kernel())
+        got2, _ = _reduce_check(tf, oracle, a, m, keep, tf.ReduceOp.Sum, oracle.SUM)
+        assert np.array_equal(got, got2), (shape, keep)                   # same bits on every run
+        perm = [int(p) for p in rng.permutation(len(keep))]                # outputs in another axis order
+        got3, ref3 = _reduce_check(tf, oracle, a, m, [keep[p] for p in perm], tf.ReduceOp.Sum, oracle.SUM)
+        assert np.array_equal(got3, ref3), (shape, keep, perm)
+    assert ran >= 10, ran
+    a = rand(rng, (37, 141, 147), dtype)
+    c0 = rand(rng, (147, 37), dtype)
+    alpha, beta = (0.5 - 2.0j, 1.5 + 0.25j) if cplx else (2.0, -0.5)
+    got, ref = _reduce_check(tf, oracle, a, [0, 1, 2], [2, 0], tf.ReduceOp.Sum, oracle.SUM, alpha=alpha, beta=beta, c0=c0)
+    assert relerr(got, ref) < TOL[dtype]
+    # the operand starts at an odd element of its buffer, so no tile starts on a 16-byte boundary
+    base = ints((37 * 141 * 147 + 3,))
+    a = base[3:].reshape(37, 141, 147)
+    got, ref = _reduce_check(tf, oracle, a, [0, 1, 2], [1], tf.ReduceOp.Sum, oracle.SUM)
+    assert np.array_equal(got, ref)
+    if not cplx:
+        a = rand(rng, (41, 83, 189), dtype)
+        for op_tf, op_or in [(tf.ReduceOp.Max, oracle.MAX), (tf.ReduceOp.Min, oracle.MIN)]:
+            for keep in ([0, 1], [2], [1], []):
+                got, ref = _reduce_check(tf, oracle, a, [0, 1, 2], keep, op_tf, op_or)
+                assert np.array_equal(got, ref), (keep, tf.last_kernel())
