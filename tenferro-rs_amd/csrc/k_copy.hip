@@ -430,23 +430,31 @@ __global__ void __launch_bounds__(NTH) copy_kernel(CopyArgs a, Op op) {
 // ---- tiles of many short axes ---------------------------------------------------------------------------------------
 // A tensor of many small extents (3^14, 2^16, [3,4]x6: spins and qubits) has no long axis to tile: four power-of-two tile
 // axes give runs of a few elements and, for extents that are no powers of two, mostly idle lanes (3^14 reversed:
-// 161 GB/s).  Here a tile is the product of WHOLE axes -- as many as it takes to reach 512-byte runs on both sides --
-// and the position-to-offset maps of a tile, which no longer are shifts and masks, come from three tables built once
-// per layout (input offset in read order; output offset and LDS position in write order) and kept in registers for
-// all the tiles a block moves.  Every tile is full by construction.
+// 161 GB/s).  Here a tile is the product of whole axes -- as many as it takes to reach 512-byte runs on both sides --
+// and, where a whole axis does not fit, of a range of its indices (one such axis per side at most: a long extent that
+// is no power of two, [27,466,1401]), and the position-to-offset maps of a tile, which no longer are shifts and masks,
+// come from tables built once per layout (input offset in read order; output offset and LDS position in write order)
+// and kept in registers for all the tiles a block moves.  Only the last range of a ranged axis is ragged: a tile
+// there looks up the coordinates of its positions along the ranged axes in two more tables and leaves out what lies
+// past the edge; every other tile is full.
 constexpr int TAB_MAX_AXES = 16;
 struct TabCopyArgs {
     const void* in;
     void* out;
-    const uint32_t* tab;   // [3][E]: input element offset of read position r; output offset and LDS position of write position w
+    // [5][E]: input element offset of read position r; output offset and LDS position of write position w; the
+    // coordinates along the two ranged axes (16 bits each) of read position r, and of write position w
+    const uint32_t* tab;
     int32_t E, ng;
     int64_t ntiles;
     int64_t g_count[MAXG], g_si[MAXG], g_so[MAXG];
+    int32_t g_slot[MAXG];    // 1, 2: the tile index along ranged axis 1, 2; 0: an axis outside the tile
+    int32_t x_n[2], x_t[2];  // extent of a ranged axis and its indices per tile (1, 1 when there is none)
 };
 struct TabBuildArgs {
     uint32_t* tab;
     int32_t E, nt;
     int32_t r_ext[TAB_MAX_AXES], w_ext[TAB_MAX_AXES], w_rpos[TAB_MAX_AXES];
+    int32_t r_slot[TAB_MAX_AXES], w_slot[TAB_MAX_AXES];   // 1, 2: a ranged axis; 0: a whole one
     int64_t r_si[TAB_MAX_AXES], w_so[TAB_MAX_AXES];
 };
 __global__ void __launch_bounds__(THREADS) tabcopy_build_kernel(TabBuildArgs b) {
@@ -454,23 +462,36 @@ __global__ void __launch_bounds__(THREADS) tabcopy_build_kernel(TabBuildArgs b) 
     if (i >= b.E) return;
     int lin = i;
     int64_t off = 0;
+    uint32_t xc = 0;
     for (int t = 0; t < b.nt; ++t) {
-        const int q = lin / b.r_ext[t];
-        off += (int64_t)(lin - q * b.r_ext[t]) * b.r_si[t];
+        const int q = lin / b.r_ext[t], c = lin - q * b.r_ext[t];
+        off += (int64_t)c * b.r_si[t];
+        if (b.r_slot[t]) xc |= (uint32_t)c << (16 * (b.r_slot[t] - 1));
         lin = q;
     }
     b.tab[i] = (uint32_t)off;
+    b.tab[3 * b.E + i] = xc;
     lin = i;
     off = 0;
+    xc = 0;
     int pos = 0;
     for (int t = 0; t < b.nt; ++t) {
         const int q = lin / b.w_ext[t], c = lin - q * b.w_ext[t];
         off += (int64_t)c * b.w_so[t];
         pos += c * b.w_rpos[t];
+        if (b.w_slot[t]) xc |= (uint32_t)c << (16 * (b.w_slot[t] - 1));
         lin = q;
     }
     b.tab[b.E + i] = (uint32_t)off;
     b.tab[2 * b.E + i] = (uint32_t)pos;
+    b.tab[4 * b.E + i] = xc;
+}
+
+// Tile t of a block on XCD x (blocks go to the XCDs in turn) -> a tile index such that every XCD moves one contiguous
+// eighth of the tiles: tiles that abut in memory share 128-byte lines at their edges, and meet in one L2.
+__device__ __forceinline__ uint64_t tab_tile_of(uint64_t slot, uint64_t ntiles) {
+    const uint64_t per = (ntiles + 7) / 8;
+    return (slot & 7) * per + (slot >> 3);
 }
 
 template <class V, int EPT>
@@ -489,30 +510,52 @@ __global__ void __launch_bounds__(THREADS) tabcopy_kernel(TabCopyArgs a) {
             lpos[j] = swz((int)a.tab[2 * E + r]);
         }
     }
-    auto origin = [&](uint64_t tile, int64_t& oi, int64_t& oo) {
+    // origin of a tile and the indices of the ranged axes it holds, packed like the coordinates in the tables
+    auto origin = [&](uint64_t tile, int64_t& oi, int64_t& oo, uint32_t& lim) {
         oi = oo = 0;
+        int l[2] = {a.x_t[0], a.x_t[1]};
         for (int g = 0; g < a.ng; ++g) {
             const uint64_t q = tile / (uint64_t)a.g_count[g];
             const int64_t c = (int64_t)(tile - q * (uint64_t)a.g_count[g]);
             tile = q;
             oi += c * a.g_si[g];
             oo += c * a.g_so[g];
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+                if (a.g_slot[g] == x + 1) {
+                    const int64_t left = (int64_t)a.x_n[x] - c * a.x_t[x];
+                    if (left < l[x]) l[x] = (int)left;
+                }
         }
         oi = uniform64(oi);
         oo = uniform64(oo);
+        lim = (uint32_t)__builtin_amdgcn_readfirstlane(l[0] | (l[1] << 16));
     };
+    const uint32_t lim_full = (uint32_t)(a.x_t[0] | (a.x_t[1] << 16));
+    auto inside = [&](uint32_t xc, uint32_t lim) { return (xc & 0xffffu) < (lim & 0xffffu) && (xc >> 16) < (lim >> 16); };
     V regs[EPT];
-    auto load = [&](int64_t oi) {
+    auto load = [&](int64_t oi, uint32_t lim) {
         const V* in = reinterpret_cast<const V*>(a.in) + oi;
+        if (lim == lim_full) {
 #pragma unroll
-        for (int j = 0; j < EPT; ++j)
-            if (tid + THREADS * j < E) regs[j] = load_stream<Pack<V, 1>>(in + roff[j]).v[0];
+            for (int j = 0; j < EPT; ++j)
+                if (tid + THREADS * j < E) regs[j] = load_stream<Pack<V, 1>>(in + roff[j]).v[0];
+        } else {   // a tile at a ragged edge: the positions past the edge are left out
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) {
+                const int r = tid + THREADS * j;
+                if (r < E && inside(a.tab[3 * E + r], lim)) regs[j] = load_stream<Pack<V, 1>>(in + roff[j]).v[0];
+            }
+        }
     };
-    uint64_t tile = blockIdx.x;
-    if (tile >= (uint64_t)a.ntiles) return;
+    const uint64_t ntiles = (uint64_t)a.ntiles, slots = (ntiles + 7) / 8 * 8;
+    uint64_t slot = blockIdx.x;
+    while (slot < slots && tab_tile_of(slot, ntiles) >= ntiles) slot += gridDim.x;
+    if (slot >= slots) return;
     int64_t oi, oo;
-    origin(tile, oi, oo);
-    load(oi);
+    uint32_t lim;
+    origin(tab_tile_of(slot, ntiles), oi, oo, lim);
+    load(oi, lim);
     for (;;) {
 #pragma unroll
         for (int j = 0; j < EPT; ++j) {
@@ -520,25 +563,40 @@ __global__ void __launch_bounds__(THREADS) tabcopy_kernel(TabCopyArgs a) {
             if (r < E) lds[swz(r)] = regs[j];
         }
         __syncthreads();
-        const uint64_t next = tile + gridDim.x;
-        const bool more = next < (uint64_t)a.ntiles;
+        uint64_t next = slot + gridDim.x;
+        while (next < slots && tab_tile_of(next, ntiles) >= ntiles) next += gridDim.x;
+        const bool more = next < slots;
         int64_t oi2 = 0, oo2 = 0;
+        uint32_t lim2 = lim_full;
         if (more) {   // the next tile's loads are in flight while this one is written out
-            origin(next, oi2, oo2);
-            load(oi2);
+            origin(tab_tile_of(next, ntiles), oi2, oo2, lim2);
+            load(oi2, lim2);
         }
         V* out = reinterpret_cast<V*>(a.out) + oo;
+        if (lim == lim_full) {
 #pragma unroll
-        for (int j = 0; j < EPT; ++j)
-            if (tid + THREADS * j < E) {
-                Pack<V, 1> x;
-                x.v[0] = lds[lpos[j]];
-                store_stream<Pack<V, 1>>(out + woff[j], x);
+            for (int j = 0; j < EPT; ++j)
+                if (tid + THREADS * j < E) {
+                    Pack<V, 1> x;
+                    x.v[0] = lds[lpos[j]];
+                    store_stream<Pack<V, 1>>(out + woff[j], x);
+                }
+        } else {
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) {
+                const int w = tid + THREADS * j;
+                if (w < E && inside(a.tab[4 * E + w], lim)) {
+                    Pack<V, 1> x;
+                    x.v[0] = lds[lpos[j]];
+                    store_stream<Pack<V, 1>>(out + woff[j], x);
+                }
             }
+        }
         if (!more) break;
         __syncthreads();
-        tile = next;
+        slot = next;
         oo = oo2;
+        lim = lim2;
     }
 }
 
@@ -956,6 +1014,405 @@ void launch_tabcopy(const TabCopyArgs& ta, int ept, dim3 grid, size_t lds, hipSt
     else TFH_LAUNCH_TIMED((tabcopy_kernel<V, 32>), grid, dim3(THREADS), lds, st, ta);
 }
 
+// ---- long extents that are no powers of two ---------------------------------------------------------------------------
+// A permutation of a tensor like [27,466,1401] has runs of kilobytes on both sides, but no power-of-two tile grid
+// fits it, and a tile small enough to keep per-element offsets in registers has runs of a few hundred bytes that
+// start anywhere: every run pays for the partly used 128-byte lines at its ends.  Here a tile is 64 KB and two-sided:
+// a group RF of axes that are dense in the input (whole axes and, last, a range of the next one) and a group WF that
+// is dense in the output.  A wave reads 64 consecutive elements of an input run per instruction -- thread t always
+// has column 64 k + t of the run, the row changes with the register -- and writes them to LDS in read order; then it
+// writes 64 consecutive elements of an output run per instruction, thread t gathering column 64 k + t of the
+// write order from LDS.  What changes from row to row is the same for all lanes (the offset of the row in memory,
+// the coordinates of the ranged axes it lies at) and comes from small tables that every block computes for itself
+// in LDS at start: nothing is kept per element, so the tile can be large.  Tiles are full except at the last range
+// of a ranged axis (two such axes at most), where lanes past the run's end and rows past the edge are left out of
+// the stores; their loads are redirected to addresses inside the tile, so that no load is conditional.
+constexpr int PERM_AXES = 8;   // axes per group
+struct PermGroup {
+    int32_t n;
+    int32_t ext[PERM_AXES];    // mixed radix, innermost first
+    int32_t lds[PERM_AXES];    // LDS position stride
+    int32_t slot[PERM_AXES];   // 1, 2: the axis is ranged axis 1, 2
+    int64_t mem[PERM_AXES];    // memory stride (elements)
+};
+struct PermArgs {
+    const void* in;
+    void* out;
+    PermGroup rs, ws, wf;      // rows of the read order (input strides), rows of the write order (output strides), write columns
+    int32_t rfn, rsn, wfn, wsn, pitch;
+    int32_t rf_slot, wf_slot;  // the ranged axis that is last in RF / WF (0: none), and the elements per index of it
+    int32_t rf_row, wf_row;
+    int32_t x_n[2], x_t[2];    // extent of a ranged axis and its indices per tile (1, 1 when there is none)
+    int32_t ng;
+    int64_t ntiles;
+    int64_t g_count[MAXG], g_si[MAXG], g_so[MAXG];
+    int32_t g_slot[MAXG];
+};
+
+// entry i of a group: memory offset, LDS position, coordinates along the ranged axes (16 bits each)
+__device__ __forceinline__ void perm_entry(const PermGroup& g, int i, uint32_t& mem, uint32_t& lds, uint32_t& xc) {
+    int64_t m = 0;
+    lds = xc = 0;
+    for (int t = 0; t < g.n; ++t) {
+        const int q = i / g.ext[t], c = i - q * g.ext[t];
+        i = q;
+        m += (int64_t)c * g.mem[t];
+        lds += (uint32_t)(c * g.lds[t]);
+        if (g.slot[t]) xc |= (uint32_t)c << (16 * (g.slot[t] - 1));
+    }
+    mem = (uint32_t)m;
+}
+
+constexpr int PERM_THREADS = 512, PERM_WAVES = PERM_THREADS / 64;
+constexpr int PERM_WSEG = 8;   // a write run is up to 8 wave instructions wide
+
+template <class V, int NSEG, int JR>
+__global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
+    prefetch_kernel_arguments<sizeof(PermArgs)>();
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    V* lds = reinterpret_cast<V*>(smem_raw);
+    uint32_t* tab = reinterpret_cast<uint32_t*>(smem_raw + (size_t)a.pitch * a.rsn * sizeof(V));
+    uint32_t* out_s = tab;                 // [wsn] output offset of a row of the write order
+    uint32_t* lw_s = out_s + a.wsn;        // [wsn] its LDS position
+    uint32_t* c_ws = lw_s + a.wsn;         // [wsn] its coordinates along the ranged axes
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    for (int i = tid; i < a.wsn; i += PERM_THREADS) perm_entry(a.ws, i, out_s[i], lw_s[i], c_ws[i]);
+    // the rows of the read order that this wave reads, the same in every tile: their input offsets and coordinates
+    uint32_t in_s[JR], c_rs[JR];
+#pragma unroll
+    for (int jj = 0; jj < JR; ++jj) {
+        const int rs = wave + PERM_WAVES * jj;
+        uint32_t l, m = 0, xc = 0;
+        if (rs < a.rsn) perm_entry(a.rs, rs, m, l, xc);
+        in_s[jj] = __builtin_amdgcn_readfirstlane(m);
+        c_rs[jj] = __builtin_amdgcn_readfirstlane(rs < a.rsn ? xc : 0xffffffffu);   // (a row past the tile: never inside)
+    }
+    uint32_t lwf[PERM_WSEG];   // LDS position of this thread's columns of the write order
+#pragma unroll
+    for (int k = 0; k < PERM_WSEG; ++k) {
+        uint32_t m, xc;
+        lwf[k] = 0;
+        if (64 * k + lane < a.wfn) perm_entry(a.wf, 64 * k + lane, m, lwf[k], xc);
+    }
+    __syncthreads();
+    auto origin = [&](uint64_t tile, int64_t& oi, int64_t& oo, uint32_t& lim) {
+        oi = oo = 0;
+        int l[2] = {a.x_t[0], a.x_t[1]};
+        for (int g = 0; g < a.ng; ++g) {
+            const uint64_t q = tile / (uint64_t)a.g_count[g];
+            const int64_t c = (int64_t)(tile - q * (uint64_t)a.g_count[g]);
+            tile = q;
+            oi += c * a.g_si[g];
+            oo += c * a.g_so[g];
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+                if (a.g_slot[g] == x + 1) {
+                    const int64_t left = (int64_t)a.x_n[x] - c * a.x_t[x];
+                    if (left < l[x]) l[x] = (int)left;
+                }
+        }
+        oi = uniform64(oi);
+        oo = uniform64(oo);
+        lim = (uint32_t)__builtin_amdgcn_readfirstlane(l[0] | (l[1] << 16));
+    };
+    const uint32_t lim_full = (uint32_t)(a.x_t[0] | (a.x_t[1] << 16));
+    auto inside = [&](uint32_t xc, uint32_t lim) { return (xc & 0xffffu) < (lim & 0xffffu) && (xc >> 16) < (lim >> 16); };
+    auto run_len = [&](int slot, int row, int full, uint32_t lim) {   // elements of a run inside the tensor at this tile
+        if (slot == 0) return full;
+        return (int)(slot == 1 ? (lim & 0xffffu) : (lim >> 16)) * row;
+    };
+    V regs[NSEG * JR];
+    auto load = [&](int64_t oi, uint32_t lim) {
+        const V* in = reinterpret_cast<const V*>(a.in) + oi;
+        const int len = run_len(a.rf_slot, a.rf_row, a.rfn, lim);
+        uint32_t col[NSEG];   // columns past the end of the run read its last element
+#pragma unroll
+        for (int k = 0; k < NSEG; ++k) col[k] = (uint32_t)(64 * k + lane < len ? 64 * k + lane : len - 1);
+#pragma unroll
+        for (int jj = 0; jj < JR; ++jj) {
+            // (a row past the edge reads row 0, which lies inside the tensor at every tile)
+            const V* row = in + (inside(c_rs[jj], lim) ? in_s[jj] : in_s[0]);
+#pragma unroll
+            for (int k = 0; k < NSEG; ++k) regs[k * JR + jj] = load_stream<Pack<V, 1>>(row + col[k]).v[0];
+        }
+    };
+    const uint64_t ntiles = (uint64_t)a.ntiles, slots = (ntiles + 7) / 8 * 8;
+    uint64_t slot = blockIdx.x;
+    while (slot < slots && tab_tile_of(slot, ntiles) >= ntiles) slot += gridDim.x;
+    if (slot >= slots) return;
+    int64_t oi, oo;
+    uint32_t lim;
+    origin(tab_tile_of(slot, ntiles), oi, oo, lim);
+    load(oi, lim);
+    for (;;) {
+#pragma unroll
+        for (int jj = 0; jj < JR; ++jj) {
+            const int rs = wave + PERM_WAVES * jj;
+            if (rs < a.rsn) {
+#pragma unroll
+                for (int k = 0; k < NSEG; ++k)
+                    if (64 * k + lane < a.rfn) lds[rs * a.pitch + 64 * k + lane] = regs[k * JR + jj];
+            }
+        }
+        __syncthreads();
+        uint64_t next = slot + gridDim.x;
+        while (next < slots && tab_tile_of(next, ntiles) >= ntiles) next += gridDim.x;
+        const bool more = next < slots;
+        int64_t oi2 = 0, oo2 = 0;
+        uint32_t lim2 = 0;
+        if (more) {   // the next tile's loads are in flight while this one is written out
+            origin(tab_tile_of(next, ntiles), oi2, oo2, lim2);
+            load(oi2, lim2);
+        }
+        V* out = reinterpret_cast<V*>(a.out) + oo;
+        if (lim == lim_full) {
+            for (int ws = wave; ws < a.wsn; ws += PERM_WAVES) {
+                const uint32_t lrow = __builtin_amdgcn_readfirstlane(lw_s[ws]);
+                V* orow = out + __builtin_amdgcn_readfirstlane(out_s[ws]);
+#pragma unroll
+                for (int k = 0; k < PERM_WSEG; ++k)
+                    if (64 * k + lane < a.wfn) {
+                        Pack<V, 1> x;
+                        x.v[0] = lds[lwf[k] + lrow];
+                        store_stream<Pack<V, 1>>(orow + (uint32_t)(64 * k + lane), x);
+                    }
+            }
+        } else {
+            const int wlen = run_len(a.wf_slot, a.wf_row, a.wfn, lim);
+            for (int ws = wave; ws < a.wsn; ws += PERM_WAVES) {
+                if (!inside(c_ws[ws], lim)) continue;
+                const uint32_t lrow = __builtin_amdgcn_readfirstlane(lw_s[ws]);
+                V* orow = out + __builtin_amdgcn_readfirstlane(out_s[ws]);
+#pragma unroll
+                for (int k = 0; k < PERM_WSEG; ++k)
+                    if (64 * k + lane < wlen) {
+                        Pack<V, 1> x;
+                        x.v[0] = lds[lwf[k] + lrow];
+                        store_stream<Pack<V, 1>>(orow + (uint32_t)(64 * k + lane), x);
+                    }
+            }
+        }
+        if (!more) break;
+        __syncthreads();
+        slot = next;
+        oo = oo2;
+        lim = lim2;
+    }
+}
+
+template <class V, int EPT>
+void launch_perm(const PermArgs& pa, int nseg, dim3 grid, size_t lds, hipStream_t st) {
+    if (nseg == 1) TFH_LAUNCH_TIMED((perm_kernel<V, 1, EPT>), grid, dim3(PERM_THREADS), lds, st, pa);
+    else if (nseg == 2) TFH_LAUNCH_TIMED((perm_kernel<V, 2, EPT / 2>), grid, dim3(PERM_THREADS), lds, st, pa);
+    else TFH_LAUNCH_TIMED((perm_kernel<V, 4, EPT / 4>), grid, dim3(PERM_THREADS), lds, st, pa);
+}
+
+// A bit-exact move of extents that the shift-and-mask tiles do not fill: two-sided 64 KB tiles.  Returns true when
+// it launched (status holds the outcome).
+bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, void* stream, int32_t& status) {
+    status = TFH_OK;
+    int64_t total = 1;
+    for (auto& x : axes) total *= x.n;
+    if (total < ((int64_t)1 << 20)) return false;
+    std::stable_sort(axes.begin(), axes.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[1]) > std::llabs(y.s[1]); });
+    fuse_axes(axes, 2);
+    const int na = (int)axes.size();
+    if (na < 2 || na > MAXG) return false;
+    for (auto& x : axes)
+        if (x.s[0] <= 0 || x.s[1] <= 0 || x.n > 0x7fffffff) return false;
+    std::vector<int> in_order(na), out_order(na);
+    for (int i = 0; i < na; ++i) in_order[i] = out_order[i] = i;
+    std::stable_sort(in_order.begin(), in_order.end(), [&](int x, int y) { return axes[x].s[0] < axes[y].s[0]; });
+    std::stable_sort(out_order.begin(), out_order.end(), [&](int x, int y) { return axes[x].s[1] < axes[y].s[1]; });
+    if (axes[in_order[0]].s[0] != 1 || axes[out_order[0]].s[1] != 1) return false;
+    const int ept = eb == 4 ? 32 : (eb == 8 ? 16 : 8);   // the registers of 512 threads hold a 64 KB tile
+    int64_t emax = (int64_t)PERM_THREADS * ept;
+    std::vector<int64_t> in_tile(na, 0);   // indices of the axis per tile (0: outside the tile)
+    int nranged = 0;
+    // a dense run of up to `cap` elements along one side's order: whole axes, then a range of the next
+    auto take_run = [&](int side, int64_t cap, int64_t& E, std::vector<char>& members) {
+        const std::vector<int>& ord = side ? out_order : in_order;
+        int64_t run = 1;
+        for (int i : ord) {
+            if (axes[i].s[side] != run) break;
+            if (in_tile[i]) {   // already in the tile through the other side
+                if (run * in_tile[i] > cap) break;
+                members[i] = 1;
+                run *= in_tile[i];
+                if (in_tile[i] != axes[i].n) break;
+                continue;
+            }
+            const int64_t room = std::min<int64_t>(cap / run, emax / E);
+            if (axes[i].n <= room) {
+                in_tile[i] = axes[i].n;
+                members[i] = 1;
+                E *= axes[i].n;
+                run *= axes[i].n;
+                continue;
+            }
+            if (room >= 2 && nranged < 2) {
+                const int64_t pieces = (axes[i].n + room - 1) / room;
+                in_tile[i] = (axes[i].n + pieces - 1) / pieces;
+                members[i] = 1;
+                E *= in_tile[i];
+                run *= in_tile[i];
+                ++nranged;
+            }
+            break;
+        }
+        return run;
+    };
+    int64_t E = 1;
+    std::vector<char> in_rf(na, 0), in_wf(na, 0);
+    // the read run first: two wave instructions wide at most (half that for 16-byte elements), then the write run in
+    // the room that the registers of a thread leave (a row per wave and register)
+    const int64_t rfn = take_run(0, eb == 16 ? 64 : 128, E, in_rf);
+    if (rfn < 16) return false;
+    const int nseg = rfn <= 64 ? 1 : (rfn <= 128 ? 2 : 4);
+    emax = std::min<int64_t>(emax, rfn * PERM_WAVES * (ept / nseg));
+    const int64_t wfn = take_run(1, 64 * PERM_WSEG, E, in_wf);
+    if (wfn < 16) return false;
+    // room left (a short output run): more of the input's fastest axes, then whole axes from either side
+    for (int side = 0, idle = 0; E * 2 <= emax && idle < 2; side ^= 1) {
+        const std::vector<int>& ord = side ? out_order : in_order;
+        int pick = -1;
+        for (int i : ord)
+            if (!in_tile[i]) { pick = i; break; }
+        if (pick < 0) { ++idle; continue; }
+        const int64_t room = emax / E;
+        if (axes[pick].n <= room) {
+            in_tile[pick] = axes[pick].n;
+            E *= axes[pick].n;
+            idle = 0;
+        } else if (room >= 2 && nranged < 2) {
+            const int64_t pieces = (axes[pick].n + room - 1) / room;
+            in_tile[pick] = (axes[pick].n + pieces - 1) / pieces;
+            E *= in_tile[pick];
+            ++nranged;
+            idle = 0;
+        } else {
+            ++idle;
+        }
+    }
+    if (E < 2048) return false;
+    PermArgs pa;
+    std::memset(&pa, 0, sizeof pa);
+    pa.x_n[0] = pa.x_n[1] = pa.x_t[0] = pa.x_t[1] = 1;
+    std::vector<int> slot(na, 0);
+    int nslots = 0;
+    for (int i = 0; i < na; ++i)
+        if (in_tile[i] && in_tile[i] != axes[i].n) {
+            slot[i] = ++nslots;
+            pa.x_n[nslots - 1] = (int32_t)axes[i].n;
+            pa.x_t[nslots - 1] = (int32_t)in_tile[i];
+            if (in_tile[i] > 0xffff) return false;
+        }
+    // a ranged axis is the last of its run: the elements per index of it
+    pa.rf_row = pa.wf_row = 1;
+    for (int i : in_order)
+        if (in_rf[i]) {
+            if (slot[i]) pa.rf_slot = slot[i];
+            else pa.rf_row *= (int32_t)in_tile[i];
+        }
+    for (int i : out_order)
+        if (in_wf[i]) {
+            if (slot[i]) pa.wf_slot = slot[i];
+            else pa.wf_row *= (int32_t)in_tile[i];
+        }
+    const int64_t wfn2 = wfn;
+    const int64_t rsn = E / rfn, wsn = E / wfn2;
+    if (rsn > PERM_WAVES * (ept / nseg)) return false;
+    const int64_t pitch = rfn | 1;
+    // LDS position strides: an axis of RF by its place in the run, a row axis by its place among the rows times the pitch
+    std::vector<int64_t> lpos(na, 0);
+    {
+        int64_t f = 1, r = 1;
+        for (int i : in_order) {
+            if (!in_tile[i]) continue;
+            if (in_rf[i]) {
+                lpos[i] = f;
+                f *= in_tile[i];
+            }
+        }
+        for (int i : in_order) {
+            if (!in_tile[i] || in_rf[i]) continue;
+            lpos[i] = r * pitch;
+            r *= in_tile[i];
+        }
+    }
+    int64_t span_in = 0, span_out = 0;
+    auto add = [&](PermGroup& g, int i, int64_t mem) {
+        if (g.n == PERM_AXES) return false;
+        g.ext[g.n] = (int32_t)in_tile[i];
+        g.lds[g.n] = (int32_t)lpos[i];
+        g.slot[g.n] = slot[i];
+        g.mem[g.n] = mem;
+        ++g.n;
+        return true;
+    };
+    for (int i : in_order) {
+        if (!in_tile[i]) continue;
+        span_in += (in_tile[i] - 1) * axes[i].s[0];
+        span_out += (in_tile[i] - 1) * axes[i].s[1];
+        if (!in_rf[i] && !add(pa.rs, i, axes[i].s[0])) return false;
+    }
+    for (int i : out_order) {
+        if (!in_tile[i]) continue;
+        if (in_wf[i]) {
+            if (!add(pa.wf, i, axes[i].s[1])) return false;
+        } else if (!add(pa.ws, i, axes[i].s[1])) {
+            return false;
+        }
+    }
+    if (span_in >= ((int64_t)1 << 32) || span_out >= ((int64_t)1 << 32)) return false;   // 32-bit element offsets
+    pa.rfn = (int32_t)rfn;
+    pa.rsn = (int32_t)rsn;
+    pa.wfn = (int32_t)wfn2;
+    pa.wsn = (int32_t)wsn;
+    pa.pitch = (int32_t)pitch;
+    pa.in = in;
+    pa.out = out;
+    int64_t ntiles = 1;
+    for (int i = na - 1; i >= 0; --i) {   // fastest tile index: the innermost axis outside the tile (neighbouring tiles abut)
+        if (in_tile[i] == axes[i].n) continue;
+        const int64_t t = in_tile[i] ? in_tile[i] : 1, count = (axes[i].n + t - 1) / t;
+        if (pa.ng == MAXG) return false;
+        pa.g_count[pa.ng] = count;
+        pa.g_si[pa.ng] = axes[i].s[0] * t;
+        pa.g_so[pa.ng] = axes[i].s[1] * t;
+        pa.g_slot[pa.ng] = slot[i];
+        ++pa.ng;
+        ntiles *= count;
+    }
+    pa.ntiles = ntiles;
+    if (ntiles < 1024) return false;   // (two tiles per block on every CU at least: smaller tensors take smaller tiles)
+    const size_t lds = (size_t)pitch * rsn * eb + (size_t)(3 * wsn) * sizeof(uint32_t);
+    if (lds > 150 * 1024) return false;
+    static const bool lds_limit_raised = [] {
+        const int cap = 160 * 1024;
+#define TFH_PERM_LDS(V, E)                                                                                                  \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 1, E>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);      \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 2, E / 2>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);  \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 4, E / 4>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+        TFH_PERM_LDS(uint32_t, 32)
+        TFH_PERM_LDS(uint64_t, 16)
+        TFH_PERM_LDS(double2, 8)
+#undef TFH_PERM_LDS
+        return true;
+    }();
+    (void)lds_limit_raised;
+    const size_t per_cu = std::max<size_t>(1, std::min<size_t>(4, (size_t)(160 * 1024) / (lds + 512)));
+    const dim3 grid((uint32_t)std::min<int64_t>((ntiles + 7) / 8 * 8, (int64_t)(256 * per_cu)));   // (a multiple of 8: a block stays on its XCD)
+    hipStream_t st = (hipStream_t)stream;
+    const int prof = prof_begin(PROF_COPY, stream);
+    if (eb == 4) launch_perm<uint32_t, 32>(pa, nseg, grid, lds, st);
+    else if (eb == 8) launch_perm<uint64_t, 16>(pa, nseg, grid, lds, st);
+    else launch_perm<double2, 8>(pa, nseg, grid, lds, st);
+    prof_end(prof, stream);
+    status = hip_check(hipGetLastError(), "copy kernel launch");
+    return true;
+}
+
 // A bit-exact move whose shift-and-mask tiles come out with short runs or mostly empty: tiles of whole axes, driven by
 // tables.  Returns true when it launched (status holds the outcome).
 bool try_table_copy(int eb, const void* in, void* out, std::vector<Axis> axes, const TilePlan& tp, void* stream, int32_t& status) {
@@ -967,7 +1424,7 @@ bool try_table_copy(int eb, const void* in, void* out, std::vector<Axis> axes, c
     double filled;
     masked_plan_quality(tp.args, run_in_old, run_out_old, filled);
     const double old_q = (double)std::min<int64_t>(std::min(run_in_old, run_out_old) * eb, 512) * (tp.all_full ? 1.0 : filled);
-    if (old_q >= 256.0) return false;
+    if (tp.all_full && old_q >= 256.0) return false;   // (tiles with a ragged edge pay a bounds check per element there)
     std::stable_sort(axes.begin(), axes.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[1]) > std::llabs(y.s[1]); });
     fuse_axes(axes, 2);
     const int na = (int)axes.size();
@@ -978,19 +1435,24 @@ bool try_table_copy(int eb, const void* in, void* out, std::vector<Axis> axes, c
     for (int i = 0; i < na; ++i) in_order[i] = out_order[i] = i;
     std::stable_sort(in_order.begin(), in_order.end(), [&](int x, int y) { return axes[x].s[0] < axes[y].s[0]; });
     std::stable_sort(out_order.begin(), out_order.end(), [&](int x, int y) { return axes[x].s[1] < axes[y].s[1]; });
-    // whole axes, alternately from the input's and the output's fastest end, while the tile fits and a side is short
-    const int64_t emax = std::min<int64_t>(61440 / eb, (int64_t)THREADS * 32);
+    // axes alternately from the input's and the output's fastest end while a side is short of `want`: whole while the
+    // tile has room for them and for what the other side still needs, else a range of the axis, which closes the side
+    // (eight elements per thread: with 16 or 32 the three offsets per element fill the register file and one block
+    // is left per CU -- [5]^9 f64 reversed 46 us with 32, 36 with 16, 24 with 8)
+    const int64_t emax = std::min<int64_t>(61440 / eb, (int64_t)THREADS * 8);
     const int64_t want = std::max<int64_t>(1, 512 / eb);
-    std::vector<char> in_tile(na, 0);
+    std::vector<int64_t> in_tile(na, 0);   // indices of the axis per tile (0: outside the tile)
     int64_t E = 1, run[2] = {1, 1};
     size_t pos[2] = {0, 0};
     bool open_[2] = {true, true};
+    int nranged = 0;
     const std::vector<int>* order[2] = {&in_order, &out_order};
     auto advance = [&](int side) {   // run of a side = product of the leading axes of its order that are in the tile
-        while (pos[side] < (size_t)na && in_tile[(*order[side])[pos[side]]]) {
-            const Axis& x = axes[(*order[side])[pos[side]]];
-            if (x.s[side] != run[side]) { open_[side] = false; break; }   // not contiguous with the run so far
-            run[side] *= x.n;
+        while (open_[side] && pos[side] < (size_t)na && in_tile[(*order[side])[pos[side]]]) {
+            const int i = (*order[side])[pos[side]];
+            if (axes[i].s[side] != run[side]) { open_[side] = false; break; }   // not contiguous with the run so far
+            run[side] *= in_tile[i];
+            if (in_tile[i] != axes[i].n) { open_[side] = false; break; }         // a range ends the run
             ++pos[side];
         }
         if (pos[side] == (size_t)na) open_[side] = false;
@@ -1003,9 +1465,23 @@ bool try_table_copy(int eb, const void* in, void* out, std::vector<Axis> axes, c
         else if (open_[1] && run[1] < want) side = 1;
         if (side < 0) break;
         const int i = (*order[side])[pos[side]];
-        if (axes[i].s[side] != run[side] || E * axes[i].n > emax) { open_[side] = false; continue; }
-        in_tile[i] = 1;
-        E *= axes[i].n;
+        if (axes[i].s[side] != run[side]) { open_[side] = false; continue; }
+        const int other = side ^ 1;
+        const int64_t need_other = (open_[other] && run[other] < want) ? (want + run[other] - 1) / run[other] : 1;
+        const int64_t room = emax / E, fair = std::max<int64_t>(1, room / need_other);
+        if (axes[i].n <= fair) {
+            in_tile[i] = axes[i].n;
+            E *= axes[i].n;
+            continue;
+        }
+        // a range of it: the room that is left, less what the other side still needs
+        const int64_t t0 = std::min<int64_t>(fair, 0xffff);
+        // (extents that the shift-and-mask tiles fill completely keep those tiles' 16-byte accesses: whole axes only)
+        if (t0 < 2 || nranged == 2 || tp.all_full) { open_[side] = false; continue; }
+        const int64_t pieces = (axes[i].n + t0 - 1) / t0;
+        in_tile[i] = (axes[i].n + pieces - 1) / pieces;
+        E *= in_tile[i];
+        ++nranged;
     }
     // runs reached with a small tile (a few short axes serve both sides): more whole axes, the input's innermost free
     // axis and the output's in turn, until a block has 2048 elements to move per tile
@@ -1015,59 +1491,82 @@ bool try_table_copy(int eb, const void* in, void* out, std::vector<Axis> axes, c
             if (!in_tile[i]) { pick = i; break; }
         if (pick < 0 || E * axes[pick].n > emax) { ++idle; continue; }
         idle = 0;
-        in_tile[pick] = 1;
+        in_tile[pick] = axes[pick].n;
         E *= axes[pick].n;
+    }
+    // the runs of the finished tile
+    for (int side = 0; side < 2; ++side) {
+        run[side] = 1;
+        for (int i : *order[side]) {
+            if (!in_tile[i] || axes[i].s[side] != run[side]) break;
+            run[side] *= in_tile[i];
+            if (in_tile[i] != axes[i].n) break;
+        }
     }
     if (E < 512) return false;
     const double new_q = (double)std::min<int64_t>(std::min(run[0], run[1]) * eb, 512);
-    if (new_q < 2.0 * old_q) return false;
+    if (tp.all_full && new_q < 2.0 * old_q) return false;   // (ragged shift-and-mask tiles lose more to their bounds checks than shorter runs cost)
     // tile axes in read order (with their LDS strides) and in write order
     TabBuildArgs tb;
     std::memset(&tb, 0, sizeof tb);
-    std::vector<int> rpos(na, 0);
+    TabCopyArgs ta;
+    std::memset(&ta, 0, sizeof ta);
+    ta.x_n[0] = ta.x_n[1] = ta.x_t[0] = ta.x_t[1] = 1;
+    std::vector<int> rpos(na, 0), slot(na, 0);
+    int nslots = 0;
+    for (int i = 0; i < na; ++i)
+        if (in_tile[i] && in_tile[i] != axes[i].n) {
+            slot[i] = ++nslots;
+            ta.x_n[nslots - 1] = (int32_t)axes[i].n;
+            ta.x_t[nslots - 1] = (int32_t)in_tile[i];
+            if (axes[i].n > 0x7fffffff) return false;
+        }
     int64_t lo = 1, span_in = 0, span_out = 0;
     std::string key = "copytab|" + std::to_string(eb);
     for (int i : in_order)
         if (in_tile[i]) {
             if (tb.nt == TAB_MAX_AXES) return false;
-            tb.r_ext[tb.nt] = (int32_t)axes[i].n;
+            tb.r_ext[tb.nt] = (int32_t)in_tile[i];
             tb.r_si[tb.nt] = axes[i].s[0];
+            tb.r_slot[tb.nt] = slot[i];
             rpos[i] = (int)lo;
-            lo *= axes[i].n;
+            lo *= in_tile[i];
             ++tb.nt;
-            span_in += (axes[i].n - 1) * axes[i].s[0];
-            span_out += (axes[i].n - 1) * axes[i].s[1];
-            key += "|" + std::to_string(axes[i].n) + "," + std::to_string(axes[i].s[0]) + "," + std::to_string(axes[i].s[1]);
+            span_in += (in_tile[i] - 1) * axes[i].s[0];
+            span_out += (in_tile[i] - 1) * axes[i].s[1];
+            key += "|" + std::to_string(in_tile[i]) + "," + std::to_string(axes[i].s[0]) + "," + std::to_string(axes[i].s[1]) + "," + std::to_string(slot[i]);
         }
     if (span_in >= ((int64_t)1 << 32) || span_out >= ((int64_t)1 << 32)) return false;   // 32-bit element offsets
     int w = 0;
     for (int i : out_order)
         if (in_tile[i]) {
-            tb.w_ext[w] = (int32_t)axes[i].n;
+            tb.w_ext[w] = (int32_t)in_tile[i];
             tb.w_so[w] = axes[i].s[1];
             tb.w_rpos[w] = rpos[i];
+            tb.w_slot[w] = slot[i];
             ++w;
         }
     tb.E = (int32_t)E;
-    TabCopyArgs ta;
-    std::memset(&ta, 0, sizeof ta);
     ta.in = in;
     ta.out = out;
     ta.E = (int32_t)E;
     int64_t ntiles = 1;
-    for (int i = na - 1; i >= 0; --i)   // fastest tile index: the innermost axis outside the tile (neighbouring tiles abut)
-        if (!in_tile[i]) {
-            ta.g_count[ta.ng] = axes[i].n;
-            ta.g_si[ta.ng] = axes[i].s[0];
-            ta.g_so[ta.ng] = axes[i].s[1];
-            ++ta.ng;
-            ntiles *= axes[i].n;
-        }
+    for (int i = na - 1; i >= 0; --i) {   // fastest tile index: the innermost axis outside the tile (neighbouring tiles abut)
+        if (in_tile[i] == axes[i].n) continue;
+        const int64_t t = in_tile[i] ? in_tile[i] : 1, count = (axes[i].n + t - 1) / t;
+        if (ta.ng == MAXG) return false;
+        ta.g_count[ta.ng] = count;
+        ta.g_si[ta.ng] = axes[i].s[0] * t;
+        ta.g_so[ta.ng] = axes[i].s[1] * t;
+        ta.g_slot[ta.ng] = slot[i];
+        ++ta.ng;
+        ntiles *= count;
+    }
     ta.ntiles = ntiles;
     if (ntiles < 8) return false;
     void* tab = nullptr;
     bool fresh = false;
-    if ((status = table_cache_get(stream, key, (size_t)3 * E * sizeof(uint32_t), &tab, &fresh)) != TFH_OK) return true;
+    if ((status = table_cache_get(stream, key, (size_t)5 * E * sizeof(uint32_t), &tab, &fresh)) != TFH_OK) return true;
     if (!tab) return false;   // no cached block to be had (cache full, stream being captured): the masked tiles do it
     hipStream_t st = (hipStream_t)stream;
     if (fresh) {
@@ -1079,7 +1578,7 @@ bool try_table_copy(int eb, const void* in, void* out, std::vector<Axis> axes, c
     const int ept = (int)((E + THREADS - 1) / THREADS);
     const size_t lds = (size_t)(E + E / 32 + 4) * eb;
     const size_t per_cu = std::max<size_t>(1, std::min<size_t>(4, (size_t)(160 * 1024) / (lds + 512)));
-    const dim3 grid((uint32_t)std::min<int64_t>(ntiles, (int64_t)(256 * per_cu)));
+    const dim3 grid((uint32_t)std::min<int64_t>((ntiles + 7) / 8 * 8, (int64_t)(256 * per_cu)));   // (a multiple of 8: a block stays on its XCD)
     const int prof = prof_begin(PROF_COPY, stream);
     if (eb == 4) launch_tabcopy<uint32_t>(ta, ept, grid, lds, st);
     else if (eb == 8) launch_tabcopy<uint64_t>(ta, ept, grid, lds, st);
@@ -1108,6 +1607,7 @@ int32_t launch_copy(int dtype, const void* in, void* out, std::vector<Axis> axes
     const bool raw = alpha.is_one() && beta.is_zero() && !(conj && cx);
     if (raw) {
         int32_t st_tab = TFH_OK;
+        if (!tp.all_full && try_perm_tiles(eb, in, out, axes, stream, st_tab)) return st_tab;
         if (try_table_copy(eb, in, out, axes, tp, stream, st_tab)) return st_tab;
         // Large tiles.  When the rows a tile touches on one side lie far apart (an axis that is contiguous on one side
         // and the slowest on the other: strides of megabytes inside every tile), 512-byte runs on that side cost 10-17 %
