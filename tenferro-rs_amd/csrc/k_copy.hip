@@ -1174,7 +1174,7 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
                     if (64 * k + lane < a.wfn) {
                         Pack<V, 1> x;
                         x.v[0] = lds[lwf[k] + lrow];
-                        store_stream<Pack<V, 1>>(orow + (uint32_t)(64 * k + lane), x);
+                        orow[(uint32_t)(64 * k + lane)] = x.v[0];   // (a cached store: the next instruction completes the 128-byte lines this one leaves partly written)
                     }
             }
         } else {
@@ -1188,7 +1188,7 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
                     if (64 * k + lane < wlen) {
                         Pack<V, 1> x;
                         x.v[0] = lds[lwf[k] + lrow];
-                        store_stream<Pack<V, 1>>(orow + (uint32_t)(64 * k + lane), x);
+                        orow[(uint32_t)(64 * k + lane)] = x.v[0];   // (a cached store: the next instruction completes the 128-byte lines this one leaves partly written)
                     }
             }
         }

@@ -44,6 +44,8 @@ def test_profile_summaries_name_their_commands_and_no_working_files():
         # every summary states the command that made it, and that command runs committed files only
         if f.startswith("host_overhead"):
             assert "python3 bench.py --host-overhead" in text, f
+        elif f.startswith("shape_sweep"):
+            assert "python3 bench.py --shape-sweep" in text, f
         else:
             assert "rocprofv3 " in text and " -- python3 bench.py" in text, f
         assert "_work/" not in text, f
