@@ -579,7 +579,7 @@ __global__ void __launch_bounds__(THREADS) tabcopy_kernel(TabCopyArgs a) {
                 if (tid + THREADS * j < E) {
                     Pack<V, 1> x;
                     x.v[0] = lds[lpos[j]];
-                    store_stream<Pack<V, 1>>(out + woff[j], x);
+                    out[woff[j]] = x.v[0];   // (a cached store: runs start anywhere, and neighbours complete the lines they share)
                 }
         } else {
 #pragma unroll
@@ -588,7 +588,7 @@ __global__ void __launch_bounds__(THREADS) tabcopy_kernel(TabCopyArgs a) {
                 if (w < E && inside(a.tab[4 * E + w], lim)) {
                     Pack<V, 1> x;
                     x.v[0] = lds[lpos[j]];
-                    store_stream<Pack<V, 1>>(out + woff[j], x);
+                    out[woff[j]] = x.v[0];   // (a cached store: runs start anywhere, and neighbours complete the lines they share)
                 }
             }
         }
@@ -1209,8 +1209,17 @@ void launch_perm(const PermArgs& pa, int nseg, dim3 grid, size_t lds, hipStream_
 
 // A bit-exact move of extents that the shift-and-mask tiles do not fill: two-sided 64 KB tiles.  Returns true when
 // it launched (status holds the outcome).
-bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, void* stream, int32_t& status) {
+bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, void* stream, int32_t& status, int attempt = 0) {
     status = TFH_OK;
+    if (attempt == 0) {
+        // the usual read run first; when that leaves the tile half empty (an innermost axis that both sides share, with
+        // one long axis behind it: the read run is all that can grow), a read run twice as long; else whatever fits
+        for (int a = 1; a <= 3; ++a)
+            if (try_perm_tiles(eb, in, out, axes, stream, status, a)) return true;
+        return false;
+    }
+    const bool want_full = attempt < 3;
+    const int64_t rf_cap = (eb == 16 ? 64 : 128) * (attempt == 2 ? 2 : 1);
     int64_t total = 1;
     for (auto& x : axes) total *= x.n;
     if (total < ((int64_t)1 << 20)) return false;
@@ -1266,7 +1275,7 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
     std::vector<char> in_rf(na, 0), in_wf(na, 0);
     // the read run first: two wave instructions wide at most (half that for 16-byte elements), then the write run in
     // the room that the registers of a thread leave (a row per wave and register)
-    const int64_t rfn = take_run(0, eb == 16 ? 64 : 128, E, in_rf);
+    const int64_t rfn = take_run(0, rf_cap, E, in_rf);
     if (rfn < 16) return false;
     const int nseg = rfn <= 64 ? 1 : (rfn <= 128 ? 2 : 4);
     emax = std::min<int64_t>(emax, rfn * PERM_WAVES * (ept / nseg));
@@ -1294,7 +1303,7 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
             ++idle;
         }
     }
-    if (E < 2048) return false;
+    if (E < 2048 || (want_full && E * 2 <= emax)) return false;
     PermArgs pa;
     std::memset(&pa, 0, sizeof pa);
     pa.x_n[0] = pa.x_n[1] = pa.x_t[0] = pa.x_t[1] = 1;
