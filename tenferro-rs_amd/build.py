@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libtenferro_hip.so")
-SOURCES = ["errors.cpp", "plan.cpp", "prims.cpp", "einsum.cpp", "contract_cache.cpp", "runtime.cpp", "k_copy.hip", "k_reduce.hip", "k_gemm.hip", "k_gemm_skinny.hip", "k_gemm_wave.hip", "k_gemm_tiny.hip", "k_gemm_bfirst.hip", "k_dot.hip", "static_scratch.hip",
+SOURCES = ["errors.cpp", "plan.cpp", "prims.cpp", "einsum.cpp", "contract_cache.cpp", "runtime.cpp", "k_copy.hip", "k_reduce.hip", "k_gemm.hip", "k_gemm_skinny.hip", "k_gemm_wave.hip", "k_gemm_tiny.hip", "k_gemm_bfirst.hip", "k_gemm_thin.hip", "k_dot.hip", "static_scratch.hip",
            "k_gemm128_f32.hip", "k_gemm128_f64.hip", "k_gemm128_c64.hip", "k_gemm128_c128.hip",
            "k_gemm64_f32.hip", "k_gemm64_f64.hip", "k_gemm64_c64.hip", "k_gemm64_c128.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -98,6 +98,10 @@ int32_t classify_contract(const std::vector<uint32_t>& ma, const int64_t* dims_a
                           const std::vector<uint32_t>& mb, const int64_t* dims_b, const int64_t* str_b,
                           const std::vector<uint32_t>& mc, const int64_t* dims_c, const int64_t* str_c,
                           ContractAxes& out);
+// C = alpha * A * B + beta * C for a long operand against a small one (at most 64 real rows, 64 KB) that the
+// register-resident streaming kernel does not take; true when it launched (k_gemm_thin.hip).
+bool try_thin_stream(int dtype, const void* a, const void* b, void* c, const struct ContractAxes& ax, Scalar alpha, Scalar beta,
+                     void* stream, bool conj_a, bool conj_b, int32_t& status);
 // Drops extent-1 axes and merges neighbours that are contiguous in every slot in [0, nslots).
 // Order is preserved (axis i+1 is "inside" axis i when they merge).
 void fuse_axes(std::vector<Axis>& ax, int nslots);

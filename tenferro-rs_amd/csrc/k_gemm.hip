@@ -779,6 +779,11 @@ int32_t launch_contract_impl(int dtype, const void* a, const void* b, void* c, C
             return st_bf;
         }
     }
+    // a long operand against a small one that is too large for the register-resident streaming kernel (k_gemm_thin.hip)
+    if (nb == 1 && std::min(M, N) <= 64 && std::max(M, N) >= 4096) {
+        int32_t st_thin = TFH_OK;
+        if (try_thin_stream(dtype, a, b, c, ax, alpha, beta, stream, conj_a, conj_b, st_thin)) return st_thin;
+    }
     // lanes of the epilogue run along n: put C's fastest axis in the N group (swap operands if needed)
     if (min_stride(ax.M, 2) < min_stride(ax.N, 2)) {
         std::swap(a, b);

@@ -3046,3 +3046,49 @@ def test_permute_two_sided_tiles_of_long_odd_extents(tf, oracle, dtype):
         assert out.to_numpy().tobytes() == ref.tobytes(), (shape, perm, tf.last_kernel())
         del a, ref, out
     assert ran >= 4, ran
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_contract_long_operand_against_a_small_one_beyond_the_register_kernel(tf, oracle, dtype):
+    # More k (over 32 16-byte chunks) than the register-resident streaming kernel holds against at most 32 real rows, far
+    # too thin for tiles: the small operand is staged in LDS as MFMA operands (complex types as the real matrix
+    # [[re, -im], [im, re]]) and every wave streams rows of the long one.  Both output orientations, either operand in
+    # either position, a long extent that ends on a partly filled unit, k that ends inside a register set, rows that
+    # are no multiple of 16, a strided small operand, general alpha / beta, and the conjugate-on-load flags.
+    rng = seeded_rng(141)
+    cplx = np.issubdtype(dtype, np.complexfloating)
+    q = 16 // (np.dtype(dtype).itemsize // (2 if cplx else 1))      # reals per 16-byte chunk
+    kq = q // (2 if cplx else 1) or 1                               # elements of k per chunk (1 for complex128)
+    mmax = 16 if cplx else 32
+    cases = [("nk", "mk", "nm", mmax, 40 * kq, 5000), ("nk", "mk", "mn", mmax, 40 * kq, 5000), ("mk", "nk", "mn", 12, 130 * kq, 4099),
+             ("mk", "nk", "nm", 9 if cplx else 17, 36 * kq, 4112), ("nk", "km", "nm", mmax - 3, 64 * kq, 8192),
+             ("mk", "nk", "mn", 5, 200 * kq, 6000), ("nk", "mk", "nm", mmax, 8 * kq, 4096 + 16)]
+    used = 0
+    for la, lb, lc, m, k, n in cases:
+        ext = dict(m=m, k=k, n=n)
+        a = rand(rng, [ext[c] for c in la], dtype)
+        b = rand(rng, [ext[c] for c in lb], dtype)
+        c0 = rand(rng, [ext[c] for c in lc], dtype)
+        for alpha, beta in [(1.0, 0.0), ((0.5 - 2j, 1.5 + 1j) if cplx else (0.5, -1.5))]:
+            ref = c0.copy()
+            oracle.contract(a, lab(la), b, lab(lb), ref, lab(lc), alpha=alpha, beta=beta)
+            dout = dev(tf, c0)
+            plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab(la), lab(lb), lab(lc)), [a.shape, b.shape, ref.shape])
+            tf.HipBackend.execute(plan, alpha, [dev(tf, a), dev(tf, b)], beta, dout)
+            used += "gemm_thin_kernel" in tf.last_kernel()
+            assert relerr(dout.to_numpy(), ref) < TOL[dtype], (la, lb, lc, m, k, n, alpha, tf.last_kernel())
+    assert used >= 10, used
+    # exact on small integers: a misplaced k, a wrong sign in the complex expansion or a dropped chunk would show
+    m, k, n = (14 if cplx else 30), 40 * kq, 4100
+    def ints(shape):
+        x = rng.integers(-4, 5, shape).astype(np.float64)
+        return (x + 1j * rng.integers(-4, 5, shape)).astype(dtype) if cplx else x.astype(dtype)
+    a, b = ints((n, k)), ints((m, k))
+    for conj_a, conj_b in ([(False, False), (True, False), (False, True), (True, True)] if cplx else [(False, False)]):
+        out = tf.Tensor.empty([n, m], tf.GpuMemory(0), tf.MemoryOrder.RowMajor, dtype)
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Contract(lab("nk"), lab("mk"), lab("nm")), [a.shape, b.shape, [n, m]])
+        da, db = dev(tf, a), dev(tf, b)
+        tf.HipBackend.execute(plan, 1.0, [da.conj_on_load() if conj_a else da, db.conj_on_load() if conj_b else db], 0.0, out)
+        assert "gemm_thin_kernel" in tf.last_kernel(), tf.last_kernel()
+        want = np.einsum("nk,mk->nm", a.conj() if conj_a else a, b.conj() if conj_b else b)
+        assert np.array_equal(out.to_numpy(), want), (conj_a, conj_b)
