@@ -271,47 +271,63 @@ bool try_thin_stream(int dtype, const void* a, const void* b, void* c, const Con
     if (m.s[2] != 1 && n.s[2] != 1) return false;
     if (m.s[slot_s] < 0 || k.s[slot_s] < 0 || m.s[2] <= 0 || n.s[2] <= 0) return false;
     const int mb = (int)((mr + 15) / 16);
-    const int64_t steps = (chunks + 3) / 4, groups = (steps + THIN_GROUP - 1) / THIN_GROUP;
-    const size_t s_bytes = (size_t)mb * groups * THIN_GROUP * 64 * 16;
-    if (s_bytes > (size_t)THIN_S_BYTES) return false;
+    // A small operand over 64 KB goes in passes over slices of k, one launch each on the same stream: the first applies
+    // beta, the later ones add to C (C is the small side of the traffic: 32 columns against k = 512 move it three times
+    // instead of once, 12 % more bytes).  A slice is a whole number of register sets of chunk steps.
+    const int64_t set_chunks = 4 * THIN_GROUP;                                  // chunks per register set and row
+    const int64_t max_sets = (int64_t)THIN_S_BYTES / ((int64_t)mb * THIN_GROUP * 64 * 16);
+    if (max_sets < 1) return false;
+    const int64_t all_sets = (chunks + set_chunks - 1) / set_chunks;
+    const int64_t passes = (all_sets + max_sets - 1) / max_sets;
+    if (passes > 8) return false;
+    const int64_t sets_per_pass = (all_sets + passes - 1) / passes;
     if (n.n > ((int64_t)1 << 40)) return false;
-    ThinArgs ta;
-    std::memset(&ta, 0, sizeof ta);
-    ta.S = S;
-    ta.L = L;
-    ta.C = c;
-    ta.ms = (int32_t)m.n;
-    ta.K = (int32_t)k.n;
-    ta.mr = (int32_t)mr;
-    ta.kr = (int32_t)kr;
-    ta.steps = (int32_t)steps;
-    ta.groups = (int32_t)groups;
-    ta.cx = cx;
-    ta.conj_s = conj_s && cx;
-    ta.conj_l = conj_l && cx;
-    ta.use_beta = !beta.is_zero();
-    ta.m_fast = m.s[2] == 1 && n.s[2] != 1;
-    ta.nl = n.n;
-    ta.units = (n.n + THIN_UNIT - 1) / THIN_UNIT;
-    ta.ss_m = m.s[slot_s];
-    ta.ss_k = k.s[slot_s];
-    ta.ls_n = n.s[slot_l];
-    ta.cs_m = m.s[2];
-    ta.cs_n = n.s[2];
-    ta.alpha_re = alpha.re; ta.alpha_im = alpha.im; ta.beta_re = beta.re; ta.beta_im = beta.im;
-    const size_t lds = s_bytes + (size_t)THIN_WAVES * THIN_UNIT * (mb * 16 + 1) * rb;
     static const bool raised = [] {
         raise_thin_lds<double>();
         raise_thin_lds<float>();
         return true;
     }();
     (void)raised;
-    const int64_t per_cu = lds <= 78 * 1024 ? 2 : 1;   // blocks that fit a CU's 160 KB of LDS
-    const int64_t blocks = std::min<int64_t>((ta.units + THIN_WAVES - 1) / THIN_WAVES, 256 * per_cu);
     hipStream_t st = (hipStream_t)stream;
     const int prof = prof_begin(PROF_CONTRACT, stream);
-    if (dbl) launch_thin_typed<double>(ta, mb, dim3((uint32_t)blocks), lds, st);
-    else launch_thin_typed<float>(ta, mb, dim3((uint32_t)blocks), lds, st);
+    for (int64_t pass = 0; pass < passes; ++pass) {
+        const int64_t c0 = pass * sets_per_pass * set_chunks, c1 = std::min<int64_t>(chunks, c0 + sets_per_pass * set_chunks);
+        if (c0 >= c1) break;
+        const int64_t kr0 = c0 * q, krn = (c1 - c0) * q;                          // the slice in reals, in elements: / nc
+        const int64_t steps = (c1 - c0 + 3) / 4, groups = (steps + THIN_GROUP - 1) / THIN_GROUP;
+        const size_t s_bytes = (size_t)mb * groups * THIN_GROUP * 64 * 16;
+        ThinArgs ta;
+        std::memset(&ta, 0, sizeof ta);
+        ta.S = (const char*)S + (kr0 / nc) * k.s[slot_s] * (int64_t)dtype_size(dtype);
+        ta.L = (const char*)L + kr0 * rb;
+        ta.C = c;
+        ta.ms = (int32_t)m.n;
+        ta.K = (int32_t)(krn / nc);
+        ta.mr = (int32_t)mr;
+        ta.kr = (int32_t)krn;
+        ta.steps = (int32_t)steps;
+        ta.groups = (int32_t)groups;
+        ta.cx = cx;
+        ta.conj_s = conj_s && cx;
+        ta.conj_l = conj_l && cx;
+        ta.use_beta = pass > 0 || !beta.is_zero();
+        ta.m_fast = m.s[2] == 1 && n.s[2] != 1;
+        ta.nl = n.n;
+        ta.units = (n.n + THIN_UNIT - 1) / THIN_UNIT;
+        ta.ss_m = m.s[slot_s];
+        ta.ss_k = k.s[slot_s];
+        ta.ls_n = n.s[slot_l];
+        ta.cs_m = m.s[2];
+        ta.cs_n = n.s[2];
+        ta.alpha_re = alpha.re; ta.alpha_im = alpha.im;
+        ta.beta_re = pass > 0 ? 1.0 : beta.re;
+        ta.beta_im = pass > 0 ? 0.0 : beta.im;
+        const size_t lds = s_bytes + (size_t)THIN_WAVES * THIN_UNIT * (mb * 16 + 1) * rb;
+        const int64_t per_cu = lds <= 78 * 1024 ? 2 : 1;   // blocks that fit a CU's 160 KB of LDS
+        const int64_t blocks = std::min<int64_t>((ta.units + THIN_WAVES - 1) / THIN_WAVES, 256 * per_cu);
+        if (dbl) launch_thin_typed<double>(ta, mb, dim3((uint32_t)blocks), lds, st);
+        else launch_thin_typed<float>(ta, mb, dim3((uint32_t)blocks), lds, st);
+    }
     prof_end(prof, stream);
     status = hip_check(hipGetLastError(), "contraction kernel launch");
     return true;

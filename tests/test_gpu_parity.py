@@ -3062,7 +3062,8 @@ def test_contract_long_operand_against_a_small_one_beyond_the_register_kernel(tf
     mmax = 16 if cplx else 32
     cases = [("nk", "mk", "nm", mmax, 40 * kq, 5000), ("nk", "mk", "mn", mmax, 40 * kq, 5000), ("mk", "nk", "mn", 12, 130 * kq, 4099),
              ("mk", "nk", "nm", 9 if cplx else 17, 36 * kq, 4112), ("nk", "km", "nm", mmax - 3, 64 * kq, 8192),
-             ("mk", "nk", "mn", 5, 200 * kq, 6000), ("nk", "mk", "nm", mmax, 8 * kq, 4096 + 16)]
+             ("mk", "nk", "mn", 5, 200 * kq, 6000), ("nk", "mk", "nm", mmax, 8 * kq, 4096 + 16),
+             ("nk", "mk", "nm", mmax, 300 * kq, 4200), ("mk", "nk", "mn", mmax - 1, 517 * kq, 4100)]   # over 64 KB: passes over slices of k
     used = 0
     for la, lb, lc, m, k, n in cases:
         ext = dict(m=m, k=k, n=n)
