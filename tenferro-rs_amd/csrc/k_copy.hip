@@ -1066,7 +1066,10 @@ __device__ __forceinline__ void perm_entry(const PermGroup& g, int i, uint32_t& 
 constexpr int PERM_THREADS = 512, PERM_WAVES = PERM_THREADS / 64;
 constexpr int PERM_WSEG = 8;   // a write run is up to 8 wave instructions wide
 
-template <class V, int NSEG, int JR>
+// WTAB: the write run is longer than PERM_WSEG wave instructions (a short innermost axis of the output inside a longer
+// dense run: batched transposes of small matrices): its LDS positions come from a table in LDS instead of registers, and
+// the (row, segment) pairs of the write order are dealt to the waves one by one.
+template <class V, int NSEG, int JR, bool WTAB>
 __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
     prefetch_kernel_arguments<sizeof(PermArgs)>();
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -1075,8 +1078,15 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
     uint32_t* out_s = tab;                 // [wsn] output offset of a row of the write order
     uint32_t* lw_s = out_s + a.wsn;        // [wsn] its LDS position
     uint32_t* c_ws = lw_s + a.wsn;         // [wsn] its coordinates along the ranged axes
+    uint32_t* lw_f = c_ws + a.wsn;         // [wfn] (WTAB) LDS position of a column of the write order
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     for (int i = tid; i < a.wsn; i += PERM_THREADS) perm_entry(a.ws, i, out_s[i], lw_s[i], c_ws[i]);
+    if (WTAB) {
+        for (int i = tid; i < a.wfn; i += PERM_THREADS) {
+            uint32_t m, xc;
+            perm_entry(a.wf, i, m, lw_f[i], xc);
+        }
+    }
     // the rows of the read order that this wave reads, the same in every tile: their input offsets and coordinates
     uint32_t in_s[JR], c_rs[JR];
 #pragma unroll
@@ -1092,7 +1102,7 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
     for (int k = 0; k < PERM_WSEG; ++k) {
         uint32_t m, xc;
         lwf[k] = 0;
-        if (64 * k + lane < a.wfn) perm_entry(a.wf, 64 * k + lane, m, lwf[k], xc);
+        if (!WTAB && 64 * k + lane < a.wfn) perm_entry(a.wf, 64 * k + lane, m, lwf[k], xc);
     }
     __syncthreads();
     auto origin = [&](uint64_t tile, int64_t& oi, int64_t& oo, uint32_t& lim) {
@@ -1165,7 +1175,15 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
             load(oi2, lim2);
         }
         V* out = reinterpret_cast<V*>(a.out) + oo;
-        if (lim == lim_full) {
+        if (WTAB) {
+            const int wlen = run_len(a.wf_slot, a.wf_row, a.wfn, lim);
+            const int nsegw = (a.wfn + 63) / 64, units = a.wsn * nsegw;
+            for (int u = wave; u < units; u += PERM_WAVES) {
+                const int ws = u / nsegw, wf = 64 * (u - ws * nsegw) + lane;
+                if (!inside(c_ws[ws], lim) || wf >= wlen) continue;
+                out[out_s[ws] + (uint32_t)wf] = lds[lw_f[wf] + lw_s[ws]];
+            }
+        } else if (lim == lim_full) {
             for (int ws = wave; ws < a.wsn; ws += PERM_WAVES) {
                 const uint32_t lrow = __builtin_amdgcn_readfirstlane(lw_s[ws]);
                 V* orow = out + __builtin_amdgcn_readfirstlane(out_s[ws]);
@@ -1188,7 +1206,7 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
                     if (64 * k + lane < wlen) {
                         Pack<V, 1> x;
                         x.v[0] = lds[lwf[k] + lrow];
-                        orow[(uint32_t)(64 * k + lane)] = x.v[0];   // (a cached store: the next instruction completes the 128-byte lines this one leaves partly written)
+                        orow[(uint32_t)(64 * k + lane)] = x.v[0];
                     }
             }
         }
@@ -1200,26 +1218,30 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
     }
 }
 
+template <class V, int EPT, bool WTAB>
+void launch_perm_w(const PermArgs& pa, int nseg, dim3 grid, size_t lds, hipStream_t st) {
+    if (nseg == 1) TFH_LAUNCH_TIMED((perm_kernel<V, 1, EPT, WTAB>), grid, dim3(PERM_THREADS), lds, st, pa);
+    else if (nseg == 2) TFH_LAUNCH_TIMED((perm_kernel<V, 2, EPT / 2, WTAB>), grid, dim3(PERM_THREADS), lds, st, pa);
+    else TFH_LAUNCH_TIMED((perm_kernel<V, 4, EPT / 4, WTAB>), grid, dim3(PERM_THREADS), lds, st, pa);
+}
 template <class V, int EPT>
-void launch_perm(const PermArgs& pa, int nseg, dim3 grid, size_t lds, hipStream_t st) {
-    if (nseg == 1) TFH_LAUNCH_TIMED((perm_kernel<V, 1, EPT>), grid, dim3(PERM_THREADS), lds, st, pa);
-    else if (nseg == 2) TFH_LAUNCH_TIMED((perm_kernel<V, 2, EPT / 2>), grid, dim3(PERM_THREADS), lds, st, pa);
-    else TFH_LAUNCH_TIMED((perm_kernel<V, 4, EPT / 4>), grid, dim3(PERM_THREADS), lds, st, pa);
+void launch_perm(const PermArgs& pa, int nseg, bool wtab, dim3 grid, size_t lds, hipStream_t st) {
+    if (wtab) launch_perm_w<V, EPT, true>(pa, nseg, grid, lds, st);
+    else launch_perm_w<V, EPT, false>(pa, nseg, grid, lds, st);
 }
 
 // A bit-exact move of extents that the shift-and-mask tiles do not fill: two-sided 64 KB tiles.  Returns true when
 // it launched (status holds the outcome).
-bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, void* stream, int32_t& status, int attempt = 0) {
-    status = TFH_OK;
-    if (attempt == 0) {
-        // the usual read run first; when that leaves the tile half empty (an innermost axis that both sides share, with
-        // one long axis behind it: the read run is all that can grow), a read run twice as long; else whatever fits
-        for (int a = 1; a <= 3; ++a)
-            if (try_perm_tiles(eb, in, out, axes, stream, status, a)) return true;
-        return false;
-    }
-    const bool want_full = attempt < 3;
-    const int64_t rf_cap = (eb == 16 ? 64 : 128) * (attempt == 2 ? 2 : 1);
+struct PermPlan {
+    PermArgs pa;
+    int nseg;
+    bool wtab;
+    size_t lds;
+    dim3 grid;
+    double score;   // bytes of the shorter of the two runs, each counted up to 1 KB, and how full the tile is
+};
+// One candidate tiling: a read run of up to rf_cap elements, a write run of up to wf_cap.
+bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, int64_t rf_cap, int64_t wf_cap, PermPlan& plan) {
     int64_t total = 1;
     for (auto& x : axes) total *= x.n;
     if (total < ((int64_t)1 << 20)) return false;
@@ -1279,7 +1301,7 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
     if (rfn < 16) return false;
     const int nseg = rfn <= 64 ? 1 : (rfn <= 128 ? 2 : 4);
     emax = std::min<int64_t>(emax, rfn * PERM_WAVES * (ept / nseg));
-    const int64_t wfn = take_run(1, 64 * PERM_WSEG, E, in_wf);
+    const int64_t wfn = take_run(1, wf_cap, E, in_wf);
     if (wfn < 16) return false;
     // room left (a short output run): more of the input's fastest axes, then whole axes from either side
     for (int side = 0, idle = 0; E * 2 <= emax && idle < 2; side ^= 1) {
@@ -1303,8 +1325,8 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
             ++idle;
         }
     }
-    if (E < 2048 || (want_full && E * 2 <= emax)) return false;
-    PermArgs pa;
+    if (E < 2048) return false;
+    PermArgs& pa = plan.pa;
     std::memset(&pa, 0, sizeof pa);
     pa.x_n[0] = pa.x_n[1] = pa.x_t[0] = pa.x_t[1] = 1;
     std::vector<int> slot(na, 0);
@@ -1395,28 +1417,57 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
     }
     pa.ntiles = ntiles;
     if (ntiles < 1024) return false;   // (two tiles per block on every CU at least: smaller tensors take smaller tiles)
-    const size_t lds = (size_t)pitch * rsn * eb + (size_t)(3 * wsn) * sizeof(uint32_t);
+    const bool wtab = wfn2 > 64 * PERM_WSEG;
+    const size_t lds = (size_t)pitch * rsn * eb + (size_t)(3 * wsn + (wtab ? wfn2 : 0)) * sizeof(uint32_t);
     if (lds > 150 * 1024) return false;
+    const size_t per_cu = std::max<size_t>(1, std::min<size_t>(4, (size_t)(160 * 1024) / (lds + 512)));
+    plan.nseg = nseg;
+    plan.wtab = wtab;
+    plan.lds = lds;
+    plan.grid = dim3((uint32_t)std::min<int64_t>((ntiles + 7) / 8 * 8, (int64_t)(256 * per_cu)));   // (a multiple of 8: a block stays on its XCD)
+    plan.score = (double)std::min<int64_t>(std::min<int64_t>(rfn, wfn2) * eb, 1024) * (0.5 + 0.5 * (double)E / (double)((int64_t)PERM_THREADS * ept)) *
+                 (wtab ? 0.8 : 1.0);   // (the table-driven write order costs an LDS read per element more)
+    return true;
+}
+
+// A bit-exact move of extents that the shift-and-mask tiles do not fill: two-sided 64 KB tiles.  Returns true when
+// it launched (status holds the outcome).
+bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, void* stream, int32_t& status) {
+    status = TFH_OK;
+    // candidates: the usual read run (two wave instructions wide, one for 16-byte elements) or one twice as long (an
+    // innermost axis that both sides share, with one long axis behind it: the read run is all that can grow), a write
+    // run held in registers or a longer one through the table (a short innermost output axis inside a longer dense run)
+    PermPlan best;
+    best.score = 0.0;
+    const int64_t rf0 = eb == 16 ? 64 : 128;
+    for (int64_t rf_cap : {rf0, 2 * rf0})
+        for (int64_t wf_cap : {(int64_t)64 * PERM_WSEG, (int64_t)8192}) {
+            PermPlan cand;
+            std::memset(&cand.pa, 0, sizeof cand.pa);
+            if (plan_perm_tiles(eb, in, out, axes, rf_cap, wf_cap, cand) && cand.score > best.score * 1.05) best = cand;
+        }
+    if (best.score <= 0.0) return false;
     static const bool lds_limit_raised = [] {
         const int cap = 160 * 1024;
-#define TFH_PERM_LDS(V, E)                                                                                                  \
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 1, E>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);      \
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 2, E / 2>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);  \
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 4, E / 4>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
-        TFH_PERM_LDS(uint32_t, 32)
-        TFH_PERM_LDS(uint64_t, 16)
-        TFH_PERM_LDS(double2, 8)
+#define TFH_PERM_LDS(V, E, W)                                                                                                  \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 1, E, W>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);      \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 2, E / 2, W>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);  \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 4, E / 4, W>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+        TFH_PERM_LDS(uint32_t, 32, false)
+        TFH_PERM_LDS(uint64_t, 16, false)
+        TFH_PERM_LDS(double2, 8, false)
+        TFH_PERM_LDS(uint32_t, 32, true)
+        TFH_PERM_LDS(uint64_t, 16, true)
+        TFH_PERM_LDS(double2, 8, true)
 #undef TFH_PERM_LDS
         return true;
     }();
     (void)lds_limit_raised;
-    const size_t per_cu = std::max<size_t>(1, std::min<size_t>(4, (size_t)(160 * 1024) / (lds + 512)));
-    const dim3 grid((uint32_t)std::min<int64_t>((ntiles + 7) / 8 * 8, (int64_t)(256 * per_cu)));   // (a multiple of 8: a block stays on its XCD)
     hipStream_t st = (hipStream_t)stream;
     const int prof = prof_begin(PROF_COPY, stream);
-    if (eb == 4) launch_perm<uint32_t, 32>(pa, nseg, grid, lds, st);
-    else if (eb == 8) launch_perm<uint64_t, 16>(pa, nseg, grid, lds, st);
-    else launch_perm<double2, 8>(pa, nseg, grid, lds, st);
+    if (eb == 4) launch_perm<uint32_t, 32>(best.pa, best.nseg, best.wtab, best.grid, best.lds, st);
+    else if (eb == 8) launch_perm<uint64_t, 16>(best.pa, best.nseg, best.wtab, best.grid, best.lds, st);
+    else launch_perm<double2, 8>(best.pa, best.nseg, best.wtab, best.grid, best.lds, st);
     prof_end(prof, stream);
     status = hip_check(hipGetLastError(), "copy kernel launch");
     return true;

@@ -3032,7 +3032,8 @@ def test_permute_two_sided_tiles_of_long_odd_extents(tf, oracle, dtype):
     rng = seeded_rng(139)
     cases = [((27, 466, 1401), (2, 0, 1)), ((193, 1255, 71), (2, 1, 0)), ((53, 42, 191, 41), (2, 0, 3, 1)),
              ((27, 90, 5, 21, 67), (1, 0, 2, 4, 3)), ((12, 10, 9, 7, 17, 5, 29), (6, 1, 2, 0, 5, 4, 3)), ((810, 592, 37), (1, 0, 2)),
-             ((33, 17, 2969, 11), (0, 2, 3, 1)), ((4099, 4111), (1, 0)), ((3, 5600001), (1, 0)), ((5600001, 3), (1, 0))]
+             ((33, 17, 2969, 11), (0, 2, 3, 1)), ((4099, 4111), (1, 0)), ((3, 5600001), (1, 0)), ((5600001, 3), (1, 0)),
+             ((14, 90, 5, 21, 134), (1, 0, 2, 4, 3)), ((9000, 45, 43), (0, 2, 1))]   # batched transposes of small matrices: the write run through its table
     ran = 0
     for shape, perm in cases:
         a = rand(rng, shape, dtype)
