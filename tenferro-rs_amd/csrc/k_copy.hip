@@ -1105,12 +1105,15 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         if (!WTAB && 64 * k + lane < a.wfn) perm_entry(a.wf, 64 * k + lane, m, lwf[k], xc);
     }
     __syncthreads();
-    auto origin = [&](uint64_t tile, int64_t& oi, int64_t& oo, uint32_t& lim) {
+    // (the skeleton below -- everything but the global loads and stores -- was 25 of a 57 us permute of 134 MB before
+    // its divisions went to 32 bits, the guards of the write segments out of the row loop and the addresses onto scalar
+    // bases: with sixteen waves per CU, instruction issue is what the memory time has to hide behind)
+    auto origin = [&](uint32_t tile, int64_t& oi, int64_t& oo, uint32_t& lim) {   // (tile counts are below 2^31)
         oi = oo = 0;
         int l[2] = {a.x_t[0], a.x_t[1]};
         for (int g = 0; g < a.ng; ++g) {
-            const uint64_t q = tile / (uint64_t)a.g_count[g];
-            const int64_t c = (int64_t)(tile - q * (uint64_t)a.g_count[g]);
+            const uint32_t n = (uint32_t)a.g_count[g], q = tile / n;
+            const int64_t c = (int64_t)(tile - q * n);
             tile = q;
             oi += c * a.g_si[g];
             oo += c * a.g_so[g];
@@ -1131,6 +1134,9 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         if (slot == 0) return full;
         return (int)(slot == 1 ? (lim & 0xffffu) : (lim >> 16)) * row;
     };
+    // rows of the read order that this wave holds, columns that this lane holds, and where they go in LDS
+    const int my_rows = __builtin_amdgcn_readfirstlane(a.rsn > wave ? (a.rsn - wave + PERM_WAVES - 1) / PERM_WAVES : 0);
+    const uint32_t lds_at = (uint32_t)(wave * a.pitch + lane), lds_step = (uint32_t)(PERM_WAVES * a.pitch);
     V regs[NSEG * JR];
     auto load = [&](int64_t oi, uint32_t lim) {
         const V* in = reinterpret_cast<const V*>(a.in) + oi;
@@ -1138,40 +1144,49 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         uint32_t col[NSEG];   // columns past the end of the run read its last element
 #pragma unroll
         for (int k = 0; k < NSEG; ++k) col[k] = (uint32_t)(64 * k + lane < len ? 64 * k + lane : len - 1);
+        if (lim == lim_full) {
 #pragma unroll
-        for (int jj = 0; jj < JR; ++jj) {
-            // (a row past the edge reads row 0, which lies inside the tensor at every tile)
-            const V* row = in + (inside(c_rs[jj], lim) ? in_s[jj] : in_s[0]);
+            for (int jj = 0; jj < JR; ++jj) {
+                const V* row = in + in_s[jj];   // (a scalar base: rows past the tile read row 0, in_s is 0 there)
 #pragma unroll
-            for (int k = 0; k < NSEG; ++k) regs[k * JR + jj] = load_stream<Pack<V, 1>>(row + col[k]).v[0];
+                for (int k = 0; k < NSEG; ++k) regs[k * JR + jj] = load_stream<Pack<V, 1>>(row + col[k]).v[0];
+            }
+        } else {
+#pragma unroll
+            for (int jj = 0; jj < JR; ++jj) {
+                // (a row past the edge reads row 0, which lies inside the tensor at every tile)
+                const V* row = in + (inside(c_rs[jj], lim) ? in_s[jj] : in_s[0]);
+#pragma unroll
+                for (int k = 0; k < NSEG; ++k) regs[k * JR + jj] = load_stream<Pack<V, 1>>(row + col[k]).v[0];
+            }
         }
     };
-    const uint64_t ntiles = (uint64_t)a.ntiles, slots = (ntiles + 7) / 8 * 8;
-    uint64_t slot = blockIdx.x;
-    while (slot < slots && tab_tile_of(slot, ntiles) >= ntiles) slot += gridDim.x;
+    const uint32_t ntiles = (uint32_t)a.ntiles, per_xcd = (ntiles + 7) / 8, slots = per_xcd * 8;
+    auto tile_of = [&](uint32_t slot) { return (slot & 7) * per_xcd + (slot >> 3); };   // every XCD a contiguous eighth
+    uint32_t slot = blockIdx.x;
+    while (slot < slots && tile_of(slot) >= ntiles) slot += gridDim.x;
     if (slot >= slots) return;
     int64_t oi, oo;
     uint32_t lim;
-    origin(tab_tile_of(slot, ntiles), oi, oo, lim);
+    origin(tile_of(slot), oi, oo, lim);
     load(oi, lim);
     for (;;) {
 #pragma unroll
         for (int jj = 0; jj < JR; ++jj) {
-            const int rs = wave + PERM_WAVES * jj;
-            if (rs < a.rsn) {
+            if (jj < my_rows) {
 #pragma unroll
                 for (int k = 0; k < NSEG; ++k)
-                    if (64 * k + lane < a.rfn) lds[rs * a.pitch + 64 * k + lane] = regs[k * JR + jj];
+                    if (64 * k + lane < a.rfn) lds[lds_at + jj * lds_step + 64 * k] = regs[k * JR + jj];
             }
         }
         __syncthreads();
-        uint64_t next = slot + gridDim.x;
-        while (next < slots && tab_tile_of(next, ntiles) >= ntiles) next += gridDim.x;
+        uint32_t next = slot + gridDim.x;
+        while (next < slots && tile_of(next) >= ntiles) next += gridDim.x;
         const bool more = next < slots;
         int64_t oi2 = 0, oo2 = 0;
         uint32_t lim2 = 0;
         if (more) {   // the next tile's loads are in flight while this one is written out
-            origin(tab_tile_of(next, ntiles), oi2, oo2, lim2);
+            origin(tile_of(next), oi2, oo2, lim2);
             load(oi2, lim2);
         }
         V* out = reinterpret_cast<V*>(a.out) + oo;
@@ -1184,16 +1199,19 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
                 out[out_s[ws] + (uint32_t)wf] = lds[lw_f[wf] + lw_s[ws]];
             }
         } else if (lim == lim_full) {
-            for (int ws = wave; ws < a.wsn; ws += PERM_WAVES) {
-                const uint32_t lrow = __builtin_amdgcn_readfirstlane(lw_s[ws]);
-                V* orow = out + __builtin_amdgcn_readfirstlane(out_s[ws]);
+            // a segment of the write run at a time: its guard is looked at once per tile, not once per row
 #pragma unroll
-                for (int k = 0; k < PERM_WSEG; ++k)
-                    if (64 * k + lane < a.wfn) {
-                        Pack<V, 1> x;
-                        x.v[0] = lds[lwf[k] + lrow];
-                        orow[(uint32_t)(64 * k + lane)] = x.v[0];   // (a cached store: the next instruction completes the 128-byte lines this one leaves partly written)
+            for (int k = 0; k < PERM_WSEG; ++k) {
+                if (64 * k >= a.wfn) break;
+                if (64 * k + lane < a.wfn) {
+                    const uint32_t wcol = (uint32_t)(64 * k + lane);
+                    for (int ws = wave; ws < a.wsn; ws += PERM_WAVES) {
+                        const uint32_t lrow = __builtin_amdgcn_readfirstlane(lw_s[ws]);
+                        V* orow = out + __builtin_amdgcn_readfirstlane(out_s[ws]);
+                        // (a cached store: the next instruction completes the 128-byte lines this one leaves partly written)
+                        orow[wcol] = lds[lwf[k] + lrow];
                     }
+                }
             }
         } else {
             const int wlen = run_len(a.wf_slot, a.wf_row, a.wfn, lim);
@@ -1203,11 +1221,7 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
                 V* orow = out + __builtin_amdgcn_readfirstlane(out_s[ws]);
 #pragma unroll
                 for (int k = 0; k < PERM_WSEG; ++k)
-                    if (64 * k + lane < wlen) {
-                        Pack<V, 1> x;
-                        x.v[0] = lds[lwf[k] + lrow];
-                        orow[(uint32_t)(64 * k + lane)] = x.v[0];
-                    }
+                    if (64 * k + lane < wlen) orow[(uint32_t)(64 * k + lane)] = lds[lwf[k] + lrow];
             }
         }
         if (!more) break;
@@ -1416,7 +1430,7 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
         ntiles *= count;
     }
     pa.ntiles = ntiles;
-    if (ntiles < 1024) return false;   // (two tiles per block on every CU at least: smaller tensors take smaller tiles)
+    if (ntiles < 1024 || ntiles >= ((int64_t)1 << 31) - 8) return false;   // (two tiles per block on every CU at least: smaller tensors take smaller tiles)
     const bool wtab = wfn2 > 64 * PERM_WSEG;
     const size_t lds = (size_t)pitch * rsn * eb + (size_t)(3 * wsn + (wtab ? wfn2 : 0)) * sizeof(uint32_t);
     if (lds > 150 * 1024) return false;
