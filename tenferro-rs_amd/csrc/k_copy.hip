@@ -1040,6 +1040,7 @@ struct PermArgs {
     void* out;
     PermGroup rs, ws, wf;      // rows of the read order (input strides), rows of the write order (output strides), write columns
     int32_t rfn, rsn, wfn, wsn, pitch;
+    int32_t nsegs, units;      // wave instructions per row of the read order, and in a tile
     int32_t rf_slot, wf_slot;  // the ranged axis that is last in RF / WF (0: none), and the elements per index of it
     int32_t rf_row, wf_row;
     int32_t x_n[2], x_t[2];    // extent of a ranged axis and its indices per tile (1, 1 when there is none)
@@ -1064,12 +1065,17 @@ __device__ __forceinline__ void perm_entry(const PermGroup& g, int i, uint32_t& 
 }
 
 constexpr int PERM_THREADS = 512, PERM_WAVES = PERM_THREADS / 64;
-constexpr int PERM_WSEG = 8;   // a write run is up to 8 wave instructions wide
+constexpr int PERM_WSEG = 8;   // a write run held in registers is up to 8 wave instructions wide
 
+// The read order is dealt to the waves in units of one wave instruction: unit u is segment u % nsegs (64 columns) of
+// row u / nsegs, wave w has units w, w + 8, ... in registers 0, 1, ...  What a unit needs (the offset of its row in
+// memory, its first column, its place in LDS, the coordinates of its row along the ranged axes) is the same for all
+// lanes: lane j of the wave computes it for the unit of register j once per block, and the loops below fetch it with
+// a lane read.  A read run of any length is covered to within one instruction, whatever its extent.
 // WTAB: the write run is longer than PERM_WSEG wave instructions (a short innermost axis of the output inside a longer
-// dense run: batched transposes of small matrices): its LDS positions come from a table in LDS instead of registers, and
-// the (row, segment) pairs of the write order are dealt to the waves one by one.
-template <class V, int NSEG, int JR, bool WTAB>
+// dense run: batched transposes of small matrices): its LDS positions come from the table in LDS instead of registers,
+// and the (row, segment) pairs of the write order are dealt to the waves one by one.
+template <class V, int EPT, bool WTAB>
 __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
     prefetch_kernel_arguments<sizeof(PermArgs)>();
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -1078,36 +1084,34 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
     uint32_t* out_s = tab;                 // [wsn] output offset of a row of the write order
     uint32_t* lw_s = out_s + a.wsn;        // [wsn] its LDS position
     uint32_t* c_ws = lw_s + a.wsn;         // [wsn] its coordinates along the ranged axes
-    uint32_t* lw_f = c_ws + a.wsn;         // [wfn] (WTAB) LDS position of a column of the write order
+    uint32_t* lw_f = c_ws + a.wsn;         // [wfn] LDS position of a column of the write order
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     for (int i = tid; i < a.wsn; i += PERM_THREADS) perm_entry(a.ws, i, out_s[i], lw_s[i], c_ws[i]);
-    if (WTAB) {
-        for (int i = tid; i < a.wfn; i += PERM_THREADS) {
-            uint32_t m, xc;
-            perm_entry(a.wf, i, m, lw_f[i], xc);
+    for (int i = tid; i < a.wfn; i += PERM_THREADS) {
+        uint32_t m, xc;
+        perm_entry(a.wf, i, m, lw_f[i], xc);
+    }
+    // the unit of register `lane` of this wave, the same in every tile
+    uint32_t u_mem = 0, u_col = 0x40000000u, u_lds = 0, u_xc = 0xffffffffu;   // (no unit: past every run, never inside)
+    {
+        const int u = wave + PERM_WAVES * lane;
+        if (lane < EPT && u < a.units) {
+            const int r = u / a.nsegs, k = u - r * a.nsegs;
+            uint32_t l;
+            perm_entry(a.rs, r, u_mem, l, u_xc);
+            u_col = (uint32_t)(64 * k);
+            u_lds = l + u_col;
         }
     }
-    // the rows of the read order that this wave reads, the same in every tile: their input offsets and coordinates
-    uint32_t in_s[JR], c_rs[JR];
-#pragma unroll
-    for (int jj = 0; jj < JR; ++jj) {
-        const int rs = wave + PERM_WAVES * jj;
-        uint32_t l, m = 0, xc = 0;
-        if (rs < a.rsn) perm_entry(a.rs, rs, m, l, xc);
-        in_s[jj] = __builtin_amdgcn_readfirstlane(m);
-        c_rs[jj] = __builtin_amdgcn_readfirstlane(rs < a.rsn ? xc : 0xffffffffu);   // (a row past the tile: never inside)
-    }
+    const int my_units = __builtin_amdgcn_readfirstlane(a.units > wave ? (a.units - wave + PERM_WAVES - 1) / PERM_WAVES : 0);
+    // (the lane reads below take values that change with the tile -- z is a zero that the compiler cannot see through,
+    // a tile index being below 2^31: it would read what stays the same once, ahead of the loop over the tiles, into
+    // more scalar registers than there are)
+    auto of_unit = [](uint32_t v, int j) { return (uint32_t)__builtin_amdgcn_readlane((int)v, j); };
+    __syncthreads();
     uint32_t lwf[PERM_WSEG];   // LDS position of this thread's columns of the write order
 #pragma unroll
-    for (int k = 0; k < PERM_WSEG; ++k) {
-        uint32_t m, xc;
-        lwf[k] = 0;
-        if (!WTAB && 64 * k + lane < a.wfn) perm_entry(a.wf, 64 * k + lane, m, lwf[k], xc);
-    }
-    __syncthreads();
-    // (the skeleton below -- everything but the global loads and stores -- was 25 of a 57 us permute of 134 MB before
-    // its divisions went to 32 bits, the guards of the write segments out of the row loop and the addresses onto scalar
-    // bases: with sixteen waves per CU, instruction issue is what the memory time has to hide behind)
+    for (int k = 0; k < PERM_WSEG; ++k) lwf[k] = (!WTAB && 64 * k + lane < a.wfn) ? lw_f[64 * k + lane] : 0u;
     auto origin = [&](uint32_t tile, int64_t& oi, int64_t& oo, uint32_t& lim) {   // (tile counts are below 2^31)
         oi = oo = 0;
         int l[2] = {a.x_t[0], a.x_t[1]};
@@ -1134,30 +1138,23 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         if (slot == 0) return full;
         return (int)(slot == 1 ? (lim & 0xffffu) : (lim >> 16)) * row;
     };
-    // rows of the read order that this wave holds, columns that this lane holds, and where they go in LDS
-    const int my_rows = __builtin_amdgcn_readfirstlane(a.rsn > wave ? (a.rsn - wave + PERM_WAVES - 1) / PERM_WAVES : 0);
-    const uint32_t lds_at = (uint32_t)(wave * a.pitch + lane), lds_step = (uint32_t)(PERM_WAVES * a.pitch);
-    V regs[NSEG * JR];
-    auto load = [&](int64_t oi, uint32_t lim) {
+    V regs[EPT];
+    // No load is conditional: a column past the end of the run reads the run's last element, a row past the edge of
+    // the tensor reads row 0 of the tile, which lies inside at every tile.
+    auto load = [&](int64_t oi, uint32_t lim, uint32_t z) {
         const V* in = reinterpret_cast<const V*>(a.in) + oi;
-        const int len = run_len(a.rf_slot, a.rf_row, a.rfn, lim);
-        uint32_t col[NSEG];   // columns past the end of the run read its last element
+        const uint32_t last = (uint32_t)run_len(a.rf_slot, a.rf_row, a.rfn, lim) - 1u;
+        // per unit, in the lane of its register: the row's offset at this tile, and the first column
+        const uint32_t t_mem = inside(u_xc, lim) ? u_mem : 0u, t_col = u_col | z;
 #pragma unroll
-        for (int k = 0; k < NSEG; ++k) col[k] = (uint32_t)(64 * k + lane < len ? 64 * k + lane : len - 1);
-        if (lim == lim_full) {
+        for (int g = 0; g < EPT; g += 8) {
+            if (g < my_units) {   // (eight units at a time: the last ones of a wave may be none, and read row 0)
 #pragma unroll
-            for (int jj = 0; jj < JR; ++jj) {
-                const V* row = in + in_s[jj];   // (a scalar base: rows past the tile read row 0, in_s is 0 there)
-#pragma unroll
-                for (int k = 0; k < NSEG; ++k) regs[k * JR + jj] = load_stream<Pack<V, 1>>(row + col[k]).v[0];
-            }
-        } else {
-#pragma unroll
-            for (int jj = 0; jj < JR; ++jj) {
-                // (a row past the edge reads row 0, which lies inside the tensor at every tile)
-                const V* row = in + (inside(c_rs[jj], lim) ? in_s[jj] : in_s[0]);
-#pragma unroll
-                for (int k = 0; k < NSEG; ++k) regs[k * JR + jj] = load_stream<Pack<V, 1>>(row + col[k]).v[0];
+                for (int j = g; j < g + 8; ++j) {
+                    const V* row = in + of_unit(t_mem, j);
+                    const uint32_t col = min(of_unit(t_col, j) + (uint32_t)lane, last);
+                    regs[j] = load_stream<Pack<V, 1>>(row + col).v[0];
+                }
             }
         }
     };
@@ -1169,14 +1166,17 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
     int64_t oi, oo;
     uint32_t lim;
     origin(tile_of(slot), oi, oo, lim);
-    load(oi, lim);
+    load(oi, lim, tile_of(slot) >> 31);
     for (;;) {
+        {
+            const uint32_t z = tile_of(slot) >> 31, t_col = u_col | z, t_lds = u_lds | z;
 #pragma unroll
-        for (int jj = 0; jj < JR; ++jj) {
-            if (jj < my_rows) {
+            for (int g = 0; g < EPT; g += 8) {
+                if (g < my_units) {
 #pragma unroll
-                for (int k = 0; k < NSEG; ++k)
-                    if (64 * k + lane < a.rfn) lds[lds_at + jj * lds_step + 64 * k] = regs[k * JR + jj];
+                    for (int j = g; j < g + 8; ++j)
+                        if (of_unit(t_col, j) + (uint32_t)lane < (uint32_t)a.rfn) lds[of_unit(t_lds, j) + (uint32_t)lane] = regs[j];
+                }
             }
         }
         __syncthreads();
@@ -1187,13 +1187,13 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         uint32_t lim2 = 0;
         if (more) {   // the next tile's loads are in flight while this one is written out
             origin(tile_of(next), oi2, oo2, lim2);
-            load(oi2, lim2);
+            load(oi2, lim2, tile_of(next) >> 31);
         }
         V* out = reinterpret_cast<V*>(a.out) + oo;
         if (WTAB) {
             const int wlen = run_len(a.wf_slot, a.wf_row, a.wfn, lim);
-            const int nsegw = (a.wfn + 63) / 64, units = a.wsn * nsegw;
-            for (int u = wave; u < units; u += PERM_WAVES) {
+            const int nsegw = (a.wfn + 63) / 64, wunits = a.wsn * nsegw;
+            for (int u = wave; u < wunits; u += PERM_WAVES) {
                 const int ws = u / nsegw, wf = 64 * (u - ws * nsegw) + lane;
                 if (!inside(c_ws[ws], lim) || wf >= wlen) continue;
                 out[out_s[ws] + (uint32_t)wf] = lds[lw_f[wf] + lw_s[ws]];
@@ -1232,23 +1232,16 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
     }
 }
 
-template <class V, int EPT, bool WTAB>
-void launch_perm_w(const PermArgs& pa, int nseg, dim3 grid, size_t lds, hipStream_t st) {
-    if (nseg == 1) TFH_LAUNCH_TIMED((perm_kernel<V, 1, EPT, WTAB>), grid, dim3(PERM_THREADS), lds, st, pa);
-    else if (nseg == 2) TFH_LAUNCH_TIMED((perm_kernel<V, 2, EPT / 2, WTAB>), grid, dim3(PERM_THREADS), lds, st, pa);
-    else TFH_LAUNCH_TIMED((perm_kernel<V, 4, EPT / 4, WTAB>), grid, dim3(PERM_THREADS), lds, st, pa);
-}
 template <class V, int EPT>
-void launch_perm(const PermArgs& pa, int nseg, bool wtab, dim3 grid, size_t lds, hipStream_t st) {
-    if (wtab) launch_perm_w<V, EPT, true>(pa, nseg, grid, lds, st);
-    else launch_perm_w<V, EPT, false>(pa, nseg, grid, lds, st);
+void launch_perm(const PermArgs& pa, bool wtab, dim3 grid, size_t lds, hipStream_t st) {
+    if (wtab) TFH_LAUNCH_TIMED((perm_kernel<V, EPT, true>), grid, dim3(PERM_THREADS), lds, st, pa);
+    else TFH_LAUNCH_TIMED((perm_kernel<V, EPT, false>), grid, dim3(PERM_THREADS), lds, st, pa);
 }
 
 // A bit-exact move of extents that the shift-and-mask tiles do not fill: two-sided 64 KB tiles.  Returns true when
 // it launched (status holds the outcome).
 struct PermPlan {
     PermArgs pa;
-    int nseg;
     bool wtab;
     size_t lds;
     dim3 grid;
@@ -1274,6 +1267,28 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     int64_t emax = (int64_t)PERM_THREADS * ept;
     std::vector<int64_t> in_tile(na, 0);   // indices of the axis per tile (0: outside the tile)
     int nranged = 0;
+    // the range of an axis of extent n behind `run` elements of whole axes, `room` indices at most: the one that
+    // covers the axis in the fewest wave instructions (64 elements each, a last partial one per run), the longest of those
+    auto best_range = [](int64_t n, int64_t run, int64_t room, bool other_run) {
+        auto cost = [&](int64_t t) {   // wave instructions per element of the axis, both sides
+            double per = (double)((run * t + 63) / 64) / (double)(run * t);
+            if (other_run) per += (double)((t + 63) / 64) / (double)t;   // (the axis is the innermost of the other side)
+            return per * (double)(t * ((n + t - 1) / t));
+        };
+        int64_t best_t = room;
+        double best_cost = cost(room);
+        for (int64_t t = room - 1; t >= std::max<int64_t>(2, room / 4); --t) {
+            const double c = cost(t);
+            if (c < best_cost * 0.999) {
+                best_cost = c;
+                best_t = t;
+            }
+        }
+        const int64_t pieces = (n + best_t - 1) / best_t;   // (equal pieces, when that costs no more)
+        const int64_t even = (n + pieces - 1) / pieces;
+        if (cost(even) <= best_cost) best_t = even;
+        return best_t;
+    };
     // a dense run of up to `cap` elements along one side's order: whole axes, then a range of the next
     auto take_run = [&](int side, int64_t cap, int64_t& E, std::vector<char>& members) {
         const std::vector<int>& ord = side ? out_order : in_order;
@@ -1296,8 +1311,7 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
                 continue;
             }
             if (room >= 2 && nranged < 2) {
-                const int64_t pieces = (axes[i].n + room - 1) / room;
-                in_tile[i] = (axes[i].n + pieces - 1) / pieces;
+                in_tile[i] = best_range(axes[i].n, run, room, axes[i].s[side ^ 1] == 1);
                 members[i] = 1;
                 E *= in_tile[i];
                 run *= in_tile[i];
@@ -1313,8 +1327,9 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     // the room that the registers of a thread leave (a row per wave and register)
     const int64_t rfn = take_run(0, rf_cap, E, in_rf);
     if (rfn < 16) return false;
-    const int nseg = rfn <= 64 ? 1 : (rfn <= 128 ? 2 : 4);
-    emax = std::min<int64_t>(emax, rfn * PERM_WAVES * (ept / nseg));
+    const int64_t nsegs = (rfn + 63) / 64, max_units = (int64_t)PERM_WAVES * ept;
+    if (nsegs > max_units) return false;
+    emax = std::min<int64_t>(emax, rfn * (max_units / nsegs));
     const int64_t wfn = take_run(1, wf_cap, E, in_wf);
     if (wfn < 16) return false;
     // room left (a short output run): more of the input's fastest axes, then whole axes from either side
@@ -1366,7 +1381,7 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
         }
     const int64_t wfn2 = wfn;
     const int64_t rsn = E / rfn, wsn = E / wfn2;
-    if (rsn > PERM_WAVES * (ept / nseg)) return false;
+    if (rsn * nsegs > max_units) return false;
     const int64_t pitch = rfn | 1;
     // LDS position strides: an axis of RF by its place in the run, a row axis by its place among the rows times the pitch
     std::vector<int64_t> lpos(na, 0);
@@ -1415,6 +1430,8 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     pa.wfn = (int32_t)wfn2;
     pa.wsn = (int32_t)wsn;
     pa.pitch = (int32_t)pitch;
+    pa.nsegs = (int32_t)nsegs;
+    pa.units = (int32_t)(rsn * nsegs);
     pa.in = in;
     pa.out = out;
     int64_t ntiles = 1;
@@ -1432,15 +1449,24 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     pa.ntiles = ntiles;
     if (ntiles < 1024 || ntiles >= ((int64_t)1 << 31) - 8) return false;   // (two tiles per block on every CU at least: smaller tensors take smaller tiles)
     const bool wtab = wfn2 > 64 * PERM_WSEG;
-    const size_t lds = (size_t)pitch * rsn * eb + (size_t)(3 * wsn + (wtab ? wfn2 : 0)) * sizeof(uint32_t);
+    const size_t lds = (size_t)pitch * rsn * eb + (size_t)(3 * wsn + wfn2) * sizeof(uint32_t);
     if (lds > 150 * 1024) return false;
-    const size_t per_cu = std::max<size_t>(1, std::min<size_t>(4, (size_t)(160 * 1024) / (lds + 512)));
-    plan.nseg = nseg;
+    // (blocks per CU: by LDS, and three of eight waves by the registers of the kernel held in registers, four of the table's)
+    const size_t per_cu = std::max<size_t>(1, std::min<size_t>(wtab ? 4 : 3, (size_t)(160 * 1024) / (lds + 512)));
     plan.wtab = wtab;
     plan.lds = lds;
     plan.grid = dim3((uint32_t)std::min<int64_t>((ntiles + 7) / 8 * 8, (int64_t)(256 * per_cu)));   // (a multiple of 8: a block stays on its XCD)
+    // the share of the lanes of the wave instructions that move an element: last partial instructions of a run, last
+    // partial ranges of an axis
+    double lanes = ((double)rfn / (double)(64 * nsegs)) * ((double)wfn2 / (double)(64 * ((wfn2 + 63) / 64)));
+    for (int i = 0; i < na; ++i)
+        if (in_tile[i] && in_tile[i] != axes[i].n) lanes *= (double)axes[i].n / (double)(in_tile[i] * ((axes[i].n + in_tile[i] - 1) / in_tile[i]));
+    // the lanes of a write instruction gather along the innermost axis of the write run: an even LDS stride there
+    // has them collide in the banks
+    const int64_t gather = pa.wf.n ? pa.wf.lds[0] : 1;
+    const double banks = (gather & 1) ? 1.0 : ((gather & 3) ? 0.8 : 0.6);
     plan.score = (double)std::min<int64_t>(std::min<int64_t>(rfn, wfn2) * eb, 1024) * (0.5 + 0.5 * (double)E / (double)((int64_t)PERM_THREADS * ept)) *
-                 (wtab ? 0.8 : 1.0);   // (the table-driven write order costs an LDS read per element more)
+                 (wtab ? 0.8 : 1.0) * lanes * banks;   // (the table-driven write order costs an LDS read per element more)
     return true;
 }
 
@@ -1454,7 +1480,7 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
     PermPlan best;
     best.score = 0.0;
     const int64_t rf0 = eb == 16 ? 64 : 128;
-    for (int64_t rf_cap : {rf0, 2 * rf0})
+    for (int64_t rf_cap : {rf0, 4 * rf0, (int64_t)16384})
         for (int64_t wf_cap : {(int64_t)64 * PERM_WSEG, (int64_t)8192}) {
             PermPlan cand;
             std::memset(&cand.pa, 0, sizeof cand.pa);
@@ -1463,10 +1489,8 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
     if (best.score <= 0.0) return false;
     static const bool lds_limit_raised = [] {
         const int cap = 160 * 1024;
-#define TFH_PERM_LDS(V, E, W)                                                                                                  \
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 1, E, W>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);      \
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 2, E / 2, W>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);  \
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, 4, E / 4, W>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+#define TFH_PERM_LDS(V, E, W) \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, E, W>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
         TFH_PERM_LDS(uint32_t, 32, false)
         TFH_PERM_LDS(uint64_t, 16, false)
         TFH_PERM_LDS(double2, 8, false)
@@ -1479,9 +1503,9 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
     (void)lds_limit_raised;
     hipStream_t st = (hipStream_t)stream;
     const int prof = prof_begin(PROF_COPY, stream);
-    if (eb == 4) launch_perm<uint32_t, 32>(best.pa, best.nseg, best.wtab, best.grid, best.lds, st);
-    else if (eb == 8) launch_perm<uint64_t, 16>(best.pa, best.nseg, best.wtab, best.grid, best.lds, st);
-    else launch_perm<double2, 8>(best.pa, best.nseg, best.wtab, best.grid, best.lds, st);
+    if (eb == 4) launch_perm<uint32_t, 32>(best.pa, best.wtab, best.grid, best.lds, st);
+    else if (eb == 8) launch_perm<uint64_t, 16>(best.pa, best.wtab, best.grid, best.lds, st);
+    else launch_perm<double2, 8>(best.pa, best.wtab, best.grid, best.lds, st);
     prof_end(prof, stream);
     status = hip_check(hipGetLastError(), "copy kernel launch");
     return true;
