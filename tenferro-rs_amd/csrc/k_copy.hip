@@ -1086,7 +1086,8 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
     uint32_t* c_ws = lw_s + a.wsn;         // [wsn] its coordinates along the ranged axes
     uint32_t* lw_f = c_ws + a.wsn;         // [wfn] LDS position of a column of the write order
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    for (int i = tid; i < a.wsn; i += PERM_THREADS) perm_entry(a.ws, i, out_s[i], lw_s[i], c_ws[i]);
+    if (!WTAB)
+        for (int i = tid; i < a.wsn; i += PERM_THREADS) perm_entry(a.ws, i, out_s[i], lw_s[i], c_ws[i]);
     for (int i = tid; i < a.wfn; i += PERM_THREADS) {
         uint32_t m, xc;
         perm_entry(a.wf, i, m, lw_f[i], xc);
@@ -1104,6 +1105,18 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         }
     }
     const int my_units = __builtin_amdgcn_readfirstlane(a.units > wave ? (a.units - wave + PERM_WAVES - 1) / PERM_WAVES : 0);
+    // WTAB: the write order in units as well, segment u % nsegw of row u / nsegw, up to 64 per wave (one per lane)
+    uint32_t w_out = 0, w_col = 0x40000000u, w_lrow = 0, w_xc = 0xffffffffu;
+    int my_wunits = 0;
+    if (WTAB) {
+        const int nsegw = (a.wfn + 63) / 64, wunits = a.wsn * nsegw, u = wave + PERM_WAVES * lane;
+        if (u < wunits) {
+            const int ws = u / nsegw, k = u - ws * nsegw;
+            perm_entry(a.ws, ws, w_out, w_lrow, w_xc);
+            w_col = (uint32_t)(64 * k);
+        }
+        my_wunits = __builtin_amdgcn_readfirstlane(wunits > wave ? (wunits - wave + PERM_WAVES - 1) / PERM_WAVES : 0);
+    }
     // (the lane reads below take values that change with the tile -- z is a zero that the compiler cannot see through,
     // a tile index being below 2^31: it would read what stays the same once, ahead of the loop over the tiles, into
     // more scalar registers than there are)
@@ -1191,12 +1204,13 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         }
         V* out = reinterpret_cast<V*>(a.out) + oo;
         if (WTAB) {
-            const int wlen = run_len(a.wf_slot, a.wf_row, a.wfn, lim);
-            const int nsegw = (a.wfn + 63) / 64, wunits = a.wsn * nsegw;
-            for (int u = wave; u < wunits; u += PERM_WAVES) {
-                const int ws = u / nsegw, wf = 64 * (u - ws * nsegw) + lane;
-                if (!inside(c_ws[ws], lim) || wf >= wlen) continue;
-                out[out_s[ws] + (uint32_t)wf] = lds[lw_f[wf] + lw_s[ws]];
+            const uint32_t wlen = (uint32_t)run_len(a.wf_slot, a.wf_row, a.wfn, lim);
+            const bool full = lim == lim_full;
+#pragma unroll 4
+            for (int j = 0; j < my_wunits; ++j) {
+                if (!full && !inside(of_unit(w_xc, j), lim)) continue;
+                const uint32_t col = of_unit(w_col, j) + (uint32_t)lane;
+                if (col < wlen) out[of_unit(w_out, j) + col] = lds[lw_f[col] + of_unit(w_lrow, j)];
             }
         } else if (lim == lim_full) {
             // a segment of the write run at a time: its guard is looked at once per tile, not once per row
@@ -1354,7 +1368,7 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
             ++idle;
         }
     }
-    if (E < 2048) return false;
+    if (E * eb < 16384) return false;   // (a quarter of the registers at least)
     PermArgs& pa = plan.pa;
     std::memset(&pa, 0, sizeof pa);
     pa.x_n[0] = pa.x_n[1] = pa.x_t[0] = pa.x_t[1] = 1;
@@ -1449,6 +1463,7 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     pa.ntiles = ntiles;
     if (ntiles < 1024 || ntiles >= ((int64_t)1 << 31) - 8) return false;   // (two tiles per block on every CU at least: smaller tensors take smaller tiles)
     const bool wtab = wfn2 > 64 * PERM_WSEG;
+    if (wtab && wsn * ((wfn2 + 63) / 64) > PERM_THREADS) return false;   // (a lane of a wave per unit of the write order)
     const size_t lds = (size_t)pitch * rsn * eb + (size_t)(3 * wsn + wfn2) * sizeof(uint32_t);
     if (lds > 150 * 1024) return false;
     // (blocks per CU: by LDS, and three of eight waves by the registers of the kernel held in registers, four of the table's)
@@ -1480,7 +1495,7 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
     PermPlan best;
     best.score = 0.0;
     const int64_t rf0 = eb == 16 ? 64 : 128;
-    for (int64_t rf_cap : {rf0, 4 * rf0, (int64_t)16384})
+    for (int64_t rf_cap : {rf0, 4 * rf0, 16 * rf0, (int64_t)16384})
         for (int64_t wf_cap : {(int64_t)64 * PERM_WSEG, (int64_t)8192}) {
             PermPlan cand;
             std::memset(&cand.pa, 0, sizeof cand.pa);
