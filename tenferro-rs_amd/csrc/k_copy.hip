@@ -12,6 +12,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -1262,7 +1263,7 @@ struct PermPlan {
     double score;   // bytes of the shorter of the two runs, each counted up to 1 KB, and how full the tile is
 };
 // One candidate tiling: a read run of up to rf_cap elements, a write run of up to wf_cap.
-bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, int64_t rf_cap, int64_t wf_cap, PermPlan& plan) {
+bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, int64_t rf_cap, int64_t wf_cap, double gain, PermPlan& plan) {
     int64_t total = 1;
     for (auto& x : axes) total *= x.n;
     if (total < ((int64_t)1 << 20)) return false;
@@ -1283,7 +1284,7 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     int nranged = 0;
     // the range of an axis of extent n behind `run` elements of whole axes, `room` indices at most: the one that
     // covers the axis in the fewest wave instructions (64 elements each, a last partial one per run), the longest of those
-    auto best_range = [](int64_t n, int64_t run, int64_t room, bool other_run) {
+    auto best_range = [gain](int64_t n, int64_t run, int64_t room, bool other_run) {
         auto cost = [&](int64_t t) {   // wave instructions per element of the axis, both sides
             double per = (double)((run * t + 63) / 64) / (double)(run * t);
             if (other_run) per += (double)((t + 63) / 64) / (double)t;   // (the axis is the innermost of the other side)
@@ -1293,7 +1294,7 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
         double best_cost = cost(room);
         for (int64_t t = room - 1; t >= std::max<int64_t>(2, room / 4); --t) {
             const double c = cost(t);
-            if (c < best_cost * 0.999) {
+            if (c < best_cost * gain) {   // (a shorter range makes the tile smaller: `gain` is what it has to save)
                 best_cost = c;
                 best_t = t;
             }
@@ -1449,8 +1450,22 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     pa.in = in;
     pa.out = out;
     int64_t ntiles = 1;
-    for (int i = na - 1; i >= 0; --i) {   // fastest tile index: the innermost axis outside the tile (neighbouring tiles abut)
-        if (in_tile[i] == axes[i].n) continue;
+    // the order of the tiles: fastest the innermost axis of the output that leaves the tile (the tiles that complete
+    // the 128-byte lines at the ends of the write runs follow at once), then the innermost such axis of the input (the
+    // same for the read runs, a few tiles later: tiles in flight on an XCD at the same time share its L2), then the
+    // rest from the output's fast end
+    std::vector<int> g_order;
+    for (int i = na - 1; i >= 0; --i)
+        if (in_tile[i] != axes[i].n) g_order.push_back(i);
+    if (g_order.size() > 2) {
+        size_t pick = 1;
+        for (size_t k = 2; k < g_order.size(); ++k)
+            if (axes[g_order[k]].s[0] < axes[g_order[pick]].s[0]) pick = k;
+        const int moved = g_order[pick];
+        g_order.erase(g_order.begin() + (long)pick);
+        g_order.insert(g_order.begin() + 1, moved);
+    }
+    for (int i : g_order) {
         const int64_t t = in_tile[i] ? in_tile[i] : 1, count = (axes[i].n + t - 1) / t;
         if (pa.ng == MAXG) return false;
         pa.g_count[pa.ng] = count;
@@ -1480,8 +1495,17 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     // has them collide in the banks
     const int64_t gather = pa.wf.n ? pa.wf.lds[0] : 1;
     const double banks = (gather & 1) ? 1.0 : ((gather & 3) ? 0.8 : 0.6);
-    plan.score = (double)std::min<int64_t>(std::min<int64_t>(rfn, wfn2) * eb, 1024) * (0.5 + 0.5 * (double)E / (double)((int64_t)PERM_THREADS * ept)) *
-                 (wtab ? 0.8 : 1.0) * lanes * banks;   // (the table-driven write order costs an LDS read per element more)
+    // What the measurements of odd shapes show, as factors: a read run pays for the partly used 128-byte lines at its
+    // ends (the tiles that follow complete those of a write run); a tile in the table-driven write order reads LDS
+    // once more per element; 4-byte elements are bound by instruction issue and gain from a third block per CU, longer
+    // ones from larger tiles; a single block per CU has nothing to overlap its two phases with; and the tiles of a CU
+    // together should hold the ~96 KB that cover the memory latency.
+    const double r_bytes = (double)(rfn * eb), w_bytes = (double)(wfn2 * eb);
+    const double blocks = (double)per_cu;
+    const double occupancy = per_cu == 1 ? 0.72 : (eb == 4 ? (per_cu == 2 ? 0.92 : 1.0) : (per_cu == 2 ? 1.0 : 0.97));
+    const double in_flight = std::min(1.0, blocks * (double)(E * eb) / 98304.0);
+    plan.score = 1000.0 * (r_bytes / (r_bytes + 128.0)) * (w_bytes / (w_bytes + 32.0)) * (wtab ? 0.85 : 1.0) * lanes * banks * occupancy *
+                 (0.4 + 0.6 * in_flight);
     return true;
 }
 
@@ -1495,12 +1519,44 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
     PermPlan best;
     best.score = 0.0;
     const int64_t rf0 = eb == 16 ? 64 : 128;
-    for (int64_t rf_cap : {rf0, 4 * rf0, 16 * rf0, (int64_t)16384})
-        for (int64_t wf_cap : {(int64_t)64 * PERM_WSEG, (int64_t)8192}) {
-            PermPlan cand;
-            std::memset(&cand.pa, 0, sizeof cand.pa);
-            if (plan_perm_tiles(eb, in, out, axes, rf_cap, wf_cap, cand) && cand.score > best.score * 1.05) best = cand;
-        }
+    // (the winner of an earlier call with the same extents and strides is kept: sixteen candidates cost tens of us)
+    struct Kept {
+        std::vector<int64_t> key;
+        PermPlan plan;
+    };
+    static std::mutex kept_mutex;
+    static std::vector<Kept> kept;
+    std::vector<int64_t> key;
+    key.push_back(eb);
+    for (auto& x : axes) {
+        key.push_back(x.n);
+        key.push_back(x.s[0]);
+        key.push_back(x.s[1]);
+    }
+    bool found = false;
+    {
+        std::lock_guard<std::mutex> lock(kept_mutex);
+        for (auto& k : kept)
+            if (k.key == key) {
+                best = k.plan;
+                found = true;
+                break;
+            }
+    }
+    if (!found) {
+        for (int64_t rf_cap : {rf0, 4 * rf0, 16 * rf0, (int64_t)16384})
+            for (int64_t wf_cap : {(int64_t)64 * PERM_WSEG, (int64_t)8192})
+                for (double gain : {0.999, 0.9}) {
+                    PermPlan cand;
+                    std::memset(&cand.pa, 0, sizeof cand.pa);
+                    if (plan_perm_tiles(eb, in, out, axes, rf_cap, wf_cap, gain, cand) && cand.score > best.score * 1.02) best = cand;
+                }
+        std::lock_guard<std::mutex> lock(kept_mutex);
+        if (kept.size() >= 64) kept.erase(kept.begin());
+        kept.push_back(Kept{key, best});
+    }
+    best.pa.in = in;
+    best.pa.out = out;
     if (best.score <= 0.0) return false;
     static const bool lds_limit_raised = [] {
         const int cap = 160 * 1024;
@@ -1664,8 +1720,22 @@ bool try_table_copy(int eb, const void* in, void* out, std::vector<Axis> axes, c
     ta.out = out;
     ta.E = (int32_t)E;
     int64_t ntiles = 1;
-    for (int i = na - 1; i >= 0; --i) {   // fastest tile index: the innermost axis outside the tile (neighbouring tiles abut)
-        if (in_tile[i] == axes[i].n) continue;
+    // the order of the tiles: fastest the innermost axis of the output that leaves the tile (the tiles that complete
+    // the 128-byte lines at the ends of the write runs follow at once), then the innermost such axis of the input (the
+    // same for the read runs, a few tiles later: tiles in flight on an XCD at the same time share its L2), then the
+    // rest from the output's fast end
+    std::vector<int> g_order;
+    for (int i = na - 1; i >= 0; --i)
+        if (in_tile[i] != axes[i].n) g_order.push_back(i);
+    if (g_order.size() > 2) {
+        size_t pick = 1;
+        for (size_t k = 2; k < g_order.size(); ++k)
+            if (axes[g_order[k]].s[0] < axes[g_order[pick]].s[0]) pick = k;
+        const int moved = g_order[pick];
+        g_order.erase(g_order.begin() + (long)pick);
+        g_order.insert(g_order.begin() + 1, moved);
+    }
+    for (int i : g_order) {
         const int64_t t = in_tile[i] ? in_tile[i] : 1, count = (axes[i].n + t - 1) / t;
         if (ta.ng == MAXG) return false;
         ta.g_count[ta.ng] = count;
