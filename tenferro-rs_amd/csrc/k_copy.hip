@@ -14,6 +14,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "internal.hpp"
@@ -1077,18 +1078,12 @@ constexpr int PERM_WSEG = 8;   // a write run held in registers is up to 8 wave 
 // dense run: batched transposes of small matrices): its LDS positions come from the table in LDS instead of registers,
 // and the (row, segment) pairs of the write order are dealt to the waves one by one.
 template <class V, int EPT, bool WTAB>
-__global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
+__global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 : 4)) perm_kernel(PermArgs a) {   // (waves per SIMD: four blocks per CU of the table's, else three of 4-byte elements, two of longer ones)
     prefetch_kernel_arguments<sizeof(PermArgs)>();
     extern __shared__ __align__(16) unsigned char smem_raw[];
     V* lds = reinterpret_cast<V*>(smem_raw);
-    uint32_t* tab = reinterpret_cast<uint32_t*>(smem_raw + (size_t)a.pitch * a.rsn * sizeof(V));
-    uint32_t* out_s = tab;                 // [wsn] output offset of a row of the write order
-    uint32_t* lw_s = out_s + a.wsn;        // [wsn] its LDS position
-    uint32_t* c_ws = lw_s + a.wsn;         // [wsn] its coordinates along the ranged axes
-    uint32_t* lw_f = c_ws + a.wsn;         // [wfn] LDS position of a column of the write order
+    uint32_t* lw_f = reinterpret_cast<uint32_t*>(smem_raw + (size_t)a.pitch * a.rsn * sizeof(V));   // [wfn] LDS position of a column of the write order
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    if (!WTAB)
-        for (int i = tid; i < a.wsn; i += PERM_THREADS) perm_entry(a.ws, i, out_s[i], lw_s[i], c_ws[i]);
     for (int i = tid; i < a.wfn; i += PERM_THREADS) {
         uint32_t m, xc;
         perm_entry(a.wf, i, m, lw_f[i], xc);
@@ -1106,11 +1101,13 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         }
     }
     const int my_units = __builtin_amdgcn_readfirstlane(a.units > wave ? (a.units - wave + PERM_WAVES - 1) / PERM_WAVES : 0);
-    // WTAB: the write order in units as well, segment u % nsegw of row u / nsegw, up to 64 per wave (one per lane)
+    // The write order the same way, one entry per lane: wave w has rows w, w + 8, ... of the write order (the offset
+    // of the row in the output, its LDS position, its coordinates); WTAB: units of one wave instruction, segment
+    // u % nsegw of row u / nsegw.  64 entries per wave at most.
     uint32_t w_out = 0, w_col = 0x40000000u, w_lrow = 0, w_xc = 0xffffffffu;
-    int my_wunits = 0;
-    if (WTAB) {
-        const int nsegw = (a.wfn + 63) / 64, wunits = a.wsn * nsegw, u = wave + PERM_WAVES * lane;
+    int my_wunits;
+    {
+        const int nsegw = WTAB ? (a.wfn + 63) / 64 : 1, wunits = a.wsn * nsegw, u = wave + PERM_WAVES * lane;
         if (u < wunits) {
             const int ws = u / nsegw, k = u - ws * nsegw;
             perm_entry(a.ws, ws, w_out, w_lrow, w_xc);
@@ -1118,9 +1115,6 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         }
         my_wunits = __builtin_amdgcn_readfirstlane(wunits > wave ? (wunits - wave + PERM_WAVES - 1) / PERM_WAVES : 0);
     }
-    // (the lane reads below take values that change with the tile -- z is a zero that the compiler cannot see through,
-    // a tile index being below 2^31: it would read what stays the same once, ahead of the loop over the tiles, into
-    // more scalar registers than there are)
     auto of_unit = [](uint32_t v, int j) { return (uint32_t)__builtin_amdgcn_readlane((int)v, j); };
     __syncthreads();
     uint32_t lwf[PERM_WSEG];   // LDS position of this thread's columns of the write order
@@ -1152,6 +1146,12 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         if (slot == 0) return full;
         return (int)(slot == 1 ? (lim & 0xffffu) : (lim >> 16)) * row;
     };
+    // (a scalar base and a 32-bit byte offset per lane: the address of a load or store takes no registers of its own)
+    auto at = [](auto* base, uint32_t i) {
+        using T = std::remove_pointer_t<decltype(base)>;
+        using B = std::conditional_t<std::is_const<T>::value, const char, char>;
+        return reinterpret_cast<T*>(reinterpret_cast<B*>(base) + i * (uint32_t)sizeof(T));
+    };
     V regs[EPT];
     // No load is conditional: a column past the end of the run reads the run's last element, a row past the edge of
     // the tensor reads row 0 of the tile, which lies inside at every tile.
@@ -1167,7 +1167,7 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
                 for (int j = g; j < g + 8; ++j) {
                     const V* row = in + of_unit(t_mem, j);
                     const uint32_t col = min(of_unit(t_col, j) + (uint32_t)lane, last);
-                    regs[j] = load_stream<Pack<V, 1>>(row + col).v[0];
+                    regs[j] = load_stream<Pack<V, 1>>(at(row, col)).v[0];
                 }
             }
         }
@@ -1207,11 +1207,27 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
         if (WTAB) {
             const uint32_t wlen = (uint32_t)run_len(a.wf_slot, a.wf_row, a.wfn, lim);
             const bool full = lim == lim_full;
-#pragma unroll 4
-            for (int j = 0; j < my_wunits; ++j) {
+            int j = 0;
+            if (full) {   // (four units at a time: their LDS reads are in flight together)
+                for (; j + 4 <= my_wunits; j += 4) {
+                    uint32_t col[4], pos[4];
+                    V v[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        col[i] = of_unit(w_col, j + i) + (uint32_t)lane;
+                        pos[i] = col[i] < wlen ? lw_f[col[i]] : 0u;
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = lds[pos[i] + of_unit(w_lrow, j + i)];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (col[i] < wlen) *at(out + of_unit(w_out, j + i), col[i]) = v[i];
+                }
+            }
+            for (; j < my_wunits; ++j) {
                 if (!full && !inside(of_unit(w_xc, j), lim)) continue;
                 const uint32_t col = of_unit(w_col, j) + (uint32_t)lane;
-                if (col < wlen) out[of_unit(w_out, j) + col] = lds[lw_f[col] + of_unit(w_lrow, j)];
+                if (col < wlen) *at(out + of_unit(w_out, j), col) = lds[lw_f[col] + of_unit(w_lrow, j)];
             }
         } else if (lim == lim_full) {
             // a segment of the write run at a time: its guard is looked at once per tile, not once per row
@@ -1220,23 +1236,30 @@ __global__ void __launch_bounds__(PERM_THREADS) perm_kernel(PermArgs a) {
                 if (64 * k >= a.wfn) break;
                 if (64 * k + lane < a.wfn) {
                     const uint32_t wcol = (uint32_t)(64 * k + lane);
-                    for (int ws = wave; ws < a.wsn; ws += PERM_WAVES) {
-                        const uint32_t lrow = __builtin_amdgcn_readfirstlane(lw_s[ws]);
-                        V* orow = out + __builtin_amdgcn_readfirstlane(out_s[ws]);
-                        // (a cached store: the next instruction completes the 128-byte lines this one leaves partly written)
-                        orow[wcol] = lds[lwf[k] + lrow];
+                    // (a cached store: the next instruction completes the 128-byte lines this one leaves partly written)
+                    // (a few rows at a time: their LDS reads are in flight together)
+                    constexpr int WU = sizeof(V) == 4 ? 2 : 4;   // (what the registers leave)
+                    int j = 0;
+                    for (; j + WU <= my_wunits; j += WU) {
+                        V v[WU];
+#pragma unroll
+                        for (int i = 0; i < WU; ++i) v[i] = lds[lwf[k] + of_unit(w_lrow, j + i)];
+#pragma unroll
+                        for (int i = 0; i < WU; ++i) *at(out + of_unit(w_out, j + i), wcol) = v[i];
                     }
+                    for (; j < my_wunits; ++j) *at(out + of_unit(w_out, j), wcol) = lds[lwf[k] + of_unit(w_lrow, j)];
                 }
             }
         } else {
             const int wlen = run_len(a.wf_slot, a.wf_row, a.wfn, lim);
-            for (int ws = wave; ws < a.wsn; ws += PERM_WAVES) {
-                if (!inside(c_ws[ws], lim)) continue;
-                const uint32_t lrow = __builtin_amdgcn_readfirstlane(lw_s[ws]);
-                V* orow = out + __builtin_amdgcn_readfirstlane(out_s[ws]);
 #pragma unroll
-                for (int k = 0; k < PERM_WSEG; ++k)
-                    if (64 * k + lane < wlen) orow[(uint32_t)(64 * k + lane)] = lds[lwf[k] + lrow];
+            for (int k = 0; k < PERM_WSEG; ++k) {
+                if (64 * k >= wlen) break;
+                if (64 * k + lane < wlen) {
+                    const uint32_t wcol = (uint32_t)(64 * k + lane);
+                    for (int j = 0; j < my_wunits; ++j)
+                        if (inside(of_unit(w_xc, j), lim)) *at(out + of_unit(w_out, j), wcol) = lds[lwf[k] + of_unit(w_lrow, j)];
+                }
             }
         }
         if (!more) break;
@@ -1478,11 +1501,11 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     pa.ntiles = ntiles;
     if (ntiles < 1024 || ntiles >= ((int64_t)1 << 31) - 8) return false;   // (two tiles per block on every CU at least: smaller tensors take smaller tiles)
     const bool wtab = wfn2 > 64 * PERM_WSEG;
-    if (wtab && wsn * ((wfn2 + 63) / 64) > PERM_THREADS) return false;   // (a lane of a wave per unit of the write order)
-    const size_t lds = (size_t)pitch * rsn * eb + (size_t)(3 * wsn + wfn2) * sizeof(uint32_t);
+    if (wsn * (wtab ? (wfn2 + 63) / 64 : 1) > PERM_THREADS) return false;   // (a lane of a wave per row or unit of the write order)
+    const size_t lds = (size_t)pitch * rsn * eb + (size_t)wfn2 * sizeof(uint32_t);
     if (lds > 150 * 1024) return false;
-    // (blocks per CU: by LDS, and three of eight waves by the registers of the kernel held in registers, four of the table's)
-    const size_t per_cu = std::max<size_t>(1, std::min<size_t>(wtab ? 4 : 3, (size_t)(160 * 1024) / (lds + 512)));
+    // (blocks per CU: by LDS, and by the registers that the kernels are compiled for)
+    const size_t per_cu = std::max<size_t>(1, std::min<size_t>(wtab ? 4 : (eb == 4 ? 3 : 2), (size_t)(160 * 1024) / (lds + 512)));
     plan.wtab = wtab;
     plan.lds = lds;
     plan.grid = dim3((uint32_t)std::min<int64_t>((ntiles + 7) / 8 * 8, (int64_t)(256 * per_cu)));   // (a multiple of 8: a block stays on its XCD)
