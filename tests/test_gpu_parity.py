@@ -3050,6 +3050,46 @@ def test_permute_two_sided_tiles_of_long_odd_extents(tf, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", ALL)
+def test_permute_two_sided_tiles_of_random_shapes_and_views(tf, oracle, dtype):
+    # Seeded random tensors of rank 3..6 with five to twelve million elements and extents off the powers of two, a random
+    # axis order each; every other input is a view that leaves out indices at both ends of two axes (rows that do not
+    # abut, bases that are not aligned).  The tile planner picks among read runs of one row or of the whole tile,
+    # write runs in registers or through the table, ranges that end ragged on one or two axes: whatever it picks, the
+    # move is bit-exact against the oracle on an output that starts as NaN.
+    rng = seeded_rng(143)
+    ran = 0
+    for case in range(8):
+        rank = int(rng.integers(3, 7))
+        target = int(rng.integers(5_000_000, 12_000_000))
+        w = rng.dirichlet(np.ones(rank)) * np.log(target)
+        shape = [max(3, int(round(np.exp(x)))) | 1 for x in w]
+        while int(np.prod(shape)) > 14_000_000:
+            shape[int(np.argmax(shape))] = shape[int(np.argmax(shape))] * 3 // 4 | 1
+        perm = [int(x) for x in rng.permutation(rank)]
+        if perm == list(range(rank)):
+            perm = perm[::-1]
+        full = rand(rng, shape, dtype)
+        a = full
+        if case % 2:
+            cut = [slice(None)] * rank
+            for ax in rng.choice(rank, 2, replace=False):
+                if shape[ax] > 8:
+                    cut[int(ax)] = slice(1, shape[ax] - 2)
+            a = full[tuple(cut)]
+        oshape = [a.shape[p] for p in perm]
+        ref = np.empty(oshape, dtype)
+        oracle.permute(np.ascontiguousarray(a), list(range(rank)), ref, list(perm))
+        assert np.array_equal(ref, np.transpose(a, perm))
+        out = dev(tf, np.full(oshape, np.nan, dtype))
+        plan = tf.HipBackend.plan(dtype, tf.PrimDescriptor.Permute(list(range(rank)), list(perm)), [list(a.shape), oshape])
+        tf.HipBackend.execute(plan, 1.0, [dev(tf, a)], 0.0, out)
+        ran += "perm_kernel" in tf.last_kernel()
+        assert out.to_numpy().tobytes() == ref.tobytes(), (shape, perm, case, tf.last_kernel())
+        del full, a, ref, out
+    assert ran >= 3, ran
+
+
+@pytest.mark.parametrize("dtype", ALL)
 def test_contract_long_operand_against_a_small_one_beyond_the_register_kernel(tf, oracle, dtype):
     # More k (over 32 16-byte chunks) than the register-resident streaming kernel holds against at most 32 real rows, far
     # too thin for tiles: the small operand is staged in LDS as MFMA operands (complex types as the real matrix
