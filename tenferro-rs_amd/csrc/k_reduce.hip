@@ -1421,10 +1421,25 @@ __global__ void __launch_bounds__(THREADS) reduce_run_fold_kernel(RunArgs a, int
     const int op = a.op;
     double re = identity(op), im = 0.0;
     if (o < outputs) {
-        for (int s = g; s < a.nsplit; s += team) {
-            const double* P = a.partial + ((int64_t)s * outputs + o) * NC;
-            re = combine(re, P[0], op);
-            if (CX) im += P[1];
+        // eight partial results in flight at a time (each is a trip to memory), added in the order of the splits
+        for (int s0 = g; s0 < a.nsplit; s0 += 8 * team) {
+            double pr[8], pi[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int s = s0 + i * team;
+                pr[i] = identity(op);
+                pi[i] = 0.0;
+                if (s < a.nsplit) {
+                    const double* P = a.partial + ((int64_t)s * outputs + o) * NC;
+                    pr[i] = P[0];
+                    if (CX) pi[i] = P[1];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                re = combine(re, pr[i], op);
+                if (CX) im += pi[i];
+            }
         }
     }
     if (team > 1) {
