@@ -629,6 +629,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity leg")
     ap.add_argument("--sweep-ops", default="permute,reduce", help="operations of --shape-sweep (permute, reduce)")
     ap.add_argument("--sweep-dtypes", default="f32,f64,c64,c128", help="dtypes of --shape-sweep")
+    ap.add_argument("--sweep-mb", type=int, default=128, help="least size of a tensor of --shape-sweep, in MB")
     ap.add_argument("--shape-sweep", action="store_true",
                     help="permutes and reductions of seeded random tensors (rank 3..7, >= 128 MB, extents that are no powers of two)")
     ap.add_argument("--host-overhead", action="store_true",
@@ -642,7 +643,7 @@ def main():
         sys.exit(2)
     h = Harness(args.steps, args.warmup, not args.no_cpu and not args.host_overhead and not args.shape_sweep)
     if args.shape_sweep:
-        shape_sweep(h, ops=tuple(args.sweep_ops.split(",")), dtypes=tuple(args.sweep_dtypes.split(",")))
+        shape_sweep(h, min_bytes=args.sweep_mb << 20, ops=tuple(args.sweep_ops.split(",")), dtypes=tuple(args.sweep_dtypes.split(",")))
         return
     if args.host_overhead:
         host_overhead(h)

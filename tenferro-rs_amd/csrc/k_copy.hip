@@ -1084,10 +1084,6 @@ __global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 :
     V* lds = reinterpret_cast<V*>(smem_raw);
     uint32_t* lw_f = reinterpret_cast<uint32_t*>(smem_raw + (size_t)a.pitch * a.rsn * sizeof(V));   // [wfn] LDS position of a column of the write order
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    for (int i = tid; i < a.wfn; i += PERM_THREADS) {
-        uint32_t m, xc;
-        perm_entry(a.wf, i, m, lw_f[i], xc);
-    }
     // the unit of register `lane` of this wave, the same in every tile
     uint32_t u_mem = 0, u_col = 0x40000000u, u_lds = 0, u_xc = 0xffffffffu;   // (no unit: past every run, never inside)
     {
@@ -1101,25 +1097,7 @@ __global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 :
         }
     }
     const int my_units = __builtin_amdgcn_readfirstlane(a.units > wave ? (a.units - wave + PERM_WAVES - 1) / PERM_WAVES : 0);
-    // The write order the same way, one entry per lane: wave w has rows w, w + 8, ... of the write order (the offset
-    // of the row in the output, its LDS position, its coordinates); WTAB: units of one wave instruction, segment
-    // u % nsegw of row u / nsegw.  64 entries per wave at most.
-    uint32_t w_out = 0, w_col = 0x40000000u, w_lrow = 0, w_xc = 0xffffffffu;
-    int my_wunits;
-    {
-        const int nsegw = WTAB ? (a.wfn + 63) / 64 : 1, wunits = a.wsn * nsegw, u = wave + PERM_WAVES * lane;
-        if (u < wunits) {
-            const int ws = u / nsegw, k = u - ws * nsegw;
-            perm_entry(a.ws, ws, w_out, w_lrow, w_xc);
-            w_col = (uint32_t)(64 * k);
-        }
-        my_wunits = __builtin_amdgcn_readfirstlane(wunits > wave ? (wunits - wave + PERM_WAVES - 1) / PERM_WAVES : 0);
-    }
     auto of_unit = [](uint32_t v, int j) { return (uint32_t)__builtin_amdgcn_readlane((int)v, j); };
-    __syncthreads();
-    uint32_t lwf[PERM_WSEG];   // LDS position of this thread's columns of the write order
-#pragma unroll
-    for (int k = 0; k < PERM_WSEG; ++k) lwf[k] = (!WTAB && 64 * k + lane < a.wfn) ? lw_f[64 * k + lane] : 0u;
     auto origin = [&](uint32_t tile, int64_t& oi, int64_t& oo, uint32_t& lim) {   // (tile counts are below 2^31)
         oi = oo = 0;
         int l[2] = {a.x_t[0], a.x_t[1]};
@@ -1181,6 +1159,29 @@ __global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 :
     uint32_t lim;
     origin(tile_of(slot), oi, oo, lim);
     load(oi, lim, tile_of(slot) >> 31);
+    // (what the write phase needs is computed while the first tile's loads are in flight)
+    for (int i = tid; i < a.wfn; i += PERM_THREADS) {
+        uint32_t m, xc;
+        perm_entry(a.wf, i, m, lw_f[i], xc);
+    }
+    // The write order the same way, one entry per lane: wave w has rows w, w + 8, ... of the write order (the offset
+    // of the row in the output, its LDS position, its coordinates); WTAB: units of one wave instruction, segment
+    // u % nsegw of row u / nsegw.  64 entries per wave at most.
+    uint32_t w_out = 0, w_col = 0x40000000u, w_lrow = 0, w_xc = 0xffffffffu;
+    int my_wunits;
+    {
+        const int nsegw = WTAB ? (a.wfn + 63) / 64 : 1, wunits = a.wsn * nsegw, u = wave + PERM_WAVES * lane;
+        if (u < wunits) {
+            const int ws = u / nsegw, k = u - ws * nsegw;
+            perm_entry(a.ws, ws, w_out, w_lrow, w_xc);
+            w_col = (uint32_t)(64 * k);
+        }
+        my_wunits = __builtin_amdgcn_readfirstlane(wunits > wave ? (wunits - wave + PERM_WAVES - 1) / PERM_WAVES : 0);
+    }
+    __syncthreads();
+    uint32_t lwf[PERM_WSEG];   // LDS position of this thread's columns of the write order
+#pragma unroll
+    for (int k = 0; k < PERM_WSEG; ++k) lwf[k] = (!WTAB && 64 * k + lane < a.wfn) ? lw_f[64 * k + lane] : 0u;
     for (;;) {
         {
             const uint32_t z = tile_of(slot) >> 31, t_col = u_col | z, t_lds = u_lds | z;
@@ -1289,7 +1290,7 @@ struct PermPlan {
 bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, int64_t rf_cap, int64_t wf_cap, double gain, PermPlan& plan) {
     int64_t total = 1;
     for (auto& x : axes) total *= x.n;
-    if (total < ((int64_t)1 << 20)) return false;
+    if (total * eb < ((int64_t)8 << 20)) return false;   // (8 MB: below, the table tiles of 2048 elements measure the same or better)
     std::stable_sort(axes.begin(), axes.end(), [](const Axis& x, const Axis& y) { return std::llabs(x.s[1]) > std::llabs(y.s[1]); });
     fuse_axes(axes, 2);
     const int na = (int)axes.size();
@@ -1302,7 +1303,12 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     std::stable_sort(out_order.begin(), out_order.end(), [&](int x, int y) { return axes[x].s[1] < axes[y].s[1]; });
     if (axes[in_order[0]].s[0] != 1 || axes[out_order[0]].s[1] != 1) return false;
     const int ept = eb == 4 ? 32 : (eb == 8 ? 16 : 8);   // the registers of 512 threads hold a 64 KB tile
-    int64_t emax = (int64_t)PERM_THREADS * ept;
+    // (a tensor too small to give every block that fits on the chip a tile of 64 KB takes smaller ones, down to
+    // 16 KB: three quarters of the blocks, since the ragged ranges of the axes add tiles; half of them, or a balance
+    // term in the score for a few tiles more than blocks, measured no better)
+    const int64_t resident = 256 * (eb == 4 ? 3 : 2);
+    const int64_t cap_bytes = std::min<int64_t>((int64_t)PERM_THREADS * ept * eb, std::max<int64_t>(16384, total * eb * 4 / (resident * 3)));
+    int64_t emax = cap_bytes / eb;
     std::vector<int64_t> in_tile(na, 0);   // indices of the axis per tile (0: outside the tile)
     int nranged = 0;
     // the range of an axis of extent n behind `run` elements of whole axes, `room` indices at most: the one that
@@ -1392,7 +1398,7 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
             ++idle;
         }
     }
-    if (E * eb < 16384) return false;   // (a quarter of the registers at least)
+    if (E * eb * 4 < cap_bytes) return false;   // (a quarter of the tile at least)
     PermArgs& pa = plan.pa;
     std::memset(&pa, 0, sizeof pa);
     pa.x_n[0] = pa.x_n[1] = pa.x_t[0] = pa.x_t[1] = 1;
@@ -1499,7 +1505,7 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
         ntiles *= count;
     }
     pa.ntiles = ntiles;
-    if (ntiles < 1024 || ntiles >= ((int64_t)1 << 31) - 8) return false;   // (two tiles per block on every CU at least: smaller tensors take smaller tiles)
+    if (ntiles < 256 || ntiles >= ((int64_t)1 << 31) - 8) return false;   // (a tile per CU at least)
     const bool wtab = wfn2 > 64 * PERM_WSEG;
     if (wsn * (wtab ? (wfn2 + 63) / 64 : 1) > PERM_THREADS) return false;   // (a lane of a wave per row or unit of the write order)
     const size_t lds = (size_t)pitch * rsn * eb + (size_t)wfn2 * sizeof(uint32_t);
@@ -1542,7 +1548,7 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
     PermPlan best;
     best.score = 0.0;
     const int64_t rf0 = eb == 16 ? 64 : 128;
-    // (the winner of an earlier call with the same extents and strides is kept: sixteen candidates cost tens of us)
+    // (the winner of an earlier call with the same extents and strides is kept: the candidates cost tens of us)
     struct Kept {
         std::vector<int64_t> key;
         PermPlan plan;

@@ -1570,7 +1570,7 @@ def test_permute_extents_with_divisor_tiles(tf, oracle, dtype):
             if fast:
                 assert copy_kernel_is_fast(tf.last_kernel()), (shape, perm, tf.last_kernel())
             else:
-                assert "tabcopy_kernel" in tf.last_kernel() or not copy_kernel_is_fast(tf.last_kernel()), (shape, perm, tf.last_kernel())
+                assert "tabcopy_kernel" in tf.last_kernel() or "perm_kernel" in tf.last_kernel() or not copy_kernel_is_fast(tf.last_kernel()), (shape, perm, tf.last_kernel())
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex128])
@@ -2806,11 +2806,11 @@ def test_permute_tensors_of_many_short_axes(tf):
             assert out.to_numpy().tobytes() == np.ascontiguousarray(x.transpose(perm)).tobytes(), (shape, perm, dtype, tf.last_kernel())
     assert used >= 14, used            # most of these shapes take the table-driven or the two-sided tiles, on both calls
     # a slice of a larger tensor: strides of the operand are not those of a dense tensor
-    big = rand(rng, (4,) + (3,) * 12, np.float64)
+    big = rand(rng, (4,) + (3,) * 11, np.float64)      # (under 4 MB: the table tiles' size)
     x = big[1]
-    perm = tuple(reversed(range(12)))
-    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute(list(range(12)), list(perm)), [[3] * 12, [3] * 12])
-    out = dev(tf, np.zeros((3,) * 12))
+    perm = tuple(reversed(range(11)))
+    plan = tf.HipBackend.plan(np.float64, tf.PrimDescriptor.Permute(list(range(11)), list(perm)), [[3] * 11, [3] * 11])
+    out = dev(tf, np.zeros((3,) * 11))
     tf.HipBackend.execute(plan, 1.0, [dev(tf, x)], 0.0, out)
     assert out.to_numpy().tobytes() == np.ascontiguousarray(x.transpose(perm)).tobytes()
     assert tf.lib().tfh_release_workspaces() == 0
@@ -2818,6 +2818,7 @@ def test_permute_tensors_of_many_short_axes(tf):
     assert "tabcopy_kernel" in tf.last_kernel() and out.to_numpy().tobytes() == np.ascontiguousarray(x.transpose(perm)).tobytes()
     # alpha/beta and conj keep the masked tiles (the table path moves raw bits only)
     z = rand(rng, (3,) * 12, np.complex128)
+    perm = tuple(reversed(range(12)))
     got = dev(tf, np.zeros((3,) * 12, np.complex128))
     tf.HipBackend.execute(tf.HipBackend.plan(np.complex128, tf.PrimDescriptor.Permute(list(range(12)), list(perm)), [[3] * 12, [3] * 12]), 2.0, [dev(tf, z)], 0.0, got)
     assert "tabcopy_kernel" not in tf.last_kernel() and np.array_equal(got.to_numpy(), 2.0 * z.transpose(perm))
