@@ -707,6 +707,23 @@ bool try_fast_reduce(int dtype, const void* a, void* c, std::vector<Axis> kept, 
         bits -= t;
     }
     if (bits != 0) return false;
+    {
+        // the contiguous bytes that a tile reads at a stretch: a tile that takes two reals of every row of 66 (an odd
+        // extent behind a factor of two) uses 8 bytes of every 64 fetched -- the dense-run kernels take such shapes
+        int64_t run = 1;
+        bool cut = false;   // the stretch ends inside an axis that goes on in memory
+        for (size_t i = 0; i < all.size(); ++i) {
+            const Ax& x = all[i];
+            const int64_t mul = i == 0 ? vec : 1;
+            if (std::llabs(x.a.s[0]) != run) break;
+            run *= ((int64_t)1 << x.tl) * mul;
+            if (((int64_t)1 << x.tl) * mul != x.a.n) {
+                cut = true;
+                break;
+            }
+        }
+        if (cut && run * rbytes < 64) return false;
+    }
     int64_t blocks = 1, r_total = 1;
     for (size_t i = 0; i < all.size(); ++i) {
         const Ax& x = all[i];
