@@ -1598,7 +1598,10 @@ bool try_run_reduce(int dtype, const void* a, void* c, const std::vector<Axis>& 
             else ch.kept_blocks *= outside, kept_in_tile *= inside;
         }
         ch.nsplit = 1;
-        if (ch.kept_blocks < 768 && walk >= 2 * minper) {
+        // (a walk of three batches of loads or fewer on 64 blocks or more stays one launch: the second launch of a
+        // split walk costs 4-5 us, as much as those batches)
+        const bool short_walk = ch.kept_blocks >= 64 && walk * ch.tile_reals * (dbl ? 8 : 4) <= 98304;
+        if (ch.kept_blocks < 768 && walk >= 2 * minper && !short_walk) {
             const int64_t outputs = ch.kept_blocks * kept_in_tile;
             ch.nsplit = std::min<int64_t>(target / ch.kept_blocks, walk / minper);
             ch.nsplit = std::min<int64_t>(ch.nsplit, std::max<int64_t>(1, total / (outputs * 48)));
