@@ -1043,6 +1043,7 @@ struct PermArgs {
     PermGroup rs, ws, wf;      // rows of the read order (input strides), rows of the write order (output strides), write columns
     int32_t rfn, rsn, wfn, wsn, pitch;
     int32_t nsegs, units;      // wave instructions per row of the read order, and in a tile
+    int32_t conj;              // complex elements: the sign of the imaginary part is flipped on the way (the only change to the bits)
     int32_t rf_slot, wf_slot;  // the ranged axis that is last in RF / WF (0: none), and the elements per index of it
     int32_t rf_row, wf_row;
     int32_t x_n[2], x_t[2];    // extent of a ranged axis and its indices per tile (1, 1 when there is none)
@@ -1130,6 +1131,17 @@ __global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 :
         using B = std::conditional_t<std::is_const<T>::value, const char, char>;
         return reinterpret_cast<T*>(reinterpret_cast<B*>(base) + i * (uint32_t)sizeof(T));
     };
+    // conjugation: the top bit of the last 32-bit word of a complex element (zero otherwise: a move of the bits)
+    const uint32_t sign = (sizeof(V) >= 8 && a.conj) ? 0x80000000u : 0u;
+    auto flip = [&](V v) {
+        if constexpr (sizeof(V) >= 8) {
+            uint32_t w[sizeof(V) / 4];
+            __builtin_memcpy(w, &v, sizeof(V));
+            w[sizeof(V) / 4 - 1] ^= sign;
+            __builtin_memcpy(&v, w, sizeof(V));
+        }
+        return v;
+    };
     V regs[EPT];
     // No load is conditional: a column past the end of the run reads the run's last element, a row past the edge of
     // the tensor reads row 0 of the tile, which lies inside at every tile.
@@ -1190,7 +1202,7 @@ __global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 :
                 if (g < my_units) {
 #pragma unroll
                     for (int j = g; j < g + 8; ++j)
-                        if (of_unit(t_col, j) + (uint32_t)lane < (uint32_t)a.rfn) lds[of_unit(t_lds, j) + (uint32_t)lane] = regs[j];
+                        if (of_unit(t_col, j) + (uint32_t)lane < (uint32_t)a.rfn) lds[of_unit(t_lds, j) + (uint32_t)lane] = flip(regs[j]);
                 }
             }
         }
@@ -1540,7 +1552,7 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
 
 // A bit-exact move of extents that the shift-and-mask tiles do not fill: two-sided 64 KB tiles.  Returns true when
 // it launched (status holds the outcome).
-bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, void* stream, int32_t& status) {
+bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, bool conj, void* stream, int32_t& status) {
     status = TFH_OK;
     // candidates: the usual read run (two wave instructions wide, one for 16-byte elements) or one twice as long (an
     // innermost axis that both sides share, with one long axis behind it: the read run is all that can grow), a write
@@ -1586,6 +1598,7 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, v
     }
     best.pa.in = in;
     best.pa.out = out;
+    best.pa.conj = conj ? 1 : 0;
     if (best.score <= 0.0) return false;
     static const bool lds_limit_raised = [] {
         const int cap = 160 * 1024;
@@ -1817,9 +1830,13 @@ int32_t launch_copy(int dtype, const void* in, void* out, std::vector<Axis> axes
     const bool vin = tp.vec_in && aligned(in, 16), vout = tp.vec_out && aligned(out, 16);
     const bool cx = is_complex(dtype);
     const bool raw = alpha.is_one() && beta.is_zero() && !(conj && cx);
+    if (!raw && alpha.is_one() && beta.is_zero() && !tp.all_full) {   // a conjugating move: the two-sided tiles flip the sign on the way
+        int32_t st_tab = TFH_OK;
+        if (try_perm_tiles(eb, in, out, axes, true, stream, st_tab)) return st_tab;
+    }
     if (raw) {
         int32_t st_tab = TFH_OK;
-        if (!tp.all_full && try_perm_tiles(eb, in, out, axes, stream, st_tab)) return st_tab;
+        if (!tp.all_full && try_perm_tiles(eb, in, out, axes, false, stream, st_tab)) return st_tab;
         if (try_table_copy(eb, in, out, axes, tp, stream, st_tab)) return st_tab;
         // Large tiles.  When the rows a tile touches on one side lie far apart (an axis that is contiguous on one side
         // and the slowest on the other: strides of megabytes inside every tile), 512-byte runs on that side cost 10-17 %

@@ -3058,7 +3058,7 @@ def test_permute_two_sided_tiles_of_random_shapes_and_views(tf, oracle, dtype):
     # write runs in registers or through the table, ranges that end ragged on one or two axes: whatever it picks, the
     # move is bit-exact against the oracle on an output that starts as NaN.
     rng = seeded_rng(143)
-    ran = 0
+    ran = conj_ran = 0
     for case in range(8):
         rank = int(rng.integers(3, 7))
         target = int(rng.integers(5_000_000, 12_000_000))
@@ -3086,8 +3086,15 @@ def test_permute_two_sided_tiles_of_random_shapes_and_views(tf, oracle, dtype):
         tf.HipBackend.execute(plan, 1.0, [dev(tf, a)], 0.0, out)
         ran += "perm_kernel" in tf.last_kernel()
         assert out.to_numpy().tobytes() == ref.tobytes(), (shape, perm, case, tf.last_kernel())
+        if np.issubdtype(dtype, np.complexfloating) and case % 3 == 0:
+            # the same move of an operand behind the conjugate-on-load flag: only the sign of the imaginary parts changes
+            out = dev(tf, np.full(oshape, np.nan, dtype))
+            tf.HipBackend.execute(plan, 1.0, [dev(tf, a).conj_on_load()], 0.0, out)
+            conj_ran += "perm_kernel" in tf.last_kernel()
+            assert out.to_numpy().tobytes() == np.conj(ref).tobytes(), (shape, perm, case, tf.last_kernel())
         del full, a, ref, out
     assert ran >= 3, ran
+    assert conj_ran >= 1 or not np.issubdtype(dtype, np.complexfloating), conj_ran
 
 
 @pytest.mark.parametrize("dtype", ALL)
