@@ -129,7 +129,9 @@ __global__ void __launch_bounds__(THIN_THREADS, 2) gemm_thin_kernel(ThinArgs a) 
         for (int t = 0; t < THIN_GROUP; ++t) {
             const int c = 4 * (grp * THIN_GROUP + t) + g;
             const int cc = c < chunks ? c : chunks - 1;
-            dst[t] = __builtin_nontemporal_load(reinterpret_cast<const Chunk*>(row) + cc);
+            // (a cached load: an instruction takes 64 bytes of each of 16 rows, the next one the other half of the same
+            // 128-byte lines -- a non-temporal load fetched them twice: 16 rows of 4 KB 964 -> 847 us)
+            dst[t] = *(reinterpret_cast<const Chunk*>(row) + cc);
         }
     };
     Acc acc[MB];
@@ -170,6 +172,30 @@ __global__ void __launch_bounds__(THIN_THREADS, 2) gemm_thin_kernel(ThinArgs a) 
         const int nn = (int)(a.nl - n0 < THIN_UNIT ? a.nl - n0 : THIN_UNIT);
         R* C = reinterpret_cast<R*>(a.C);
         const int count = a.ms * THIN_UNIT;            // elements of the unit
+        if (!a.use_beta) {
+            // A fixed number of unconditional stores (lanes past the unit's elements or rows past the end of L write
+            // the last element again): the waits for the loads that were issued before them can then count them,
+            // instead of waiting for every store of the wave to be acknowledged.
+            constexpr int SI = MB * 16 * THIN_UNIT / 64;
+#pragma unroll
+            for (int it = 0; it < SI; ++it) {
+                int e = lane + 64 * it;
+                e = e < count ? e : count - 1;
+                const int m = a.m_fast ? e % a.ms : e / THIN_UNIT;
+                int nl = a.m_fast ? e / a.ms : e % THIN_UNIT;
+                nl = nl < nn ? nl : nn - 1;
+                R* dst = C + ((int64_t)m * a.cs_m + (n0 + nl) * a.cs_n) * nc;
+                if (a.cx) {
+                    const double re = tile[nl * TP + 2 * m], im = tile[nl * TP + 2 * m + 1];
+                    dst[0] = (R)(a.alpha_re * re - a.alpha_im * im);
+                    dst[1] = (R)(a.alpha_re * im + a.alpha_im * re);
+                } else {
+                    dst[0] = (R)(a.alpha_re * (double)tile[nl * TP + m]);
+                }
+            }
+            thin_wave_sync();
+            return;
+        }
         for (int e = lane; e < count; e += 64) {
             // m fastest when C is contiguous along m, n fastest otherwise
             const int m = a.m_fast ? e % a.ms : e / THIN_UNIT, nl = a.m_fast ? e / a.ms : e % THIN_UNIT;
@@ -201,12 +227,15 @@ __global__ void __launch_bounds__(THIN_THREADS, 2) gemm_thin_kernel(ThinArgs a) 
             u_mm += nwaves;
         }
     };
+    // Every pass issues its loads whether or not a set is left (past the wave's last unit the loads read the last row
+    // of L again): with a fixed number of loads between a set's issue and its use the wait for it can leave the
+    // newer ones in flight; a conditional issue makes every wait one for all of them, and loads and MFMAs take turns.
     issue(buf[0]);
     for (int64_t f = 0; f < total; f += 2) {
-        if (f + 1 < total) issue(buf[1]);
+        issue(buf[1]);
         step(buf[0]);
         if (f + 1 >= total) break;
-        if (f + 2 < total) issue(buf[0]);
+        issue(buf[0]);
         step(buf[1]);
     }
 }
