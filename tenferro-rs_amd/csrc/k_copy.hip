@@ -1078,7 +1078,15 @@ constexpr int PERM_WSEG = 8;   // a write run held in registers is up to 8 wave 
 // WTAB: the write run is longer than PERM_WSEG wave instructions (a short innermost axis of the output inside a longer
 // dense run: batched transposes of small matrices): its LDS positions come from the table in LDS instead of registers,
 // and the (row, segment) pairs of the write order are dealt to the waves one by one.
-template <class V, int EPT, bool WTAB>
+// W: elements per lane of a read instruction (2 for 8-byte elements when the read run is longer than one instruction
+// of single elements: half the load and LDS-write instructions; the pair starts at any element, so its load is aligned
+// to the element only and its two LDS writes are one ds_write2).
+template <class V> struct PermPair;
+template <> struct PermPair<uint32_t> { typedef uint32_t type __attribute__((ext_vector_type(2), aligned(4))); };
+template <> struct PermPair<uint64_t> { typedef uint64_t type __attribute__((ext_vector_type(2), aligned(8))); };
+template <> struct PermPair<double2> { typedef uint64_t type __attribute__((ext_vector_type(2), aligned(8))); };   // (never used: W = 1)
+
+template <class V, int EPT, bool WTAB, int W = 1>
 __global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 : 4)) perm_kernel(PermArgs a) {   // (waves per SIMD: four blocks per CU of the table's, else three of 4-byte elements, two of longer ones)
     prefetch_kernel_arguments<sizeof(PermArgs)>();
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -1089,11 +1097,11 @@ __global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 :
     uint32_t u_mem = 0, u_col = 0x40000000u, u_lds = 0, u_xc = 0xffffffffu;   // (no unit: past every run, never inside)
     {
         const int u = wave + PERM_WAVES * lane;
-        if (lane < EPT && u < a.units) {
+        if (lane < EPT / W && u < a.units) {
             const int r = u / a.nsegs, k = u - r * a.nsegs;
             uint32_t l;
             perm_entry(a.rs, r, u_mem, l, u_xc);
-            u_col = (uint32_t)(64 * k);
+            u_col = (uint32_t)(64 * W * k);
             u_lds = l + u_col;
         }
     }
@@ -1151,13 +1159,23 @@ __global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 :
         // per unit, in the lane of its register: the row's offset at this tile, and the first column
         const uint32_t t_mem = inside(u_xc, lim) ? u_mem : 0u, t_col = u_col | z;
 #pragma unroll
-        for (int g = 0; g < EPT; g += 8) {
+        for (int g = 0; g < EPT / W; g += 8) {
             if (g < my_units) {   // (eight units at a time: the last ones of a wave may be none, and read row 0)
 #pragma unroll
                 for (int j = g; j < g + 8; ++j) {
                     const V* row = in + of_unit(t_mem, j);
-                    const uint32_t col = min(of_unit(t_col, j) + (uint32_t)lane, last);
-                    regs[j] = load_stream<Pack<V, 1>>(at(row, col)).v[0];
+                    if constexpr (W == 1) {
+                        const uint32_t col = min(of_unit(t_col, j) + (uint32_t)lane, last);
+                        regs[j] = load_stream<Pack<V, 1>>(at(row, col)).v[0];
+                    } else {
+                        // a pair that starts at the run's last element is read one element earlier (its second
+                        // element is the one wanted); runs are 16 elements and more
+                        typedef typename PermPair<V>::type Pair;
+                        const uint32_t col = of_unit(t_col, j) + 2u * (uint32_t)lane, from = min(col, last - 1u);
+                        const Pair pr = __builtin_nontemporal_load(reinterpret_cast<const Pair*>(at(row, from)));
+                        regs[2 * j] = col > from ? (V)pr[1] : (V)pr[0];
+                        regs[2 * j + 1] = (V)pr[1];
+                    }
                 }
             }
         }
@@ -1198,11 +1216,22 @@ __global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 :
         {
             const uint32_t z = tile_of(slot) >> 31, t_col = u_col | z, t_lds = u_lds | z;
 #pragma unroll
-            for (int g = 0; g < EPT; g += 8) {
+            for (int g = 0; g < EPT / W; g += 8) {
                 if (g < my_units) {
 #pragma unroll
-                    for (int j = g; j < g + 8; ++j)
-                        if (of_unit(t_col, j) + (uint32_t)lane < (uint32_t)a.rfn) lds[of_unit(t_lds, j) + (uint32_t)lane] = flip(regs[j]);
+                    for (int j = g; j < g + 8; ++j) {
+                        if constexpr (W == 1) {
+                            if (of_unit(t_col, j) + (uint32_t)lane < (uint32_t)a.rfn) lds[of_unit(t_lds, j) + (uint32_t)lane] = flip(regs[j]);
+                        } else {
+                            const uint32_t col = of_unit(t_col, j) + 2u * (uint32_t)lane, pos = of_unit(t_lds, j) + 2u * (uint32_t)lane;
+                            if (col + 1u < (uint32_t)a.rfn) {
+                                lds[pos] = flip(regs[2 * j]);
+                                lds[pos + 1u] = flip(regs[2 * j + 1]);
+                            } else if (col < (uint32_t)a.rfn) {
+                                lds[pos] = flip(regs[2 * j]);
+                            }
+                        }
+                    }
                 }
             }
         }
@@ -1284,7 +1313,14 @@ __global__ void __launch_bounds__(PERM_THREADS, WTAB ? 8 : (sizeof(V) == 4 ? 6 :
 }
 
 template <class V, int EPT>
-void launch_perm(const PermArgs& pa, bool wtab, dim3 grid, size_t lds, hipStream_t st) {
+void launch_perm(const PermArgs& pa, bool wtab, int w, dim3 grid, size_t lds, hipStream_t st) {
+    if constexpr (sizeof(V) <= 8) {
+        if (w == 2) {
+            if (wtab) TFH_LAUNCH_TIMED((perm_kernel<V, EPT, true, 2>), grid, dim3(PERM_THREADS), lds, st, pa);
+            else TFH_LAUNCH_TIMED((perm_kernel<V, EPT, false, 2>), grid, dim3(PERM_THREADS), lds, st, pa);
+            return;
+        }
+    }
     if (wtab) TFH_LAUNCH_TIMED((perm_kernel<V, EPT, true>), grid, dim3(PERM_THREADS), lds, st, pa);
     else TFH_LAUNCH_TIMED((perm_kernel<V, EPT, false>), grid, dim3(PERM_THREADS), lds, st, pa);
 }
@@ -1294,6 +1330,7 @@ void launch_perm(const PermArgs& pa, bool wtab, dim3 grid, size_t lds, hipStream
 struct PermPlan {
     PermArgs pa;
     bool wtab;
+    int w;          // elements per lane of a read instruction
     size_t lds;
     dim3 grid;
     double score;   // bytes of the shorter of the two runs, each counted up to 1 KB, and how full the tile is
@@ -1488,6 +1525,22 @@ bool plan_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, 
     pa.pitch = (int32_t)pitch;
     pa.nsegs = (int32_t)nsegs;
     pa.units = (int32_t)(rsn * nsegs);
+    // pairs per lane in the read phase: a read run of more than one instruction of single elements, rows that still
+    // fit the registers, and no tile whose read run is a single element (the pair would reach past it)
+    plan.w = 1;
+    {
+        const int64_t nsegs2 = (rfn + 127) / 128;
+        bool short_run = false;
+        if (pa.rf_slot) {
+            const int64_t n = pa.x_n[pa.rf_slot - 1], t = pa.x_t[pa.rf_slot - 1];
+            short_run = (n % t) * pa.rf_row == 1;
+        }
+        if (eb == 8 && rfn > 64 && rsn * nsegs2 <= max_units / 2 && !short_run) {   // (4-byte elements measured 2 points slower with pairs, 8-byte ones 3 faster)
+            plan.w = 2;
+            pa.nsegs = (int32_t)nsegs2;
+            pa.units = (int32_t)(rsn * nsegs2);
+        }
+    }
     pa.in = in;
     pa.out = out;
     int64_t ntiles = 1;
@@ -1603,7 +1656,9 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, b
     static const bool lds_limit_raised = [] {
         const int cap = 160 * 1024;
 #define TFH_PERM_LDS(V, E, W) \
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, E, W>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, E, W>), hipFuncAttributeMaxDynamicSharedMemorySize, cap); \
+    if constexpr (sizeof(V) <= 8) \
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&perm_kernel<V, E, W, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, cap);
         TFH_PERM_LDS(uint32_t, 32, false)
         TFH_PERM_LDS(uint64_t, 16, false)
         TFH_PERM_LDS(double2, 8, false)
@@ -1616,9 +1671,9 @@ bool try_perm_tiles(int eb, const void* in, void* out, std::vector<Axis> axes, b
     (void)lds_limit_raised;
     hipStream_t st = (hipStream_t)stream;
     const int prof = prof_begin(PROF_COPY, stream);
-    if (eb == 4) launch_perm<uint32_t, 32>(best.pa, best.wtab, best.grid, best.lds, st);
-    else if (eb == 8) launch_perm<uint64_t, 16>(best.pa, best.wtab, best.grid, best.lds, st);
-    else launch_perm<double2, 8>(best.pa, best.wtab, best.grid, best.lds, st);
+    if (eb == 4) launch_perm<uint32_t, 32>(best.pa, best.wtab, best.w, best.grid, best.lds, st);
+    else if (eb == 8) launch_perm<uint64_t, 16>(best.pa, best.wtab, best.w, best.grid, best.lds, st);
+    else launch_perm<double2, 8>(best.pa, best.wtab, best.w, best.grid, best.lds, st);
     prof_end(prof, stream);
     status = hip_check(hipGetLastError(), "copy kernel launch");
     return true;
